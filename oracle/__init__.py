@@ -1,0 +1,40 @@
+"""CPU oracle for the GRPO logprob + loss hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing under ``rl_amd/`` may import this package;
+it is used by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` as the checker / reported CPU baseline.
+
+Every function is a plain-PyTorch (CPU, fp32 unless stated) restatement of the
+arithmetic of the reference implementation, cited per function as
+``<reference file>:<lines>`` relative to the NeMo-RL source tree.  The
+primitives the reference relies on (``log_softmax``, ``gather``, ``sort``,
+``cumsum``, ``topk``, ``matmul``) are PyTorch's own, so torch on the CPU is
+the legitimate ground truth for them.
+
+Pinning status (what fixes each function besides its own text):
+
+* ``logprob.*``            pinned: textbook ``log_softmax(x).gather`` identity,
+                           autograd of that form, brute force on tiny vocab,
+                           chunk == no-chunk, packed == per-sequence.
+* ``sampling.*``           pinned by properties (outside top-k is -inf, kept
+                           probabilities reach top_p, keep_mask == ~isinf) and
+                           brute force.  PARITY UNPINNED for which of several
+                           exactly tied values at the top-p boundary survives
+                           (the reference sorts unstably); this oracle keeps
+                           torch's stable ascending order.
+* ``loss.calculate_kl``    pinned: golden vectors of the reference's unit tests.
+* ``loss.masked_mean``     pinned: closed form.
+* ``loss.clipped_pg_loss`` pinned: closed-form losses of the reference's unit
+                           tests (PPO clip, REINFORCE, on-policy, CISPO, KL,
+                           IS/TIS/ICE-POP/seq-mask-tis, dual clip, GSPO).
+                           PARITY UNPINNED for the diagnostics the reference
+                           never tests numerically (token_mult_prob_error,
+                           gen_kl_error, policy_kl_error, js_divergence_error,
+                           sampling_importance_ratio, probs_ratio*): restated
+                           from the source text and checked against
+                           independent float64 formulas only.
+* ``advantage.*``          pinned: golden vectors of the reference's unit tests.
+* ``lmhead.*``             PARITY UNPINNED against the reference (its only test
+                           needs Megatron, two GPUs and a model download);
+                           pinned here to ``logprob(hidden @ W.T)`` in fp32.
+"""

@@ -1,0 +1,80 @@
+"""Pins the advantage oracle to the reference's golden vectors (CPU only)."""
+
+import pytest
+import torch
+
+from oracle import advantage as A
+from helpers import load_golden
+
+BASE = load_golden("baseline_cases.json")
+ADV = load_golden("grpo_adv_cases.json")
+
+
+@pytest.mark.parametrize("case", BASE["cases"], ids=[c["name"] for c in BASE["cases"]])
+def test_baseline_std_golden(case):
+    r = torch.tensor(case["rewards"], dtype=torch.float32)
+    p = torch.tensor(case["prompts"])
+    v = torch.tensor(case["valid"], dtype=torch.float32)
+    baseline, std = A.baseline_and_std_per_prompt(p, r, v)
+    assert torch.allclose(baseline, torch.tensor(case["baseline"], dtype=torch.float32), rtol=BASE["rtol"])
+    if case["std"] is None:
+        assert torch.isfinite(std).all()
+    else:
+        assert torch.allclose(std, torch.tensor(case["std"], dtype=torch.float32), rtol=BASE["rtol"])
+
+
+def test_baseline_empty():
+    b, s = A.baseline_and_std_per_prompt(torch.empty(0, 3, dtype=torch.long), torch.tensor([]), torch.tensor([]))
+    assert b.shape == (0,) and s.shape == (0,)
+
+
+def test_group_ids_brute_force():
+    torch.manual_seed(0)
+    p = torch.randint(0, 2, (40, 3))
+    gid = A.group_ids_by_prompt(p)
+    for i in range(40):
+        for j in range(40):
+            assert (gid[i] == gid[j]).item() == bool((p[i] == p[j]).all())
+
+
+def test_non_loo_is_plain_mean_and_bessel_std():
+    """Without leave-one-out the baseline is the group mean and std the unbiased
+    sample std (library routine)."""
+    torch.manual_seed(1)
+    r = torch.randn(12)
+    p = torch.arange(3).repeat_interleave(4).unsqueeze(-1)
+    b, s = A.baseline_and_std_per_prompt(p, r, torch.ones(12), leave_one_out_baseline=False)
+    for g in range(3):
+        grp = r[g * 4 : g * 4 + 4]
+        assert torch.allclose(b[g * 4 : g * 4 + 4], grp.mean().expand(4), atol=1e-6)
+        assert torch.allclose(s[g * 4 : g * 4 + 4], grp.std(unbiased=True).expand(4), rtol=1e-3)
+
+
+def test_loo_matches_brute_force():
+    torch.manual_seed(2)
+    r = torch.randn(10)
+    p = torch.tensor([[0]] * 6 + [[7]] * 4)
+    b, s = A.baseline_and_std_per_prompt(p, r, torch.ones(10))
+    for lo, hi in ((0, 6), (6, 10)):
+        for i in range(lo, hi):
+            others = torch.cat([r[lo:i], r[i + 1 : hi]])
+            assert b[i].item() == pytest.approx(others.mean().item(), abs=1e-6)
+            assert s[i].item() == pytest.approx(others.std(unbiased=True).item(), rel=2e-3)
+
+
+@pytest.mark.parametrize("case", ADV["cases"], ids=[c["name"] for c in ADV["cases"]])
+def test_grpo_advantage_golden(case):
+    out = A.grpo_advantages(
+        torch.tensor(case["prompt_ids"]), torch.tensor(case["rewards"], dtype=torch.float32),
+        torch.ones(*case["mask_shape"]), leave_one_out_baseline=False, normalize_rewards=True,
+    )
+    assert tuple(out.shape) == tuple(case["mask_shape"])
+    assert (out == out[:, :1]).all()
+    if case["expected_col"] is not None:
+        exp = torch.tensor(case["expected_col"], dtype=torch.float32)
+        assert torch.allclose(out[:, 0], exp, rtol=case["rtol"], atol=1e-6)
+    elif case["name"] == "symmetry":
+        assert out[0, 0] < 0 and abs(out[1, 0]) < 1e-5 and out[2, 0] > 0
+        assert torch.allclose(out[0], -out[2], rtol=1e-5)
+    else:
+        assert abs(out.mean()) < 1e-5
