@@ -1,0 +1,187 @@
+/*
+ * nrl_hip.h - C ABI of librl_amd_hip.so: the GRPO logits -> logprob -> loss hot path
+ * as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - every entry point enqueues work on `stream` (a hipStream_t passed as void*) and returns
+ *     without synchronising; nothing is allocated or freed inside the library;
+ *   - sizes and strides are in ELEMENTS (not bytes); the vocabulary axis is contiguous;
+ *   - return value: 0 = ok, negative = NRL_E_* below; nrl_last_error() gives the text for the
+ *     calling thread;
+ *   - the library keeps no state between calls: entry points may be called from any host
+ *     thread (forward pass and autograd thread alike).
+ *
+ * The reference (NVIDIA NeMo-RL) has no FFI; each entry point names the Python code whose
+ * arithmetic it replaces (paths relative to the reference tree).
+ */
+#ifndef NRL_HIP_H
+#define NRL_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NRL_OK 0
+#define NRL_E_INVALID (-1)     /* bad argument (shape, stride, dtype, null pointer)   */
+#define NRL_E_UNSUPPORTED (-2) /* combination not built                                */
+#define NRL_E_LAUNCH (-3)      /* hipLaunchKernel / runtime error                      */
+#define NRL_E_WORKSPACE (-4)   /* workspace too small                                  */
+
+enum nrl_dtype { NRL_F32 = 0, NRL_BF16 = 1, NRL_F16 = 2 };
+
+/* how the temperature divide is rounded (nemo_rl/models/automodel/train.py:180-194 divides the
+ * logits in place in their own dtype):  DIV = round(x / T), what torch does on the CPU;
+ * RCP = round(x * (1/T)) with 1/T rounded to fp32 first, what torch does on the GPU. */
+enum nrl_temp_mode { NRL_TEMP_DIV = 0, NRL_TEMP_RCP = 1 };
+
+int nrl_version(void);
+const char* nrl_last_error(void);
+
+/* Row addressing shared by the logprob entry points.  Row (o, i), 0 <= o < n_outer,
+ * 0 <= i < n_inner, lives at logits + o*stride_outer + i*stride_inner and has `vocab` contiguous
+ * elements.  Its target id is targets[o*tgt_stride_outer + i*tgt_stride_inner].  Passing
+ * targets = input_ids + 1 with n_inner = S-1 gives the reference's roll(-1) + drop-last-column
+ * without materialising either. */
+typedef struct nrl_rows {
+    const void* logits;
+    int32_t dtype; /* nrl_dtype */
+    int64_t n_outer, n_inner, vocab;
+    int64_t stride_outer, stride_inner;
+    const int64_t* targets;
+    int64_t tgt_stride_outer, tgt_stride_inner;
+    int64_t vocab_start, vocab_end; /* targets outside [start, end) -> logprob 0, no one-hot */
+    float temperature;              /* 1.0 = off */
+    int32_t temp_mode;              /* nrl_temp_mode */
+} nrl_rows;
+
+/* K1  logits -> token logprob, one streaming pass per row (online log-sum-exp + gather).
+ * Replaces DistributedLogprob.forward / ChunkedDistributedLogprob.forward
+ * (nemo_rl/distributed/model_utils.py:136-165, 289-331) and the log_softmax + gather of
+ * get_next_token_logprobs_from_logits (:1677-1693) at TP = CP = 1.
+ * logprob_out, lse_out: fp32 [n_outer * n_inner]; lse_out may be NULL (inference_only). */
+int nrl_logprob_fwd(const nrl_rows* rows, float* logprob_out, float* lse_out, void* stream);
+
+/* K2  dlogits = g * (onehot(target) - exp(x - lse)), written once in the logits' dtype.
+ * Replaces DistributedLogprob.backward / ChunkedDistributedLogprob.backward (:167-207, 333-380).
+ * grad: fp32 upstream gradient of the logprobs, element (o, i) at
+ * grad[o*grad_stride_outer + i*grad_stride_inner].
+ * dlogits: same dtype as the logits; row (o, i) at dlogits + o*d_stride_outer + i*d_stride_inner
+ * for 0 <= i < d_n_inner; rows with i >= rows->n_inner (positions the forward dropped) are
+ * zero-filled.  dlogits may alias the logits (in-place gradient).  Rows whose g is exactly 0 are
+ * zero-filled without reading the logits. */
+int nrl_logprob_bwd(const nrl_rows* rows, const float* lse, const float* grad,
+                    int64_t grad_stride_outer, int64_t grad_stride_inner, void* dlogits,
+                    int64_t d_n_inner, int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
+
+/* Packed sequences (one [1, T, V] row of logits, sequences delimited by cu_seqlens_padded).
+ * Replaces from_parallel_logits_to_logprobs_packed_sequences (model_utils.py:1085-1196) at
+ * CP = 1: position p of sequence s (start = cu[s], len = cu[s+1]-cu[s]) uses target
+ * targets[start + (p+1) % len] unless pre_rolled (then targets[start + p]); the last position of
+ * every sequence is dropped; out[s, p] for p < min(len-1, unpacked_seqlen-1), zero elsewhere.
+ * logits: [T, vocab] contiguous rows of stride `row_stride`.  cu_seqlens: int32 [n_seq+1] device.
+ * out: fp32 [n_seq, unpacked_seqlen-1];  lse_out: fp32 [T] or NULL. */
+int nrl_logprob_packed_fwd(const void* logits, int32_t dtype, int64_t total_tokens, int64_t vocab,
+                           int64_t row_stride, const int64_t* targets, int32_t pre_rolled,
+                           const int32_t* cu_seqlens, int64_t n_seq, int64_t unpacked_seqlen,
+                           int64_t vocab_start, int64_t vocab_end, float temperature,
+                           int32_t temp_mode, float* out, float* lse_out, void* stream);
+
+/* Backward of the packed entry point: grad is fp32 [n_seq, unpacked_seqlen-1]; dlogits [T, vocab]
+ * (rows of stride d_row_stride); dropped / padded positions are zero-filled. */
+int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t total_tokens, int64_t vocab,
+                           int64_t row_stride, const int64_t* targets, int32_t pre_rolled,
+                           const int32_t* cu_seqlens, int64_t n_seq, int64_t unpacked_seqlen,
+                           int64_t vocab_start, int64_t vocab_end, float temperature,
+                           int32_t temp_mode, const float* lse, const float* grad, void* dlogits,
+                           int64_t d_row_stride, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * K4  ClippedPGLossFn (nemo_rl/algorithms/loss/loss_functions.py:374-788) with calculate_kl and
+ * masked_mean (nemo_rl/algorithms/utils.py:42-101, 212-224) fused: loss, its gradient with
+ * respect to the token logprobs, and every metric, in two launches.
+ * ------------------------------------------------------------------------------------------ */
+enum nrl_tis_type { NRL_TIS_NONE = 0, NRL_TIS_TIS = 1, NRL_TIS_ICEPOP = 2, NRL_TIS_SEQ_MASK = 3 };
+
+typedef struct nrl_grpo_cfg {
+    int32_t token_level_loss;
+    int32_t disable_ppo_ratio;
+    int32_t force_on_policy_ratio;
+    int32_t use_cispo;
+    int32_t sequence_level_importance_ratios;
+    int32_t use_importance_sampling_correction;
+    int32_t use_on_policy_kl_approximation;
+    int32_t tis_type;       /* nrl_tis_type */
+    int32_t kl_type;        /* 1, 2, 3 = k1, k2, k3 */
+    int32_t has_kl;         /* reference_policy_kl_penalty != 0 */
+    int32_t has_kl_input_clamp, has_kl_output_clamp;
+    int32_t has_dual_clip;  /* ratio_clip_c is not None */
+    int32_t has_nll;        /* positive_example_nll_weight > 0 and "rewards" given */
+    float ratio_clip_min, ratio_clip_max, ratio_clip_c;
+    float kl_beta, kl_input_clamp, kl_output_clamp;
+    float tis_max, tis_min;
+    float nll_weight;
+} nrl_grpo_cfg;
+
+/* metric slots of the fp32 metrics_out array (NRL_GRPO_N_METRICS entries) */
+enum nrl_grpo_metric {
+    NRL_M_LOSS = 0, NRL_M_PROBS_RATIO, NRL_M_PROBS_RATIO_CLAMPED, NRL_M_PROBS_RATIO_MIN,
+    NRL_M_PROBS_RATIO_MAX, NRL_M_PROBS_RATIO_CLAMPED_MIN, NRL_M_PROBS_RATIO_CLAMPED_MAX,
+    NRL_M_KL, /* the reduced kl term (beta included); kl_penalty = this / beta */
+    NRL_M_TOKEN_MULT_PROB_ERROR, NRL_M_GEN_KL_ERROR, NRL_M_POLICY_KL_ERROR, NRL_M_JS_DIVERGENCE_ERROR,
+    NRL_M_SAMPLING_IMPORTANCE_RATIO, NRL_M_NUM_VALID_SAMPLES, NRL_M_APPROX_ENTROPY, NRL_M_IS_OOB_RATIO,
+    NRL_M_POSITIVE_NLL_LOSS, NRL_M_ACTOR_LOSS, NRL_M_N_MASKED_TOKENS, NRL_GRPO_N_METRICS = 24
+};
+
+/* Every [B, Sm1] input is fp32 with unit column stride and its own row stride (so the
+ * reference's data[...][:, 1:] slices are passed as pointer + 1 with row stride S). */
+typedef struct nrl_grpo_inputs {
+    int64_t batch, sm1;
+    const float* lp;  int64_t lp_stride;   /* current-policy logprobs (requires grad)        */
+    const float* lpu; int64_t lpu_stride;  /* unfiltered logprobs for the KL, NULL = use lp  */
+    const float* prev; int64_t prev_stride; /* NULL allowed when force_on_policy_ratio        */
+    const float* gen; int64_t gen_stride;
+    const float* ref; int64_t ref_stride;  /* NULL allowed when !has_kl                      */
+    const float* adv; int64_t adv_stride;
+    const float* token_mask; int64_t token_mask_stride;
+    const float* sample_mask;   /* [B] */
+    const float* correct_mask;  /* [B] (rewards > 0), NULL unless has_nll */
+    const float* global_valid;  /* device [2]: {global_valid_seqs, global_valid_toks} */
+} nrl_grpo_inputs;
+
+int64_t nrl_grpo_loss_workspace_bytes(int64_t batch);
+
+/* loss_out: fp32 [1]; dlp_out: fp32 [B, Sm1] contiguous (d loss / d lp); dlpu_out: fp32 [B, Sm1]
+ * or NULL (required iff in->lpu != NULL and cfg->has_kl); metrics_out: fp32 [NRL_GRPO_N_METRICS];
+ * workspace: nrl_grpo_loss_workspace_bytes(B) bytes, 8-byte aligned. */
+int nrl_grpo_loss_fwd_bwd(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out,
+                          float* dlp_out, float* dlpu_out, float* metrics_out, void* workspace,
+                          int64_t workspace_bytes, void* stream);
+
+/* NLLLossFn scalar branch (loss_functions.py:818-842): loss = -sum(lp*mask)/(Gt+1e-8);
+ * metrics_out[0..2] = {loss, num_unmasked_tokens, num_valid_samples}; dlp_out = -mask/(Gt+1e-8). */
+int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,
+                         float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * K5  calculate_baseline_and_std_per_prompt (nemo_rl/algorithms/utils.py:104-198) and
+ * GRPOAdvantageEstimator.compute_advantage (nemo_rl/algorithms/advantage_estimator.py:82-98).
+ * prompts: int64 [B, Sp] rows of stride prompt_stride; rows are grouped by exact equality.
+ * group_out (int32 [B], may be NULL): index of the first row of each row's group.
+ * std_rewards may be NULL (= rewards).  adv_out (fp32 [B]) may be NULL; when given it holds
+ * (r - baseline), divided by (std + 1e-6) where std > 0 if `normalize`.
+ * workspace: nrl_group_workspace_bytes(B) bytes.
+ * ------------------------------------------------------------------------------------------ */
+int64_t nrl_group_workspace_bytes(int64_t batch);
+int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int64_t prompt_len,
+                           int64_t prompt_stride, const float* rewards, const float* valid,
+                           const float* std_rewards, int32_t leave_one_out, int32_t normalize,
+                           float* baseline_out, float* std_out, float* adv_out, int32_t* group_out,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NRL_HIP_H */

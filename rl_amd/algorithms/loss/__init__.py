@@ -1,0 +1,16 @@
+"""Loss functions of the GRPO hot path (counterpart of ``nemo_rl/algorithms/loss/__init__.py``)."""
+
+from .interfaces import LossFunction, LossInputType, LossType, MetricNormalizer
+from .loss_functions import ClippedPGLossConfig, ClippedPGLossFn, NLLLossFn
+from .utils import prepare_loss_input, prepare_packed_loss_input
+from .wrapper import (
+    SequencePackingFusionLossWrapper,
+    SequencePackingLossWrapper,
+    wrap_loss_fn_with_input_preparation,
+)
+
+__all__ = [
+    "ClippedPGLossConfig", "ClippedPGLossFn", "NLLLossFn", "LossFunction", "LossInputType", "LossType",
+    "MetricNormalizer", "prepare_loss_input", "prepare_packed_loss_input", "SequencePackingFusionLossWrapper",
+    "SequencePackingLossWrapper", "wrap_loss_fn_with_input_preparation",
+]

@@ -1,0 +1,320 @@
+"""Clipped policy-gradient loss (GRPO / PPO-clip / DAPO clip-higher / REINFORCE / GSPO / CISPO)
+and the NLL loss, computed by the fused HIP loss kernel.
+
+Counterpart of ``nemo_rl/algorithms/loss/loss_functions.py:111-842``: same configuration fields,
+constructor checks, call signature, returned metrics and ``metric_normalizations`` table.  One
+call is two kernel launches and one device->host copy of the metrics record, instead of a few
+dozen element-wise kernels and a synchronisation per metric.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+from pydantic import BaseModel
+
+from ... import ops as _ops  # noqa: F401
+from ..._lib import METRIC_SLOTS, NRL_TIS
+from .interfaces import LossFunction, LossInputType, LossType, MetricNormalizer
+
+_OPS = torch.ops.rl_amd
+_KL_TYPES = {"k1": 1, "k2": 2, "k3": 3}
+
+
+class ClippedPGLossConfig(BaseModel, extra="allow"):
+    """Field names and defaults of the reference configuration (``loss_functions.py:111-164``)."""
+
+    disable_ppo_ratio: bool = False
+    token_level_loss: bool = True
+    sequence_level_importance_ratios: bool = False
+    ratio_clip_min: float = 0.2
+    ratio_clip_max: float = 0.2
+    ratio_clip_c: Optional[float] = None
+    reference_policy_kl_penalty: float = 0.01
+    reference_policy_kl_type: str = "k3"
+    kl_input_clamp_value: Optional[float] = 20.0
+    kl_output_clamp_value: Optional[float] = 10.0
+    use_kl_in_reward: bool = False
+    use_importance_sampling_correction: bool = False
+    truncated_importance_sampling_type: Optional[str] = None
+    truncated_importance_sampling_ratio: Optional[float] = None
+    truncated_importance_sampling_ratio_min: Optional[float] = None
+    use_on_policy_kl_approximation: bool = False
+    force_on_policy_ratio: bool = False
+    use_cispo: bool = False
+    positive_example_nll_weight: float = 0.0
+
+
+def _gpu_for(t: torch.Tensor) -> torch.device:
+    if t.is_cuda:
+        return t.device
+    if not torch.cuda.is_available():
+        raise RuntimeError("rl_amd needs an MI355X: no GPU is visible and there is no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _f32(t, dev):
+    return t.to(device=dev, dtype=torch.float32)
+
+
+def _global_valid(seqs, toks, dev) -> torch.Tensor:
+    parts = []
+    for v in (seqs, toks):
+        if isinstance(v, torch.Tensor):
+            parts.append(v.detach().reshape(()).to(device=dev, dtype=torch.float32))
+        else:
+            parts.append(torch.tensor(float(v), dtype=torch.float32, device=dev))
+    return torch.stack(parts)
+
+
+class _FusedLoss(torch.autograd.Function):
+    """loss, metrics = kernel(lp, lpu, ...); the kernel also returns d loss / d lp (and / d lpu), so the
+    backward is a scalar multiply."""
+
+    @staticmethod
+    def forward(ctx, lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct, global_valid, iflags, fparams):
+        loss, dlp, dlpu, metrics = _OPS.grpo_loss(
+            lp.detach(), None if lpu is None else lpu.detach(), prev, gen, ref, adv, token_mask, sample_mask, correct,
+            global_valid, iflags, fparams,
+        )
+        ctx.save_for_backward(dlp, dlpu)
+        ctx.has_lpu = lpu is not None and dlpu.numel() > 0
+        ctx.mark_non_differentiable(metrics)
+        return loss, metrics
+
+    @staticmethod
+    def backward(ctx, grad_loss, _grad_metrics):
+        dlp, dlpu = ctx.saved_tensors
+        g_lp = dlp * grad_loss if ctx.needs_input_grad[0] else None
+        g_lpu = dlpu * grad_loss if (ctx.has_lpu and ctx.needs_input_grad[1]) else None
+        return (g_lp, g_lpu) + (None,) * 10
+
+
+class ClippedPGLossFn(LossFunction):
+    """Generalised clipped policy-gradient loss with KL regularisation.
+
+    ``L = E_t[max(-A r, -A clip(r, 1-eps_lo, 1+eps_hi))] + beta * KL(pi || pi_ref)`` with the variants
+    selected by the configuration flags (see ``ClippedPGLossConfig``)."""
+
+    input_type = LossInputType.LOGPROB
+
+    def __init__(self, cfg, use_fused_linear_logprobs: bool = False):
+        if isinstance(cfg, dict):
+            cfg = ClippedPGLossConfig(**cfg)
+        self.use_fused_linear_logprobs = use_fused_linear_logprobs
+        self.disable_ppo_ratio = cfg.disable_ppo_ratio
+        self.ratio_clip_min = cfg.ratio_clip_min
+        self.ratio_clip_max = cfg.ratio_clip_max
+        self.ratio_clip_c = cfg.ratio_clip_c
+        self.reference_policy_kl_penalty = cfg.reference_policy_kl_penalty if not cfg.use_kl_in_reward else 0
+        self.reference_policy_kl_type = cfg.reference_policy_kl_type
+        self.kl_input_clamp_value = cfg.kl_input_clamp_value
+        self.kl_output_clamp_value = cfg.kl_output_clamp_value
+        self.use_importance_sampling_correction = cfg.use_importance_sampling_correction
+        self.truncated_importance_sampling_type = cfg.truncated_importance_sampling_type
+        self.truncated_importance_sampling_ratio = cfg.truncated_importance_sampling_ratio
+        self.truncated_importance_sampling_ratio_min = cfg.truncated_importance_sampling_ratio_min
+        self.use_on_policy_kl_approximation = cfg.use_on_policy_kl_approximation
+        self.force_on_policy_ratio = cfg.force_on_policy_ratio
+        self.sequence_level_importance_ratios = cfg.sequence_level_importance_ratios
+        self.positive_example_nll_weight = cfg.positive_example_nll_weight
+        self.use_cispo = cfg.use_cispo
+        self.loss_type = LossType.TOKEN_LEVEL if cfg.token_level_loss else LossType.SEQUENCE_LEVEL
+        self._check_flags()
+        self.metric_normalizations = self._normalizations()
+
+    # -- constructor checks, loss_functions.py:265-324 ------------------------------------------
+    def _check_flags(self) -> None:
+        if self.sequence_level_importance_ratios:
+            assert self.loss_type == LossType.SEQUENCE_LEVEL, (
+                "sequence-level importance sampling (e.g. GSPO) is mutually exclusive with token-level loss"
+            )
+        if self.use_cispo:
+            assert not self.disable_ppo_ratio, "use_cispo is incompatible with disable_ppo_ratio"
+            assert not self.force_on_policy_ratio, "use_cispo is incompatible with force_on_policy_ratio"
+            assert not self.sequence_level_importance_ratios, (
+                "use_cispo is incompatible with sequence_level_importance_ratios"
+            )
+            assert self.ratio_clip_c is None, "use_cispo is incompatible with dual clipping (ratio_clip_c)"
+            assert self.loss_type == LossType.TOKEN_LEVEL, "use_cispo requires token_level_loss=True"
+        kind = self.truncated_importance_sampling_type
+        if kind is not None:
+            assert self.use_importance_sampling_correction, (
+                "truncated importance sampling is only supported when use_importance_sampling_correction is True"
+            )
+            assert kind in ("tis", "icepop", "seq-mask-tis"), (
+                f"truncated_importance_sampling_type must be 'tis', 'icepop', or 'seq-mask-tis', got {kind}"
+            )
+            hi, lo = self.truncated_importance_sampling_ratio, self.truncated_importance_sampling_ratio_min
+            assert hi is not None and hi > 0, "truncated_importance_sampling_ratio should be positive"
+            if lo is not None:
+                assert lo <= hi, (
+                    "truncated_importance_sampling_ratio_min must be <= truncated_importance_sampling_ratio"
+                )
+            if kind in ("icepop", "seq-mask-tis"):
+                assert lo is not None, (
+                    "truncated_importance_sampling_ratio_min should be set when "
+                    "truncated_importance_sampling_type is 'icepop' or 'seq-mask-tis'"
+                )
+            if kind == "seq-mask-tis":
+                assert not self.sequence_level_importance_ratios, (
+                    "seq-mask-tis is incompatible with sequence_level_importance_ratios=True"
+                )
+
+    # -- per-metric denominators, loss_functions.py:331-372 --------------------------------------
+    def _normalizations(self) -> dict[str, MetricNormalizer]:
+        tok, seq, none = MetricNormalizer.TOKENS, MetricNormalizer.SEQUENCES, MetricNormalizer.NONE
+        like_grad = tok if self.loss_type == LossType.TOKEN_LEVEL else seq
+        table = {"loss": like_grad, "kl_penalty": like_grad}
+        for key in ("probs_ratio", "probs_ratio_clamped", "token_mult_prob_error", "gen_kl_error",
+                    "policy_kl_error", "js_divergence_error", "approx_entropy"):
+            table[key] = tok
+        table["sampling_importance_ratio"] = seq if self.sequence_level_importance_ratios else tok
+        for key in ("num_valid_samples", "positive_nll_loss", "probs_ratio_min", "probs_ratio_max",
+                    "probs_ratio_clamped_min", "probs_ratio_clamped_max"):
+            table[key] = none
+        if self.truncated_importance_sampling_type is not None:
+            table["is_oob_ratio"] = seq if self.truncated_importance_sampling_type == "seq-mask-tis" else tok
+        return table
+
+    def _kernel_config(self, has_nll: bool) -> tuple[list[int], list[float]]:
+        kind = self.truncated_importance_sampling_type
+        if self.truncated_importance_sampling_ratio is not None and kind not in ("tis", "icepop", "seq-mask-tis"):
+            raise ValueError(f"Invalid truncated importance sampling type: {kind}")
+        if self.reference_policy_kl_type not in _KL_TYPES:
+            raise ValueError(f"Invalid KL type: {self.reference_policy_kl_type}")
+        if self.ratio_clip_c is not None:
+            assert self.ratio_clip_c > 1, (
+                f"ratio_clip_c must exceed 1 representing a lower bound of the ratios, got {self.ratio_clip_c}."
+            )
+        use_tis = self.truncated_importance_sampling_ratio is not None
+        lo = self.truncated_importance_sampling_ratio_min
+        iflags = [
+            int(self.loss_type == LossType.TOKEN_LEVEL), int(self.disable_ppo_ratio), int(self.force_on_policy_ratio),
+            int(self.use_cispo), int(self.sequence_level_importance_ratios),
+            int(self.use_importance_sampling_correction), int(self.use_on_policy_kl_approximation),
+            NRL_TIS[kind] if use_tis else 0, _KL_TYPES[self.reference_policy_kl_type],
+            int(self.reference_policy_kl_penalty != 0), int(self.kl_input_clamp_value is not None),
+            int(self.kl_output_clamp_value is not None), int(self.ratio_clip_c is not None), int(has_nll),
+        ]
+        fparams = [
+            self.ratio_clip_min, self.ratio_clip_max, self.ratio_clip_c or 0.0, float(self.reference_policy_kl_penalty),
+            self.kl_input_clamp_value or 0.0, self.kl_output_clamp_value or 0.0,
+            self.truncated_importance_sampling_ratio or 0.0, 0.0 if lo is None else lo,
+            float(self.positive_example_nll_weight),
+        ]
+        return iflags, fparams
+
+    def __call__(
+        self,
+        next_token_logprobs: torch.Tensor,
+        data: Any,
+        global_valid_seqs: torch.Tensor,
+        global_valid_toks: torch.Tensor,
+    ) -> tuple[torch.Tensor, dict]:
+        """``loss_functions.py:374-788``.  ``data`` is any mapping with the reference's keys."""
+        lp_in = next_token_logprobs
+        home = lp_in.device
+        dev = _gpu_for(lp_in)
+        beta = self.reference_policy_kl_penalty
+
+        sample_mask_in = data["sample_mask"]
+        lp = _f32(lp_in, dev)
+        token_mask = _f32(data["token_mask"][:, 1:], dev)
+        sample_mask = _f32(sample_mask_in, dev)
+        adv = _f32(data["advantages"][:, 1:], dev)
+        prev = None if self.force_on_policy_ratio else _f32(data["prev_logprobs"][:, 1:], dev)
+        gen = _f32(data["generation_logprobs"][:, 1:], dev)
+        ref = lpu = None
+        if beta != 0:
+            ref = _f32(data["reference_policy_logprobs"][:, 1:], dev)
+            unfiltered = data.get("curr_logprobs_unfiltered", None)
+            if unfiltered is not None and unfiltered is not lp_in:
+                lpu = _f32(unfiltered, dev)
+        correct = None
+        has_nll = self.positive_example_nll_weight > 0 and "rewards" in data
+        if has_nll:
+            correct = (data["rewards"] > 0).to(device=dev, dtype=torch.float32)
+        iflags, fparams = self._kernel_config(has_nll)
+
+        loss, metrics = _FusedLoss.apply(
+            lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct,
+            _global_valid(global_valid_seqs, global_valid_toks, dev), iflags, fparams,
+        )
+        if home != dev:
+            loss = loss.to(home)
+        m = metrics.cpu().tolist()  # the one synchronisation of the call
+        get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
+        n_valid = get("num_valid_samples")
+        out = {
+            "loss": get("loss"),
+            "probs_ratio": get("probs_ratio"),
+            "probs_ratio_clamped": get("probs_ratio_clamped"),
+            "probs_ratio_min": get("probs_ratio_min"),
+            "probs_ratio_max": get("probs_ratio_max"),
+            "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
+            "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
+            "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
+            "token_mult_prob_error": get("token_mult_prob_error"),
+            "gen_kl_error": get("gen_kl_error"),
+            "policy_kl_error": get("policy_kl_error"),
+            "js_divergence_error": get("js_divergence_error"),
+            "sampling_importance_ratio": get("sampling_importance_ratio"),
+            "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
+            "approx_entropy": get("approx_entropy"),
+        }
+        if self.truncated_importance_sampling_ratio is not None:
+            out["is_oob_ratio"] = get("is_oob_ratio")
+        out["positive_nll_loss"] = get("positive_nll_loss")
+        return loss, out
+
+
+class _FusedNll(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, lp, token_mask, sample_mask, global_valid):
+        loss, dlp, metrics = _OPS.nll_loss(lp.detach(), token_mask, sample_mask, global_valid)
+        ctx.save_for_backward(dlp)
+        ctx.mark_non_differentiable(metrics)
+        return loss, metrics
+
+    @staticmethod
+    def backward(ctx, grad_loss, _grad_metrics):
+        (dlp,) = ctx.saved_tensors
+        return dlp * grad_loss, None, None, None
+
+
+class NLLLossFn(LossFunction):
+    """Negative log-likelihood over the masked tokens (``loss_functions.py:791-842``, scalar branch)."""
+
+    loss_type = LossType.TOKEN_LEVEL
+    input_type = LossInputType.LOGPROB
+
+    def __init__(self, use_fused_linear_logprobs: bool = False):
+        self.use_fused_linear_logprobs = use_fused_linear_logprobs
+        self.metric_normalizations = {
+            "loss": MetricNormalizer.TOKENS,
+            "num_unmasked_tokens": MetricNormalizer.NONE,
+            "num_valid_samples": MetricNormalizer.NONE,
+        }
+
+    def __call__(self, next_token_logprobs, data, global_valid_seqs, global_valid_toks,
+                 dpo_loss: bool = False, dpo_average_log_probs: bool = False):
+        if dpo_loss:
+            raise NotImplementedError("the per-sample DPO reduction is outside the GRPO hot path")
+        home = next_token_logprobs.device
+        dev = _gpu_for(next_token_logprobs)
+        sample_mask_in, token_mask_in = data["sample_mask"], data["token_mask"]
+        loss, metrics = _FusedNll.apply(
+            _f32(next_token_logprobs, dev), _f32(token_mask_in[:, 1:], dev), _f32(sample_mask_in, dev),
+            _global_valid(1.0, global_valid_toks, dev),
+        )
+        if home != dev:
+            loss = loss.to(home)
+        m = metrics.cpu().tolist()
+        integral = not (sample_mask_in.is_floating_point() or token_mask_in.is_floating_point())
+        return loss, {
+            "loss": m[0],
+            "num_unmasked_tokens": int(m[1]) if integral else m[1],
+            "num_valid_samples": m[2] if sample_mask_in.is_floating_point() else int(m[2]),
+        }

@@ -1,0 +1,194 @@
+// Shared device helpers for the gfx950 kernels: element decoding for fp32 / bf16 / fp16 rows,
+// round-to-nearest-even narrowing, wave64 / workgroup reductions and the host-side error slot.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/nrl_hip.h"
+
+namespace nrl {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kWave = 64;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------------------------
+// host: per-thread error text
+// ---------------------------------------------------------------------------------------------
+char* error_slot();
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+// ---------------------------------------------------------------------------------------------
+// scalar conversions
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
+
+// fp32 -> bf16 bits, round to nearest even (NaN stays a quiet NaN)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t lo16) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(lo16)));
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(f)));
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// torch.max / torch.min semantics: NaN propagates
+__device__ __forceinline__ float nan_max(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ __forceinline__ float nan_min(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+
+// ---------------------------------------------------------------------------------------------
+// Row element traits.  DT is an nrl_dtype.  A 16-byte vector holds EPV elements.
+// TEMP: 0 = no temperature, 1 = round(x / T), 2 = round(x * rcpT); the rounding is to the row's
+// own dtype, mirroring an in-place divide of the logits tensor.
+// ---------------------------------------------------------------------------------------------
+template <int DT> struct Row;
+
+template <> struct Row<NRL_F32> {
+    static constexpr int EPV = 4;
+    static constexpr int BYTES = 4;
+    __device__ static __forceinline__ float round_self(float v) { return v; }
+    __device__ static __forceinline__ void decode(const u32x4& r, float (&v)[4]) {
+        v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y);
+        v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
+    }
+    __device__ static __forceinline__ u32x4 encode(const float (&v)[4]) {
+        u32x4 r;
+        r.x = __float_as_uint(v[0]); r.y = __float_as_uint(v[1]);
+        r.z = __float_as_uint(v[2]); r.w = __float_as_uint(v[3]);
+        return r;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float v) { static_cast<float*>(p)[i] = v; }
+};
+
+template <> struct Row<NRL_BF16> {
+    static constexpr int EPV = 8;
+    static constexpr int BYTES = 2;
+    __device__ static __forceinline__ float round_self(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+    __device__ static __forceinline__ void decode(const u32x4& r, float (&v)[8]) {
+        v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+        v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+        v[4] = __uint_as_float(r.z << 16); v[5] = __uint_as_float(r.z & 0xffff0000u);
+        v[6] = __uint_as_float(r.w << 16); v[7] = __uint_as_float(r.w & 0xffff0000u);
+    }
+    __device__ static __forceinline__ u32x4 encode(const float (&v)[8]) {
+        u32x4 r;
+        r.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+        r.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+        r.z = f32_to_bf16_bits(v[4]) | (f32_to_bf16_bits(v[5]) << 16);
+        r.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
+        return r;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+        return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float v) {
+        static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+    }
+};
+
+template <> struct Row<NRL_F16> {
+    static constexpr int EPV = 8;
+    static constexpr int BYTES = 2;
+    __device__ static __forceinline__ float round_self(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
+    __device__ static __forceinline__ void decode(const u32x4& r, float (&v)[8]) {
+        v[0] = f16_bits_to_f32(r.x & 0xffffu); v[1] = f16_bits_to_f32(r.x >> 16);
+        v[2] = f16_bits_to_f32(r.y & 0xffffu); v[3] = f16_bits_to_f32(r.y >> 16);
+        v[4] = f16_bits_to_f32(r.z & 0xffffu); v[5] = f16_bits_to_f32(r.z >> 16);
+        v[6] = f16_bits_to_f32(r.w & 0xffffu); v[7] = f16_bits_to_f32(r.w >> 16);
+    }
+    __device__ static __forceinline__ u32x4 encode(const float (&v)[8]) {
+        u32x4 r;
+        r.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+        r.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+        r.z = f32_to_f16_bits(v[4]) | (f32_to_f16_bits(v[5]) << 16);
+        r.w = f32_to_f16_bits(v[6]) | (f32_to_f16_bits(v[7]) << 16);
+        return r;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+        return f16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float v) {
+        static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(f32_to_f16_bits(v));
+    }
+};
+
+// temperature applied the way an in-place divide of the logits tensor rounds it
+template <int DT, int TEMP> __device__ __forceinline__ float scale_logit(float x, float tparam) {
+    if constexpr (TEMP == 0) return x;
+    else if constexpr (TEMP == 1) return Row<DT>::round_self(__fdiv_rn(x, tparam));
+    else return Row<DT>::round_self(x * tparam);
+}
+
+// ---------------------------------------------------------------------------------------------
+// reductions (wave64)
+// ---------------------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Sum over a workgroup of NW waves; every thread receives the total.  `smem` holds NW entries.
+// Lanes are combined in a fixed butterfly order and waves in ascending order, so the result
+// depends only on the values and the workgroup shape.
+template <typename T, int NW> __device__ __forceinline__ T block_sum(T v, T* smem) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    T t = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) t += smem[i];
+    return t;
+}
+template <int NW> __device__ __forceinline__ float block_max(float v, float* smem) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float t = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) t = fmaxf(t, smem[i]);
+    return t;
+}
+template <int NW> __device__ __forceinline__ float block_min(float v, float* smem) {
+    v = wave_min(v);
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float t = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) t = fminf(t, smem[i]);
+    return t;
+}
+
+}  // namespace nrl

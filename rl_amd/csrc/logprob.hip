@@ -1,0 +1,508 @@
+// K1 / K2: vocabulary logits -> token logprob (forward) and softmax-minus-onehot gradient
+// (backward) for gfx950.
+//
+// One workgroup of 256 threads (4 wave64) owns one logits row.  The forward is a single
+// streaming pass: every lane reads 16-byte vectors (coalesced, 1 KiB per wave per load), keeps a
+// running (max, sum-of-exp) pair in registers, and the pairs are merged with a wave butterfly and
+// a 4-entry LDS exchange.  The reduction order of a row depends only on the vocabulary size,
+// never on how many rows are in the launch, so a row's result is bit-identical whatever batch it
+// arrives in.  The backward re-reads the row once and writes the gradient once, narrowing from
+// fp32 with a single round-to-nearest-even; probabilities are never stored.
+//
+// Algorithmic HBM traffic: forward V*sizeof(logit) per row, backward 2*V*sizeof(logit) per row.
+
+#include <float.h>
+
+#include "common.hpp"
+
+namespace nrl {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+constexpr int kUnroll = 4;
+
+struct Lse {
+    float m;  // running maximum
+    float s;  // sum of exp(x - m)
+};
+
+__device__ __forceinline__ Lse lse_merge(Lse a, Lse b) {
+    const float m = fmaxf(a.m, b.m);
+    Lse r;
+    r.m = m;
+    r.s = a.s * fast_exp2((a.m - m) * kLog2e) + b.s * fast_exp2((b.m - m) * kLog2e);
+    return r;
+}
+
+template <int N> __device__ __forceinline__ void lse_push(Lse& acc, const float (&v)[N]) {
+    float vm = v[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) vm = fmaxf(vm, v[k]);
+    const float mn = fmaxf(acc.m, vm);
+    float part = 0.f;
+#pragma unroll
+    for (int k = 0; k < N; ++k) part += fast_exp2((v[k] - mn) * kLog2e);
+    acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + part;
+    acc.m = mn;
+}
+
+__device__ __forceinline__ void lse_push1(Lse& acc, float x) {
+    const float mn = fmaxf(acc.m, x);
+    acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((x - mn) * kLog2e);
+    acc.m = mn;
+}
+
+// number of leading elements before the first 16-byte boundary of a row
+template <int DT> __device__ __forceinline__ int64_t row_head(const void* row, int64_t vocab) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(row);
+    const int64_t h = static_cast<int64_t>(((16 - (a & 15)) & 15) / Row<DT>::BYTES);
+    return h < vocab ? h : vocab;
+}
+
+// Online log-sum-exp of one row; every thread returns the row's (max, sum).
+template <int DT, int TEMP>
+__device__ __forceinline__ Lse row_online_lse(const void* row, int64_t vocab, float tparam, Lse* smem) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    Lse acc;
+    acc.m = -FLT_MAX;
+    acc.s = 0.f;
+
+    const int64_t head = row_head<DT>(row, vocab);
+    const int64_t nvec = (vocab - head) / EPV;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(row) + head * Row<DT>::BYTES);
+
+    int64_t base = 0;
+    for (; base + kUnroll * kBlock <= nvec; base += kUnroll * kBlock) {
+        u32x4 r[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) r[u] = __builtin_nontemporal_load(xv + base + u * kBlock + tid);
+        float v[kUnroll * EPV];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float t[EPV];
+            Row<DT>::decode(r[u], t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) v[u * EPV + k] = scale_logit<DT, TEMP>(t[k], tparam);
+        }
+        lse_push<kUnroll * EPV>(acc, v);
+    }
+    for (int64_t i = base + tid; i < nvec; i += kBlock) {
+        float t[EPV];
+        Row<DT>::decode(__builtin_nontemporal_load(xv + i), t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) t[k] = scale_logit<DT, TEMP>(t[k], tparam);
+        lse_push<EPV>(acc, t);
+    }
+    // unaligned head and the tail shorter than one vector
+    if (tid < head) lse_push1(acc, scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), tparam));
+    const int64_t tail0 = head + nvec * EPV;
+    if (tail0 + tid < vocab) lse_push1(acc, scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), tparam));
+
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        Lse o;
+        o.m = __shfl_xor(acc.m, off, kWave);
+        o.s = __shfl_xor(acc.s, off, kWave);
+        acc = lse_merge(acc, o);
+    }
+    const int lane = tid & (kWave - 1), w = tid / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = acc;
+    __syncthreads();
+    Lse tot = smem[0];
+#pragma unroll
+    for (int i = 1; i < kWaves; ++i) tot = lse_merge(tot, smem[i]);
+    return tot;
+}
+
+template <int DT> __device__ __forceinline__ void row_zero(void* row, int64_t vocab) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const int64_t head = row_head<DT>(row, vocab);
+    const int64_t nvec = (vocab - head) / EPV;
+    u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(row) + head * Row<DT>::BYTES);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int64_t i = tid; i < nvec; i += kBlock) __builtin_nontemporal_store(z, ov + i);
+    if (tid < head) Row<DT>::store1(row, tid, 0.f);
+    const int64_t tail0 = head + nvec * EPV;
+    if (tail0 + tid < vocab) Row<DT>::store1(row, tail0 + tid, 0.f);
+}
+
+// gradient of one element: g * (onehot - softmax), narrowed once to the row dtype; with a fused
+// temperature the chain rule through the in-place divide rounds a second time, as autograd does.
+template <int DT, int TEMP>
+__device__ __forceinline__ float grad_elem(float x, bool is_target, float lse, float g, float tparam) {
+    const float p = fast_exp2((scale_logit<DT, TEMP>(x, tparam) - lse) * kLog2e);
+    float d = ((is_target ? 1.f : 0.f) - p) * g;
+    if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), tparam);
+    if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * tparam;
+    return d;
+}
+
+template <int DT, int TEMP>
+__device__ __forceinline__ void row_write_grad(const void* row, void* out, int64_t vocab, float lse, float g,
+                                               int64_t tgt, float tparam) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const int64_t head = row_head<DT>(row, vocab);
+    if (row_head<DT>(out, vocab) != head) {
+        // input and output rows are not congruent modulo 16 bytes: element-wise path
+        for (int64_t i = tid; i < vocab; i += kBlock)
+            Row<DT>::store1(out, i, grad_elem<DT, TEMP>(Row<DT>::load1(row, i), i == tgt, lse, g, tparam));
+        return;
+    }
+    const int64_t nvec = (vocab - head) / EPV;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(row) + head * Row<DT>::BYTES);
+    u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(out) + head * Row<DT>::BYTES);
+    const int64_t tvec = tgt >= head ? (tgt - head) / EPV : -1;  // vector that holds the target
+    const int tsub = tgt >= head ? static_cast<int>((tgt - head) % EPV) : -1;
+
+    int64_t base = 0;
+    for (; base + kUnroll * kBlock <= nvec; base += kUnroll * kBlock) {
+        u32x4 r[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) r[u] = __builtin_nontemporal_load(xv + base + u * kBlock + tid);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int64_t vi = base + u * kBlock + tid;
+            float t[EPV];
+            Row<DT>::decode(r[u], t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) t[k] = grad_elem<DT, TEMP>(t[k], vi == tvec && k == tsub, lse, g, tparam);
+            __builtin_nontemporal_store(Row<DT>::encode(t), ov + vi);
+        }
+    }
+    for (int64_t vi = base + tid; vi < nvec; vi += kBlock) {
+        float t[EPV];
+        Row<DT>::decode(__builtin_nontemporal_load(xv + vi), t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) t[k] = grad_elem<DT, TEMP>(t[k], vi == tvec && k == tsub, lse, g, tparam);
+        __builtin_nontemporal_store(Row<DT>::encode(t), ov + vi);
+    }
+    if (tid < head) Row<DT>::store1(out, tid, grad_elem<DT, TEMP>(Row<DT>::load1(row, tid), tid == tgt, lse, g, tparam));
+    const int64_t tail0 = head + nvec * EPV;
+    if (tail0 + tid < vocab) {
+        const int64_t i = tail0 + tid;
+        Row<DT>::store1(out, i, grad_elem<DT, TEMP>(Row<DT>::load1(row, i), i == tgt, lse, g, tparam));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// strided [n_outer, n_inner] rows
+// ---------------------------------------------------------------------------------------------
+struct RowArgs {
+    const void* logits;
+    int64_t n_inner, vocab, stride_outer, stride_inner;
+    const int64_t* targets;
+    int64_t ts_outer, ts_inner, vstart, vend;
+    float tparam;
+};
+
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kBlock) void logprob_fwd_kernel(RowArgs a, float* __restrict__ logprob,
+                                                             float* __restrict__ lse_out) {
+    __shared__ Lse smem[kWaves];
+    const int64_t r = blockIdx.x;
+    const int64_t o = r / a.n_inner, i = r - o * a.n_inner;
+    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+    const Lse t = row_online_lse<DT, TEMP>(row, a.vocab, a.tparam, smem);
+    if (threadIdx.x == 0) {
+        const float log_s = logf(t.s);
+        const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
+        float lp = 0.f;
+        if (tg >= a.vstart && tg < a.vend) {
+            const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(row, tg - a.vstart), a.tparam);
+            lp = (xt - t.m) - log_s;
+        }
+        logprob[r] = lp;
+        if (lse_out) lse_out[r] = t.m + log_s;
+    }
+}
+
+struct GradArgs {
+    const float* lse;
+    const float* grad;
+    int64_t gs_outer, gs_inner;
+    void* dlogits;
+    int64_t d_n_inner, ds_outer, ds_inner;
+};
+
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kBlock) void logprob_bwd_kernel(RowArgs a, GradArgs ga) {
+    const int64_t r = blockIdx.x;
+    const int64_t o = r / ga.d_n_inner, i = r - o * ga.d_n_inner;
+    char* out = static_cast<char*>(ga.dlogits) + (o * ga.ds_outer + i * ga.ds_inner) * Row<DT>::BYTES;
+    float g = 0.f;
+    if (i < a.n_inner) g = ga.grad[o * ga.gs_outer + i * ga.gs_inner];
+    if (g == 0.f) {  // dropped position or masked token: the gradient row is exactly zero
+        row_zero<DT>(out, a.vocab);
+        return;
+    }
+    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+    const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
+    const int64_t tloc = (tg >= a.vstart && tg < a.vend) ? tg - a.vstart : -1;
+    row_write_grad<DT, TEMP>(row, out, a.vocab, ga.lse[o * a.n_inner + i], g, tloc, a.tparam);
+}
+
+// ---------------------------------------------------------------------------------------------
+// packed sequences: row p of a [T, V] buffer belongs to the sequence s with cu[s] <= p < cu[s+1]
+// ---------------------------------------------------------------------------------------------
+struct PackedArgs {
+    const void* logits;
+    int64_t total, vocab, row_stride;
+    const int64_t* targets;
+    int pre_rolled;
+    const int32_t* cu;
+    int64_t n_seq, unpacked_seqlen, vstart, vend;
+    float tparam;
+};
+
+// sequence index of packed position p, or -1 if p lies outside every sequence
+__device__ __forceinline__ int64_t find_seq(const int32_t* cu, int64_t n_seq, int64_t p) {
+    if (n_seq <= 0 || p < cu[0] || p >= cu[n_seq]) return -1;
+    int64_t lo = 0, hi = n_seq;  // invariant: cu[lo] <= p < cu[hi]
+    while (hi - lo > 1) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (cu[mid] <= p) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+struct PackedPos {
+    int64_t seq, pos, len, start;
+};
+
+__device__ __forceinline__ PackedPos locate(const PackedArgs& a, int64_t p, PackedPos* sh) {
+    if (threadIdx.x == 0) {
+        PackedPos q;
+        q.seq = find_seq(a.cu, a.n_seq, p);
+        q.start = q.seq >= 0 ? a.cu[q.seq] : 0;
+        q.len = q.seq >= 0 ? a.cu[q.seq + 1] - q.start : 0;
+        q.pos = p - q.start;
+        *sh = q;
+    }
+    __syncthreads();
+    return *sh;
+}
+
+__device__ __forceinline__ int64_t packed_target(const PackedArgs& a, const PackedPos& q) {
+    const int64_t j = a.pre_rolled ? q.pos : (q.pos + 1 == q.len ? 0 : q.pos + 1);
+    return a.targets[q.start + j];
+}
+
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kBlock) void logprob_packed_fwd_kernel(PackedArgs a, float* __restrict__ out,
+                                                                    float* __restrict__ lse_out) {
+    __shared__ Lse smem[kWaves];
+    __shared__ PackedPos sh;
+    const int64_t p = blockIdx.x;
+    const PackedPos q = locate(a, p, &sh);
+    // positions whose logprob is never used still get an LSE only when the caller keeps it
+    const bool emitted = q.seq >= 0 && q.pos + 1 < q.len && q.pos < a.unpacked_seqlen - 1;
+    if (!emitted) {
+        if (lse_out && threadIdx.x == 0) lse_out[p] = 0.f;
+        return;
+    }
+    const char* row = static_cast<const char*>(a.logits) + p * a.row_stride * Row<DT>::BYTES;
+    const Lse t = row_online_lse<DT, TEMP>(row, a.vocab, a.tparam, smem);
+    if (threadIdx.x == 0) {
+        const float log_s = logf(t.s);
+        const int64_t tg = packed_target(a, q);
+        float lp = 0.f;
+        if (tg >= a.vstart && tg < a.vend) {
+            const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(row, tg - a.vstart), a.tparam);
+            lp = (xt - t.m) - log_s;
+        }
+        out[q.seq * (a.unpacked_seqlen - 1) + q.pos] = lp;
+        if (lse_out) lse_out[p] = t.m + log_s;
+    }
+}
+
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kBlock) void logprob_packed_bwd_kernel(PackedArgs a, const float* __restrict__ lse,
+                                                                    const float* __restrict__ grad, void* dlogits,
+                                                                    int64_t d_row_stride) {
+    __shared__ PackedPos sh;
+    const int64_t p = blockIdx.x;
+    const PackedPos q = locate(a, p, &sh);
+    char* out = static_cast<char*>(dlogits) + p * d_row_stride * Row<DT>::BYTES;
+    const bool emitted = q.seq >= 0 && q.pos + 1 < q.len && q.pos < a.unpacked_seqlen - 1;
+    const float g = emitted ? grad[q.seq * (a.unpacked_seqlen - 1) + q.pos] : 0.f;
+    if (g == 0.f) {
+        row_zero<DT>(out, a.vocab);
+        return;
+    }
+    const char* row = static_cast<const char*>(a.logits) + p * a.row_stride * Row<DT>::BYTES;
+    const int64_t tg = packed_target(a, q);
+    const int64_t tloc = (tg >= a.vstart && tg < a.vend) ? tg - a.vstart : -1;
+    row_write_grad<DT, TEMP>(row, out, a.vocab, lse[p], g, tloc, a.tparam);
+}
+
+// zero-fill of the unpacked [n_seq, L] output before the packed forward scatters into it
+__global__ void fill_zero_f32(float* p, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------
+static int temp_code(float temperature, int mode, float* tparam) {
+    if (temperature == 1.0f) { *tparam = 1.f; return 0; }
+    if (mode == NRL_TEMP_DIV) { *tparam = temperature; return 1; }
+    *tparam = 1.0f / temperature;
+    return 2;
+}
+
+static int check_rows(const nrl_rows* r) {
+    if (!r) return fail(NRL_E_INVALID, "rows is NULL");
+    if (r->dtype != NRL_F32 && r->dtype != NRL_BF16 && r->dtype != NRL_F16)
+        return fail(NRL_E_INVALID, "unknown logits dtype %d", r->dtype);
+    if (r->n_outer < 0 || r->n_inner < 0 || r->vocab <= 0)
+        return fail(NRL_E_INVALID, "bad shape [%lld, %lld, %lld]", (long long)r->n_outer, (long long)r->n_inner,
+                    (long long)r->vocab);
+    if (r->n_outer * r->n_inner > 0 && (!r->logits || !r->targets)) return fail(NRL_E_INVALID, "null logits or targets");
+    if (r->vocab_end - r->vocab_start != r->vocab)
+        return fail(NRL_E_INVALID, "vocab range [%lld, %lld) does not span %lld columns", (long long)r->vocab_start,
+                    (long long)r->vocab_end, (long long)r->vocab);
+    if (!(r->temperature > 0.f)) return fail(NRL_E_INVALID, "temperature must be positive");
+    if (r->temp_mode != NRL_TEMP_DIV && r->temp_mode != NRL_TEMP_RCP) return fail(NRL_E_INVALID, "bad temp_mode");
+    if (r->n_outer * r->n_inner >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    return NRL_OK;
+}
+
+static RowArgs make_row_args(const nrl_rows* r, float tparam) {
+    RowArgs a;
+    a.logits = r->logits;
+    a.n_inner = r->n_inner;
+    a.vocab = r->vocab;
+    a.stride_outer = r->stride_outer;
+    a.stride_inner = r->stride_inner;
+    a.targets = r->targets;
+    a.ts_outer = r->tgt_stride_outer;
+    a.ts_inner = r->tgt_stride_inner;
+    a.vstart = r->vocab_start;
+    a.vend = r->vocab_end;
+    a.tparam = tparam;
+    return a;
+}
+
+#define NRL_DISPATCH(DT_, TC_, ...)                                                         \
+    switch ((DT_) * 3 + (TC_)) {                                                            \
+        case NRL_F32 * 3 + 0: { constexpr int DT = NRL_F32, TEMP = 0; __VA_ARGS__; break; }        \
+        case NRL_F32 * 3 + 1: { constexpr int DT = NRL_F32, TEMP = 1; __VA_ARGS__; break; }        \
+        case NRL_F32 * 3 + 2: { constexpr int DT = NRL_F32, TEMP = 2; __VA_ARGS__; break; }        \
+        case NRL_BF16 * 3 + 0: { constexpr int DT = NRL_BF16, TEMP = 0; __VA_ARGS__; break; }      \
+        case NRL_BF16 * 3 + 1: { constexpr int DT = NRL_BF16, TEMP = 1; __VA_ARGS__; break; }      \
+        case NRL_BF16 * 3 + 2: { constexpr int DT = NRL_BF16, TEMP = 2; __VA_ARGS__; break; }      \
+        case NRL_F16 * 3 + 0: { constexpr int DT = NRL_F16, TEMP = 0; __VA_ARGS__; break; }        \
+        case NRL_F16 * 3 + 1: { constexpr int DT = NRL_F16, TEMP = 1; __VA_ARGS__; break; }        \
+        default: { constexpr int DT = NRL_F16, TEMP = 2; __VA_ARGS__; break; }                     \
+    }
+
+}  // namespace nrl
+
+using namespace nrl;
+
+extern "C" int nrl_logprob_fwd(const nrl_rows* rows, float* logprob_out, float* lse_out, void* stream) {
+    if (int e = check_rows(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!logprob_out) return fail(NRL_E_INVALID, "logprob_out is NULL");
+    float tparam;
+    const int tc = temp_code(rows->temperature, rows->temp_mode, &tparam);
+    const RowArgs a = make_row_args(rows, tparam);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(rows->dtype, tc, logprob_fwd_kernel<DT, TEMP><<<dim3((unsigned)n), dim3(kBlock), 0, s>>>(a, logprob_out, lse_out));
+    return check_launch("logprob_fwd");
+}
+
+extern "C" int nrl_logprob_bwd(const nrl_rows* rows, const float* lse, const float* grad, int64_t grad_stride_outer,
+                               int64_t grad_stride_inner, void* dlogits, int64_t d_n_inner, int64_t d_stride_outer,
+                               int64_t d_stride_inner, void* stream) {
+    if (int e = check_rows(rows)) return e;
+    if (d_n_inner < rows->n_inner) return fail(NRL_E_INVALID, "d_n_inner %lld < n_inner %lld", (long long)d_n_inner,
+                                               (long long)rows->n_inner);
+    const int64_t n = rows->n_outer * d_n_inner;
+    if (n == 0) return NRL_OK;
+    if (n >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    if (!dlogits || (rows->n_outer * rows->n_inner > 0 && (!lse || !grad)))
+        return fail(NRL_E_INVALID, "null lse, grad or dlogits");
+    float tparam;
+    const int tc = temp_code(rows->temperature, rows->temp_mode, &tparam);
+    const RowArgs a = make_row_args(rows, tparam);
+    GradArgs ga;
+    ga.lse = lse;
+    ga.grad = grad;
+    ga.gs_outer = grad_stride_outer;
+    ga.gs_inner = grad_stride_inner;
+    ga.dlogits = dlogits;
+    ga.d_n_inner = d_n_inner;
+    ga.ds_outer = d_stride_outer;
+    ga.ds_inner = d_stride_inner;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(rows->dtype, tc, logprob_bwd_kernel<DT, TEMP><<<dim3((unsigned)n), dim3(kBlock), 0, s>>>(a, ga));
+    return check_launch("logprob_bwd");
+}
+
+static int check_packed(const void* logits, int32_t dtype, int64_t total, int64_t vocab, const int64_t* targets,
+                        const int32_t* cu, int64_t n_seq, int64_t unpacked_seqlen, int64_t vstart, int64_t vend,
+                        float temperature, int32_t temp_mode) {
+    if (dtype != NRL_F32 && dtype != NRL_BF16 && dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype %d", dtype);
+    if (total < 0 || vocab <= 0 || n_seq < 0 || unpacked_seqlen < 1) return fail(NRL_E_INVALID, "bad packed shape");
+    if (total > 0 && (!logits || !targets || !cu)) return fail(NRL_E_INVALID, "null logits, targets or cu_seqlens");
+    if (vend - vstart != vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
+    if (!(temperature > 0.f)) return fail(NRL_E_INVALID, "temperature must be positive");
+    if (temp_mode != NRL_TEMP_DIV && temp_mode != NRL_TEMP_RCP) return fail(NRL_E_INVALID, "bad temp_mode");
+    if (total >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    return NRL_OK;
+}
+
+extern "C" int nrl_logprob_packed_fwd(const void* logits, int32_t dtype, int64_t total_tokens, int64_t vocab,
+                                      int64_t row_stride, const int64_t* targets, int32_t pre_rolled,
+                                      const int32_t* cu_seqlens, int64_t n_seq, int64_t unpacked_seqlen,
+                                      int64_t vocab_start, int64_t vocab_end, float temperature, int32_t temp_mode,
+                                      float* out, float* lse_out, void* stream) {
+    if (int e = check_packed(logits, dtype, total_tokens, vocab, targets, cu_seqlens, n_seq, unpacked_seqlen,
+                             vocab_start, vocab_end, temperature, temp_mode))
+        return e;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t n_out = n_seq * (unpacked_seqlen - 1);
+    if (n_out > 0) {
+        if (!out) return fail(NRL_E_INVALID, "out is NULL");
+        fill_zero_f32<<<dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s>>>(out, n_out);
+    }
+    if (total_tokens == 0 || n_out == 0) return check_launch("logprob_packed_fwd");
+    PackedArgs a;
+    a.logits = logits; a.total = total_tokens; a.vocab = vocab; a.row_stride = row_stride; a.targets = targets;
+    a.pre_rolled = pre_rolled; a.cu = cu_seqlens; a.n_seq = n_seq; a.unpacked_seqlen = unpacked_seqlen;
+    a.vstart = vocab_start; a.vend = vocab_end;
+    const int tc = temp_code(temperature, temp_mode, &a.tparam);
+    NRL_DISPATCH(dtype, tc,
+                 logprob_packed_fwd_kernel<DT, TEMP><<<dim3((unsigned)total_tokens), dim3(kBlock), 0, s>>>(a, out, lse_out));
+    return check_launch("logprob_packed_fwd");
+}
+
+extern "C" int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t total_tokens, int64_t vocab,
+                                      int64_t row_stride, const int64_t* targets, int32_t pre_rolled,
+                                      const int32_t* cu_seqlens, int64_t n_seq, int64_t unpacked_seqlen,
+                                      int64_t vocab_start, int64_t vocab_end, float temperature, int32_t temp_mode,
+                                      const float* lse, const float* grad, void* dlogits, int64_t d_row_stride,
+                                      void* stream) {
+    if (int e = check_packed(logits, dtype, total_tokens, vocab, targets, cu_seqlens, n_seq, unpacked_seqlen,
+                             vocab_start, vocab_end, temperature, temp_mode))
+        return e;
+    if (total_tokens == 0) return NRL_OK;
+    if (!dlogits || !lse || (n_seq * (unpacked_seqlen - 1) > 0 && !grad)) return fail(NRL_E_INVALID, "null lse, grad or dlogits");
+    PackedArgs a;
+    a.logits = logits; a.total = total_tokens; a.vocab = vocab; a.row_stride = row_stride; a.targets = targets;
+    a.pre_rolled = pre_rolled; a.cu = cu_seqlens; a.n_seq = n_seq; a.unpacked_seqlen = unpacked_seqlen;
+    a.vstart = vocab_start; a.vend = vocab_end;
+    const int tc = temp_code(temperature, temp_mode, &a.tparam);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(dtype, tc,
+                 logprob_packed_bwd_kernel<DT, TEMP><<<dim3((unsigned)total_tokens), dim3(kBlock), 0, s>>>(
+                     a, lse, grad, dlogits, d_row_stride));
+    return check_launch("logprob_packed_bwd");
+}

@@ -1,0 +1,298 @@
+"""Logits -> token log-probabilities on one MI355X.
+
+Single-GPU counterpart of ``nemo_rl/distributed/model_utils.py``: the same public names and
+argument lists, with the chain of PyTorch ops (fp32 cast, amax, exp, sum, log, gather and their
+backward) replaced by one streaming HIP kernel per direction (``torch.ops.rl_amd.logprob_fwd`` /
+``logprob_bwd``).  Tensor-parallel and context-parallel groups are accepted for signature
+compatibility but must span a single rank; this build runs on one GPU.
+
+What each function mirrors is cited as ``model_utils.py:<lines>`` of the reference file.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+
+from .. import ops as _ops  # noqa: F401  (registers torch.ops.rl_amd.*)
+from .._lib import NRL_TEMP_RCP
+from ..algorithms.logits_sampling_utils import (
+    TrainingSamplingParams,
+    need_top_k_or_top_p_filtering,
+)
+
+_OPS = torch.ops.rl_amd
+
+
+def _group_size(group) -> int:
+    if group is None or not torch.distributed.is_available() or not torch.distributed.is_initialized():
+        return 1
+    return torch.distributed.get_world_size(group)
+
+
+def _require_single_rank(group, what: str) -> None:
+    n = _group_size(group)
+    if n != 1:
+        raise NotImplementedError(
+            f"{what}: a {n}-rank process group was given; this build computes the full vocabulary on one GPU"
+        )
+
+
+def _to_device(t: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
+    return t if t.device == like.device else t.to(like.device)
+
+
+def _prep_rows(logits, targets):
+    if logits.dim() != 3:
+        raise ValueError(f"expected logits [B, S, V], got {tuple(logits.shape)}")
+    if logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    targets = _to_device(targets, logits)
+    if targets.dtype != torch.int64:
+        targets = targets.long()
+    return logits, targets
+
+
+def _fwd_rows(ctx, logits, targets, n_inner, vocab_start, vocab_end, inference_only, temperature):
+    """Shared forward: saves the logits (no copy), the targets and one fp32 log-sum-exp per row;
+    the softmax is never materialised."""
+    logits, targets = _prep_rows(logits.detach(), targets)
+    save = (not inference_only) and ctx.needs_input_grad[0]
+    out, lse = _OPS.logprob_fwd(logits, targets, n_inner, vocab_start, vocab_end, temperature, NRL_TEMP_RCP, save)
+    if save:
+        ctx.save_for_backward(logits, targets, lse)
+        ctx.meta = (n_inner, vocab_start, vocab_end, temperature)
+    ctx.saved = save
+    return out
+
+
+def _bwd_rows(ctx, grad_out):
+    """Shared backward: the gradient comes back in the logits' dtype, rows >= n_inner zeroed."""
+    if not ctx.saved:
+        raise RuntimeError("backward through a logprob computed with inference_only=True")
+    logits, targets, lse = ctx.saved_tensors
+    n_inner, vocab_start, vocab_end, temperature = ctx.meta
+    grad = grad_out if grad_out.dtype == torch.float32 else grad_out.float()
+    return _OPS.logprob_bwd(logits, targets, lse, grad, n_inner, vocab_start, vocab_end, temperature, NRL_TEMP_RCP)
+
+
+class _RowsLogprob(torch.autograd.Function):
+    """logits [B,S,V], targets [B,>=n_inner] (already aligned to the rows) -> fp32 [B,n_inner]."""
+
+    @staticmethod
+    def forward(ctx, logits, targets, n_inner, vocab_start, vocab_end, inference_only, temperature):
+        return _fwd_rows(ctx, logits, targets, n_inner, vocab_start, vocab_end, inference_only, temperature)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        return _bwd_rows(ctx, grad_out), None, None, None, None, None, None
+
+
+def _rows_logprob(logits, targets, n_inner, vocab_start, vocab_end, inference_only, temperature=1.0):
+    return _RowsLogprob.apply(logits, targets, n_inner, vocab_start, vocab_end, inference_only, float(temperature))
+
+
+class DistributedLogprob(torch.autograd.Function):
+    """``model_utils.py:120-207``.  ``apply(logits, target, vocab_start_index, vocab_end_index, group,
+    inference_only=False)`` with ``target`` already shifted; every position is computed."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, target, vocab_start_index, vocab_end_index, group, inference_only=False):
+        _require_single_rank(group, "DistributedLogprob")
+        return _fwd_rows(
+            ctx, vocab_parallel_logits, target, target.shape[1], vocab_start_index, vocab_end_index, inference_only, 1.0
+        )
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        return _bwd_rows(ctx, grad_outputs[0]), None, None, None, None, None
+
+
+class ChunkedDistributedLogprob(torch.autograd.Function):
+    """``model_utils.py:267-380``.  The sequence-chunk loop only bounds the reference's working set;
+    the streaming kernel has none, so ``chunk_size`` does not change the launch and chunked and
+    unchunked results are bit-identical."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, target, vocab_start_index, vocab_end_index, chunk_size, tp_group,
+                inference_only=False):
+        _require_single_rank(tp_group, "ChunkedDistributedLogprob")
+        if chunk_size is None or int(chunk_size) < 1:
+            raise ValueError(f"chunk_size must be a positive int, got {chunk_size}")
+        return _fwd_rows(
+            ctx, vocab_parallel_logits, target, target.shape[1], vocab_start_index, vocab_end_index, inference_only, 1.0
+        )
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        return _bwd_rows(ctx, grad_outputs[0]), None, None, None, None, None, None
+
+
+def _get_tokens_on_this_cp_rank(input_ids, cp_rank: int, cp_size: int, seq_dim: int = 1):
+    """``model_utils.py:1199-1233`` for the only context-parallel size this build runs with."""
+    if cp_size != 1:
+        raise NotImplementedError("context parallelism spans more than one GPU")
+    return input_ids
+
+
+def from_parallel_logits_to_logprobs(
+    vocab_parallel_logits: torch.Tensor,
+    target: torch.Tensor,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    tp_group: Any,
+    inference_only: bool = False,
+    cp_group: Optional[Any] = None,
+    chunk_size: Optional[int] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+) -> torch.Tensor:
+    """``model_utils.py:947-1042``: ``target`` is unshifted ``[B, S]``; returns ``[B, S-1]`` fp32.
+
+    The roll by -1 and the dropped last column become pointer arithmetic: row ``(b, i)`` reads
+    ``target[b, i+1]`` and only ``S-1`` rows per sequence are launched.  Logits longer than the
+    targets (context-parallel padding in the reference, ``:984-986``) are ignored beyond ``S``."""
+    _require_single_rank(tp_group, "from_parallel_logits_to_logprobs")
+    _require_single_rank(cp_group, "from_parallel_logits_to_logprobs")
+    b, s = target.shape
+    if vocab_parallel_logits.shape[1] < s:
+        raise ValueError(f"logits cover {vocab_parallel_logits.shape[1]} positions, targets {s}")
+    if need_top_k_or_top_p_filtering(sampling_params):
+        from .sampling_logprob import rows_logprob_sampled
+
+        return rows_logprob_sampled(
+            vocab_parallel_logits, target[:, 1:], s - 1, sampling_params.top_k, sampling_params.top_p, inference_only
+        )
+    if s - 1 == 0:
+        return torch.zeros((b, 0), dtype=torch.float32, device=vocab_parallel_logits.device)
+    return _rows_logprob(
+        vocab_parallel_logits, target[:, 1:], s - 1, vocab_start_index, vocab_end_index, inference_only
+    )
+
+
+def get_next_token_logprobs_from_logits(
+    input_ids: torch.Tensor,
+    next_token_logits: torch.Tensor,
+    seq_index: Optional[torch.Tensor] = None,
+    vocab_parallel_rank: Optional[int] = None,
+    vocab_parallel_group: Optional[Any] = None,
+    context_parallel_group: Optional[Any] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+    chunk_size: Optional[int] = None,
+) -> torch.Tensor:
+    """``model_utils.py:1611-1695``.  All three branches of the reference reduce to the same maths
+    on one GPU.  The reference first casts the logits to fp32 (``:1648-1649``); the kernel reads
+    bf16/fp16 directly and accumulates in fp32, which is the same arithmetic without the copy, and
+    autograd receives the gradient already narrowed (one rounding, as the cast's backward does)."""
+    if vocab_parallel_group is not None:
+        assert vocab_parallel_rank is not None, (
+            "vocab_parallel_rank must be provided when vocab_parallel_group is provided"
+        )
+        _require_single_rank(vocab_parallel_group, "get_next_token_logprobs_from_logits")
+    _require_single_rank(context_parallel_group, "get_next_token_logprobs_from_logits")
+    if seq_index is not None:
+        raise NotImplementedError("seq_index belongs to context-parallel DTensor logits (more than one GPU)")
+    if hasattr(next_token_logits, "to_local"):
+        next_token_logits = next_token_logits.to_local()
+    vocab = next_token_logits.shape[-1]
+    rank = vocab_parallel_rank or 0
+    inference_only = not (torch.is_grad_enabled() and next_token_logits.requires_grad)
+    return from_parallel_logits_to_logprobs(
+        next_token_logits,
+        input_ids,
+        vocab_start_index=rank * vocab,
+        vocab_end_index=(rank + 1) * vocab,
+        tp_group=vocab_parallel_group,
+        inference_only=inference_only,
+        cp_group=context_parallel_group,
+        chunk_size=None,
+        sampling_params=sampling_params,
+    )[:, : input_ids.shape[1] - 1]
+
+
+# ------------------------------------------------------------------------------------------------
+# packed sequences
+# ------------------------------------------------------------------------------------------------
+class _PackedLogprob(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, inference_only):
+        save = (not inference_only) and ctx.needs_input_grad[0]
+        out, lse = _OPS.logprob_packed_fwd(
+            logits2d.detach(), targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, 1.0,
+            NRL_TEMP_RCP, save,
+        )
+        if save:
+            ctx.save_for_backward(logits2d.detach(), targets1d, cu_dev, lse)
+            ctx.meta = (pre_rolled, unpacked_seqlen, vocab_start, vocab_end)
+        ctx.saved = save
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if not ctx.saved:
+            raise RuntimeError("backward through a logprob computed with inference_only=True")
+        logits2d, targets1d, cu_dev, lse = ctx.saved_tensors
+        pre_rolled, unpacked_seqlen, vocab_start, vocab_end = ctx.meta
+        d = _OPS.logprob_packed_bwd(
+            logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, 1.0, NRL_TEMP_RCP,
+            lse, grad_out.float(),
+        )
+        return d, None, None, None, None, None, None, None
+
+
+def _checked_cu_seqlens(cu_seqlens_padded: torch.Tensor, total: int, n_targets: int, device) -> torch.Tensor:
+    """One host read of the sequence boundaries (the reference reads them per sequence): they must be
+    non-decreasing and stay inside the packed buffers, because the kernels index with them."""
+    host = cu_seqlens_padded.detach().to("cpu", torch.int64)
+    if host.dim() != 1 or host.numel() < 1:
+        raise ValueError("cu_seqlens_padded must be a 1-D tensor with at least one entry")
+    if host.numel() > 1 and bool((host[1:] < host[:-1]).any()):
+        raise ValueError("cu_seqlens_padded must be non-decreasing")
+    if int(host[0]) < 0 or int(host[-1]) > total or int(host[-1]) > n_targets:
+        raise ValueError(
+            f"cu_seqlens_padded spans [{int(host[0])}, {int(host[-1])}) but the packed row has {total} positions "
+            f"and {n_targets} targets"
+        )
+    return host.to(torch.int32).to(device)
+
+
+def from_parallel_logits_to_logprobs_packed_sequences(
+    vocab_parallel_logits: torch.Tensor,
+    target: torch.Tensor,
+    cu_seqlens_padded: torch.Tensor,
+    unpacked_seqlen: int,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    group: Any,
+    inference_only: bool = False,
+    cp_group: Optional[Any] = None,
+    chunk_size: Optional[int] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+    target_is_pre_rolled: bool = False,
+) -> torch.Tensor:
+    """``model_utils.py:1045-1196``: packed ``[1, T, V]`` logits -> unpacked ``[B, unpacked_seqlen-1]``.
+
+    The per-sequence roll, the dropped last position of every sequence and the unpacking are index
+    arithmetic inside the kernel (a binary search of ``cu_seqlens_padded`` per row); positions that
+    never reach the output are not read at all."""
+    _require_single_rank(group, "from_parallel_logits_to_logprobs_packed_sequences")
+    _require_single_rank(cp_group, "from_parallel_logits_to_logprobs_packed_sequences")
+    if vocab_parallel_logits.dim() != 3 or vocab_parallel_logits.shape[0] != 1:
+        raise ValueError(f"expected packed logits [1, T, V], got {tuple(vocab_parallel_logits.shape)}")
+    logits2d = vocab_parallel_logits.squeeze(0)
+    if logits2d.stride(-1) != 1:
+        logits2d = logits2d.contiguous()
+    targets1d = _to_device(target, logits2d).reshape(-1).long().contiguous()
+    total = logits2d.shape[0]
+    cu_dev = _checked_cu_seqlens(cu_seqlens_padded, total, targets1d.shape[0], logits2d.device)
+    if need_top_k_or_top_p_filtering(sampling_params):
+        from .sampling_logprob import packed_logprob_sampled
+
+        return packed_logprob_sampled(
+            logits2d, targets1d, target_is_pre_rolled, cu_dev, int(unpacked_seqlen), sampling_params.top_k,
+            sampling_params.top_p, inference_only,
+        )
+    return _PackedLogprob.apply(
+        logits2d, targets1d, bool(target_is_pre_rolled), cu_dev, int(unpacked_seqlen), vocab_start_index,
+        vocab_end_index, inference_only,
+    )

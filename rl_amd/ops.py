@@ -1,0 +1,342 @@
+"""PyTorch custom ops (``torch.ops.rl_amd.*``) over the C-ABI HIP library.
+
+PyTorch supplies device memory and the current stream; every computation is a kernel in
+``librl_amd_hip.so``.  Each op validates shapes on the host before a launch and raises on
+anything the kernels do not assume (CPU tensors, non-contiguous vocabulary axis, wrong dtype).
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.NRL_F32, torch.bfloat16: _lib.NRL_BF16, torch.float16: _lib.NRL_F16}
+
+_LIB = torch.library.Library("rl_amd", "DEF")
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _need_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("rl_amd ops run on the GPU only (got a CPU tensor); there is no CPU fallback")
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise ValueError(f"unsupported logits dtype {t.dtype}") from None
+
+
+def _rows(logits, targets, n_inner, vocab_start, vocab_end, temperature, temp_mode) -> _lib.NrlRows:
+    """logits [B, S, V] (unit stride on V), targets [B, >= n_inner] int64 view."""
+    if logits.dim() != 3 or targets.dim() != 2:
+        raise ValueError(f"expected logits [B,S,V] and targets [B,S'], got {tuple(logits.shape)}, {tuple(targets.shape)}")
+    if logits.stride(2) != 1 and logits.shape[2] > 1:
+        raise ValueError("the vocabulary axis of the logits must be contiguous")
+    if targets.dtype != torch.int64:
+        raise ValueError(f"targets must be int64, got {targets.dtype}")
+    b, s, v = logits.shape
+    if targets.shape[0] != b or n_inner > s or n_inner > targets.shape[1] or n_inner < 0:
+        raise ValueError(
+            f"rows [{b}, {n_inner}] do not fit logits {tuple(logits.shape)} / targets {tuple(targets.shape)}"
+        )
+    r = _lib.NrlRows()
+    r.logits = logits.data_ptr()
+    r.dtype = _dtype_code(logits)
+    r.n_outer, r.n_inner, r.vocab = b, n_inner, v
+    r.stride_outer, r.stride_inner = logits.stride(0), logits.stride(1)
+    r.targets = targets.data_ptr()
+    r.tgt_stride_outer, r.tgt_stride_inner = targets.stride(0), targets.stride(1)
+    r.vocab_start, r.vocab_end = vocab_start, vocab_end
+    r.temperature, r.temp_mode = temperature, temp_mode
+    return r
+
+
+# ------------------------------------------------------------------------------------------------
+# K1 / K2
+# ------------------------------------------------------------------------------------------------
+_LIB.define(
+    "logprob_fwd(Tensor logits, Tensor targets, int n_inner, int vocab_start, int vocab_end, "
+    "float temperature, int temp_mode, bool save_lse) -> (Tensor, Tensor)"
+)
+_LIB.define(
+    "logprob_bwd(Tensor logits, Tensor targets, Tensor lse, Tensor grad, int n_inner, int vocab_start, "
+    "int vocab_end, float temperature, int temp_mode) -> Tensor"
+)
+_LIB.define(
+    "logprob_bwd_(Tensor(a!) logits, Tensor targets, Tensor lse, Tensor grad, int n_inner, int vocab_start, "
+    "int vocab_end, float temperature, int temp_mode) -> ()"
+)
+
+
+def _logprob_fwd(logits, targets, n_inner, vocab_start, vocab_end, temperature, temp_mode, save_lse):
+    _need_gpu(logits, targets)
+    rows = _rows(logits, targets, n_inner, vocab_start, vocab_end, temperature, temp_mode)
+    b = logits.shape[0]
+    with torch.cuda.device(logits.device):
+        out = torch.empty((b, n_inner), dtype=torch.float32, device=logits.device)
+        lse = torch.empty((b, n_inner) if save_lse else (0,), dtype=torch.float32, device=logits.device)
+        code = _lib.load().nrl_logprob_fwd(C.byref(rows), _ptr(out), _ptr(lse if save_lse else None), _stream())
+    _lib.check(code, "nrl_logprob_fwd")
+    return out, lse
+
+
+def _logprob_bwd(logits, targets, lse, grad, n_inner, vocab_start, vocab_end, temperature, temp_mode, in_place=False):
+    _need_gpu(logits, targets, lse, grad)
+    rows = _rows(logits, targets, n_inner, vocab_start, vocab_end, temperature, temp_mode)
+    b, s, v = logits.shape
+    if tuple(lse.shape) != (b, n_inner) or not lse.is_contiguous() or lse.dtype != torch.float32:
+        raise ValueError("lse must be a contiguous fp32 [B, n_inner] tensor")
+    if tuple(grad.shape) != (b, n_inner) or grad.dtype != torch.float32:
+        raise ValueError(f"grad must be fp32 [B, n_inner], got {grad.dtype} {tuple(grad.shape)}")
+    with torch.cuda.device(logits.device):
+        d = logits if in_place else torch.empty((b, s, v), dtype=logits.dtype, device=logits.device)
+        code = _lib.load().nrl_logprob_bwd(
+            C.byref(rows), _ptr(lse), _ptr(grad), grad.stride(0), grad.stride(1),
+            _ptr(d), s, d.stride(0), d.stride(1), _stream(),
+        )
+    _lib.check(code, "nrl_logprob_bwd")
+    return d
+
+
+def _logprob_bwd_inplace(logits, targets, lse, grad, n_inner, vocab_start, vocab_end, temperature, temp_mode):
+    """The gradient overwrites the logits buffer (for callers that no longer need the logits)."""
+    _logprob_bwd(logits, targets, lse, grad, n_inner, vocab_start, vocab_end, temperature, temp_mode, in_place=True)
+
+
+for _name, _fn in (("logprob_fwd", _logprob_fwd), ("logprob_bwd", _logprob_bwd), ("logprob_bwd_", _logprob_bwd_inplace)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")  # raises: there is no CPU path
+
+
+# ------------------------------------------------------------------------------------------------
+# packed sequences
+# ------------------------------------------------------------------------------------------------
+_LIB.define(
+    "logprob_packed_fwd(Tensor logits, Tensor targets, bool pre_rolled, Tensor cu_seqlens, int unpacked_seqlen, "
+    "int vocab_start, int vocab_end, float temperature, int temp_mode, bool save_lse) -> (Tensor, Tensor)"
+)
+_LIB.define(
+    "logprob_packed_bwd(Tensor logits, Tensor targets, bool pre_rolled, Tensor cu_seqlens, int unpacked_seqlen, "
+    "int vocab_start, int vocab_end, float temperature, int temp_mode, Tensor lse, Tensor grad) -> Tensor"
+)
+
+
+def _check_packed(logits, targets, cu_seqlens, unpacked_seqlen):
+    _need_gpu(logits, targets, cu_seqlens)
+    if logits.dim() != 2 or (logits.stride(1) != 1 and logits.shape[1] > 1):
+        raise ValueError("packed logits must be [T, V] with a contiguous vocabulary axis")
+    if targets.dtype != torch.int64 or targets.dim() != 1 or not targets.is_contiguous():
+        raise ValueError("packed targets must be a contiguous int64 [T] tensor")
+    if targets.shape[0] < logits.shape[0]:
+        raise ValueError(f"{targets.shape[0]} targets for {logits.shape[0]} packed positions")
+    if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or not cu_seqlens.is_contiguous():
+        raise ValueError("cu_seqlens must be a contiguous int32 [n_seq+1] tensor")
+    if cu_seqlens.shape[0] < 1 or unpacked_seqlen < 1:
+        raise ValueError("cu_seqlens needs at least one entry and unpacked_seqlen >= 1")
+
+
+def _logprob_packed_fwd(logits, targets, pre_rolled, cu_seqlens, unpacked_seqlen, vocab_start, vocab_end,
+                        temperature, temp_mode, save_lse):
+    _check_packed(logits, targets, cu_seqlens, unpacked_seqlen)
+    t, v = logits.shape
+    n_seq = cu_seqlens.shape[0] - 1
+    with torch.cuda.device(logits.device):
+        out = torch.empty((n_seq, unpacked_seqlen - 1), dtype=torch.float32, device=logits.device)
+        lse = torch.empty((t,) if save_lse else (0,), dtype=torch.float32, device=logits.device)
+        code = _lib.load().nrl_logprob_packed_fwd(
+            _ptr(logits), _dtype_code(logits), t, v, logits.stride(0), _ptr(targets), int(pre_rolled),
+            _ptr(cu_seqlens), n_seq, unpacked_seqlen, vocab_start, vocab_end, temperature, temp_mode,
+            _ptr(out), _ptr(lse if save_lse else None), _stream(),
+        )
+    _lib.check(code, "nrl_logprob_packed_fwd")
+    return out, lse
+
+
+def _logprob_packed_bwd(logits, targets, pre_rolled, cu_seqlens, unpacked_seqlen, vocab_start, vocab_end,
+                        temperature, temp_mode, lse, grad):
+    _check_packed(logits, targets, cu_seqlens, unpacked_seqlen)
+    _need_gpu(lse, grad)
+    t, v = logits.shape
+    n_seq = cu_seqlens.shape[0] - 1
+    if tuple(lse.shape) != (t,) or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise ValueError("lse must be a contiguous fp32 [T] tensor")
+    if tuple(grad.shape) != (n_seq, unpacked_seqlen - 1) or grad.dtype != torch.float32:
+        raise ValueError("grad must be fp32 [n_seq, unpacked_seqlen-1]")
+    grad = grad.contiguous()
+    with torch.cuda.device(logits.device):
+        d = torch.empty((t, v), dtype=logits.dtype, device=logits.device)
+        code = _lib.load().nrl_logprob_packed_bwd(
+            _ptr(logits), _dtype_code(logits), t, v, logits.stride(0), _ptr(targets), int(pre_rolled),
+            _ptr(cu_seqlens), n_seq, unpacked_seqlen, vocab_start, vocab_end, temperature, temp_mode,
+            _ptr(lse), _ptr(grad), _ptr(d), d.stride(0), _stream(),
+        )
+    _lib.check(code, "nrl_logprob_packed_bwd")
+    return d
+
+
+for _name, _fn in (("logprob_packed_fwd", _logprob_packed_fwd), ("logprob_packed_bwd", _logprob_packed_bwd)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
+# ------------------------------------------------------------------------------------------------
+# K4
+# ------------------------------------------------------------------------------------------------
+_LIB.define(
+    "grpo_loss(Tensor lp, Tensor? lpu, Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, Tensor token_mask, "
+    "Tensor sample_mask, Tensor? correct_mask, Tensor global_valid, int[] iflags, float[] fparams) "
+    "-> (Tensor, Tensor, Tensor, Tensor)"
+)
+_LIB.define(
+    "nll_loss(Tensor lp, Tensor token_mask, Tensor sample_mask, Tensor global_valid) -> (Tensor, Tensor, Tensor)"
+)
+
+_CFG_INT = [n for n, _ in _lib.NrlGrpoCfg._fields_[:14]]
+_CFG_FLT = [n for n, _ in _lib.NrlGrpoCfg._fields_[14:]]
+
+
+def _rowmat(t, b, n, name):
+    """fp32 [B, n] with unit column stride -> (tensor kept alive, row stride)."""
+    if t is None:
+        return None, 0
+    if t.dtype != torch.float32 or tuple(t.shape) != (b, n):
+        raise ValueError(f"{name} must be fp32 [{b}, {n}], got {t.dtype} {tuple(t.shape)}")
+    if n > 1 and t.stride(1) != 1:
+        t = t.contiguous()
+    return t, (t.stride(0) if b > 1 else n)
+
+
+def _vec(t, b, name):
+    if t is None:
+        return None
+    if t.dtype != torch.float32 or tuple(t.shape) != (b,):
+        raise ValueError(f"{name} must be fp32 [{b}], got {t.dtype} {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def _grpo_inputs(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_mask, global_valid):
+    _need_gpu(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_mask, global_valid)
+    if lp.dim() != 2:
+        raise ValueError(f"logprobs must be [B, S-1], got {tuple(lp.shape)}")
+    b, n = lp.shape
+    keep = []
+    inp = _lib.NrlGrpoInputs()
+    inp.batch, inp.sm1 = b, n
+    for field, t in (("lp", lp), ("lpu", lpu), ("prev", prev), ("gen", gen), ("ref", ref), ("adv", adv),
+                     ("token_mask", token_mask)):
+        t, stride = _rowmat(t, b, n, field)
+        keep.append(t)
+        setattr(inp, field, 0 if t is None else t.data_ptr())
+        setattr(inp, field + "_stride", stride)
+    sm, cm = _vec(sample_mask, b, "sample_mask"), _vec(correct_mask, b, "correct_mask")
+    if global_valid.dtype != torch.float32 or tuple(global_valid.shape) != (2,):
+        raise ValueError("global_valid must be fp32 [2] = (valid_seqs, valid_toks)")
+    gv = global_valid.contiguous()
+    keep += [sm, cm, gv]
+    inp.sample_mask = sm.data_ptr()
+    inp.correct_mask = 0 if cm is None else cm.data_ptr()
+    inp.global_valid = gv.data_ptr()
+    return inp, keep, b, n
+
+
+def _grpo_loss(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_mask, global_valid, iflags, fparams):
+    if len(iflags) != len(_CFG_INT) or len(fparams) != len(_CFG_FLT):
+        raise ValueError("malformed loss configuration")
+    inp, keep, b, n = _grpo_inputs(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_mask, global_valid)
+    cfg = _lib.NrlGrpoCfg()
+    for name, v in zip(_CFG_INT, iflags):
+        setattr(cfg, name, int(v))
+    for name, v in zip(_CFG_FLT, fparams):
+        setattr(cfg, name, float(v))
+    lib = _lib.load()
+    dev = lp.device
+    split = lpu is not None and cfg.has_kl
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dlp = torch.empty((b, n), dtype=torch.float32, device=dev)
+        dlpu = torch.empty((b, n) if split else (0,), dtype=torch.float32, device=dev)
+        metrics = torch.empty((_lib.NRL_GRPO_N_METRICS,), dtype=torch.float32, device=dev)
+        ws_bytes = lib.nrl_grpo_loss_workspace_bytes(b)
+        ws = torch.empty((ws_bytes // 8,), dtype=torch.float64, device=dev)
+        code = lib.nrl_grpo_loss_fwd_bwd(
+            C.byref(cfg), C.byref(inp), _ptr(loss), _ptr(dlp), _ptr(dlpu if split else None), _ptr(metrics),
+            _ptr(ws), ws_bytes, _stream(),
+        )
+    _lib.check(code, "nrl_grpo_loss_fwd_bwd")
+    del keep
+    return loss, dlp, dlpu, metrics
+
+
+def _nll_loss(lp, token_mask, sample_mask, global_valid):
+    inp, keep, b, n = _grpo_inputs(lp, None, None, None, None, None, token_mask, sample_mask, None, global_valid)
+    lib = _lib.load()
+    dev = lp.device
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dlp = torch.empty((b, n), dtype=torch.float32, device=dev)
+        metrics = torch.empty((3,), dtype=torch.float32, device=dev)
+        ws_bytes = lib.nrl_grpo_loss_workspace_bytes(b)
+        ws = torch.empty((ws_bytes // 8,), dtype=torch.float64, device=dev)
+        code = lib.nrl_nll_loss_fwd_bwd(C.byref(inp), _ptr(loss), _ptr(dlp), _ptr(metrics), _ptr(ws), ws_bytes, _stream())
+    _lib.check(code, "nrl_nll_loss_fwd_bwd")
+    del keep
+    return loss, dlp, metrics
+
+
+for _name, _fn in (("grpo_loss", _grpo_loss), ("nll_loss", _nll_loss)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
+# ------------------------------------------------------------------------------------------------
+# K5
+# ------------------------------------------------------------------------------------------------
+_LIB.define(
+    "group_baseline_std(Tensor prompts, Tensor rewards, Tensor valid, Tensor? std_rewards, bool leave_one_out, "
+    "bool normalize) -> (Tensor, Tensor, Tensor, Tensor)"
+)
+
+
+def _group_baseline_std(prompts, rewards, valid, std_rewards, leave_one_out, normalize):
+    _need_gpu(prompts, rewards, valid, std_rewards)
+    if prompts.dim() == 1:
+        prompts = prompts.unsqueeze(-1)
+    if prompts.dim() != 2 or prompts.dtype != torch.int64:
+        raise ValueError(f"prompts must be int64 [B, Sp], got {prompts.dtype} {tuple(prompts.shape)}")
+    b, sp = prompts.shape
+    if sp > 1 and prompts.stride(1) != 1:
+        prompts = prompts.contiguous()
+    rewards, valid, std_rewards = _vec(rewards, b, "rewards"), _vec(valid, b, "valid_mask"), _vec(std_rewards, b, "std_rewards")
+    lib = _lib.load()
+    dev = rewards.device
+    with torch.cuda.device(dev):
+        baseline = torch.empty((b,), dtype=torch.float32, device=dev)
+        std = torch.empty((b,), dtype=torch.float32, device=dev)
+        adv = torch.empty((b,), dtype=torch.float32, device=dev)
+        group = torch.empty((b,), dtype=torch.int32, device=dev)
+        ws_bytes = lib.nrl_group_workspace_bytes(b)
+        ws = torch.empty(((ws_bytes + 7) // 8,), dtype=torch.float64, device=dev)
+        code = lib.nrl_group_baseline_std(
+            _ptr(prompts), b, sp, prompts.stride(0) if b > 1 else sp, _ptr(rewards), _ptr(valid), _ptr(std_rewards),
+            int(leave_one_out), int(normalize), _ptr(baseline), _ptr(std), _ptr(adv), _ptr(group), _ptr(ws),
+            ws.numel() * 8, _stream(),
+        )
+    _lib.check(code, "nrl_group_baseline_std")
+    return baseline, std, adv, group
+
+
+_LIB.impl("group_baseline_std", _group_baseline_std, "CUDA")
+_LIB.impl("group_baseline_std", _group_baseline_std, "CPU")

@@ -1,0 +1,341 @@
+"""GPU parity: fused HIP GRPO loss and advantage kernels against the golden vectors of the
+reference's unit tests and against the CPU oracle (loss and gradients within 1e-4 relative;
+masks, counts and group indices exact)."""
+
+import math
+
+import pytest
+import torch
+
+from helpers import exact_logits_for_logprobs, golden_case_to_inputs, load_golden, synthetic_grpo_batch
+from oracle import advantage as OA
+from oracle import logprob as OL
+from oracle import loss as O
+from rl_amd.algorithms.advantage_estimator import AdvEstimatorConfig, GRPOAdvantageEstimator
+from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn, NLLLossFn, prepare_loss_input
+from rl_amd.algorithms.utils import calculate_baseline_and_std_per_prompt
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+PG = load_golden("clipped_pg_cases.json")
+BASE = load_golden("baseline_cases.json")
+ADV = load_golden("grpo_adv_cases.json")
+
+
+def _to_dev(data):
+    return {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in data.items()}
+
+
+def _close(a, b, rel=1e-4, abs_=1e-6):
+    if math.isinf(b) or math.isinf(a):
+        return a == b
+    return abs(a - b) <= rel * abs(b) + abs_
+
+
+@pytest.mark.parametrize("case", PG["cases"], ids=[c["name"] for c in PG["cases"]])
+def test_golden_cases_through_prepare_and_loss(case):
+    """Same flow as the reference's tests: exact logits -> prepare_loss_input -> loss."""
+    lp, data, gs, gt = golden_case_to_inputs(case)
+    vocab = 8
+    data["input_ids"] = torch.randint(0, vocab, data["input_ids"].shape, generator=torch.Generator().manual_seed(1))
+    logits = exact_logits_for_logprobs(lp, data["input_ids"], vocab)
+    fn = ClippedPGLossFn(ClippedPGLossConfig(**case["cfg"]))
+    ddev = _to_dev(data)
+    loss_input, ddev = prepare_loss_input(logits.to(DEV).requires_grad_(True), ddev, fn)
+    torch.testing.assert_close(loss_input["next_token_logprobs"].detach().cpu(), lp, rtol=1e-5, atol=1e-5)
+    loss, metrics = fn(data=ddev, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    assert loss.is_cuda and loss.dim() == 0
+    if "expected_loss" in case:
+        exp = case["expected_loss"]
+        assert abs(loss.item() - exp) <= case.get("rtol", 0.0) * abs(exp) + case.get("atol", 1e-6)
+        assert metrics["loss"] == pytest.approx(loss.item())
+    for k, v in case.get("expected_metrics_exact", {}).items():
+        assert metrics[k] == v, (k, metrics[k])
+    for k, v in case.get("expected_metrics_approx", {}).items():
+        assert metrics[k] == pytest.approx(v, rel=1e-5)
+    if case.get("property") == "loss is finite":
+        assert math.isfinite(loss.item())
+    # and against the oracle on the same inputs: loss, every metric, gradient
+    lpo = lp.clone().requires_grad_(True)
+    want, wm = O.clipped_pg_loss(O.LossConfig(**case["cfg"]), lpo, data, gs, gt)
+    if math.isfinite(want.item()):
+        assert _close(loss.item(), want.item())
+    assert set(metrics) == set(wm)
+    for k in wm:
+        assert _close(float(metrics[k]), float(wm[k])), (k, metrics[k], wm[k])
+    lpg = lp.to(DEV).requires_grad_(True)
+    l2, _ = fn(next_token_logprobs=lpg, data=ddev, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV))
+    l2.backward()
+    if lpo.requires_grad and want.requires_grad and math.isfinite(want.item()):
+        want.backward()
+        torch.testing.assert_close(lpg.grad.cpu(), lpo.grad, rtol=1e-4, atol=1e-7)
+
+
+def test_zero_mask_gives_exact_zero_and_sentinels():
+    lp, data, gs, gt = golden_case_to_inputs(PG["cases"][0])
+    data["token_mask"] = torch.zeros_like(data["token_mask"])
+    gt = torch.sum(data["sample_mask"].unsqueeze(-1) * data["token_mask"])
+    fn = ClippedPGLossFn(ClippedPGLossConfig(reference_policy_kl_penalty=0.1))
+    loss, m = fn(lp.to(DEV), _to_dev(data), gs.to(DEV), gt.to(DEV))
+    assert loss.item() == 0.0
+    assert m["probs_ratio_min"] == float("inf") and m["probs_ratio_max"] == float("-inf")
+
+
+@pytest.mark.parametrize("approx", [False, True])
+def test_kl_gradient_includes_sampling_term(approx):
+    c = PG["kl_gradient_case"]
+    t = lambda k: torch.tensor(c[k])  # noqa: E731
+    z = torch.zeros(1, 1)
+
+    def grad(beta):
+        lp = t("curr").to(DEV).requires_grad_(True)
+        data = _to_dev({
+            "token_mask": torch.tensor([[0, 1, 1]]), "sample_mask": torch.tensor([1]),
+            "advantages": torch.cat([z, t("adv")], -1), "prev_logprobs": torch.cat([z, t("prev")], -1),
+            "generation_logprobs": torch.cat([z, t("gen")], -1),
+            "reference_policy_logprobs": torch.cat([z, t("ref")], -1),
+        })
+        fn = ClippedPGLossFn(ClippedPGLossConfig(reference_policy_kl_penalty=beta, use_on_policy_kl_approximation=approx))
+        loss, _ = fn(next_token_logprobs=lp, data=data, global_valid_seqs=torch.tensor(1), global_valid_toks=torch.tensor(2))
+        loss.backward()
+        return lp.grad.cpu()
+
+    got = grad(c["beta"]) - grad(0.0)
+    logr = t("ref") - t("curr")
+    kl = torch.exp(logr) - 1 - logr
+    w = torch.exp(t("curr") - t("gen")) if approx else torch.ones_like(logr)
+    torch.testing.assert_close(got, c["beta"] * w * (kl + 1 - torch.exp(logr)) / 2, rtol=1e-4, atol=1e-7)
+
+
+CONFIG_MATRIX = [
+    dict(),
+    dict(reference_policy_kl_penalty=0.05, reference_policy_kl_type="k1"),
+    dict(reference_policy_kl_penalty=0.05, reference_policy_kl_type="k2", kl_input_clamp_value=0.05, kl_output_clamp_value=0.001),
+    dict(reference_policy_kl_penalty=0.05, kl_input_clamp_value=None, kl_output_clamp_value=None, use_on_policy_kl_approximation=True),
+    dict(token_level_loss=False, reference_policy_kl_penalty=0.001),
+    dict(token_level_loss=False, sequence_level_importance_ratios=True, use_importance_sampling_correction=True),
+    dict(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0),
+    dict(ratio_clip_c=3.0, use_importance_sampling_correction=True),
+    dict(use_cispo=True, use_importance_sampling_correction=True),
+    dict(disable_ppo_ratio=True),
+    dict(force_on_policy_ratio=True, reference_policy_kl_penalty=0.02),
+    dict(use_importance_sampling_correction=True, truncated_importance_sampling_type="tis", truncated_importance_sampling_ratio=1.02),
+    dict(use_importance_sampling_correction=True, truncated_importance_sampling_type="icepop",
+         truncated_importance_sampling_ratio=1.03, truncated_importance_sampling_ratio_min=0.97),
+    dict(use_importance_sampling_correction=True, truncated_importance_sampling_type="seq-mask-tis",
+         truncated_importance_sampling_ratio=1.002, truncated_importance_sampling_ratio_min=0.998),
+    dict(token_level_loss=False, use_importance_sampling_correction=True, truncated_importance_sampling_type="tis",
+         truncated_importance_sampling_ratio=1.5, truncated_importance_sampling_ratio_min=0.5, sequence_level_importance_ratios=True),
+    dict(positive_example_nll_weight=0.3),
+]
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.int64, torch.float32])
+@pytest.mark.parametrize("cfg", CONFIG_MATRIX, ids=[str(i) for i in range(len(CONFIG_MATRIX))])
+def test_random_batches_match_oracle(cfg, mask_dtype):
+    g = torch.Generator().manual_seed(100 + len(cfg))
+    b, s = 6, 300
+    lp = -torch.rand(b, s - 1, generator=g) * 3
+    noise = lambda: torch.cat([torch.zeros(b, 1), lp + 0.05 * torch.randn(b, s - 1, generator=g)], 1)  # noqa: E731
+    tm = torch.zeros(b, s, dtype=mask_dtype)
+    for i in range(b):
+        tm[i, int(torch.randint(1, s - 1, (1,), generator=g)):] = 1
+    tm[3] = 0  # a sequence without any valid token
+    data = {
+        "token_mask": tm, "sample_mask": torch.tensor([1, 1, 0, 1, 1, 1], dtype=mask_dtype),
+        "advantages": torch.randn(b, 1, generator=g).expand(b, s), "prev_logprobs": noise(),
+        "generation_logprobs": noise(), "reference_policy_logprobs": noise(),
+        "rewards": torch.tensor([1.0, 0.0, 1.0, 0.0, 1.0, 1.0]),
+    }
+    gs = data["sample_mask"].sum()
+    gt = (data["token_mask"][:, 1:] * data["sample_mask"].unsqueeze(-1)).sum() * 2  # pretend a second microbatch
+    lpo = lp.clone().requires_grad_(True)
+    want, wm = O.clipped_pg_loss(O.LossConfig(**cfg), lpo, data, gs, gt)
+    want.backward()
+    lpg = lp.to(DEV).requires_grad_(True)
+    got, gm = ClippedPGLossFn(ClippedPGLossConfig(**cfg))(lpg, _to_dev(data), gs.to(DEV), gt.to(DEV))
+    (got * 3.0).backward()
+    assert _close(got.item(), want.item()), (got.item(), want.item())
+    assert set(gm) == set(wm)
+    for k in wm:
+        assert _close(float(gm[k]), float(wm[k]), rel=1e-4, abs_=1e-7), (k, gm[k], wm[k])
+    assert type(gm["num_valid_samples"]) is type(wm["num_valid_samples"])
+    scale = lpo.grad.abs().max().item()
+    assert (lpg.grad.cpu() / 3.0 - lpo.grad).abs().max().item() <= 1e-4 * scale
+
+
+def test_unfiltered_logprobs_get_their_own_gradient():
+    g = torch.Generator().manual_seed(3)
+    b, s = 3, 40
+    lp = -torch.rand(b, s - 1, generator=g)
+    lpu = lp - 0.1 * torch.rand(b, s - 1, generator=g)
+    base = {
+        "token_mask": torch.cat([torch.zeros(b, 1), torch.ones(b, s - 1)], 1), "sample_mask": torch.ones(b),
+        "advantages": torch.randn(b, s, generator=g), "prev_logprobs": -torch.rand(b, s, generator=g),
+        "generation_logprobs": -torch.rand(b, s, generator=g), "reference_policy_logprobs": -torch.rand(b, s, generator=g),
+    }
+    cfg = dict(reference_policy_kl_penalty=0.1)
+    a, u = lp.clone().requires_grad_(True), lpu.clone().requires_grad_(True)
+    want, _ = O.clipped_pg_loss(O.LossConfig(**cfg), a, {**base, "curr_logprobs_unfiltered": u}, torch.tensor(3.0), torch.tensor(117.0))
+    want.backward()
+    ag, ug = lp.to(DEV).requires_grad_(True), lpu.to(DEV).requires_grad_(True)
+    got, _ = ClippedPGLossFn(ClippedPGLossConfig(**cfg))(
+        ag, {**_to_dev(base), "curr_logprobs_unfiltered": ug}, torch.tensor(3.0), torch.tensor(117.0))
+    got.backward()
+    assert _close(got.item(), want.item())
+    torch.testing.assert_close(ag.grad.cpu(), a.grad, rtol=1e-4, atol=1e-8)
+    torch.testing.assert_close(ug.grad.cpu(), u.grad, rtol=1e-4, atol=1e-8)
+
+
+def test_split_rescale_matches_sync_normalisation():
+    # tests/unit/algorithms/test_loss_functions.py:2768-2838 of the reference
+    from rl_amd.algorithms.loss import MetricNormalizer
+
+    torch.manual_seed(1234)
+    cfg = ClippedPGLossConfig(token_level_loss=True, use_importance_sampling_correction=True,
+                              truncated_importance_sampling_type="seq-mask-tis",
+                              truncated_importance_sampling_ratio=1.5, truncated_importance_sampling_ratio_min=0.7)
+    fn = ClippedPGLossFn(cfg)
+    b, s = 4, 8
+    mbs = []
+    for _ in range(2):
+        tm = torch.ones(b, s, dtype=torch.int64)
+        tm[:, 0] = 0
+        tm[0, -2:] = 0
+        data = _to_dev({
+            "token_mask": tm, "sample_mask": torch.tensor([1, 1, 1, 0]), "advantages": torch.randn(b, s),
+            "prev_logprobs": -torch.rand(b, s), "generation_logprobs": -torch.rand(b, s),
+            "reference_policy_logprobs": -torch.rand(b, s),
+        })
+        mbs.append((data, (-torch.rand(b, s - 1)).to(DEV)))
+    tot_s = sum(d["sample_mask"].sum() for d, _ in mbs).float()
+    tot_t = sum((d["token_mask"][:, 1:] * d["sample_mask"].unsqueeze(-1)).sum() for d, _ in mbs).float()
+    sync, raw = {}, {}
+    for d, lp in mbs:
+        for k, v in fn(lp, d, tot_s, tot_t)[1].items():
+            sync[k] = sync.get(k, 0.0) + v
+        for k, v in fn(lp, d, torch.tensor(1.0), torch.tensor(1.0))[1].items():
+            raw[k] = raw.get(k, 0.0) + v
+    for k, kind in fn.metric_normalizations.items():
+        if kind is MetricNormalizer.NONE:
+            continue
+        den = tot_t if kind is MetricNormalizer.TOKENS else tot_s
+        assert raw[k] / den.item() == pytest.approx(sync[k], rel=1e-5, abs=1e-7), k
+    assert raw["num_valid_samples"] == pytest.approx(sync["num_valid_samples"])
+
+
+def test_nll_loss_matches_oracle():
+    g = torch.Generator().manual_seed(4)
+    b, s = 5, 77
+    lp = -torch.rand(b, s - 1, generator=g) * 4
+    data = {"token_mask": (torch.rand(b, s, generator=g) > 0.3).long(), "sample_mask": torch.tensor([1, 0, 1, 1, 1])}
+    gt = (data["token_mask"][:, 1:] * data["sample_mask"].unsqueeze(-1)).sum()
+    a = lp.clone().requires_grad_(True)
+    want, wm = O.nll_loss(a, data, gt)
+    want.backward()
+    ag = lp.to(DEV).requires_grad_(True)
+    got, gm = NLLLossFn()(ag, _to_dev(data), None, gt.to(DEV))
+    got.backward()
+    assert _close(got.item(), want.item())
+    assert gm["num_unmasked_tokens"] == wm["num_unmasked_tokens"] and gm["num_valid_samples"] == wm["num_valid_samples"]
+    torch.testing.assert_close(ag.grad.cpu(), a.grad, rtol=1e-5, atol=1e-9)
+
+
+# ---- advantages ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("case", BASE["cases"], ids=[c["name"] for c in BASE["cases"]])
+@pytest.mark.parametrize("where", ["cpu", "cuda"])
+def test_baseline_std_golden(case, where):
+    r = torch.tensor(case["rewards"], dtype=torch.float32, device=where)
+    p = torch.tensor(case["prompts"], device=where)
+    v = torch.tensor(case["valid"], dtype=torch.float32, device=where)
+    baseline, std = calculate_baseline_and_std_per_prompt(p, r, v)
+    assert baseline.device.type == where and std.device.type == where
+    assert torch.allclose(baseline.cpu(), torch.tensor(case["baseline"], dtype=torch.float32), rtol=BASE["rtol"])
+    if case["std"] is None:
+        assert torch.isfinite(std).all()
+    else:
+        assert torch.allclose(std.cpu(), torch.tensor(case["std"], dtype=torch.float32), rtol=BASE["rtol"])
+
+
+def test_baseline_empty_input():
+    b, s = calculate_baseline_and_std_per_prompt(torch.empty(0, 3, dtype=torch.long), torch.tensor([]), torch.tensor([]))
+    assert b.shape == (0,) and s.shape == (0,)
+
+
+@pytest.mark.parametrize("case", ADV["cases"], ids=[c["name"] for c in ADV["cases"]])
+def test_grpo_advantage_golden(case):
+    est = GRPOAdvantageEstimator(AdvEstimatorConfig(use_leave_one_out_baseline=False, normalize_rewards=True), None)
+    out = est.compute_advantage(
+        prompt_ids=torch.tensor(case["prompt_ids"]), rewards=torch.tensor(case["rewards"], dtype=torch.float32),
+        mask=torch.ones(*case["mask_shape"]))
+    assert tuple(out.shape) == tuple(case["mask_shape"])
+    if case["expected_col"] is not None:
+        assert torch.allclose(out[:, 0], torch.tensor(case["expected_col"]), rtol=case["rtol"], atol=1e-6)
+    elif case["name"] == "symmetry":
+        assert out[0, 0] < 0 and abs(out[1, 0]) < 1e-5 and out[2, 0] > 0 and torch.allclose(out[0], -out[2], rtol=1e-5)
+    else:
+        assert abs(out.mean()) < 1e-5
+
+
+@pytest.mark.parametrize("loo", [True, False])
+def test_groups_and_advantages_match_oracle_bit_exact_decisions(loo):
+    """Random prompts with duplicates, shuffled; Bernoulli rewards (the BASELINE workload): group
+    indices, std > 0 decisions and values must agree with the oracle."""
+    g = torch.Generator().manual_seed(12)
+    n_prompts, group, plen = 37, 8, 33
+    base = torch.randint(0, 5, (n_prompts, plen), generator=g)  # small alphabet: near-duplicate prompts
+    base[1] = base[0]
+    base[1, -1] += 1  # differs from prompt 0 in the last token only
+    prompts = base.repeat_interleave(group, 0)
+    perm = torch.randperm(prompts.shape[0], generator=g)
+    prompts = prompts[perm]
+    rewards = (torch.rand(prompts.shape[0], generator=g) < 0.5).float()
+    valid = (torch.rand(prompts.shape[0], generator=g) < 0.9).float()
+    wb, ws = OA.baseline_and_std_per_prompt(prompts, rewards, valid, loo)
+    gb, gs_, _, gid = torch.ops.rl_amd.group_baseline_std(prompts.to(DEV), rewards.to(DEV), valid.to(DEV), None, loo, False)
+    want_gid = OA.group_ids_by_prompt(prompts)
+    first = {}
+    for i, v in enumerate(want_gid.tolist()):
+        first.setdefault(v, i)
+    assert gid.cpu().tolist() == [first[v] for v in want_gid.tolist()]  # index of the group's first row
+    assert torch.equal((gs_.cpu() > 0), (ws > 0)) and torch.equal((gs_.cpu() != 0), (ws != 0))
+    torch.testing.assert_close(gb.cpu(), wb, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(gs_.cpu(), ws, rtol=1e-5, atol=1e-7)
+    want_adv = OA.grpo_advantages(prompts, rewards, torch.ones(prompts.shape[0], 3), loo, True)
+    est = GRPOAdvantageEstimator(AdvEstimatorConfig(use_leave_one_out_baseline=loo), None)
+    got_adv = est.compute_advantage(prompts, rewards, torch.ones(prompts.shape[0], 3))
+    torch.testing.assert_close(got_adv, want_adv, rtol=1e-5, atol=1e-6)
+
+
+def test_config1_end_to_end_small():
+    """BASELINE config 1 at reduced size: advantages -> logprobs -> loss -> dlogits, fp32 logits."""
+    w = synthetic_grpo_batch(4, 4, 64, 2048, seed=1001)
+    ids, logits = w["input_ids"], w["logits"]
+    adv = OA.grpo_advantages(w["prompt_ids"], w["rewards"], w["token_mask"])
+    xo = logits.clone().requires_grad_(True)
+    lpo = OL.next_token_logprobs(ids, xo)
+    g = w["generator"]
+    prev = torch.cat([torch.zeros(16, 1), lpo.detach() + 0.05 * torch.randn(16, 63, generator=g)], 1)
+    ref = torch.cat([torch.zeros(16, 1), lpo.detach() + 0.05 * torch.randn(16, 63, generator=g)], 1)
+    data = {"input_ids": ids, "token_mask": w["token_mask"], "sample_mask": w["sample_mask"], "advantages": adv,
+            "prev_logprobs": prev, "generation_logprobs": prev, "reference_policy_logprobs": ref}
+    gs = w["sample_mask"].sum()
+    gt = (w["token_mask"][:, 1:] * w["sample_mask"].unsqueeze(-1)).sum()
+    want, wm = O.clipped_pg_loss(O.LossConfig(), lpo, data, gs, gt)
+    want.backward()
+
+    est = GRPOAdvantageEstimator(AdvEstimatorConfig(), None)
+    adv_g = est.compute_advantage(w["prompt_ids"], w["rewards"], w["token_mask"])
+    torch.testing.assert_close(adv_g, adv, rtol=1e-5, atol=1e-6)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    xg = logits.to(DEV).requires_grad_(True)
+    ddev = _to_dev({**data, "advantages": adv_g})
+    loss_input, ddev = prepare_loss_input(xg, ddev, fn)
+    assert (loss_input["next_token_logprobs"].cpu() - lpo.detach()).abs().max().item() <= 1e-5
+    got, gm = fn(data=ddev, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    got.backward()
+    assert _close(got.item(), want.item())
+    for k in wm:
+        assert _close(float(gm[k]), float(wm[k]), rel=1e-4, abs_=1e-7), k
+    scale = xo.grad.abs().max().item()
+    assert (xg.grad.cpu() - xo.grad).abs().max().item() <= 1e-4 * scale

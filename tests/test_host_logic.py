@@ -1,0 +1,115 @@
+"""CPU-only tests of the host-side mirror of the reference interface."""
+
+import pytest
+import torch
+
+import rl_amd
+from helpers import load_golden
+from oracle import logprob as OL
+from rl_amd.algorithms.loss import (
+    ClippedPGLossConfig,
+    ClippedPGLossFn,
+    LossInputType,
+    LossType,
+    MetricNormalizer,
+    NLLLossFn,
+)
+from rl_amd.algorithms.loss.utils import _pack_input_ids
+from rl_amd.algorithms.logits_sampling_utils import TrainingSamplingParams, need_top_k_or_top_p_filtering
+
+PG = load_golden("clipped_pg_cases.json")
+
+
+@pytest.mark.parametrize("bad", PG["config_asserts"]["must_raise_assertion"])
+def test_constructor_asserts(bad):
+    with pytest.raises(AssertionError):
+        ClippedPGLossFn(ClippedPGLossConfig(**bad))
+
+
+def test_tis_min_above_max_message():
+    cfg = ClippedPGLossConfig(
+        use_importance_sampling_correction=True, truncated_importance_sampling_type="tis",
+        truncated_importance_sampling_ratio=1.0, truncated_importance_sampling_ratio_min=2.0,
+    )
+    with pytest.raises(AssertionError, match="truncated_importance_sampling_ratio_min must be <= truncated_importance_sampling_ratio"):
+        ClippedPGLossFn(cfg)
+
+
+def test_metric_normalizations_table():
+    # tests/unit/algorithms/test_loss_functions.py:2688-2765 of the reference
+    n = ClippedPGLossFn(ClippedPGLossConfig()).metric_normalizations
+    assert n["loss"] is MetricNormalizer.TOKENS and n["kl_penalty"] is MetricNormalizer.TOKENS
+    assert n["sampling_importance_ratio"] is MetricNormalizer.TOKENS
+    for k in ("probs_ratio", "probs_ratio_clamped", "token_mult_prob_error", "gen_kl_error", "policy_kl_error",
+              "js_divergence_error", "approx_entropy"):
+        assert n[k] is MetricNormalizer.TOKENS
+    for k in ("num_valid_samples", "positive_nll_loss", "probs_ratio_min", "probs_ratio_max"):
+        assert n[k] is MetricNormalizer.NONE
+    assert "is_oob_ratio" not in n
+    n = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, sequence_level_importance_ratios=True,
+                                            use_importance_sampling_correction=True)).metric_normalizations
+    assert n["loss"] is MetricNormalizer.SEQUENCES and n["sampling_importance_ratio"] is MetricNormalizer.SEQUENCES
+    assert n["token_mult_prob_error"] is MetricNormalizer.TOKENS
+    n = ClippedPGLossFn(ClippedPGLossConfig(
+        token_level_loss=True, use_importance_sampling_correction=True,
+        truncated_importance_sampling_type="seq-mask-tis", truncated_importance_sampling_ratio=2.0,
+        truncated_importance_sampling_ratio_min=0.5)).metric_normalizations
+    assert n["loss"] is MetricNormalizer.TOKENS and n["is_oob_ratio"] is MetricNormalizer.SEQUENCES
+    n = ClippedPGLossFn(ClippedPGLossConfig(
+        token_level_loss=False, use_importance_sampling_correction=True,
+        truncated_importance_sampling_type="tis", truncated_importance_sampling_ratio=2.0)).metric_normalizations
+    assert n["loss"] is MetricNormalizer.SEQUENCES and n["is_oob_ratio"] is MetricNormalizer.TOKENS
+    n = NLLLossFn().metric_normalizations
+    assert n["loss"] is MetricNormalizer.TOKENS and n["num_unmasked_tokens"] is MetricNormalizer.NONE
+
+
+def test_loss_attributes_and_pickle():
+    import pickle
+
+    fn = ClippedPGLossFn(ClippedPGLossConfig(use_kl_in_reward=True), use_fused_linear_logprobs=True)
+    assert fn.input_type is LossInputType.LOGPROB and fn.loss_type is LossType.TOKEN_LEVEL
+    assert fn.reference_policy_kl_penalty == 0 and fn.use_fused_linear_logprobs
+    clone = pickle.loads(pickle.dumps(fn))  # the driver ships the loss object to every worker
+    assert clone.ratio_clip_min == fn.ratio_clip_min and clone.metric_normalizations == fn.metric_normalizations
+
+
+def test_sampling_predicates():
+    assert not need_top_k_or_top_p_filtering(None)
+    assert not need_top_k_or_top_p_filtering(TrainingSamplingParams())
+    assert not need_top_k_or_top_p_filtering(TrainingSamplingParams(top_k=-1, top_p=1.0))
+    assert need_top_k_or_top_p_filtering(TrainingSamplingParams(top_k=5))
+    assert need_top_k_or_top_p_filtering(TrainingSamplingParams(top_p=0.9))
+
+
+@pytest.mark.parametrize("roll", [0, -1])
+def test_pack_input_ids_matches_oracle(roll):
+    torch.manual_seed(0)
+    ids = torch.randint(1, 50, (4, 12))
+    cu = torch.tensor([0, 5, 17, 17, 26])       # lengths 5, 12, 0, 9
+    cup = torch.tensor([0, 8, 24, 24, 36])      # padded to multiples of 4 (with an empty sequence)
+    got = _pack_input_ids(ids, cu, cup, roll_shift=roll)
+    assert torch.equal(got, OL.pack_input_ids(ids, cu, cup, roll_shift=roll))
+    # a sequence whose recorded length exceeds the row width copies only the real tokens
+    cu2, cup2 = torch.tensor([0, 5, 20]), torch.tensor([0, 8, 24])
+    assert torch.equal(_pack_input_ids(ids[:2], cu2, cup2, roll_shift=roll),
+                       OL.pack_input_ids(ids[:2], cu2, cup2, roll_shift=roll))
+
+
+def test_install_aliases_reference_paths():
+    assert rl_amd.install() in ("aliased", "patched")
+    import nemo_rl.algorithms.loss_functions as short
+    from nemo_rl.algorithms.loss import ClippedPGLossFn as A
+    from nemo_rl.algorithms.loss.loss_functions import ClippedPGLossFn as B
+    from nemo_rl.distributed.model_utils import from_parallel_logits_to_logprobs  # noqa: F401
+    from nemo_rl.algorithms.utils import calculate_baseline_and_std_per_prompt  # noqa: F401
+    from nemo_rl.algorithms.advantage_estimator import GRPOAdvantageEstimator  # noqa: F401
+
+    assert A is B is short.ClippedPGLossFn is ClippedPGLossFn
+
+
+def test_multi_rank_groups_are_rejected(monkeypatch):
+    from rl_amd.distributed import model_utils as mu
+
+    monkeypatch.setattr(mu, "_group_size", lambda g: 2 if g == "tp2" else 1)
+    with pytest.raises(NotImplementedError, match="one GPU"):
+        mu.from_parallel_logits_to_logprobs(torch.zeros(1, 2, 4), torch.zeros(1, 2, dtype=torch.long), 0, 4, "tp2")
