@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the GRPO logprob + loss hot path on one MI355X.
+
+One step = one pass of the hot path over one synthetic batch of the workload: for every
+microbatch, logits -> token logprobs (K1), clipped-PG loss forward+backward (K4), dlogits (K2),
+through the public API (``prepare_loss_input`` -> ``ClippedPGLossFn`` -> autograd).  Inputs are
+resident in HBM before the timed region.  Prints ONE JSON line.
+
+Default workload (BASELINE config 2): 16 prompts x 8 generations = 128 sequences x 4096 tokens,
+V = 151936, bf16 logits ~ N(0,3) with a +8 spike at the target id with p = 0.3, prompt prefix
+U[256,1024] masked out; run as microbatches of 16 sequences (19.9 GB of logits each).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+WORKLOADS = {
+    # name: (sequences, seq_len, vocab, dtype, sequences per microbatch, logit std, spike p)
+    "c2": dict(seqs=128, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=3.0, spike_p=0.3,
+               desc="BASELINE config 2: 16 prompts x 8 = 128 seq x 4096 tok, V=151936 bf16, fwd+bwd to dlogits"),
+    "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
+               desc="BASELINE config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--seqs", type=int, default=None, help="override the number of sequences (smaller test runs)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    return ap.parse_args()
+
+
+class EventTimer:
+    """Records HIP events on the current stream around each kernel launch of the timed region."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.open = {}
+        self.pairs = {}
+
+    def start(self, name):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.open[name] = ev
+
+    def stop(self, name):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.pairs.setdefault(name, []).append((self.open.pop(name), ev))
+
+    def summary(self):
+        out = {}
+        for name, pairs in self.pairs.items():
+            ms = [a.elapsed_time(b) for a, b in pairs]
+            out[name] = dict(launches=len(ms), avg_ms=sum(ms) / len(ms), total_ms=sum(ms))
+        return out
+
+
+def make_microbatch(torch, w, n_seq, seed, dev):
+    """Synthetic microbatch generated on the GPU (the CPU-generated variant of the same recipe is what
+    the parity tests use)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    s, v = w["seq_len"], w["vocab"]
+    dtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    logits = torch.empty((n_seq, s, v), dtype=dtype, device=dev)
+    logits.normal_(0.0, w["std"], generator=g)
+    ids = torch.randint(0, v, (n_seq, s), generator=g, device=dev)
+    if w["spike_p"] > 0:
+        hit = (torch.rand((n_seq, s - 1), generator=g, device=dev) < w["spike_p"]).to(dtype) * 8.0
+        view = logits[:, :-1]
+        idx = ids[:, 1:].unsqueeze(-1)
+        view.scatter_add_(-1, idx, hit.unsqueeze(-1))
+    lo, hi = (256, 1024) if s >= 2048 else (max(1, s // 8), max(2, s // 4))
+    prefix = torch.randint(lo, hi + 1, (n_seq,), generator=g, device=dev)
+    token_mask = (torch.arange(s, device=dev).unsqueeze(0) >= prefix.unsqueeze(-1)).to(torch.int64)
+    token_mask[:, 0] = 0
+    sample_mask = torch.ones(n_seq, dtype=torch.float32, device=dev)
+    adv = torch.randn((n_seq, 1), generator=g, device=dev).expand(n_seq, s).contiguous()
+    base = -torch.rand((n_seq, s), generator=g, device=dev) * 3
+    noise = lambda: base + 0.05 * torch.randn((n_seq, s), generator=g, device=dev)  # noqa: E731
+    return dict(logits=logits, data={
+        "input_ids": ids, "token_mask": token_mask, "sample_mask": sample_mask, "advantages": adv,
+        "prev_logprobs": base, "generation_logprobs": base, "reference_policy_logprobs": noise(),
+    })
+
+
+def cpu_baseline(torch, w, seconds):
+    """The oracle (pure PyTorch restatement of the reference op sequence) on the host cores, on a
+    bounded sample of the same workload: real vocabulary and dtype, fewer rows."""
+    from oracle import logprob as OL
+    from oracle import loss as O
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    dtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    v = w["vocab"]
+
+    def run(n_seq, s):
+        g = torch.Generator().manual_seed(1002)
+        logits = (torch.randn(n_seq, s, v, generator=g) * w["std"]).to(dtype).requires_grad_(True)
+        ids = torch.randint(0, v, (n_seq, s), generator=g)
+        base = -torch.rand(n_seq, s, generator=g) * 3
+        tm = torch.ones(n_seq, s, dtype=torch.int64)
+        tm[:, : s // 8] = 0
+        data = {"token_mask": tm, "sample_mask": torch.ones(n_seq), "advantages": torch.randn(n_seq, 1, generator=g).expand(n_seq, s),
+                "prev_logprobs": base, "generation_logprobs": base, "reference_policy_logprobs": base + 0.05}
+        t0 = time.perf_counter()
+        lp = OL.next_token_logprobs(ids, logits)
+        loss, _ = O.clipped_pg_loss(O.LossConfig(), lp, data, torch.tensor(float(n_seq)), tm[:, 1:].sum().float())
+        loss.backward()
+        return time.perf_counter() - t0
+
+    s, n_seq = 64, 64
+    run(1, s)  # warm-up
+    times = []
+    while sum(times) < seconds or len(times) < 3:
+        times.append(run(n_seq, s))
+    times.sort()
+    t = times[len(times) // 2]
+    rows = n_seq * s
+    return dict(value=rows / t, unit="tokens/s", cores=threads, kind="port",
+                sample=f"{rows} rows of V={v} {w['dtype']} per iteration, oracle fwd+loss+bwd, median of {len(times)} "
+                       f"iterations ({sum(times):.1f} s total), {threads} threads of {cores} host cores")
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from rl_amd import _lib, ops
+    from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn, prepare_loss_input
+
+    _lib.load()
+    w = dict(WORKLOADS[args.workload])
+    if args.seqs:
+        w["seqs"] = args.seqs
+        w["mb_seqs"] = min(w["mb_seqs"], args.seqs)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    elt = 2 if w["dtype"] == "bf16" else 4
+    n_mb = (w["seqs"] + w["mb_seqs"] - 1) // w["mb_seqs"]
+    mb_bytes = w["mb_seqs"] * w["seq_len"] * w["vocab"] * elt
+    free, _total = torch.cuda.mem_get_info()
+    # logits of every microbatch stay resident if they fit next to one gradient buffer; otherwise
+    # the microbatches cycle through as many distinct buffers as fit
+    n_buf = max(1, min(n_mb, int((free * 0.9 - mb_bytes * 1.2) // mb_bytes)))
+    mbs = [make_microbatch(torch, w, w["mb_seqs"], 1002 + i, dev) for i in range(n_buf)]
+    torch.cuda.synchronize()
+
+    fn = ClippedPGLossFn(ClippedPGLossConfig())  # eps 0.2/0.2, k3 KL beta 0.01, token-level mean
+    tot_seqs = torch.tensor(float(w["seqs"]), device=dev)
+    tot_toks = sum((m["data"]["token_mask"][:, 1:].sum() for m in mbs)) * (n_mb / n_buf)
+    tot_toks = tot_toks.float()
+
+    def step():
+        for i in range(n_mb):
+            m = mbs[i % n_buf]
+            logits = m["logits"].requires_grad_(True)
+            loss_input, data = prepare_loss_input(logits, m["data"], fn)
+            loss, _metrics = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+            (dlogits,) = torch.autograd.grad(loss, logits)
+            del dlogits, loss, loss_input
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = EventTimer(torch)
+    ops.KERNEL_TIMER = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    kernels = timer.summary()
+
+    tokens_per_step = w["seqs"] * w["seq_len"]
+    rows_per_launch = w["mb_seqs"] * w["seq_len"]
+    row_bytes = w["vocab"] * elt
+    bwd = kernels.get("logprob_bwd", dict(avg_ms=float("nan")))
+    fwd = kernels.get("logprob_fwd", dict(avg_ms=float("nan")))
+    bwd_gbs = 2 * row_bytes * rows_per_launch / (bwd["avg_ms"] * 1e-3) / 1e9
+    fwd_gbs = row_bytes * w["mb_seqs"] * (w["seq_len"] - 1) / (fwd["avg_ms"] * 1e-3) / 1e9
+    result = {
+        "metric": "GRPO logprob+loss fwd/bwd tokens/s at V=151936; % of HBM peak",
+        "value": tokens_per_step * args.steps / elapsed,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w["dtype"],
+        "data": "synthetic",
+        "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
+                   "microbatches": n_mb, "resident_logit_buffers": n_buf,
+                   "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level"},
+        "hbm_frac_end_to_end": 3 * row_bytes * tokens_per_step * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "logprob_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "avg_launch_ms": bwd["avg_ms"], "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
+        "roofline_fwd": {"bound": "hbm", "kernel": "logprob_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
+        "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -4,9 +4,9 @@ Test infrastructure only (see ``oracle/__init__.py``).
 
 Single-GPU (TP = CP = 1) restatement of ``nemo_rl/distributed/model_utils.py``:
 the collectives at ``:50-54, 61-65, 152-156`` reduce over one rank and vanish.
-Gradients come from torch autograd over the same fp32 expression the reference
-differentiates by hand, so ``dlogits = g * (onehot - softmax)`` falls out of
-the definition instead of being retyped.
+The backward of the row op restates the reference's hand-written one (it differs from
+plain autograd only for targets outside the vocabulary shard); the tests pin it to
+torch autograd of ``log_softmax(x).gather(t)`` for in-range targets.
 """
 
 from __future__ import annotations
@@ -35,26 +35,39 @@ def stable_log_softmax(x32: torch.Tensor) -> torch.Tensor:
     return shifted - shifted.exp().sum(-1, keepdim=True).log()
 
 
+class _RowsLogprob(torch.autograd.Function):
+    """``DistributedLogprob`` on one rank (``model_utils.py:136-207``).  The hand-written backward is
+    ``-softmax * g`` for every row plus ``g`` at the target of the rows whose target is inside the
+    shard (``:193-197``): a row whose target lies in another shard returns 0 in the forward but still
+    receives the softmax term, because the full-vocabulary logprob is the sum over shards."""
+
+    @staticmethod
+    def forward(ctx, logits, target, vocab_start, vocab_end):
+        outside = (target < vocab_start) | (target >= vocab_end)
+        local = (target - vocab_start).masked_fill(outside, 0)
+        logp = stable_log_softmax(logits.to(torch.float32))
+        picked = torch.gather(logp, -1, local.unsqueeze(-1)).squeeze(-1)
+        ctx.save_for_backward(logp.exp(), outside, local)
+        return picked.masked_fill(outside, 0.0)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        softmax, outside, local = ctx.saved_tensors
+        onehot = torch.nn.functional.one_hot(local, num_classes=softmax.shape[-1]) * (~outside).unsqueeze(-1)
+        return (onehot.float() - softmax) * grad_output.unsqueeze(-1), None, None, None
+
+
 def rows_logprob(
     logits: torch.Tensor,
     target: torch.Tensor,
     vocab_start: int = 0,
     vocab_end: Optional[int] = None,
 ) -> torch.Tensor:
-    """``DistributedLogprob.forward`` (``model_utils.py:136-165``) on one rank.
-
-    ``logits [..., V]`` any float dtype, ``target [...]`` int64, already shifted.
-    Targets outside ``[vocab_start, vocab_end)`` give 0 and no one-hot term in
-    the gradient (``:137-150, 196-197``).
-    """
-    vocab = logits.shape[-1]
+    """``logits [..., V]`` any float dtype, ``target [...]`` int64, already shifted.  Targets outside
+    ``[vocab_start, vocab_end)`` give 0 (``model_utils.py:137-150``)."""
     if vocab_end is None:
-        vocab_end = vocab_start + vocab
-    outside = (target < vocab_start) | (target >= vocab_end)
-    local = (target - vocab_start).masked_fill(outside, 0)
-    logp = stable_log_softmax(logits.to(torch.float32))
-    picked = torch.gather(logp, -1, local.unsqueeze(-1)).squeeze(-1)
-    return picked.masked_fill(outside, 0.0)
+        vocab_end = vocab_start + logits.shape[-1]
+    return _RowsLogprob.apply(logits, target, vocab_start, vocab_end)
 
 
 def rows_logprob_seq_chunked(logits, target, chunk_size, vocab_start=0, vocab_end=None):

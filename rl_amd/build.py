@@ -22,6 +22,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-std=c++17",
     "-fPIC",
+    "-ffp-contract=off",  # token arithmetic mirrors separate fp32 PyTorch ops: no fused multiply-add
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 

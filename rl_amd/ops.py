@@ -17,6 +17,24 @@ _DTYPES = {torch.float32: _lib.NRL_F32, torch.bfloat16: _lib.NRL_BF16, torch.flo
 
 _LIB = torch.library.Library("rl_amd", "DEF")
 
+# Optional per-launch timing: an object with ``start(name)`` / ``stop(name)`` that records events on
+# the current stream around a kernel launch (used by the benchmark harness); None in normal use.
+KERNEL_TIMER = None
+
+
+class _timed:
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        if KERNEL_TIMER is not None:
+            KERNEL_TIMER.start(self.name)
+
+    def __exit__(self, *exc):
+        if KERNEL_TIMER is not None:
+            KERNEL_TIMER.stop(self.name)
+        return False
+
 
 def _stream() -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -88,7 +106,8 @@ def _logprob_fwd(logits, targets, n_inner, vocab_start, vocab_end, temperature, 
     with torch.cuda.device(logits.device):
         out = torch.empty((b, n_inner), dtype=torch.float32, device=logits.device)
         lse = torch.empty((b, n_inner) if save_lse else (0,), dtype=torch.float32, device=logits.device)
-        code = _lib.load().nrl_logprob_fwd(C.byref(rows), _ptr(out), _ptr(lse if save_lse else None), _stream())
+        with _timed("logprob_fwd"):
+            code = _lib.load().nrl_logprob_fwd(C.byref(rows), _ptr(out), _ptr(lse if save_lse else None), _stream())
     _lib.check(code, "nrl_logprob_fwd")
     return out, lse
 
@@ -103,10 +122,11 @@ def _logprob_bwd(logits, targets, lse, grad, n_inner, vocab_start, vocab_end, te
         raise ValueError(f"grad must be fp32 [B, n_inner], got {grad.dtype} {tuple(grad.shape)}")
     with torch.cuda.device(logits.device):
         d = logits if in_place else torch.empty((b, s, v), dtype=logits.dtype, device=logits.device)
-        code = _lib.load().nrl_logprob_bwd(
-            C.byref(rows), _ptr(lse), _ptr(grad), grad.stride(0), grad.stride(1),
-            _ptr(d), s, d.stride(0), d.stride(1), _stream(),
-        )
+        with _timed("logprob_bwd"):
+            code = _lib.load().nrl_logprob_bwd(
+                C.byref(rows), _ptr(lse), _ptr(grad), grad.stride(0), grad.stride(1),
+                _ptr(d), s, d.stride(0), d.stride(1), _stream(),
+            )
     _lib.check(code, "nrl_logprob_bwd")
     return d
 
@@ -271,10 +291,11 @@ def _grpo_loss(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_ma
         metrics = torch.empty((_lib.NRL_GRPO_N_METRICS,), dtype=torch.float32, device=dev)
         ws_bytes = lib.nrl_grpo_loss_workspace_bytes(b)
         ws = torch.empty((ws_bytes // 8,), dtype=torch.float64, device=dev)
-        code = lib.nrl_grpo_loss_fwd_bwd(
-            C.byref(cfg), C.byref(inp), _ptr(loss), _ptr(dlp), _ptr(dlpu if split else None), _ptr(metrics),
-            _ptr(ws), ws_bytes, _stream(),
-        )
+        with _timed("grpo_loss"):
+            code = lib.nrl_grpo_loss_fwd_bwd(
+                C.byref(cfg), C.byref(inp), _ptr(loss), _ptr(dlp), _ptr(dlpu if split else None), _ptr(metrics),
+                _ptr(ws), ws_bytes, _stream(),
+            )
     _lib.check(code, "nrl_grpo_loss_fwd_bwd")
     del keep
     return loss, dlp, dlpu, metrics

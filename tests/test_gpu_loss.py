@@ -27,6 +27,8 @@ def _to_dev(data):
 
 
 def _close(a, b, rel=1e-4, abs_=1e-6):
+    if math.isnan(a) or math.isnan(b):
+        return math.isnan(a) and math.isnan(b)
     if math.isinf(b) or math.isinf(a):
         return a == b
     return abs(a - b) <= rel * abs(b) + abs_
@@ -38,11 +40,14 @@ def test_golden_cases_through_prepare_and_loss(case):
     lp, data, gs, gt = golden_case_to_inputs(case)
     vocab = 8
     data["input_ids"] = torch.randint(0, vocab, data["input_ids"].shape, generator=torch.Generator().manual_seed(1))
-    logits = exact_logits_for_logprobs(lp, data["input_ids"], vocab)
     fn = ClippedPGLossFn(ClippedPGLossConfig(**case["cfg"]))
     ddev = _to_dev(data)
-    loss_input, ddev = prepare_loss_input(logits.to(DEV).requires_grad_(True), ddev, fn)
-    torch.testing.assert_close(loss_input["next_token_logprobs"].detach().cpu(), lp, rtol=1e-5, atol=1e-5)
+    if bool((lp <= 0).all()):
+        logits = exact_logits_for_logprobs(lp, data["input_ids"], vocab)
+        loss_input, ddev = prepare_loss_input(logits.to(DEV).requires_grad_(True), ddev, fn)
+        torch.testing.assert_close(loss_input["next_token_logprobs"].detach().cpu(), lp, rtol=1e-5, atol=1e-5)
+    else:  # the reference passes these (positive) logprobs straight to the loss
+        loss_input = {"next_token_logprobs": lp.to(DEV)}
     loss, metrics = fn(data=ddev, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
     assert loss.is_cuda and loss.dim() == 0
     if "expected_loss" in case:
