@@ -25,6 +25,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (scaled by the same counters on a 4 GiB copy), valid for one microbatch of the named workload
+MEASURED_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}
+
 WORKLOADS = {
     # name: (sequences, seq_len, vocab, dtype, sequences per microbatch, logit std, spike p)
     "c2": dict(seqs=128, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=3.0, spike_p=0.3,
@@ -42,6 +46,8 @@ def parse_args():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--seqs", type=int, default=None, help="override the number of sequences (smaller test runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 4 GiB device-to-device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     return ap.parse_args()
 
@@ -92,11 +98,18 @@ def make_microbatch(torch, w, n_seq, seed, dev):
     token_mask[:, 0] = 0
     sample_mask = torch.ones(n_seq, dtype=torch.float32, device=dev)
     adv = torch.randn((n_seq, 1), generator=g, device=dev).expand(n_seq, s).contiguous()
-    base = -torch.rand((n_seq, s), generator=g, device=dev) * 3
-    noise = lambda: base + 0.05 * torch.randn((n_seq, s), generator=g, device=dev)  # noqa: E731
+    # prev / generation / reference logprobs = current-policy logprobs + N(0, 0.05), as in a real step
+    # where the policy has moved only slightly since the rollout
+    from rl_amd.distributed.model_utils import get_next_token_logprobs_from_logits
+
+    with torch.no_grad():
+        cur = get_next_token_logprobs_from_logits(ids, logits)
+    cur = torch.cat([torch.zeros((n_seq, 1), device=dev), cur], dim=1)
+    noise = lambda: cur + 0.05 * torch.randn((n_seq, s), generator=g, device=dev)  # noqa: E731
+    prev = noise()
     return dict(logits=logits, data={
         "input_ids": ids, "token_mask": token_mask, "sample_mask": sample_mask, "advantages": adv,
-        "prev_logprobs": base, "generation_logprobs": base, "reference_policy_logprobs": noise(),
+        "prev_logprobs": prev, "generation_logprobs": prev, "reference_policy_logprobs": noise(),
     })
 
 
@@ -219,12 +232,19 @@ def main():
                    "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level"},
         "hbm_frac_end_to_end": 3 * row_bytes * tokens_per_step * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": "logprob_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if not args.seqs else None,
                      "avg_launch_ms": bwd["avg_ms"], "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
         "roofline_fwd": {"bound": "hbm", "kernel": "logprob_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
     }
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)  # 4 GiB
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        result["copy_calibration_bytes"] = src.numel() * 4
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_seconds)
     print(json.dumps(result))
