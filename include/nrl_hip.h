@@ -99,6 +99,38 @@ int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t total_toke
                            int64_t d_row_stride, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * K3  Token logprobs under top-k / top-p filtering.  Replaces apply_top_k_top_p
+ * (nemo_rl/algorithms/logits_sampling_utils.py:69-285) followed by log_softmax + gather, i.e.
+ * DistributedLogprobWithSampling / ChunkedDistributedLogprobWithSampling at TP = 1
+ * (nemo_rl/distributed/model_utils.py:383-719) and the filtered plain branch (:1677-1693), without
+ * sorting the vocabulary.  rows->vocab_start must be 0 and vocab_end == vocab.
+ * top_k <= 0 and top_p >= 1 switch the respective filter off (at least one must be on).
+ * Per row the forward emits the keep predicate (thr_out, tie_out): element v is kept iff
+ * x_v > thr, or x_v == thr and v >= tie; and lse_kept_out, the log-sum-exp over the kept set.
+ * logprob_out (may be NULL, then rows->targets may be NULL): x_t - lse_kept, or -inf when the target
+ * was filtered out.  logprob_unfiltered_out / lse_full_out (may be NULL): the same row's unfiltered
+ * logprob (what the KL penalty needs, loss/utils.py:104-118) from the same pass.
+ * overflow_flag: device int32 set to 1 if some row's kept set exceeded the on-chip candidate list
+ * (4096 entries; such rows come back as NaN).  top_k above 2048 is not supported.
+ * ------------------------------------------------------------------------------------------ */
+int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
+                              float* thr_out, int32_t* tie_out, float* lse_kept_out,
+                              float* logprob_unfiltered_out, float* lse_full_out,
+                              int32_t* overflow_flag, void* stream);
+
+/* dlogits_v = keep_v * g * (onehot_v - exp(x_v - lse_kept)); layout arguments as nrl_logprob_bwd. */
+int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,
+                              const float* lse_kept, const float* grad, int64_t grad_stride_outer,
+                              int64_t grad_stride_inner, void* dlogits, int64_t d_n_inner,
+                              int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
+
+/* Materialises apply_top_k_top_p's outputs from a forward's (thr, tie): filtered logits (-inf outside
+ * the kept set, same dtype, row (o,i) at filtered_out + o*f_stride_outer + i*f_stride_inner) and the
+ * keep mask (uint8 [rows, vocab], may be NULL). */
+int nrl_topk_topp_filter(const nrl_rows* rows, const float* thr, const int32_t* tie, void* filtered_out,
+                         int64_t f_stride_outer, int64_t f_stride_inner, uint8_t* keep_out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * K4  ClippedPGLossFn (nemo_rl/algorithms/loss/loss_functions.py:374-788) with calculate_kl and
  * masked_mean (nemo_rl/algorithms/utils.py:42-101, 212-224) fused: loss, its gradient with
  * respect to the token logprobs, and every metric, in two launches.

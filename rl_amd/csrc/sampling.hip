@@ -1,0 +1,557 @@
+// K3: token logprobs under top-k / top-p (nucleus) filtering, forward and backward, for gfx950.
+//
+// The reference sorts every 151 936-wide row (values + int64 indices).  Here one workgroup of 512
+// threads owns a row and never sorts it:
+//   pass 1 (HBM)   streams the row keeping 2048 chunk maxima in registers (and, when the caller
+//                  wants the unfiltered logprob too, the online log-sum-exp of the full row);
+//   select         the k-th largest chunk maximum is a lower bound of the k-th largest element
+//                  (radix select over the 2048 maxima in LDS); for top-p alone the bound is
+//                  lse + log((1-p)/V): everything below it is dropped whatever the order;
+//   pass 2 (cache) re-reads the row and appends the few elements above the bound to an LDS list;
+//   finish         bitonic sort of the list by (value, index), top-k threshold with ties kept,
+//                  softmax over the kept values, ascending cumulative mass > 1 - top_p, the
+//                  renormalised log-sum-exp, the target's logprob (-inf when it was filtered).
+// Per row the forward saves (threshold value, tie index, kept log-sum-exp): element v is kept iff
+// x_v > thr, or x_v == thr and v >= tie index.  Among exactly tied values at the top-p boundary the
+// larger vocabulary indices survive (ascending stable order); all ties at the top-k threshold are
+// kept.  The backward streams the row once more: d_v = keep_v * g * (onehot_v - exp(x_v - lse_kept)).
+//
+// Rows whose candidate list would exceed the LDS capacity (very flat distributions under top-p
+// alone, or thousands of exact ties) raise the overflow flag instead of producing a wrong result.
+
+#include <float.h>
+#include <math.h>
+
+#include "common.hpp"
+
+namespace nrl {
+
+constexpr int kSelBlock = 512;
+constexpr int kSelWaves = kSelBlock / kWave;
+constexpr int kSub = 4;                      // chunk maxima per thread
+constexpr int kChunks = kSelBlock * kSub;    // 2048
+constexpr int kCap = 4096;                   // candidate capacity (LDS)
+
+struct Lse2 {
+    float m, s;
+};
+__device__ __forceinline__ Lse2 lse2_merge(Lse2 a, Lse2 b) {
+    const float m = fmaxf(a.m, b.m);
+    Lse2 r;
+    r.m = m;
+    r.s = a.s * fast_exp2((a.m - m) * kLog2e) + b.s * fast_exp2((b.m - m) * kLog2e);
+    return r;
+}
+
+// monotone map float -> uint32 (larger float, larger key)
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+template <int DT> __device__ __forceinline__ int64_t sel_row_head(const void* row, int64_t vocab) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(row);
+    const int64_t h = static_cast<int64_t>(((16 - (a & 15)) & 15) / Row<DT>::BYTES);
+    return h < vocab ? h : vocab;
+}
+
+struct SelShared {
+    uint32_t maxima[kChunks];
+    unsigned long long cand[kCap];
+    float expv[kCap];
+    uint32_t hist[256];
+    Lse2 lse_w[kSelWaves];
+    int count;
+    uint32_t sel_prefix;
+    int sel_k;
+    float bound;
+    float thr;
+    int tie;
+    float lse_kept;
+    int n_keep;
+};
+
+// k-th largest (1-based) of the kChunks keys in sh.maxima; every thread returns it
+__device__ __forceinline__ uint32_t select_kth_largest(SelShared& sh, int k) {
+    const int tid = threadIdx.x;
+    if (tid == 0) { sh.sel_prefix = 0u; sh.sel_k = k; }
+    uint32_t mask = 0u;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) sh.hist[tid] = 0u;
+        __syncthreads();
+        const uint32_t prefix = sh.sel_prefix;
+        for (int i = tid; i < kChunks; i += kSelBlock) {
+            const uint32_t key = sh.maxima[i];
+            if ((key & mask) == prefix) atomicAdd(&sh.hist[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int need = sh.sel_k;
+            int b = 255;
+            for (; b > 0; --b) {
+                const int c = static_cast<int>(sh.hist[b]);
+                if (c >= need) break;
+                need -= c;
+            }
+            sh.sel_prefix = prefix | (static_cast<uint32_t>(b) << shift);
+            sh.sel_k = need;
+        }
+        mask |= 0xffu << shift;
+        __syncthreads();
+    }
+    return sh.sel_prefix;
+}
+
+// descending bitonic sort of sh.cand[0 .. n_pad)
+__device__ __forceinline__ void sort_candidates_desc(SelShared& sh, int n_pad) {
+    const int tid = threadIdx.x;
+    for (int size = 2; size <= n_pad; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = tid; i < (n_pad >> 1); i += kSelBlock) {
+                const int lo = ((i / stride) * (stride << 1)) + (i % stride);
+                const int hi = lo + stride;
+                const bool desc = ((lo & size) == 0);
+                const unsigned long long a = sh.cand[lo], b = sh.cand[hi];
+                if ((a < b) == desc) { sh.cand[lo] = b; sh.cand[hi] = a; }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+struct SelArgs {
+    const void* logits;
+    int64_t n_inner, vocab, stride_outer, stride_inner;
+    const int64_t* targets;  // may be NULL (filter only)
+    int64_t ts_outer, ts_inner;
+    float tparam;
+    int top_k;    // <= 0: off
+    float top_p;  // >= 1: off
+    float* logprob;      // [rows] or NULL
+    float* thr;          // [rows]
+    int32_t* tie;        // [rows]
+    float* lse_kept;     // [rows]
+    float* logprob_full; // [rows] or NULL: unfiltered logprob of the target
+    float* lse_full;     // [rows] or NULL
+    int32_t* overflow;   // device flag
+};
+
+template <int DT, int TEMP, bool FULL_LSE>
+__global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
+    __shared__ SelShared sh;
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const int64_t r = blockIdx.x;
+    const int64_t o = r / a.n_inner, i_in = r - o * a.n_inner;
+    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i_in * a.stride_inner) * Row<DT>::BYTES;
+    const int64_t vocab = a.vocab;
+    const int64_t head = sel_row_head<DT>(row, vocab);
+    const int64_t nvec = (vocab - head) / EPV;
+    const int64_t tail0 = head + nvec * EPV;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(row + head * Row<DT>::BYTES);
+
+    // ---- pass 1: chunk maxima (+ full-row online log-sum-exp) ----
+    float mx[kSub];
+#pragma unroll
+    for (int u = 0; u < kSub; ++u) mx[u] = -FLT_MAX;
+    Lse2 acc;
+    acc.m = -FLT_MAX;
+    acc.s = 0.f;
+    int64_t base = 0;
+    for (; base + kSub * kSelBlock <= nvec; base += kSub * kSelBlock) {
+        u32x4 q[kSub];
+#pragma unroll
+        for (int u = 0; u < kSub; ++u) q[u] = xv[base + u * kSelBlock + tid];
+        float v[kSub * EPV];
+#pragma unroll
+        for (int u = 0; u < kSub; ++u) {
+            float t[EPV];
+            Row<DT>::decode(q[u], t);
+            float vm = -FLT_MAX;
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) {
+                t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+                v[u * EPV + k] = t[k];
+                vm = fmaxf(vm, t[k]);
+            }
+            mx[u] = fmaxf(mx[u], vm);
+        }
+        if (FULL_LSE) {
+            float vm = fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3]));
+            const float mn = fmaxf(acc.m, vm);
+            float part = 0.f;
+#pragma unroll
+            for (int k = 0; k < kSub * EPV; ++k) part += fast_exp2((v[k] - mn) * kLog2e);
+            acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + part;
+            acc.m = mn;
+        }
+    }
+    for (int64_t vi = base + tid; vi < nvec; vi += kSelBlock) {
+        float t[EPV];
+        Row<DT>::decode(xv[vi], t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) {
+            t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+            mx[0] = fmaxf(mx[0], t[k]);
+            if (FULL_LSE) {
+                const float mn = fmaxf(acc.m, t[k]);
+                acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((t[k] - mn) * kLog2e);
+                acc.m = mn;
+            }
+        }
+    }
+    {
+        const int64_t e0 = tid < head ? tid : -1;
+        const int64_t e1 = tail0 + tid < vocab ? tail0 + tid : -1;
+        for (int w = 0; w < 2; ++w) {
+            const int64_t e = w == 0 ? e0 : e1;
+            if (e < 0) continue;
+            const float x = scale_logit<DT, TEMP>(Row<DT>::load1(row, e), a.tparam);
+            mx[0] = fmaxf(mx[0], x);
+            if (FULL_LSE) {
+                const float mn = fmaxf(acc.m, x);
+                acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((x - mn) * kLog2e);
+                acc.m = mn;
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kSub; ++u) sh.maxima[u * kSelBlock + tid] = order_key(mx[u]);
+    float lse_full = 0.f;
+    if (FULL_LSE) {
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            Lse2 other;
+            other.m = __shfl_xor(acc.m, off, kWave);
+            other.s = __shfl_xor(acc.s, off, kWave);
+            acc = lse2_merge(acc, other);
+        }
+        if ((tid & (kWave - 1)) == 0) sh.lse_w[tid / kWave] = acc;
+    }
+    if (tid == 0) sh.count = 0;
+    __syncthreads();
+    if (FULL_LSE) {
+        Lse2 tot = sh.lse_w[0];
+#pragma unroll
+        for (int w = 1; w < kSelWaves; ++w) tot = lse2_merge(tot, sh.lse_w[w]);
+        lse_full = tot.m + logf(tot.s);
+    }
+
+    // ---- lower bound of everything that can be kept ----
+    const bool use_k = a.top_k > 0;
+    const bool use_p = a.top_p < 1.0f;
+    uint32_t bound_key = 0u;
+    if (use_k) {
+        if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, a.top_k);
+    } else {
+        // top-p alone: elements with probability <= (1-p)/V sum to at most 1-p and are the smallest
+        const float b = lse_full + logf((1.0f - a.top_p) / static_cast<float>(vocab));
+        bound_key = order_key(b) + 1u;  // strictly above the bound
+    }
+
+    // ---- pass 2: collect candidates ----
+    for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
+        float t[EPV];
+        Row<DT>::decode(xv[vi], t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) {
+            const uint32_t key = order_key(scale_logit<DT, TEMP>(t[k], a.tparam));
+            if (key >= bound_key) {
+                const int pos = atomicAdd(&sh.count, 1);
+                if (pos < kCap)
+                    sh.cand[pos] = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(head + vi * EPV + k);
+            }
+        }
+    }
+    for (int w = 0; w < 2; ++w) {
+        const int64_t e = w == 0 ? (tid < head ? tid : -1) : (tail0 + tid < vocab ? tail0 + tid : -1);
+        if (e < 0) continue;
+        const uint32_t key = order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, e), a.tparam));
+        if (key >= bound_key) {
+            const int pos = atomicAdd(&sh.count, 1);
+            if (pos < kCap) sh.cand[pos] = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(e);
+        }
+    }
+    __syncthreads();
+    const int n = sh.count;
+    if (n > kCap || n == 0) {
+        // the kept set does not fit the candidate list (or the row holds no finite value)
+        if (tid == 0) {
+            if (n > kCap) atomicExch(a.overflow, 1);
+            a.thr[r] = __builtin_nanf("");
+            a.tie[r] = 0;
+            a.lse_kept[r] = __builtin_nanf("");
+            if (a.logprob) a.logprob[r] = __builtin_nanf("");
+            if (a.lse_full) a.lse_full[r] = lse_full;
+            if (a.logprob_full) a.logprob_full[r] = __builtin_nanf("");
+        }
+        return;
+    }
+    int n_pad = 1;
+    while (n_pad < n) n_pad <<= 1;
+    for (int i = n + tid; i < n_pad; i += kSelBlock) sh.cand[i] = 0ull;  // sorts last
+    sort_candidates_desc(sh, n_pad);
+
+    // ---- top-k threshold (ties kept), softmax over the kept values ----
+    int n_k = n;
+    if (use_k) {
+        const int kk = a.top_k < n ? a.top_k : n;
+        const uint32_t thr_key = static_cast<uint32_t>(sh.cand[kk - 1] >> 32);
+        int cnt = 0;
+        for (int i = tid; i < n; i += kSelBlock) cnt += (static_cast<uint32_t>(sh.cand[i] >> 32) >= thr_key) ? 1 : 0;
+        __shared__ int cnt_w[kSelWaves];
+        n_k = block_sum<int, kSelWaves>(cnt, cnt_w);
+    }
+    const float m = key_value(static_cast<uint32_t>(sh.cand[0] >> 32));
+    for (int i = tid; i < n_k; i += kSelBlock)
+        sh.expv[i] = expf(key_value(static_cast<uint32_t>(sh.cand[i] >> 32)) - m);
+    __syncthreads();
+    if (tid == 0) {
+        int n_keep = n_k;
+        if (use_p) {
+            float s_k = 0.f;
+            for (int i = n_k - 1; i >= 0; --i) s_k += sh.expv[i];
+            // ascending cumulative probability, smallest kept value first; keep while it exceeds 1 - p
+            const float cut = 1.0f - a.top_p;
+            float cum = 0.f;
+            if (!use_k) {
+                // top-p alone normalises over the whole row: the elements below the candidate bound
+                // come first in ascending order and contribute their (small) mass to the running sum
+                const float s_full = expf(lse_full - m);
+                cum = fmaxf(0.f, (s_full - s_k) / s_full);
+                s_k = s_full;
+            }
+            n_keep = 1;
+            for (int i = n_k - 1; i >= 1; --i) {
+                cum += sh.expv[i] / s_k;
+                if (cum > cut) { n_keep = i + 1; break; }
+            }
+        }
+        float s = 0.f;
+        for (int i = n_keep - 1; i >= 0; --i) s += sh.expv[i];
+        const unsigned long long last = sh.cand[n_keep - 1];
+        const uint32_t last_key = static_cast<uint32_t>(last >> 32);
+        int tie = 0;
+        if (n_keep < n && static_cast<uint32_t>(sh.cand[n_keep] >> 32) == last_key) tie = static_cast<int>(last & 0xffffffffu);
+        sh.thr = key_value(last_key);
+        sh.tie = tie;
+        sh.lse_kept = m + logf(s);
+        sh.n_keep = n_keep;
+        a.thr[r] = sh.thr;
+        a.tie[r] = tie;
+        a.lse_kept[r] = sh.lse_kept;
+        if (a.lse_full) a.lse_full[r] = lse_full;
+        if (a.targets && a.logprob) {
+            const int64_t tg = a.targets[o * a.ts_outer + i_in * a.ts_inner];
+            float lp = -INFINITY, lpf = 0.f;
+            if (tg >= 0 && tg < vocab) {
+                const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(row, tg), a.tparam);
+                const bool kept = xt > sh.thr || (xt == sh.thr && tg >= tie);
+                if (kept) lp = xt - sh.lse_kept;
+                lpf = xt - lse_full;
+            }
+            a.logprob[r] = lp;
+            if (a.logprob_full) a.logprob_full[r] = lpf;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward / materialisation: one streaming pass with the saved keep predicate
+// ---------------------------------------------------------------------------------------------
+struct SelBwdArgs {
+    const void* logits;
+    int64_t n_inner, vocab, stride_outer, stride_inner;
+    const int64_t* targets;
+    int64_t ts_outer, ts_inner;
+    float tparam;
+    const float* thr;
+    const int32_t* tie;
+    const float* lse_kept;
+    const float* grad;
+    int64_t gs_outer, gs_inner;
+    void* out;  // dlogits, or filtered logits
+    int64_t d_n_inner, ds_outer, ds_inner;
+    uint8_t* keep_out;  // [rows, vocab] or NULL (filter mode)
+};
+
+// MODE 0: gradient, MODE 1: filtered logits (-inf outside the kept set) + keep mask
+template <int DT, int TEMP, int MODE>
+__global__ __launch_bounds__(kSelBlock) void topk_topp_stream_kernel(SelBwdArgs a) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const int64_t r = blockIdx.x;
+    const int64_t o = r / a.d_n_inner, i_in = r - o * a.d_n_inner;
+    char* out = static_cast<char*>(a.out) + (o * a.ds_outer + i_in * a.ds_inner) * Row<DT>::BYTES;
+    const int64_t vocab = a.vocab;
+    float g = 0.f;
+    if (MODE == 0 && i_in < a.n_inner) g = a.grad[o * a.gs_outer + i_in * a.gs_inner];
+    if (MODE == 0 && g == 0.f) {
+        for (int64_t e = tid; e < vocab; e += kSelBlock) Row<DT>::store1(out, e, 0.f);
+        return;
+    }
+    const int64_t rr = o * a.n_inner + i_in;
+    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i_in * a.stride_inner) * Row<DT>::BYTES;
+    const float thr = a.thr[rr], lse = a.lse_kept[rr];
+    const int64_t tie = a.tie[rr];
+    int64_t tg = -1;
+    if (MODE == 0) tg = a.targets[o * a.ts_outer + i_in * a.ts_inner];
+    uint8_t* keep_row = (MODE == 1 && a.keep_out) ? a.keep_out + rr * vocab : nullptr;
+
+    auto elem = [&](float x_raw, int64_t idx, bool& keep) -> float {
+        const float x = scale_logit<DT, TEMP>(x_raw, a.tparam);
+        keep = x > thr || (x == thr && idx >= tie);
+        if (MODE == 1) return keep ? x : -INFINITY;
+        if (!keep) return 0.f;
+        float d = ((idx == tg ? 1.f : 0.f) - fast_exp2((x - lse) * kLog2e)) * g;
+        if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
+        if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
+        return d;
+    };
+
+    const int64_t head = sel_row_head<DT>(row, vocab);
+    if (sel_row_head<DT>(out, vocab) != head) {
+        for (int64_t e = tid; e < vocab; e += kSelBlock) {
+            bool keep;
+            Row<DT>::store1(out, e, elem(Row<DT>::load1(row, e), e, keep));
+            if (keep_row) keep_row[e] = keep ? 1 : 0;
+        }
+        return;
+    }
+    const int64_t nvec = (vocab - head) / EPV;
+    const int64_t tail0 = head + nvec * EPV;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(row + head * Row<DT>::BYTES);
+    u32x4* ov = reinterpret_cast<u32x4*>(out + head * Row<DT>::BYTES);
+    for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
+        float t[EPV];
+        Row<DT>::decode(__builtin_nontemporal_load(xv + vi), t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) {
+            bool keep;
+            const int64_t idx = head + vi * EPV + k;
+            t[k] = elem(t[k], idx, keep);
+            if (keep_row) keep_row[idx] = keep ? 1 : 0;
+        }
+        __builtin_nontemporal_store(Row<DT>::encode(t), ov + vi);
+    }
+    for (int w = 0; w < 2; ++w) {
+        const int64_t e = w == 0 ? (tid < head ? tid : -1) : (tail0 + tid < vocab ? tail0 + tid : -1);
+        if (e < 0) continue;
+        bool keep;
+        Row<DT>::store1(out, e, elem(Row<DT>::load1(row, e), e, keep));
+        if (keep_row) keep_row[e] = keep ? 1 : 0;
+    }
+}
+
+static int temp_code3(float temperature, int mode, float* tparam) {
+    if (temperature == 1.0f) { *tparam = 1.f; return 0; }
+    if (mode == NRL_TEMP_DIV) { *tparam = temperature; return 1; }
+    *tparam = 1.0f / temperature;
+    return 2;
+}
+
+static int check_sel_rows(const nrl_rows* r, bool need_targets) {
+    if (!r) return fail(NRL_E_INVALID, "rows is NULL");
+    if (r->dtype != NRL_F32 && r->dtype != NRL_BF16 && r->dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype %d", r->dtype);
+    if (r->n_outer < 0 || r->n_inner < 0 || r->vocab <= 0) return fail(NRL_E_INVALID, "bad shape");
+    if (r->vocab >= (1ll << 31)) return fail(NRL_E_INVALID, "vocabulary too large");
+    if (r->n_outer * r->n_inner > 0 && (!r->logits || (need_targets && !r->targets))) return fail(NRL_E_INVALID, "null logits or targets");
+    if (r->vocab_start != 0 || r->vocab_end != r->vocab) return fail(NRL_E_UNSUPPORTED, "top-k/top-p needs the full vocabulary on this GPU");
+    if (!(r->temperature > 0.f)) return fail(NRL_E_INVALID, "temperature must be positive");
+    if (r->n_outer * r->n_inner >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    return NRL_OK;
+}
+
+#define NRL_SEL_DISPATCH(DT_, TC_, ...)                                                     \
+    switch ((DT_) * 3 + (TC_)) {                                                            \
+        case NRL_F32 * 3 + 0: { constexpr int DT = NRL_F32, TEMP = 0; __VA_ARGS__; break; }  \
+        case NRL_F32 * 3 + 1: { constexpr int DT = NRL_F32, TEMP = 1; __VA_ARGS__; break; }  \
+        case NRL_F32 * 3 + 2: { constexpr int DT = NRL_F32, TEMP = 2; __VA_ARGS__; break; }  \
+        case NRL_BF16 * 3 + 0: { constexpr int DT = NRL_BF16, TEMP = 0; __VA_ARGS__; break; } \
+        case NRL_BF16 * 3 + 1: { constexpr int DT = NRL_BF16, TEMP = 1; __VA_ARGS__; break; } \
+        case NRL_BF16 * 3 + 2: { constexpr int DT = NRL_BF16, TEMP = 2; __VA_ARGS__; break; } \
+        case NRL_F16 * 3 + 0: { constexpr int DT = NRL_F16, TEMP = 0; __VA_ARGS__; break; }  \
+        case NRL_F16 * 3 + 1: { constexpr int DT = NRL_F16, TEMP = 1; __VA_ARGS__; break; }  \
+        default: { constexpr int DT = NRL_F16, TEMP = 2; __VA_ARGS__; break; }              \
+    }
+
+}  // namespace nrl
+
+using namespace nrl;
+
+extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
+                                         float* thr_out, int32_t* tie_out, float* lse_kept_out,
+                                         float* logprob_unfiltered_out, float* lse_full_out, int32_t* overflow_flag,
+                                         void* stream) {
+    if (int e = check_sel_rows(rows, logprob_out != nullptr)) return e;
+    const bool use_k = top_k > 0, use_p = top_p < 1.0f;
+    if (!use_k && !use_p) return fail(NRL_E_INVALID, "neither top-k nor top-p is active");
+    if (use_p && !(top_p > 0.f)) return fail(NRL_E_INVALID, "top_p must be in (0, 1]");
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!thr_out || !tie_out || !lse_kept_out || !overflow_flag) return fail(NRL_E_INVALID, "null state output");
+    SelArgs a;
+    a.logits = rows->logits; a.n_inner = rows->n_inner; a.vocab = rows->vocab;
+    a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
+    a.targets = rows->targets; a.ts_outer = rows->tgt_stride_outer; a.ts_inner = rows->tgt_stride_inner;
+    a.top_k = use_k ? static_cast<int>(top_k > (1ll << 30) ? (1ll << 30) : top_k) : 0;
+    a.top_p = use_p ? top_p : 1.0f;
+    a.logprob = logprob_out; a.thr = thr_out; a.tie = tie_out; a.lse_kept = lse_kept_out;
+    a.logprob_full = logprob_unfiltered_out; a.lse_full = lse_full_out; a.overflow = overflow_flag;
+    const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
+    const bool full = !use_k || logprob_unfiltered_out != nullptr || lse_full_out != nullptr;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (full) {
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    } else {
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, false><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    }
+    return check_launch("topk_topp_logprob_fwd");
+}
+
+extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,
+                                         const float* lse_kept, const float* grad, int64_t grad_stride_outer,
+                                         int64_t grad_stride_inner, void* dlogits, int64_t d_n_inner,
+                                         int64_t d_stride_outer, int64_t d_stride_inner, void* stream) {
+    if (int e = check_sel_rows(rows, true)) return e;
+    if (d_n_inner < rows->n_inner) return fail(NRL_E_INVALID, "d_n_inner < n_inner");
+    const int64_t n = rows->n_outer * d_n_inner;
+    if (n == 0) return NRL_OK;
+    if (n >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    if (!dlogits || (rows->n_outer * rows->n_inner > 0 && (!thr || !tie || !lse_kept || !grad))) return fail(NRL_E_INVALID, "null argument");
+    SelBwdArgs a;
+    a.logits = rows->logits; a.n_inner = rows->n_inner; a.vocab = rows->vocab;
+    a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
+    a.targets = rows->targets; a.ts_outer = rows->tgt_stride_outer; a.ts_inner = rows->tgt_stride_inner;
+    a.thr = thr; a.tie = tie; a.lse_kept = lse_kept; a.grad = grad;
+    a.gs_outer = grad_stride_outer; a.gs_inner = grad_stride_inner;
+    a.out = dlogits; a.d_n_inner = d_n_inner; a.ds_outer = d_stride_outer; a.ds_inner = d_stride_inner;
+    a.keep_out = nullptr;
+    const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 0><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    return check_launch("topk_topp_logprob_bwd");
+}
+
+extern "C" int nrl_topk_topp_filter(const nrl_rows* rows, const float* thr, const int32_t* tie, void* filtered_out,
+                                    int64_t f_stride_outer, int64_t f_stride_inner, uint8_t* keep_out, void* stream) {
+    if (int e = check_sel_rows(rows, false)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!thr || !tie || !filtered_out) return fail(NRL_E_INVALID, "null argument");
+    SelBwdArgs a;
+    a.logits = rows->logits; a.n_inner = rows->n_inner; a.vocab = rows->vocab;
+    a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
+    a.targets = nullptr; a.ts_outer = 0; a.ts_inner = 0;
+    a.thr = thr; a.tie = tie; a.lse_kept = thr; a.grad = nullptr; a.gs_outer = 0; a.gs_inner = 0;
+    a.out = filtered_out; a.d_n_inner = rows->n_inner; a.ds_outer = f_stride_outer; a.ds_inner = f_stride_inner;
+    a.keep_out = keep_out;
+    const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 1><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    return check_launch("topk_topp_filter");
+}

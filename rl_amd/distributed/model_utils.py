@@ -129,6 +129,42 @@ class ChunkedDistributedLogprob(torch.autograd.Function):
         return _bwd_rows(ctx, grad_outputs[0]), None, None, None, None, None, None
 
 
+class DistributedLogprobWithSampling(torch.autograd.Function):
+    """``model_utils.py:383-510`` on one rank: ``apply(logits, target, tp_group, top_k, top_p,
+    inference_only=False)`` with ``target`` already shifted.  No all-to-all and no sort: the selection
+    kernel finds the kept set of every row on chip."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, target, tp_group, top_k, top_p, inference_only=False):
+        from .sampling_logprob import _sampled_fwd
+
+        _require_single_rank(tp_group, "DistributedLogprobWithSampling")
+        return _sampled_fwd(ctx, vocab_parallel_logits, target, target.shape[1], top_k, top_p, inference_only)
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        from .sampling_logprob import _sampled_bwd
+
+        return _sampled_bwd(ctx, grad_outputs[0]), None, None, None, None, None
+
+
+class ChunkedDistributedLogprobWithSampling(torch.autograd.Function):
+    """``model_utils.py:513-719``; ``chunk_size`` bounds the reference's sort buffers and has no effect here."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, target, tp_group, top_k, top_p, chunk_size, inference_only=False):
+        from .sampling_logprob import _sampled_fwd
+
+        _require_single_rank(tp_group, "ChunkedDistributedLogprobWithSampling")
+        return _sampled_fwd(ctx, vocab_parallel_logits, target, target.shape[1], top_k, top_p, inference_only)
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        from .sampling_logprob import _sampled_bwd
+
+        return _sampled_bwd(ctx, grad_outputs[0]), None, None, None, None, None, None
+
+
 def _get_tokens_on_this_cp_rank(input_ids, cp_rank: int, cp_size: int, seq_dim: int = 1):
     """``model_utils.py:1199-1233`` for the only context-parallel size this build runs with."""
     if cp_size != 1:

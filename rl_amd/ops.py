@@ -213,6 +213,94 @@ for _name, _fn in (("logprob_packed_fwd", _logprob_packed_fwd), ("logprob_packed
 
 
 # ------------------------------------------------------------------------------------------------
+# K3: top-k / top-p
+# ------------------------------------------------------------------------------------------------
+_LIB.define(
+    "topk_topp_logprob_fwd(Tensor logits, Tensor? targets, int n_inner, int top_k, float top_p, float temperature, "
+    "int temp_mode, bool want_unfiltered) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)"
+)
+_LIB.define(
+    "topk_topp_logprob_bwd(Tensor logits, Tensor targets, Tensor thr, Tensor tie, Tensor lse_kept, Tensor grad, "
+    "int n_inner, float temperature, int temp_mode) -> Tensor"
+)
+_LIB.define(
+    "topk_topp_filter(Tensor logits, Tensor thr, Tensor tie, float temperature, int temp_mode) -> (Tensor, Tensor)"
+)
+
+
+def _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, temp_mode, want_unfiltered):
+    """-> (logprob [B,n] (empty without targets), thr, tie, lse_kept, unfiltered logprob (or empty), overflow flag)."""
+    _need_gpu(logits, targets)
+    b, s, v = logits.shape
+    dummy = targets if targets is not None else torch.zeros((b, max(n_inner, 1)), dtype=torch.int64, device=logits.device)
+    rows = _rows(logits, dummy, n_inner, 0, v, temperature, temp_mode)
+    if targets is None:
+        rows.targets = 0
+    dev = logits.device
+    with torch.cuda.device(dev):
+        f32 = dict(dtype=torch.float32, device=dev)
+        lp = torch.empty((b, n_inner) if targets is not None else (0,), **f32)
+        thr = torch.empty((b, n_inner), **f32)
+        tie = torch.empty((b, n_inner), dtype=torch.int32, device=dev)
+        lse = torch.empty((b, n_inner), **f32)
+        lpu = torch.empty((b, n_inner) if want_unfiltered else (0,), **f32)
+        flag = torch.zeros((1,), dtype=torch.int32, device=dev)
+        with _timed("topk_topp_fwd"):
+            code = _lib.load().nrl_topk_topp_logprob_fwd(
+                C.byref(rows), int(top_k), float(top_p), _ptr(lp if targets is not None else None), _ptr(thr), _ptr(tie),
+                _ptr(lse), _ptr(lpu if want_unfiltered else None), None, _ptr(flag), _stream(),
+            )
+    _lib.check(code, "nrl_topk_topp_logprob_fwd")
+    return lp, thr, tie, lse, lpu, flag
+
+
+def _topk_topp_logprob_bwd(logits, targets, thr, tie, lse_kept, grad, n_inner, temperature, temp_mode):
+    _need_gpu(logits, targets, thr, tie, lse_kept, grad)
+    b, s, v = logits.shape
+    rows = _rows(logits, targets, n_inner, 0, v, temperature, temp_mode)
+    for t, name in ((thr, "thr"), (tie, "tie"), (lse_kept, "lse_kept")):
+        if tuple(t.shape) != (b, n_inner) or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous [B, n_inner] tensor")
+    if thr.dtype != torch.float32 or lse_kept.dtype != torch.float32 or tie.dtype != torch.int32:
+        raise ValueError("thr / lse_kept must be fp32 and tie int32")
+    if tuple(grad.shape) != (b, n_inner) or grad.dtype != torch.float32:
+        raise ValueError("grad must be fp32 [B, n_inner]")
+    with torch.cuda.device(logits.device):
+        d = torch.empty((b, s, v), dtype=logits.dtype, device=logits.device)
+        with _timed("topk_topp_bwd"):
+            code = _lib.load().nrl_topk_topp_logprob_bwd(
+                C.byref(rows), _ptr(thr), _ptr(tie), _ptr(lse_kept), _ptr(grad), grad.stride(0), grad.stride(1),
+                _ptr(d), s, d.stride(0), d.stride(1), _stream(),
+            )
+    _lib.check(code, "nrl_topk_topp_logprob_bwd")
+    return d
+
+
+def _topk_topp_filter(logits, thr, tie, temperature, temp_mode):
+    _need_gpu(logits, thr, tie)
+    b, s, v = logits.shape
+    dummy = torch.zeros((b, max(s, 1)), dtype=torch.int64, device=logits.device)
+    rows = _rows(logits, dummy, s, 0, v, temperature, temp_mode)
+    rows.targets = 0
+    if tuple(thr.shape) != (b, s) or tuple(tie.shape) != (b, s) or not thr.is_contiguous() or not tie.is_contiguous():
+        raise ValueError("thr / tie must be contiguous [B, S]")
+    with torch.cuda.device(logits.device):
+        out = torch.empty((b, s, v), dtype=logits.dtype, device=logits.device)
+        keep = torch.empty((b, s, v), dtype=torch.uint8, device=logits.device)
+        code = _lib.load().nrl_topk_topp_filter(
+            C.byref(rows), _ptr(thr), _ptr(tie), _ptr(out), out.stride(0), out.stride(1), _ptr(keep), _stream()
+        )
+    _lib.check(code, "nrl_topk_topp_filter")
+    return out, keep
+
+
+for _name, _fn in (("topk_topp_logprob_fwd", _topk_topp_logprob_fwd), ("topk_topp_logprob_bwd", _topk_topp_logprob_bwd),
+                   ("topk_topp_filter", _topk_topp_filter)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
+# ------------------------------------------------------------------------------------------------
 # K4
 # ------------------------------------------------------------------------------------------------
 _LIB.define(
