@@ -213,6 +213,31 @@ int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int64_t prompt
                            float* baseline_out, float* std_out, float* adv_out, int32_t* group_out,
                            void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * K6  Fused lm_head -> token logprob on the bf16 matrix cores (MFMA), never materialising the
+ * [N, V] logits.  Replaces ChunkedDistributedHiddenStatesToLogprobs
+ * (nemo_rl/distributed/model_utils.py:2137-2316) at TP = 1.
+ * hidden: bf16 [N, H] rows of stride ldh (token order is the caller's); weight: bf16 [V, H] rows of
+ * stride ldw; both 16-byte aligned, H and the strides multiples of 8.  targets: int64 [N], already
+ * shifted.  The logits of a tile are rounded to bf16 before the softmax, as the reference's bf16
+ * matmul does.  logprob_out / lse_out: fp32 [N] (lse_out may be NULL).
+ * Backward: grad fp32 [N] -> dhidden_out fp32 [N, H] (row stride ld_dh) and dweight_out bf16 [V, H]
+ * (row stride ld_dw), accumulated in fp32 and narrowed once.  Tokens are processed in chunks of 4096:
+ * per chunk the gradient of the logits exists as bf16 [chunk, V] (twice, one transposed).
+ * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
+ * ------------------------------------------------------------------------------------------ */
+int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab);
+int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
+                           const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
+                           int64_t vocab_start, int64_t vocab_end, float* logprob_out, float* lse_out,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab);
+int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
+                           const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
+                           int64_t vocab_start, int64_t vocab_end, const float* lse, const float* grad,
+                           float* dhidden_out, int64_t ld_dh, void* dweight_out, int64_t ld_dw,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,10 @@ SIGNATURES = {
     "nrl_grpo_loss_workspace_bytes": (_I64, [_I64]),
     "nrl_grpo_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _I64, _P]),
+    "nrl_lmhead_fwd_workspace_bytes": (_I64, [_I64, _I64]),
+    "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P]),
+    "nrl_lmhead_bwd_workspace_bytes": (_I64, [_I64, _I64, _I64]),
+    "nrl_lmhead_logprob_bwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _P, _I64, _P]),
     "nrl_group_workspace_bytes": (_I64, [_I64]),
     "nrl_group_baseline_std": (C.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _I32, _I32, _P, _P, _P, _P, _P, _I64, _P]),
 }

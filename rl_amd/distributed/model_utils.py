@@ -332,3 +332,66 @@ def from_parallel_logits_to_logprobs_packed_sequences(
         logits2d, targets1d, bool(target_is_pre_rolled), cu_dev, int(unpacked_seqlen), vocab_start_index,
         vocab_end_index, inference_only,
     )
+
+
+# ------------------------------------------------------------------------------------------------
+# fused lm_head: hidden states -> logprobs
+# ------------------------------------------------------------------------------------------------
+class ChunkedDistributedHiddenStatesToLogprobs(torch.autograd.Function):
+    """``model_utils.py:2137-2316`` on one rank: ``apply(hidden [S,B,H], target [B,S] (already shifted),
+    output_weight [V,H], vocab_start_index, vocab_end_index, chunk_size, tp_group, inference_only)``
+    -> fp32 ``[B,S]``.  The product runs on the bf16 matrix cores with the softmax folded into the
+    GEMM epilogue; ``chunk_size`` (the reference's sequence chunk) is not needed to bound memory in the
+    forward, and the backward chunks tokens on its own."""
+
+    @staticmethod
+    def forward(ctx, tensor_parallel_hidden_states, target, output_weight_layer, vocab_start_index, vocab_end_index,
+                chunk_size, tp_group, inference_only=False):
+        _require_single_rank(tp_group, "ChunkedDistributedHiddenStatesToLogprobs")
+        hidden = tensor_parallel_hidden_states.detach()
+        if hidden.dim() != 3:
+            raise ValueError(f"expected hidden states [S, B, H], got {tuple(hidden.shape)}")
+        s, b, h = hidden.shape
+        hidden2d = hidden.reshape(s * b, h)
+        weight = output_weight_layer.detach()
+        tgt = _to_device(target, hidden).long().t().contiguous().reshape(-1)  # token order of the hidden rows: (s, b)
+        lp, lse = _OPS.lmhead_logprob_fwd(hidden2d, weight, tgt, vocab_start_index, vocab_end_index)
+        ctx.saved = (not inference_only) and (ctx.needs_input_grad[0] or ctx.needs_input_grad[2])
+        if ctx.saved:
+            ctx.save_for_backward(hidden2d, weight, tgt, lse)
+            ctx.meta = (s, b, h, vocab_start_index, vocab_end_index, tensor_parallel_hidden_states.dtype,
+                        output_weight_layer.dtype)
+        return lp.view(s, b).t().contiguous()
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        if not ctx.saved:
+            raise RuntimeError("backward through a logprob computed with inference_only=True")
+        hidden2d, weight, tgt, lse = ctx.saved_tensors
+        s, b, h, v0, v1, h_dtype, w_dtype = ctx.meta
+        grad = grad_outputs[0].float().t().contiguous().reshape(-1)
+        dh, dw = _OPS.lmhead_logprob_bwd(hidden2d, weight, tgt, lse, grad, v0, v1)
+        return dh.view(s, b, h).to(h_dtype), None, dw.to(w_dtype), None, None, None, None, None
+
+
+def from_parallel_hidden_states_to_logprobs(
+    tensor_parallel_hidden_states: torch.Tensor,
+    output_weight_layer: torch.Tensor,
+    runtime_gather_output: bool,
+    target: torch.Tensor,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    tp_group: Any,
+    inference_only: bool = False,
+    cp_group: Optional[Any] = None,
+    chunk_size: Optional[int] = None,
+) -> torch.Tensor:
+    """``model_utils.py:2106-2134``: hidden ``[S,B,H]`` (sequence first), weight ``[V,H]``, unshifted
+    ``target [B,S]`` -> ``[B, S-1]`` fp32."""
+    assert _group_size(cp_group) == 1, "Context parallelism is not supported for linear CE fusion loss"
+    rolled = target.roll(shifts=-1, dims=-1)
+    logprobs = ChunkedDistributedHiddenStatesToLogprobs.apply(
+        tensor_parallel_hidden_states, rolled, output_weight_layer, vocab_start_index, vocab_end_index, chunk_size,
+        tp_group, inference_only,
+    )
+    return logprobs[:, :-1]

@@ -449,3 +449,83 @@ def _group_baseline_std(prompts, rewards, valid, std_rewards, leave_one_out, nor
 
 _LIB.impl("group_baseline_std", _group_baseline_std, "CUDA")
 _LIB.impl("group_baseline_std", _group_baseline_std, "CPU")
+
+
+# ------------------------------------------------------------------------------------------------
+# K6: fused lm_head
+# ------------------------------------------------------------------------------------------------
+_LIB.define(
+    "lmhead_logprob_fwd(Tensor hidden, Tensor weight, Tensor targets, int vocab_start, int vocab_end) -> (Tensor, Tensor)"
+)
+_LIB.define(
+    "lmhead_logprob_bwd(Tensor hidden, Tensor weight, Tensor targets, Tensor lse, Tensor grad, int vocab_start, "
+    "int vocab_end) -> (Tensor, Tensor)"
+)
+
+
+def _check_lmhead(hidden, weight, targets):
+    _need_gpu(hidden, weight, targets)
+    if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
+        raise ValueError(f"expected hidden [N,H] and weight [V,H], got {tuple(hidden.shape)}, {tuple(weight.shape)}")
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("the fused lm_head path runs on bf16 hidden states and weights")
+    if hidden.shape[1] % 8:
+        raise ValueError("the hidden size must be a multiple of 8")
+    if targets.dtype != torch.int64 or tuple(targets.shape) != (hidden.shape[0],) or not targets.is_contiguous():
+        raise ValueError("targets must be a contiguous int64 [N] tensor")
+    hidden = hidden if hidden.stride(1) == 1 and hidden.stride(0) % 8 == 0 and hidden.data_ptr() % 16 == 0 else hidden.contiguous()
+    weight = weight if weight.stride(1) == 1 and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0 else weight.contiguous()
+    return hidden, weight
+
+
+def _ws(nbytes, dev):
+    return torch.empty(((nbytes + 255) // 256 * 32,), dtype=torch.float64, device=dev)  # 256-byte granules
+
+
+def _lmhead_logprob_fwd(hidden, weight, targets, vocab_start, vocab_end):
+    hidden, weight = _check_lmhead(hidden, weight, targets)
+    n, h = hidden.shape
+    v = weight.shape[0]
+    lib = _lib.load()
+    dev = hidden.device
+    with torch.cuda.device(dev):
+        lp = torch.empty((n,), dtype=torch.float32, device=dev)
+        lse = torch.empty((n,), dtype=torch.float32, device=dev)
+        nbytes = lib.nrl_lmhead_fwd_workspace_bytes(n, v)
+        ws = _ws(nbytes, dev)
+        with _timed("lmhead_fwd"):
+            code = lib.nrl_lmhead_logprob_fwd(
+                _ptr(hidden), n, h, hidden.stride(0), _ptr(weight), v, weight.stride(0), _ptr(targets), vocab_start,
+                vocab_end, _ptr(lp), _ptr(lse), _ptr(ws), ws.numel() * 8, _stream(),
+            )
+    _lib.check(code, "nrl_lmhead_logprob_fwd")
+    return lp, lse
+
+
+def _lmhead_logprob_bwd(hidden, weight, targets, lse, grad, vocab_start, vocab_end):
+    hidden, weight = _check_lmhead(hidden, weight, targets)
+    _need_gpu(lse, grad)
+    n, h = hidden.shape
+    v = weight.shape[0]
+    for t, name in ((lse, "lse"), (grad, "grad")):
+        if t.dtype != torch.float32 or tuple(t.shape) != (n,) or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous fp32 [N] tensor")
+    lib = _lib.load()
+    dev = hidden.device
+    with torch.cuda.device(dev):
+        dh = torch.empty((n, h), dtype=torch.float32, device=dev)
+        dw = torch.empty((v, h), dtype=torch.bfloat16, device=dev)
+        nbytes = lib.nrl_lmhead_bwd_workspace_bytes(n, h, v)
+        ws = _ws(nbytes, dev)
+        with _timed("lmhead_bwd"):
+            code = lib.nrl_lmhead_logprob_bwd(
+                _ptr(hidden), n, h, hidden.stride(0), _ptr(weight), v, weight.stride(0), _ptr(targets), vocab_start,
+                vocab_end, _ptr(lse), _ptr(grad), _ptr(dh), h, _ptr(dw), h, _ptr(ws), ws.numel() * 8, _stream(),
+            )
+    _lib.check(code, "nrl_lmhead_logprob_bwd")
+    return dh, dw
+
+
+for _name, _fn in (("lmhead_logprob_fwd", _lmhead_logprob_fwd), ("lmhead_logprob_bwd", _lmhead_logprob_bwd)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
