@@ -33,6 +33,8 @@ WORKLOADS = {
     # name: (sequences, seq_len, vocab, dtype, sequences per microbatch, logit std, spike p)
     "c2": dict(seqs=128, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=3.0, spike_p=0.3,
                desc="BASELINE config 2: 16 prompts x 8 = 128 seq x 4096 tok, V=151936 bf16, fwd+bwd to dlogits"),
+    "c3": dict(seqs=16, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=0.0, spike_p=0.0, hidden=4096,
+               desc="BASELINE config 3: fused lm_head + logprob, hidden [65536,4096] bf16, W [151936,4096] bf16, fwd+bwd (dH, dW)"),
     "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
                desc="BASELINE config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
 }
@@ -153,6 +155,74 @@ def cpu_baseline(torch, w, seconds):
                        f"iterations ({sum(times):.1f} s total), {threads} threads of {cores} host cores")
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
+
+
+def bench_lmhead(args, torch, w):
+    """Config 3: hidden states -> logprobs -> loss -> (dH, dW) through the fused MFMA path."""
+    from rl_amd import ops
+    from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn
+    from rl_amd.distributed.model_utils import from_parallel_hidden_states_to_logprobs
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    b, s, h, v = (args.seqs or w["seqs"]), w["seq_len"], w["hidden"], w["vocab"]
+    g = torch.Generator(device=dev).manual_seed(1003)
+    hidden = torch.randn((s, b, h), generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+    weight = (torch.randn((v, h), generator=g, device=dev) * 0.02).to(torch.bfloat16).requires_grad_(True)
+    ids = torch.randint(0, v, (b, s), generator=g, device=dev)
+    with torch.no_grad():
+        cur = from_parallel_hidden_states_to_logprobs(hidden, weight, False, ids, 0, v, None, inference_only=True)
+    cur = torch.cat([torch.zeros((b, 1), device=dev), cur], dim=1)
+    prev = cur + 0.05 * torch.randn((b, s), generator=g, device=dev)
+    tm = (torch.arange(s, device=dev).unsqueeze(0) >= torch.randint(256, 1025, (b, 1), generator=g, device=dev)).long()
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": torch.ones(b, device=dev),
+            "advantages": torch.randn((b, 1), generator=g, device=dev).expand(b, s).contiguous(),
+            "prev_logprobs": prev, "generation_logprobs": prev,
+            "reference_policy_logprobs": cur + 0.05 * torch.randn((b, s), generator=g, device=dev)}
+    fn = ClippedPGLossFn(ClippedPGLossConfig(), use_fused_linear_logprobs=True)
+    gs, gt = torch.tensor(float(b), device=dev), tm[:, 1:].sum().float()
+
+    def step():
+        lp = from_parallel_hidden_states_to_logprobs(hidden, weight, False, ids, 0, v, None)
+        loss, _ = fn(next_token_logprobs=lp, data=data, global_valid_seqs=gs, global_valid_toks=gt)
+        dh, dw = torch.autograd.grad(loss, (hidden, weight))
+        del dh, dw
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = EventTimer(torch)
+    ops.KERNEL_TIMER = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    k = timer.summary()
+    n = b * s
+    fwd_ms, bwd_ms = k["lmhead_fwd"]["avg_ms"], k["lmhead_bwd"]["avg_ms"]
+    fwd_tf = 2.0 * n * h * v / (fwd_ms * 1e-3) / 1e12
+    bwd_alg_tf = 4.0 * n * h * v / (bwd_ms * 1e-3) / 1e12       # dH + dW
+    bwd_exec_tf = 6.0 * n * h * v / (bwd_ms * 1e-3) / 1e12      # + recomputed logits
+    result = {
+        "metric": "fused lm_head + GRPO loss fwd/bwd tokens/s; % of bf16 MFMA peak",
+        "value": n * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["desc"], "tokens": n, "hidden": h, "vocab": v},
+        "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tf, "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "avg_launch_ms": fwd_ms},
+        "roofline_bwd": {"bound": "mfma", "kernel": "lmhead backward (grad + dH + dW GEMMs)", "achieved": bwd_alg_tf,
+                         "achieved_incl_recompute": bwd_exec_tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": bwd_alg_tf / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": bwd_ms},
+        "algorithmic_tflops_end_to_end": 6.0 * n * h * v * args.steps / elapsed / 1e12,
+        "kernel_ms": {kk: round(vv["avg_ms"], 4) for kk, vv in k.items()},
+    }
+    print(json.dumps(result))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -165,6 +235,8 @@ def main():
 
     _lib.load()
     w = dict(WORKLOADS[args.workload])
+    if args.workload == "c3":
+        return bench_lmhead(args, torch, w)
     if args.seqs:
         w["seqs"] = args.seqs
         w["mb_seqs"] = min(w["mb_seqs"], args.seqs)

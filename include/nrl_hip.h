@@ -192,6 +192,24 @@ int nrl_grpo_loss_fwd_bwd(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, fl
                           float* dlp_out, float* dlpu_out, float* metrics_out, void* workspace,
                           int64_t workspace_bytes, void* stream);
 
+/* Fused variant: one pass over the logits computes the token logprob (as K1), the loss terms and
+ * d loss / d logprob of that token (as K4) and writes dlogits (as K2) from the row held on chip:
+ * the logits are read once and the gradient written once.  Replaces, for a single-GPU worker,
+ * prepare_loss_input + ClippedPGLossFn + the backward of the logprob op
+ * (nemo_rl/algorithms/loss/wrapper.py:292-322 with loss_functions.py:374-788 and
+ * nemo_rl/distributed/model_utils.py:120-207).  `in` is as for nrl_grpo_loss_fwd_bwd with lp / lpu
+ * ignored (batch = rows->n_outer, sm1 = rows->n_inner).  dlogits holds loss_scale * d loss / d logits
+ * (layout as in nrl_logprob_bwd; may alias the logits).  logprob_out: fp32 [B, n_inner]; positions
+ * whose mask is zero are not evaluated (logprob 0, zero gradient row, logits not read).
+ * Returns NRL_E_UNSUPPORTED for what cannot be fused: sequence-level probability ratios (GSPO), the
+ * positive-example NLL term, rows that are not 16-byte aligned or longer than 20480 16-byte vectors.
+ * workspace: nrl_fused_workspace_bytes(B, n_inner) bytes, 8-byte aligned. */
+int64_t nrl_fused_workspace_bytes(int64_t batch, int64_t n_inner);
+int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
+                               float loss_scale, void* dlogits, int64_t d_n_inner, int64_t d_stride_outer,
+                               int64_t d_stride_inner, float* logprob_out, float* loss_out,
+                               float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* NLLLossFn scalar branch (loss_functions.py:818-842): loss = -sum(lp*mask)/(Gt+1e-8);
  * metrics_out[0..2] = {loss, num_unmasked_tokens, num_valid_samples}; dlp_out = -mask/(Gt+1e-8). */
 int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,

@@ -76,6 +76,9 @@ SIGNATURES = {
     "nrl_topk_topp_filter": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P, _I64, _I64, _P, _P]),
     "nrl_grpo_loss_workspace_bytes": (_I64, [_I64]),
     "nrl_grpo_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _P, _I64, _P]),
+    "nrl_fused_workspace_bytes": (_I64, [_I64, _I64]),
+    "nrl_fused_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _F, _P, _I64,
+                                             _I64, _I64, _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _I64, _P]),
     "nrl_lmhead_fwd_workspace_bytes": (_I64, [_I64, _I64]),
     "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P]),

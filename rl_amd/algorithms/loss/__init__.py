@@ -1,5 +1,6 @@
 """Loss functions of the GRPO hot path (counterpart of ``nemo_rl/algorithms/loss/__init__.py``)."""
 
+from .fused import fused_logits_clipped_pg_loss, why_not_fusable
 from .interfaces import LossFunction, LossInputType, LossType, MetricNormalizer
 from .loss_functions import ClippedPGLossConfig, ClippedPGLossFn, NLLLossFn
 from .utils import prepare_loss_input, prepare_packed_loss_input
@@ -10,7 +11,7 @@ from .wrapper import (
 )
 
 __all__ = [
-    "ClippedPGLossConfig", "ClippedPGLossFn", "NLLLossFn", "LossFunction", "LossInputType", "LossType",
+    "fused_logits_clipped_pg_loss", "why_not_fusable", "ClippedPGLossConfig", "ClippedPGLossFn", "NLLLossFn", "LossFunction", "LossInputType", "LossType",
     "MetricNormalizer", "prepare_loss_input", "prepare_packed_loss_input", "SequencePackingFusionLossWrapper",
     "SequencePackingLossWrapper", "wrap_loss_fn_with_input_preparation",
 ]

@@ -1,0 +1,143 @@
+"""Single-pass path: logits -> clipped-PG loss -> dlogits in one kernel.
+
+``fused_logits_clipped_pg_loss`` does what ``prepare_loss_input`` + ``ClippedPGLossFn`` + the
+backward of the logprob op do (``nemo_rl/algorithms/loss/wrapper.py:292-322``), but the logits are
+read once and the gradient written once: the kernel keeps each row on chip between the
+log-sum-exp and the gradient and evaluates the token's loss terms in between.  The gradient exists
+as soon as the forward returns; ``backward`` hands it to autograd (scaled if the upstream gradient
+is not the ``loss_scale`` it was computed with).
+"""
+
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+
+from ... import ops as _ops  # noqa: F401
+from ..._lib import METRIC_SLOTS
+from .interfaces import LossType
+from .loss_functions import ClippedPGLossFn, _f32, _global_valid
+
+_OPS = torch.ops.rl_amd
+
+
+def why_not_fusable(loss_fn, logits, data, sampling_params=None) -> Optional[str]:
+    """None if the fused kernel covers this call, else the reason it does not."""
+    from ..logits_sampling_utils import need_top_k_or_top_p_filtering
+
+    if type(loss_fn) is not ClippedPGLossFn:
+        return "not a ClippedPGLossFn"
+    if getattr(loss_fn, "use_fused_linear_logprobs", False):
+        return "the model already returned logprobs"
+    if need_top_k_or_top_p_filtering(sampling_params):
+        return "top-k/top-p filtering"
+    if loss_fn.sequence_level_importance_ratios and not (loss_fn.disable_ppo_ratio or loss_fn.force_on_policy_ratio):
+        return "sequence-level probability ratios"
+    if loss_fn.force_on_policy_ratio and (
+        loss_fn.sequence_level_importance_ratios or loss_fn.truncated_importance_sampling_type == "seq-mask-tis"
+    ):
+        return "sequence-level importance weights of the current policy"
+    if loss_fn.positive_example_nll_weight > 0 and "rewards" in data:
+        return "positive-example NLL term"
+    if not isinstance(logits, torch.Tensor) or not logits.is_cuda or logits.dim() != 3:
+        return "logits are not a [B, S, V] GPU tensor"
+    elt = logits.element_size()
+    if logits.dtype not in (torch.float32, torch.bfloat16, torch.float16) or logits.stride(2) != 1:
+        return "unsupported logits dtype or layout"
+    vocab = logits.shape[2]
+    if (vocab * elt) % 16 or vocab * elt > 20480 * 16:
+        return "vocabulary row does not fit the on-chip path"
+    if logits.data_ptr() % 16 or (logits.stride(0) * elt) % 16 or (logits.stride(1) * elt) % 16:
+        return "rows are not 16-byte aligned"
+    if logits.shape[1] < data["input_ids"].shape[1]:
+        return "logits shorter than input_ids"
+    return None
+
+
+class _FusedLogitsLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams,
+                loss_scale, in_place):
+        x = logits.detach()
+        if in_place:
+            loss, lp, metrics = _OPS.fused_logits_grpo_loss_(
+                x, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams, loss_scale)
+            dlogits = x  # the caller declared the logits dead; their storage now holds the gradient
+        else:
+            loss, dlogits, lp, metrics = _OPS.fused_logits_grpo_loss(
+                x, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams, loss_scale)
+        ctx.save_for_backward(dlogits)
+        ctx.loss_scale = loss_scale
+        ctx.mark_non_differentiable(lp, metrics)
+        return loss, lp, metrics
+
+    @staticmethod
+    def backward(ctx, grad_loss, _g_lp, _g_metrics):
+        (dlogits,) = ctx.saved_tensors
+        factor = float(grad_loss) / ctx.loss_scale
+        if factor != 1.0:
+            dlogits = (dlogits.float() * factor).to(dlogits.dtype)
+        return (dlogits,) + (None,) * 13
+
+
+def fused_logits_clipped_pg_loss(
+    logits: torch.Tensor,
+    data: Any,
+    loss_fn: ClippedPGLossFn,
+    global_valid_seqs,
+    global_valid_toks,
+    *,
+    loss_scale: float = 1.0,
+    in_place: bool = False,
+):
+    """``(loss, metrics)`` exactly as ``loss_fn(prepare_loss_input(logits, data, loss_fn))`` would return them.
+
+    ``loss_scale`` is the gradient the caller will send into ``loss.backward()`` (1 for a plain
+    ``backward()``, ``dp_size * cp_size`` when the worker scales the loss first); with it the stored
+    gradient is final and ``backward`` moves no data.  ``in_place=True`` writes the gradient over the
+    logits buffer instead of allocating a second ``[B, S, V]`` tensor (the logits are dead after the
+    loss in the training step).  The metrics do not include values for masked positions, which are
+    never evaluated."""
+    reason = why_not_fusable(loss_fn, logits, data)
+    if reason is not None:
+        raise NotImplementedError(f"fused logits->loss path: {reason}")
+    dev = logits.device
+    ids = data["input_ids"].to(dev)
+    if ids.dtype != torch.int64:
+        ids = ids.long()
+    n_inner = ids.shape[1] - 1
+    beta = loss_fn.reference_policy_kl_penalty
+    sample_mask_in = data["sample_mask"]
+    prev = None if loss_fn.force_on_policy_ratio else _f32(data["prev_logprobs"][:, 1:], dev)
+    ref = _f32(data["reference_policy_logprobs"][:, 1:], dev) if beta != 0 else None
+    iflags, fparams = loss_fn._kernel_config(False)
+    loss, _lp, metrics = _FusedLogitsLoss.apply(
+        logits, ids[:, 1:], n_inner, prev, _f32(data["generation_logprobs"][:, 1:], dev), ref,
+        _f32(data["advantages"][:, 1:], dev), _f32(data["token_mask"][:, 1:], dev), _f32(sample_mask_in, dev),
+        _global_valid(global_valid_seqs, global_valid_toks, dev), iflags, fparams, float(loss_scale), bool(in_place),
+    )
+    m = metrics.cpu().tolist()
+    get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
+    n_valid = get("num_valid_samples")
+    out = {
+        "loss": get("loss"),
+        "probs_ratio": get("probs_ratio"),
+        "probs_ratio_clamped": get("probs_ratio_clamped"),
+        "probs_ratio_min": get("probs_ratio_min"),
+        "probs_ratio_max": get("probs_ratio_max"),
+        "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
+        "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
+        "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
+        "token_mult_prob_error": get("token_mult_prob_error"),
+        "gen_kl_error": get("gen_kl_error"),
+        "policy_kl_error": get("policy_kl_error"),
+        "js_divergence_error": get("js_divergence_error"),
+        "sampling_importance_ratio": get("sampling_importance_ratio"),
+        "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
+        "approx_entropy": get("approx_entropy"),
+    }
+    if loss_fn.truncated_importance_sampling_ratio is not None:
+        out["is_oob_ratio"] = get("is_oob_ratio")
+    out["positive_nll_loss"] = get("positive_nll_loss")
+    return loss, out

@@ -105,7 +105,18 @@ def wrap_loss_fn_with_input_preparation(next_token_logits, data, global_valid_se
                                         vocab_parallel_rank: Optional[int] = None,
                                         vocab_parallel_group: Optional[Any] = None,
                                         context_parallel_group: Optional[Any] = None):
-    """``wrapper.py:292-322``: prepare, then call the loss."""
+    """``wrapper.py:292-322``: prepare, then call the loss.  When the loss is a ``ClippedPGLossFn`` whose
+    per-token gradient does not need other tokens' logprobs and the logits are a plain GPU tensor, both
+    steps (and the later backward through the logprob op) run as one fused pass over the logits."""
+    from .fused import fused_logits_clipped_pg_loss, why_not_fusable
+    from .utils import prepare_loss_input
+
+    if (prepare_fn is prepare_loss_input and torch.is_grad_enabled() and isinstance(next_token_logits, torch.Tensor)
+            and next_token_logits.requires_grad and why_not_fusable(loss_fn, next_token_logits, data) is None):
+        from ...distributed.model_utils import _group_size
+
+        if _group_size(vocab_parallel_group) == 1 and _group_size(context_parallel_group) == 1:
+            return fused_logits_clipped_pg_loss(next_token_logits, data, loss_fn, global_valid_seqs, global_valid_toks)
     loss_input, data = prepare_fn(
         logits=next_token_logits, data=data, loss_fn=loss_fn, vocab_parallel_rank=vocab_parallel_rank,
         vocab_parallel_group=vocab_parallel_group, context_parallel_group=context_parallel_group,

@@ -16,52 +16,40 @@
 #include <math.h>
 
 #include "common.hpp"
+#include "grpo_token.hpp"
 
 namespace nrl {
 
 constexpr int kLossBlock = 256;
 constexpr int kLossWaves = kLossBlock / kWave;
 
-// per-row partial slots
-enum {
-    P_ACTOR = 0, P_KL, P_MULT_ERR, P_GEN_KL, P_POLICY_KL, P_JS, P_SAMPLING, P_ENTROPY, P_RATIO, P_RATIO_CL,
-    P_OOB, P_NLL, P_N_CORRECT, P_SAMPLE_MASK, P_N_SELECTED, P_SEQ_W, P_R_MIN, P_R_MAX, P_RC_MIN, P_RC_MAX,
-    P_COUNT
-};
-
-struct GrpoArgs {
-    nrl_grpo_cfg cfg;
-    nrl_grpo_inputs in;
-    float* dlp;
-    float* dlpu;
-    double* parts;  // [B, P_COUNT]
-};
-
-__device__ __forceinline__ float finite_or_zero(float x) { return (x - x == 0.f) ? x : 0.f; }
-
-__device__ __forceinline__ float kl_value(int type, float logr) {
-    if (type == 1) return -logr;
-    if (type == 2) return (logr * logr) / 2.f;
-    return (expf(logr) - 1.f) - logr;
-}
-
-// d kl / d logr
-__device__ __forceinline__ float kl_slope(int type, float logr) {
-    if (type == 1) return -1.f;
-    if (type == 2) return logr;
-    return expf(logr) - 1.f;
-}
-
-__device__ __forceinline__ float clampf(float x, float lo, float hi) {
-    // torch.clamp: min(max(x, lo), hi) with NaN propagating
-    if (x != x) return x;
-    return fminf(fmaxf(x, lo), hi);
-}
-
-// gradient share of the larger (or, for SMALLER, the smaller) of two values: 1, 1/2 on a tie, 0
-__device__ __forceinline__ float pick_weight(float self, float other, bool want_max) {
-    if (self == other) return 0.5f;
-    return (want_max ? self > other : self < other) ? 1.f : 0.f;
+// Workgroup-wide reduction of one sequence's accumulators into its row of partials.
+__device__ __forceinline__ void store_row_parts(const nrl_grpo_cfg& c, double* out, double (&acc)[P_R_MIN], float r_min,
+                                                float r_max, float rc_min, float rc_max, const SeqStats& st, float smv,
+                                                double* sm_d, float* sm_f) {
+    const int tid = threadIdx.x;
+    const float tis_floor = c.tis_min;
+#pragma unroll
+    for (int k = 0; k < P_R_MIN; ++k) {
+        const double tot = block_sum<double, kLossWaves>(acc[k], sm_d);
+        if (tid == 0) out[k] = tot;
+    }
+    const float mn = block_min<kLossWaves>(r_min, sm_f), mx = block_max<kLossWaves>(r_max, sm_f);
+    const float cmn = block_min<kLossWaves>(rc_min, sm_f), cmx = block_max<kLossWaves>(rc_max, sm_f);
+    if (tid == 0) {
+        const float seq_w = st.seq_w, seq_keep = st.seq_keep;
+        if (!c.token_level_loss) {  // sequence-level: masked mean over tokens, then weight by sample_mask
+            out[P_ACTOR] = static_cast<double>(static_cast<float>(out[P_ACTOR]) / st.seq_den) * smv;
+            out[P_KL] = static_cast<double>(static_cast<float>(out[P_KL]) / st.seq_den) * smv;
+        }
+        out[P_SAMPLE_MASK] = smv;
+        out[P_SEQ_W] = c.tis_type == NRL_TIS_SEQ_MASK ? seq_w * seq_keep : seq_w;
+        if (c.sequence_level_importance_ratios && c.tis_type == NRL_TIS_TIS) out[P_SEQ_W] = clampf(seq_w, tis_floor, c.tis_max);
+        if (c.sequence_level_importance_ratios && c.tis_type == NRL_TIS_ICEPOP)
+            out[P_SEQ_W] = (seq_w >= c.tis_min && seq_w <= c.tis_max) ? seq_w : 0.f;
+        if (c.tis_type == NRL_TIS_SEQ_MASK) out[P_OOB] = (1.f - seq_keep) * smv;
+        out[P_R_MIN] = mn; out[P_R_MAX] = mx; out[P_RC_MIN] = cmn; out[P_RC_MAX] = cmx;
+    }
 }
 
 template <bool GSPO>
@@ -106,130 +94,27 @@ __global__ __launch_bounds__(kLossBlock) void grpo_rows_kernel(GrpoArgs a) {
         const float geo = expf(static_cast<float>(block_sum<double, kLossWaves>(s_geo, sm_d)) / seq_den);
         seq_keep = (geo >= c.tis_min && geo <= c.tis_max) ? 1.f : 0.f;
     }
-    const float tis_floor = c.tis_min;  // host passes 0 when the lower bound is unset
-
-    const float clip_lo = 1.0f - c.ratio_clip_min, clip_hi = 1.0f + c.ratio_clip_max;
-
     double acc[P_R_MIN];
 #pragma unroll
     for (int k = 0; k < P_R_MIN; ++k) acc[k] = 0;
     float r_min = INFINITY, r_max = -INFINITY, rc_min = INFINITY, rc_max = -INFINITY;
     double gspo_k = 0;  // sum_t coef * w * d clip / d ratio  (GSPO only)
 
+    SeqStats st;
+    st.seq_den = seq_den; st.seq_ratio = seq_ratio; st.seq_w = seq_w; st.seq_keep = seq_keep;
     for (int64_t t = tid; t < n; t += kLossBlock) {
-        const float lp = lp_row[t], lpu = lpu_row[t], prev = prev_row[t], gen = gen_row[t];
-        const float adv = adv_row[t], tm = tm_row[t];
-        const float mask = tm * smv;
-        // gradient coefficient of a per-token value in the reduced loss
-        const float coef = c.token_level_loss ? mask / den_t : (tm / seq_den) * (smv / den_s);
-
-        // ---- diagnostics on (gen, prev) ----
-        acc[P_MULT_ERR] += expf(fabsf(gen - prev) * mask) * mask;
-        acc[P_GEN_KL] += kl_value(c.kl_type, prev - gen) * mask;
-        acc[P_POLICY_KL] += kl_value(c.kl_type, gen - prev) * mask;
-        {
-            const float log_mix = logf(0.5f * expf(prev) + 0.5f * expf(gen));
-            const float dp = prev - log_mix, dg = gen - log_mix;
-            const float kp = (expf(dp) - dp) - 1.f, kg = (expf(dg) - dg) - 1.f;
-            acc[P_JS] += (0.5f * kp + 0.5f * kg) * mask;
+        TokenIn ti;
+        ti.lp = lp_row[t]; ti.lpu = lpu_row[t]; ti.prev = prev_row[t]; ti.gen = gen_row[t];
+        ti.ref = c.has_kl ? ref_row[t] : 0.f; ti.adv = adv_row[t]; ti.tm = tm_row[t]; ti.smv = smv; ti.correct = correct;
+        ti.den_t = den_t; ti.den_s = den_s;
+        const TokenOut o = token_eval<GSPO>(c, st, ti);
+#pragma unroll
+        for (int k = 0; k < P_SAMPLE_MASK; ++k) acc[k] += o.term[k];
+        if (o.selected) {
+            r_min = fminf(r_min, o.ratio); r_max = fmaxf(r_max, o.ratio);
+            rc_min = fminf(rc_min, o.ratio_cl); rc_max = fmaxf(rc_max, o.ratio_cl);
         }
-
-        // ---- KL to the reference policy ----
-        float d_lpu = 0.f;
-        if (c.has_kl) {
-            const float ref = ref_row[t];
-            const float w_raw = c.use_on_policy_kl_approximation ? expf(lpu - gen) : expf(lpu - lpu);
-            const float w = finite_or_zero(w_raw);
-            float w_slope = w;  // d w / d lpu (zero where nan_to_num replaced the value)
-            float logr = ref - lpu;
-            float in_range = 1.f;
-            if (c.has_kl_input_clamp) {
-                const float cl = clampf(logr, -c.kl_input_clamp, c.kl_input_clamp);
-                if (!(logr == cl)) { w_slope = 0.f; in_range = 0.f; }
-                logr = cl;
-            }
-            const float k = kl_value(c.kl_type, logr);
-            float v = w * k;
-            // d v / d lpu: weight term + kl term (d logr / d lpu = -1)
-            float dv = w_slope * k + w * (-kl_slope(c.kl_type, logr)) * in_range;
-            if (c.has_kl_output_clamp) {
-                const float vc = clampf(v, -c.kl_output_clamp, c.kl_output_clamp);
-                if (!(v >= -c.kl_output_clamp && v <= c.kl_output_clamp)) dv = 0.f;
-                v = vc;
-            }
-            const float klt = c.kl_beta * v;
-            acc[P_KL] += c.token_level_loss ? klt * mask : (klt * tm);
-            d_lpu = coef * (c.kl_beta * dv);
-        }
-
-        // ---- probability ratio and clipped surrogate ----
-        float ratio, ratio_cl, d_clip;  // d_clip = d clip_loss / d lp (non-GSPO) or / d ratio (GSPO)
-        float clip;
-        if (c.force_on_policy_ratio) {
-            ratio = expf(lp - lp);
-            ratio_cl = ratio;
-            clip = nan_max(-adv * ratio, -adv * ratio_cl);
-            d_clip = -adv * ratio;
-        } else if (!c.disable_ppo_ratio) {
-            ratio = GSPO ? seq_ratio : expf(lp - prev);
-            ratio_cl = clampf(ratio, clip_lo, clip_hi);
-            if (c.use_cispo) {
-                clip = -adv * ratio_cl * lp;
-                d_clip = -adv * ratio_cl;
-            } else {
-                const float l1 = -adv * ratio, l2 = -adv * ratio_cl;
-                clip = nan_max(l1, l2);
-                const float inside = (ratio >= clip_lo && ratio <= clip_hi) ? 1.f : 0.f;
-                const float share = pick_weight(l1, l2, true) + pick_weight(l2, l1, true) * inside;
-                d_clip = -adv * share * (GSPO ? 1.f : ratio);
-            }
-        } else {
-            ratio = lp;
-            ratio_cl = lp;
-            clip = nan_max(-adv * ratio, -adv * ratio_cl);
-            d_clip = -adv;
-        }
-        if (c.has_dual_clip) {
-            const float l3 = -adv * c.ratio_clip_c;
-            if (adv < 0.f) {
-                d_clip *= pick_weight(clip, l3, false);
-                clip = nan_min(clip, l3);
-            }
-        }
-
-        // ---- off-policy importance weight ----
-        float w_is = c.sequence_level_importance_ratios ? seq_w : finite_or_zero(expf(prev - gen));
-        if (c.tis_type == NRL_TIS_TIS) {
-            acc[P_OOB] += ((w_is > c.tis_max || w_is < tis_floor) ? 1.f : 0.f) * mask;
-            w_is = clampf(w_is, tis_floor, c.tis_max);
-        } else if (c.tis_type == NRL_TIS_ICEPOP) {
-            const bool kept = w_is >= c.tis_min && w_is <= c.tis_max;
-            acc[P_OOB] += (kept ? 0.f : 1.f) * mask;
-            w_is = kept ? w_is : 0.f;
-        } else if (c.tis_type == NRL_TIS_SEQ_MASK) {
-            w_is = w_is * seq_keep;
-        }
-        const float w_use = c.use_importance_sampling_correction ? w_is : 1.f;
-
-        const float actor_t = w_use * clip;
-        acc[P_ACTOR] += c.token_level_loss ? actor_t * mask : actor_t * tm;
-        if (!c.sequence_level_importance_ratios) acc[P_SAMPLING] += w_is * mask;
-        acc[P_ENTROPY] += (expf(lp - gen) * lp) * mask;
-        acc[P_RATIO] += ratio * mask;
-        acc[P_RATIO_CL] += ratio_cl * mask;
-        if (c.has_nll) {
-            const float cm = mask * correct;
-            acc[P_NLL] += (-lp) * cm;
-            acc[P_N_CORRECT] += cm;
-        }
-        if (mask != 0.f) {
-            acc[P_N_SELECTED] += 1.0;
-            r_min = fminf(r_min, ratio); r_max = fmaxf(r_max, ratio);
-            rc_min = fminf(rc_min, ratio_cl); rc_max = fmaxf(rc_max, ratio_cl);
-        }
-
-        // ---- gradient ----
-        const float d_actor = coef * w_use * d_clip;
+        const float d_actor = o.d_actor, d_lpu = o.d_lpu;
         if (GSPO) {
             gspo_k += d_actor;
             if (a.dlpu) a.dlpu[b * n + t] = d_lpu;
@@ -252,28 +137,7 @@ __global__ __launch_bounds__(kLossBlock) void grpo_rows_kernel(GrpoArgs a) {
         }
     }
 
-    // ---- row partials ----
-    double* out = a.parts + b * P_COUNT;
-#pragma unroll
-    for (int k = 0; k < P_R_MIN; ++k) {
-        const double tot = block_sum<double, kLossWaves>(acc[k], sm_d);
-        if (tid == 0) out[k] = tot;
-    }
-    const float mn = block_min<kLossWaves>(r_min, sm_f), mx = block_max<kLossWaves>(r_max, sm_f);
-    const float cmn = block_min<kLossWaves>(rc_min, sm_f), cmx = block_max<kLossWaves>(rc_max, sm_f);
-    if (tid == 0) {
-        if (!c.token_level_loss) {  // sequence-level: masked mean over tokens, then weight by sample_mask
-            out[P_ACTOR] = static_cast<double>(static_cast<float>(out[P_ACTOR]) / seq_den) * smv;
-            out[P_KL] = static_cast<double>(static_cast<float>(out[P_KL]) / seq_den) * smv;
-        }
-        out[P_SAMPLE_MASK] = smv;
-        out[P_SEQ_W] = c.tis_type == NRL_TIS_SEQ_MASK ? seq_w * seq_keep : seq_w;
-        if (c.sequence_level_importance_ratios && c.tis_type == NRL_TIS_TIS) out[P_SEQ_W] = clampf(seq_w, tis_floor, c.tis_max);
-        if (c.sequence_level_importance_ratios && c.tis_type == NRL_TIS_ICEPOP)
-            out[P_SEQ_W] = (seq_w >= c.tis_min && seq_w <= c.tis_max) ? seq_w : 0.f;
-        if (c.tis_type == NRL_TIS_SEQ_MASK) out[P_OOB] = (1.f - seq_keep) * smv;
-        out[P_R_MIN] = mn; out[P_R_MAX] = mx; out[P_RC_MIN] = cmn; out[P_RC_MAX] = cmx;
-    }
+    store_row_parts(c, a.parts + b * P_COUNT, acc, r_min, r_max, rc_min, rc_max, st, smv, sm_d, sm_f);
 }
 
 // Fixed-order reduction of the row partials and normalisation into the metrics record.
@@ -383,6 +247,214 @@ __global__ __launch_bounds__(kLossBlock) void nll_finish_kernel(nrl_grpo_inputs 
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fused pass: logits row -> log-sum-exp -> token logprob -> loss terms and d loss / d logprob ->
+// dlogits, with the row held on chip (registers plus an LDS slice) between the reduction and the
+// gradient, so the logits are read once and the gradient written once (2 * V * sizeof(logit) per
+// token instead of 3).  Valid when d loss / d logprob of a token depends only on that token and on
+// per-sequence quantities that do not involve the current logprobs: everything except sequence-level
+// probability ratios (GSPO) and the positive-example NLL term.  Tokens whose mask is zero are not
+// evaluated: their gradient row is zero-filled without reading the logits and their logprob is
+// reported as 0.
+// ---------------------------------------------------------------------------------------------
+constexpr int kFusedBlock = 1024;
+constexpr int kFusedWaves = kFusedBlock / kWave;
+constexpr int kFusedRegVec = 16;  // 16-byte vectors per lane held in registers ...
+constexpr int kFusedLdsVec = 4;   // ... and in LDS (64 KiB per workgroup)
+constexpr int kFusedVec = kFusedRegVec + kFusedLdsVec;
+constexpr int T_RATIO = P_SAMPLE_MASK, T_RATIO_CL = P_SAMPLE_MASK + 1, T_SELECTED = P_SAMPLE_MASK + 2, T_COUNT = 20;
+static_assert(P_SAMPLE_MASK + 3 <= T_COUNT, "token term record too small");
+
+struct FusedArgs {
+    nrl_grpo_cfg cfg;
+    nrl_grpo_inputs in;  // lp / lpu unused
+    const void* logits;
+    int64_t n_inner, d_n_inner, vocab, stride_outer, stride_inner;
+    const int64_t* targets;
+    int64_t ts_outer, ts_inner, vstart, vend;
+    float tparam, loss_scale;
+    void* dlogits;
+    int64_t ds_outer, ds_inner;
+    float* lp_out;     // [B, n_inner]
+    float* seq_stats;  // [B, 3]: seq_den, seq_w, seq_keep
+    float* terms;      // [B * n_inner, T_COUNT]
+    double* parts;     // [B, P_COUNT]
+};
+
+__global__ __launch_bounds__(kLossBlock) void grpo_seq_stats_kernel(FusedArgs a) {
+    __shared__ double sm_d[kLossWaves];
+    const nrl_grpo_cfg& c = a.cfg;
+    const nrl_grpo_inputs& in = a.in;
+    const int64_t b = blockIdx.x, n = in.sm1;
+    const float smv = in.sample_mask[b];
+    double s_tm = 0, s_is = 0, s_geo = 0;
+    const bool need_prev = c.sequence_level_importance_ratios || c.tis_type == NRL_TIS_SEQ_MASK;
+    for (int64_t t = threadIdx.x; t < n; t += kLossBlock) {
+        const float tm = in.token_mask[b * in.token_mask_stride + t];
+        s_tm += tm;
+        if (need_prev) {
+            const float d = in.prev[b * in.prev_stride + t] - in.gen[b * in.gen_stride + t];
+            s_is += d * (tm * smv);
+            s_geo += finite_or_zero(d) * tm;
+        }
+    }
+    const float seq_den = static_cast<float>(block_sum<double, kLossWaves>(s_tm, sm_d)) + 1e-8f;
+    float seq_w = 1.f, seq_keep = 1.f;
+    if (c.sequence_level_importance_ratios) seq_w = finite_or_zero(expf(static_cast<float>(block_sum<double, kLossWaves>(s_is, sm_d))));
+    if (c.tis_type == NRL_TIS_SEQ_MASK) {
+        const float geo = expf(static_cast<float>(block_sum<double, kLossWaves>(s_geo, sm_d)) / seq_den);
+        seq_keep = (geo >= c.tis_min && geo <= c.tis_max) ? 1.f : 0.f;
+    }
+    if (threadIdx.x == 0) {
+        a.seq_stats[b * 3] = seq_den;
+        a.seq_stats[b * 3 + 1] = seq_w;
+        a.seq_stats[b * 3 + 2] = seq_keep;
+    }
+}
+
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArgs a) {
+    constexpr int EPV = Row<DT>::EPV;
+    __shared__ u32x4 stash[kFusedLdsVec * kFusedBlock];
+    __shared__ float sm_f[kFusedWaves];
+    __shared__ float sh_g, sh_lse;
+    const nrl_grpo_cfg& c = a.cfg;
+    const nrl_grpo_inputs& in = a.in;
+    const int tid = threadIdx.x;
+    const int64_t r = blockIdx.x;
+    const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+    u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(a.dlogits) + (o * a.ds_outer + i * a.ds_inner) * Row<DT>::BYTES);
+    const int64_t nvec = a.vocab / EPV;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    float tm = 0.f, smv = 0.f;
+    if (i < a.n_inner) {
+        tm = in.token_mask[o * in.token_mask_stride + i];
+        smv = in.sample_mask[o];
+    }
+    const int64_t tok = o * a.n_inner + i;
+    if (tm * smv == 0.f) {  // dropped position or masked token
+        for (int64_t v = tid; v < nvec; v += kFusedBlock) __builtin_nontemporal_store(zero, ov + v);
+        if (i < a.n_inner && tid < T_COUNT) a.terms[tok * T_COUNT + tid] = 0.f;
+        if (i < a.n_inner && tid == 0) a.lp_out[tok] = 0.f;
+        return;
+    }
+    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(row);
+    u32x4 regs[kFusedRegVec];
+#pragma unroll
+    for (int j = 0; j < kFusedRegVec; ++j) {
+        const int64_t v = tid + static_cast<int64_t>(j) * kFusedBlock;
+        regs[j] = v < nvec ? __builtin_nontemporal_load(xv + v) : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < kFusedLdsVec; ++j) {
+        const int64_t v = tid + static_cast<int64_t>(kFusedRegVec + j) * kFusedBlock;
+        if (v < nvec) stash[j * kFusedBlock + tid] = __builtin_nontemporal_load(xv + v);
+    }
+    // every lane only ever touches its own stash slots, so no barrier is needed around them
+    auto fetch = [&](int j) -> u32x4 { return j < kFusedRegVec ? regs[j] : stash[(j - kFusedRegVec) * kFusedBlock + tid]; };
+
+    // row maximum, then the sum of exponentials (the data are on chip: no online rescaling needed)
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < kFusedVec; ++j) {
+        if (tid + static_cast<int64_t>(j) * kFusedBlock < nvec) {
+            float t[EPV];
+            Row<DT>::decode(fetch(j), t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) mx = fmaxf(mx, scale_logit<DT, TEMP>(t[k], a.tparam));
+        }
+    }
+    const float m = block_max<kFusedWaves>(mx, sm_f);
+    float part = 0.f;
+#pragma unroll
+    for (int j = 0; j < kFusedVec; ++j) {
+        if (tid + static_cast<int64_t>(j) * kFusedBlock < nvec) {
+            float t[EPV];
+            Row<DT>::decode(fetch(j), t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) part += fast_exp2((scale_logit<DT, TEMP>(t[k], a.tparam) - m) * kLog2e);
+        }
+    }
+    const float ssum = block_sum<float, kFusedWaves>(part, sm_f);
+    const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
+    const int64_t tloc = (tg >= a.vstart && tg < a.vend) ? tg - a.vstart : -1;
+    if (tid == 0) {
+        const float log_s = logf(ssum);
+        float lp = 0.f;
+        if (tloc >= 0) lp = (scale_logit<DT, TEMP>(Row<DT>::load1(row, tloc), a.tparam) - m) - log_s;
+        SeqStats st;
+        st.seq_den = a.seq_stats[o * 3]; st.seq_ratio = 1.f; st.seq_w = a.seq_stats[o * 3 + 1]; st.seq_keep = a.seq_stats[o * 3 + 2];
+        TokenIn ti;
+        ti.lp = lp; ti.lpu = lp;
+        ti.prev = c.force_on_policy_ratio ? lp : in.prev[o * in.prev_stride + i];
+        ti.gen = in.gen[o * in.gen_stride + i];
+        ti.ref = c.has_kl ? in.ref[o * in.ref_stride + i] : 0.f;
+        ti.adv = in.adv[o * in.adv_stride + i];
+        ti.tm = tm; ti.smv = smv; ti.correct = 0.f;
+        ti.den_s = in.global_valid[0] + 1e-8f;
+        ti.den_t = in.global_valid[1] + 1e-8f;
+        const TokenOut out = token_eval<false>(c, st, ti);
+        float* rec = a.terms + tok * T_COUNT;
+#pragma unroll
+        for (int k = 0; k < P_SAMPLE_MASK; ++k) rec[k] = out.term[k];
+        rec[T_RATIO] = out.ratio;
+        rec[T_RATIO_CL] = out.ratio_cl;
+        rec[T_SELECTED] = out.selected ? 1.f : 0.f;
+        a.lp_out[tok] = lp;
+        sh_g = (out.d_actor + out.d_lpu) * a.loss_scale;
+        sh_lse = m + log_s;
+    }
+    __syncthreads();
+    const float g = sh_g, lse = sh_lse;
+    if (g == 0.f) {
+        for (int64_t v = tid; v < nvec; v += kFusedBlock) __builtin_nontemporal_store(zero, ov + v);
+        return;
+    }
+    const int64_t tvec = tloc >= 0 ? tloc / EPV : -1;
+    const int tsub = tloc >= 0 ? static_cast<int>(tloc % EPV) : -1;
+#pragma unroll
+    for (int j = 0; j < kFusedVec; ++j) {
+        const int64_t v = tid + static_cast<int64_t>(j) * kFusedBlock;
+        if (v < nvec) {
+            float t[EPV];
+            Row<DT>::decode(fetch(j), t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) {
+                const float p = fast_exp2((scale_logit<DT, TEMP>(t[k], a.tparam) - lse) * kLog2e);
+                float d = (((v == tvec && k == tsub) ? 1.f : 0.f) - p) * g;
+                if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
+                if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
+                t[k] = d;
+            }
+            __builtin_nontemporal_store(Row<DT>::encode(t), ov + v);
+        }
+    }
+}
+
+// one workgroup per sequence: token term records -> the sequence's row of partials
+__global__ __launch_bounds__(kLossBlock) void grpo_terms_reduce_kernel(FusedArgs a) {
+    __shared__ double sm_d[kLossWaves];
+    __shared__ float sm_f[kLossWaves];
+    const int64_t b = blockIdx.x, n = a.n_inner;
+    double acc[P_R_MIN];
+#pragma unroll
+    for (int k = 0; k < P_R_MIN; ++k) acc[k] = 0;
+    float r_min = INFINITY, r_max = -INFINITY, rc_min = INFINITY, rc_max = -INFINITY;
+    for (int64_t t = threadIdx.x; t < n; t += kLossBlock) {
+        const float* rec = a.terms + (b * n + t) * T_COUNT;
+#pragma unroll
+        for (int k = 0; k < P_SAMPLE_MASK; ++k) acc[k] += rec[k];
+        if (rec[T_SELECTED] != 0.f) {
+            r_min = fminf(r_min, rec[T_RATIO]); r_max = fmaxf(r_max, rec[T_RATIO]);
+            rc_min = fminf(rc_min, rec[T_RATIO_CL]); rc_max = fmaxf(rc_max, rec[T_RATIO_CL]);
+        }
+    }
+    SeqStats st;
+    st.seq_den = a.seq_stats[b * 3]; st.seq_ratio = 1.f; st.seq_w = a.seq_stats[b * 3 + 1]; st.seq_keep = a.seq_stats[b * 3 + 2];
+    store_row_parts(a.cfg, a.parts + b * P_COUNT, acc, r_min, r_max, rc_min, rc_max, st, a.in.sample_mask[b], sm_d, sm_f);
+}
+
 static int check_inputs(const nrl_grpo_inputs* in, bool need_prev, bool need_ref, bool need_adv) {
     if (!in) return fail(NRL_E_INVALID, "inputs is NULL");
     if (in->batch < 0 || in->sm1 < 0) return fail(NRL_E_INVALID, "bad shape [%lld, %lld]", (long long)in->batch, (long long)in->sm1);
@@ -451,4 +523,97 @@ extern "C" int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, 
     if (in->batch > 0) nll_rows_kernel<<<dim3((unsigned)in->batch), dim3(kLossBlock), 0, s>>>(*in, dlp_out, parts);
     nll_finish_kernel<<<dim3(1), dim3(kLossBlock), 0, s>>>(*in, parts, loss_out, metrics_out);
     return check_launch("nll_loss_fwd_bwd");
+}
+
+static int64_t align8(int64_t v) { return (v + 7) / 8 * 8; }
+
+extern "C" int64_t nrl_fused_workspace_bytes(int64_t batch, int64_t n_inner) {
+    const int64_t b = batch < 1 ? 1 : batch, n = n_inner < 1 ? 1 : n_inner;
+    return align8(b * 3 * 4) + align8(b * n * T_COUNT * 4) + b * P_COUNT * 8;
+}
+
+extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
+                                          float loss_scale, void* dlogits, int64_t d_n_inner, int64_t d_stride_outer,
+                                          int64_t d_stride_inner, float* logprob_out, float* loss_out, float* metrics_out,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!rows || !cfg || !in) return fail(NRL_E_INVALID, "null argument");
+    if (rows->dtype != NRL_F32 && rows->dtype != NRL_BF16 && rows->dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype");
+    if (rows->n_outer < 0 || rows->n_inner < 0 || rows->vocab <= 0 || d_n_inner < rows->n_inner) return fail(NRL_E_INVALID, "bad shape");
+    if (in->batch != rows->n_outer || in->sm1 != rows->n_inner) return fail(NRL_E_INVALID, "loss inputs and logits rows disagree");
+    if (rows->vocab_end - rows->vocab_start != rows->vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
+    if (!(rows->temperature > 0.f)) return fail(NRL_E_INVALID, "temperature must be positive");
+    const bool gspo = cfg->sequence_level_importance_ratios && !cfg->disable_ppo_ratio && !cfg->force_on_policy_ratio;
+    if (gspo) return fail(NRL_E_UNSUPPORTED, "sequence-level probability ratios need every logprob of a sequence first");
+    if (cfg->has_nll) return fail(NRL_E_UNSUPPORTED, "the positive-example NLL term is not fused");
+    // sequence-level importance weights are sums over prev - gen; with force_on_policy_ratio prev is the
+    // current logprob itself, which does not exist before the pass
+    const bool seq_weights = cfg->sequence_level_importance_ratios || cfg->tis_type == NRL_TIS_SEQ_MASK;
+    if (seq_weights && cfg->force_on_policy_ratio)
+        return fail(NRL_E_UNSUPPORTED, "sequence-level importance weights with force_on_policy_ratio depend on the current logprobs");
+    if (seq_weights && rows->n_outer * rows->n_inner > 0 && !in->prev) return fail(NRL_E_INVALID, "prev_logprobs is NULL");
+    if (cfg->kl_type < 1 || cfg->kl_type > 3 || cfg->tis_type < 0 || cfg->tis_type > 3) return fail(NRL_E_INVALID, "bad kl_type or tis_type");
+    const int bytes = rows->dtype == NRL_F32 ? 4 : 2, epv = 16 / bytes;
+    if (rows->vocab % epv || rows->vocab / epv > static_cast<int64_t>(kFusedVec) * kFusedBlock)
+        return fail(NRL_E_UNSUPPORTED, "row does not fit the on-chip path (vocab %lld)", (long long)rows->vocab);
+    if ((reinterpret_cast<uintptr_t>(rows->logits) & 15) || (reinterpret_cast<uintptr_t>(dlogits) & 15) ||
+        (rows->stride_outer * bytes) % 16 || (rows->stride_inner * bytes) % 16 || (d_stride_outer * bytes) % 16 ||
+        (d_stride_inner * bytes) % 16)
+        return fail(NRL_E_UNSUPPORTED, "rows must be 16-byte aligned");
+    const int64_t n_rows = rows->n_outer * d_n_inner;
+    if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    if (!loss_out || !metrics_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
+    if (workspace_bytes < nrl_fused_workspace_bytes(rows->n_outer, rows->n_inner)) return fail(NRL_E_WORKSPACE, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7) return fail(NRL_E_INVALID, "workspace must be 8-byte aligned");
+    if (n_rows > 0) {
+        if (!rows->logits || !rows->targets || !dlogits || !logprob_out) return fail(NRL_E_INVALID, "null logits, targets or output");
+        if (!in->gen || !in->adv || !in->token_mask || !in->sample_mask || !in->global_valid) return fail(NRL_E_INVALID, "null loss input");
+        if (!cfg->force_on_policy_ratio && !in->prev) return fail(NRL_E_INVALID, "prev_logprobs is NULL");
+        if (cfg->has_kl && !in->ref) return fail(NRL_E_INVALID, "reference_policy_logprobs is NULL");
+    }
+    FusedArgs a;
+    a.cfg = *cfg;
+    a.in = *in;
+    a.in.lp = nullptr; a.in.lpu = nullptr;
+    a.logits = rows->logits; a.n_inner = rows->n_inner; a.d_n_inner = d_n_inner; a.vocab = rows->vocab;
+    a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
+    a.targets = rows->targets; a.ts_outer = rows->tgt_stride_outer; a.ts_inner = rows->tgt_stride_inner;
+    a.vstart = rows->vocab_start; a.vend = rows->vocab_end;
+    a.loss_scale = loss_scale;
+    a.dlogits = dlogits; a.ds_outer = d_stride_outer; a.ds_inner = d_stride_inner;
+    a.lp_out = logprob_out;
+    char* ws = static_cast<char*>(workspace);
+    a.seq_stats = reinterpret_cast<float*>(ws); ws += align8(rows->n_outer * 3 * 4);
+    a.terms = reinterpret_cast<float*>(ws); ws += align8(rows->n_outer * (rows->n_inner < 1 ? 1 : rows->n_inner) * T_COUNT * 4);
+    a.parts = reinterpret_cast<double*>(ws);
+    int tc = 0;
+    a.tparam = 1.f;
+    if (rows->temperature != 1.0f) {
+        if (rows->temp_mode == NRL_TEMP_DIV) { tc = 1; a.tparam = rows->temperature; }
+        else { tc = 2; a.tparam = 1.0f / rows->temperature; }
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned nb = static_cast<unsigned>(rows->n_outer);
+    if (nb > 0) grpo_seq_stats_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);
+    if (n_rows > 0) {
+        const dim3 grid((unsigned)n_rows), block(kFusedBlock);
+        switch (rows->dtype * 3 + tc) {
+            case NRL_F32 * 3 + 0: fused_logits_loss_kernel<NRL_F32, 0><<<grid, block, 0, s>>>(a); break;
+            case NRL_F32 * 3 + 1: fused_logits_loss_kernel<NRL_F32, 1><<<grid, block, 0, s>>>(a); break;
+            case NRL_F32 * 3 + 2: fused_logits_loss_kernel<NRL_F32, 2><<<grid, block, 0, s>>>(a); break;
+            case NRL_BF16 * 3 + 0: fused_logits_loss_kernel<NRL_BF16, 0><<<grid, block, 0, s>>>(a); break;
+            case NRL_BF16 * 3 + 1: fused_logits_loss_kernel<NRL_BF16, 1><<<grid, block, 0, s>>>(a); break;
+            case NRL_BF16 * 3 + 2: fused_logits_loss_kernel<NRL_BF16, 2><<<grid, block, 0, s>>>(a); break;
+            case NRL_F16 * 3 + 0: fused_logits_loss_kernel<NRL_F16, 0><<<grid, block, 0, s>>>(a); break;
+            case NRL_F16 * 3 + 1: fused_logits_loss_kernel<NRL_F16, 1><<<grid, block, 0, s>>>(a); break;
+            default: fused_logits_loss_kernel<NRL_F16, 2><<<grid, block, 0, s>>>(a); break;
+        }
+    }
+    if (nb > 0) grpo_terms_reduce_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);
+    GrpoArgs fa;
+    fa.cfg = *cfg;
+    fa.in = *in;
+    fa.dlp = nullptr; fa.dlpu = nullptr;
+    fa.parts = a.parts;
+    grpo_finish_kernel<<<dim3(1), dim3(kLossBlock), 0, s>>>(fa, loss_out, metrics_out);
+    return check_launch("fused_logits_grpo_loss");
 }

@@ -389,6 +389,65 @@ def _grpo_loss(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_ma
     return loss, dlp, dlpu, metrics
 
 
+_LIB.define(
+    "fused_logits_grpo_loss(Tensor logits, Tensor targets, int n_inner, Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, "
+    "Tensor token_mask, Tensor sample_mask, Tensor global_valid, int[] iflags, float[] fparams, float loss_scale) "
+    "-> (Tensor, Tensor, Tensor, Tensor)"
+)
+_LIB.define(
+    "fused_logits_grpo_loss_(Tensor(a!) logits, Tensor targets, int n_inner, Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, "
+    "Tensor token_mask, Tensor sample_mask, Tensor global_valid, int[] iflags, float[] fparams, float loss_scale) "
+    "-> (Tensor, Tensor, Tensor)"
+)
+
+
+def _fused_logits_grpo_loss(logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags,
+                            fparams, loss_scale, in_place=False):
+    """-> (loss, dlogits, logprobs [B, n_inner], metrics)."""
+    if len(iflags) != len(_CFG_INT) or len(fparams) != len(_CFG_FLT):
+        raise ValueError("malformed loss configuration")
+    _need_gpu(logits, targets)
+    b, s, v = logits.shape
+    rows = _rows(logits, targets, n_inner, 0, v, 1.0, _lib.NRL_TEMP_RCP)
+    dev = logits.device
+    lp_shape = torch.empty((b, n_inner), dtype=torch.float32, device=dev)
+    inp, keep, _, _ = _grpo_inputs(lp_shape, None, prev, gen, ref, adv, token_mask, sample_mask, None, global_valid)
+    cfg = _lib.NrlGrpoCfg()
+    for name, val in zip(_CFG_INT, iflags):
+        setattr(cfg, name, int(val))
+    for name, val in zip(_CFG_FLT, fparams):
+        setattr(cfg, name, float(val))
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        metrics = torch.empty((_lib.NRL_GRPO_N_METRICS,), dtype=torch.float32, device=dev)
+        d = logits if in_place else torch.empty((b, s, v), dtype=logits.dtype, device=dev)
+        ws_bytes = lib.nrl_fused_workspace_bytes(b, n_inner)
+        ws = torch.empty(((ws_bytes + 7) // 8,), dtype=torch.float64, device=dev)
+        with _timed("fused_logits_loss"):
+            code = lib.nrl_fused_logits_grpo_loss(
+                C.byref(rows), C.byref(cfg), C.byref(inp), float(loss_scale), _ptr(d), s, d.stride(0), d.stride(1),
+                _ptr(lp_shape), _ptr(loss), _ptr(metrics), _ptr(ws), ws.numel() * 8, _stream(),
+            )
+    if code == -2:
+        raise NotImplementedError(lib.nrl_last_error().decode(errors="replace"))
+    _lib.check(code, "nrl_fused_logits_grpo_loss")
+    del keep
+    return loss, d, lp_shape, metrics
+
+
+def _fused_logits_grpo_loss_inplace(logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid,
+                                    iflags, fparams, loss_scale):
+    loss, _, lp, metrics = _fused_logits_grpo_loss(logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask,
+                                                   global_valid, iflags, fparams, loss_scale, in_place=True)
+    return loss, lp, metrics
+
+
+for _name, _fn in (("fused_logits_grpo_loss", _fused_logits_grpo_loss), ("fused_logits_grpo_loss_", _fused_logits_grpo_loss_inplace)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
 def _nll_loss(lp, token_mask, sample_mask, global_valid):
     inp, keep, b, n = _grpo_inputs(lp, None, None, None, None, None, token_mask, sample_mask, None, global_valid)
     lib = _lib.load()

@@ -1,0 +1,174 @@
+"""GPU parity of the single-pass path (logits -> loss -> dlogits in one kernel) against the
+three-kernel HIP path and the CPU oracle.  Tolerances: loss / metrics 1e-4 relative, gradients as in
+``test_gpu_logprob.py``."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import logprob as OL
+from oracle import loss as O
+from rl_amd.algorithms.loss import (
+    ClippedPGLossConfig,
+    ClippedPGLossFn,
+    fused_logits_clipped_pg_loss,
+    prepare_loss_input,
+    why_not_fusable,
+    wrap_loss_fn_with_input_preparation,
+)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _batch(b, s, vocab, dtype, seed, float_masks=False):
+    g = torch.Generator().manual_seed(seed)
+    logits = (torch.randn(b, s, vocab, generator=g) * 2.5).to(dtype)
+    ids = torch.randint(0, vocab, (b, s), generator=g)
+    cur = OL.next_token_logprobs(ids, logits.float())
+    pad = lambda t: torch.cat([torch.zeros(b, 1), t], 1)  # noqa: E731
+    tm = torch.zeros(b, s, dtype=torch.float32 if float_masks else torch.int64)
+    for i in range(b):
+        tm[i, int(torch.randint(1, s - 2, (1,), generator=g)):] = 1
+    if b > 2:
+        tm[2] = 0
+    sm = torch.ones(b, dtype=torch.float32 if float_masks else torch.int64)
+    if b > 1:
+        sm[1] = 0
+    prev = pad(cur + 0.05 * torch.randn(b, s - 1, generator=g))
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm,
+            "advantages": torch.randn(b, 1, generator=g).expand(b, s).contiguous(), "prev_logprobs": prev,
+            "generation_logprobs": pad(cur + 0.05 * torch.randn(b, s - 1, generator=g)),
+            "reference_policy_logprobs": pad(cur + 0.05 * torch.randn(b, s - 1, generator=g))}
+    gs = sm.sum()
+    gt = (tm[:, 1:] * sm.unsqueeze(-1)).sum()
+    return logits, data, gs, gt
+
+
+def _close(a, b, rel=1e-4, abs_=1e-6):
+    if math.isinf(a) or math.isinf(b):
+        return a == b
+    return abs(a - b) <= rel * abs(b) + abs_
+
+
+FUSABLE = [
+    dict(),
+    dict(reference_policy_kl_penalty=0.0, ratio_clip_min=0.2, ratio_clip_max=0.28),
+    dict(reference_policy_kl_penalty=0.05, reference_policy_kl_type="k2", use_on_policy_kl_approximation=True),
+    dict(token_level_loss=False, reference_policy_kl_penalty=0.001),
+    dict(ratio_clip_c=3.0, use_importance_sampling_correction=True),
+    dict(use_cispo=True),
+    dict(disable_ppo_ratio=True),
+    dict(force_on_policy_ratio=True),
+    dict(use_importance_sampling_correction=True, truncated_importance_sampling_type="tis", truncated_importance_sampling_ratio=1.02),
+    dict(use_importance_sampling_correction=True, truncated_importance_sampling_type="seq-mask-tis",
+         truncated_importance_sampling_ratio=1.01, truncated_importance_sampling_ratio_min=0.99),
+    dict(token_level_loss=False, use_importance_sampling_correction=True, sequence_level_importance_ratios=True,
+         disable_ppo_ratio=True),
+]
+
+
+@pytest.mark.parametrize("cfg", FUSABLE, ids=[str(i) for i in range(len(FUSABLE))])
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 2000), (torch.bfloat16, 4096)])
+def test_fused_matches_oracle_and_unfused(cfg, dtype, vocab):
+    logits, data, gs, gt = _batch(4, 24, vocab, dtype, seed=len(cfg) + vocab)
+    xo = logits.to(torch.float32, copy=True).requires_grad_(True)
+    want, wm = O.clipped_pg_loss(O.LossConfig(**cfg), OL.next_token_logprobs(data["input_ids"], xo), data, gs, gt)
+    want.backward()
+
+    fn = ClippedPGLossFn(ClippedPGLossConfig(**cfg))
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    xg = logits.to(DEV).requires_grad_(True)
+    assert why_not_fusable(fn, xg, ddev) is None
+    got, gm = fused_logits_clipped_pg_loss(xg, ddev, fn, gs.to(DEV), gt.to(DEV))
+    got.backward()
+    assert _close(got.item(), want.item()), (got.item(), want.item())
+    assert set(gm) == set(wm)
+    for k in wm:
+        assert _close(float(gm[k]), float(wm[k]), rel=1e-4, abs_=1e-6), (k, gm[k], wm[k])
+
+    xu = logits.to(DEV).requires_grad_(True)
+    loss_input, d2 = prepare_loss_input(xu, dict(ddev), fn)
+    un, um = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    un.backward()
+    assert _close(got.item(), un.item(), rel=1e-5)
+    scale = xo.grad.abs().max().item() + 1e-30
+    gf, gu = xg.grad.float().cpu(), xu.grad.float().cpu()
+    if dtype == torch.float32:
+        assert (gf - xo.grad).abs().max().item() <= 1e-4 * scale
+        assert (gf - gu).abs().max().item() <= 1e-5 * scale
+    else:
+        ulp = 2.0 ** -8
+        assert bool(((gf - xo.grad).abs() <= xo.grad.abs() * (ulp + 1e-4) + 1e-4 * scale * ulp + 1e-30).all())
+        assert (gf == gu).float().mean().item() > 0.995
+    # masked tokens and the dropped last position receive exactly zero
+    mask = (data["token_mask"][:, 1:] * data["sample_mask"].unsqueeze(-1)) != 0
+    assert torch.all(gf[:, :-1][~mask] == 0) and torch.all(gf[:, -1] == 0)
+
+
+def test_fused_in_place_and_loss_scale():
+    logits, data, gs, gt = _batch(3, 16, 1024, torch.bfloat16, seed=5)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    x1 = logits.to(DEV).requires_grad_(True)
+    l1, _ = fused_logits_clipped_pg_loss(x1, ddev, fn, gs.to(DEV), gt.to(DEV))
+    (g1,) = torch.autograd.grad(l1, x1)
+    # the upstream gradient is folded in at forward time ...
+    x2 = logits.to(DEV).requires_grad_(True)
+    l2, _ = fused_logits_clipped_pg_loss(x2, ddev, fn, gs.to(DEV), gt.to(DEV), loss_scale=4.0)
+    (g2,) = torch.autograd.grad(l2 * 4.0, x2)
+    assert l1.item() == l2.item()
+    torch.testing.assert_close(g2.float(), g1.float() * 4.0, rtol=2 ** -7, atol=0)
+    # ... or applied afterwards when it was not announced
+    x3 = logits.to(DEV).requires_grad_(True)
+    l3, _ = fused_logits_clipped_pg_loss(x3, ddev, fn, gs.to(DEV), gt.to(DEV))
+    (g3,) = torch.autograd.grad(l3 * 4.0, x3)
+    torch.testing.assert_close(g3.float(), g1.float() * 4.0, rtol=2 ** -7, atol=0)
+    # in place: the logits buffer ends up holding the gradient
+    base = logits.to(DEV)
+    leaf = base.clone().requires_grad_(True)
+    work = leaf * 1                      # a non-leaf, like a model output
+    l4, _ = fused_logits_clipped_pg_loss(work, ddev, fn, gs.to(DEV), gt.to(DEV), in_place=True)
+    (g4,) = torch.autograd.grad(l4, leaf)
+    assert l4.item() == l1.item() and torch.equal(g4, g1)
+
+
+def test_unfusable_configs_fall_back_in_the_wrapper():
+    logits, data, gs, gt = _batch(3, 12, 512, torch.float32, seed=9)
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    gspo = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, sequence_level_importance_ratios=True))
+    assert why_not_fusable(gspo, logits.to(DEV), ddev) is not None
+    on_policy_seq = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, sequence_level_importance_ratios=True,
+                                                        force_on_policy_ratio=True))
+    assert why_not_fusable(on_policy_seq, logits.to(DEV), ddev) is not None
+    with pytest.raises(NotImplementedError):
+        fused_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, gspo, gs, gt)
+    for fn in (gspo, ClippedPGLossFn(ClippedPGLossConfig())):
+        xw = logits.to(DEV).requires_grad_(True)
+        lw, mw = wrap_loss_fn_with_input_preparation(xw, dict(ddev), gs.to(DEV), gt.to(DEV), fn, prepare_loss_input)
+        lw.backward()
+        xu = logits.to(DEV).requires_grad_(True)
+        li, d2 = prepare_loss_input(xu, dict(ddev), fn)
+        lu, mu = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **li)
+        lu.backward()
+        assert _close(lw.item(), lu.item(), rel=1e-5)
+        assert set(mw) == set(mu)
+        torch.testing.assert_close(xw.grad, xu.grad, rtol=1e-4, atol=1e-9)
+
+
+def test_fused_c2_slice_bf16_full_vocab():
+    logits, data, gs, gt = _batch(2, 10, 151936, torch.bfloat16, seed=1002)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    xg = logits.to(DEV).requires_grad_(True)
+    got, gm = fused_logits_clipped_pg_loss(xg, ddev, fn, gs.to(DEV), gt.to(DEV))
+    got.backward()
+    xo = logits.to(torch.float32, copy=True).requires_grad_(True)
+    want, wm = O.clipped_pg_loss(O.LossConfig(), OL.next_token_logprobs(data["input_ids"], xo), data, gs, gt)
+    want.backward()
+    assert _close(got.item(), want.item())
+    for k in wm:
+        assert _close(float(gm[k]), float(wm[k]), rel=2e-4, abs_=1e-6), (k, gm[k], wm[k])
+    scale = xo.grad.abs().max().item()
+    assert bool(((xg.grad.float().cpu() - xo.grad).abs() <= xo.grad.abs() * (2.0 ** -8 + 1e-4) + 1e-4 * scale * 2.0 ** -8 + 1e-30).all())
