@@ -311,6 +311,38 @@ def main():
                          "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
     }
+    # ---- the single-pass path (its own row: 2 * V * sizeof per token, gradient emitted by the forward launch) ----
+    from rl_amd.algorithms.loss import wrap_loss_fn_with_input_preparation
+
+    def fused_step():
+        for i in range(n_mb):
+            m = mbs[i % n_buf]
+            logits = m["logits"].requires_grad_(True)
+            loss, _metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare_loss_input)
+            (dlogits,) = torch.autograd.grad(loss, logits)
+            del dlogits, loss
+
+    for _ in range(args.warmup):
+        fused_step()
+    torch.cuda.synchronize()
+    ftimer = EventTimer(torch)
+    ops.KERNEL_TIMER = ftimer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fused_step()
+    torch.cuda.synchronize()
+    f_elapsed = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    fk = ftimer.summary().get("fused_logits_loss", dict(avg_ms=float("nan")))
+    f_gbs = 2 * row_bytes * rows_per_launch / (fk["avg_ms"] * 1e-3) / 1e9
+    result["fused_single_pass"] = {
+        "value": tokens_per_step * args.steps / f_elapsed, "unit": "tokens/s", "ms_per_step": f_elapsed / args.steps * 1e3,
+        "api": "wrap_loss_fn_with_input_preparation -> fused_logits_grpo_loss (seq stats + fused pass + term reduce + finish)",
+        "algorithmic_bytes_per_token": 2 * row_bytes,
+        "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel", "achieved": f_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": f_gbs / HBM_PEAK_GBS, "avg_launch_ms": fk["avg_ms"],
+                     "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
+    }
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)  # 4 GiB
         dst = torch.empty_like(src)
