@@ -29,9 +29,13 @@ _ALIASES = {
 # attributes replaced on a real NeMo-RL install (module -> names)
 _PATCHED = {
     "nemo_rl.distributed.model_utils": [
-        "DistributedLogprob", "ChunkedDistributedLogprob", "from_parallel_logits_to_logprobs",
-        "from_parallel_logits_to_logprobs_packed_sequences", "get_next_token_logprobs_from_logits",
+        "DistributedLogprob", "ChunkedDistributedLogprob", "DistributedLogprobWithSampling",
+        "ChunkedDistributedLogprobWithSampling", "ChunkedDistributedHiddenStatesToLogprobs",
+        "from_parallel_logits_to_logprobs", "from_parallel_logits_to_logprobs_packed_sequences",
+        "from_parallel_hidden_states_to_logprobs", "get_next_token_logprobs_from_logits",
     ],
+    "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
+    "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],
     "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
