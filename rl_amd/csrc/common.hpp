@@ -29,12 +29,22 @@ int check_launch(const char* what);
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
 
-// fp32 -> bf16 bits, round to nearest even (NaN stays a quiet NaN)
+// fp32 -> bf16 / fp16 bits, round to nearest even (NaN stays a quiet NaN), through the hardware
+// converts (v_cvt_pk_bf16_f32, v_cvt_pk_f16_f32): one instruction per pair
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<__bf16>(f)));
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t lo16) {
@@ -88,10 +98,10 @@ template <> struct Row<NRL_BF16> {
     }
     __device__ static __forceinline__ u32x4 encode(const float (&v)[8]) {
         u32x4 r;
-        r.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-        r.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
-        r.z = f32_to_bf16_bits(v[4]) | (f32_to_bf16_bits(v[5]) << 16);
-        r.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
+        r.x = pack_bf16x2(v[0], v[1]);
+        r.y = pack_bf16x2(v[2], v[3]);
+        r.z = pack_bf16x2(v[4], v[5]);
+        r.w = pack_bf16x2(v[6], v[7]);
         return r;
     }
     __device__ static __forceinline__ float load1(const void* p, int64_t i) {
@@ -114,10 +124,10 @@ template <> struct Row<NRL_F16> {
     }
     __device__ static __forceinline__ u32x4 encode(const float (&v)[8]) {
         u32x4 r;
-        r.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-        r.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-        r.z = f32_to_f16_bits(v[4]) | (f32_to_f16_bits(v[5]) << 16);
-        r.w = f32_to_f16_bits(v[6]) | (f32_to_f16_bits(v[7]) << 16);
+        r.x = pack_f16x2(v[0], v[1]);
+        r.y = pack_f16x2(v[2], v[3]);
+        r.z = pack_f16x2(v[4], v[5]);
+        r.w = pack_f16x2(v[6], v[7]);
         return r;
     }
     __device__ static __forceinline__ float load1(const void* p, int64_t i) {
@@ -189,6 +199,101 @@ template <int NW> __device__ __forceinline__ float block_min(float v, float* sme
 #pragma unroll
     for (int i = 1; i < NW; ++i) t = fminf(t, smem[i]);
     return t;
+}
+
+// Running (maximum, sum of exp(x - maximum)) pair of an online log-sum-exp.
+struct Lse {
+    float m;  // running maximum
+    float s;  // sum of exp(x - m)
+};
+
+__device__ __forceinline__ Lse lse_merge(Lse a, Lse b) {
+    const float m = fmaxf(a.m, b.m);
+    Lse r;
+    r.m = m;
+    r.s = a.s * fast_exp2((a.m - m) * kLog2e) + b.s * fast_exp2((b.m - m) * kLog2e);
+    return r;
+}
+
+template <int N> __device__ __forceinline__ void lse_push(Lse& acc, const float (&v)[N]) {
+    float vm = v[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) vm = fmaxf(vm, v[k]);
+    const float mn = fmaxf(acc.m, vm);
+    const float mn2 = mn * kLog2e;
+    float part = 0.f;
+#pragma unroll
+    for (int k = 0; k < N; ++k) part += fast_exp2(__builtin_fmaf(v[k], kLog2e, -mn2));
+    acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + part;
+    acc.m = mn;
+}
+
+__device__ __forceinline__ void lse_push1(Lse& acc, float x) {
+    const float mn = fmaxf(acc.m, x);
+    acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((x - mn) * kLog2e);
+    acc.m = mn;
+}
+
+// merge over the wave, then over the workgroup's NW waves; every thread returns the total
+template <int NW> __device__ __forceinline__ Lse block_lse(Lse acc, Lse* smem) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        Lse o;
+        o.m = __shfl_xor(acc.m, off, kWave);
+        o.s = __shfl_xor(acc.s, off, kWave);
+        acc = lse_merge(acc, o);
+    }
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = acc;
+    __syncthreads();
+    Lse tot = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) tot = lse_merge(tot, smem[i]);
+    return tot;
+}
+
+// ---------------------------------------------------------------------------------------------
+// d logprob / d logits of one row, times the incoming gradient g: g * (onehot - softmax), narrowed
+// once to the row dtype; with a fused temperature the chain rule through the in-place divide rounds
+// a second time, as autograd does.  RowGrad carries the per-row constants.
+// ---------------------------------------------------------------------------------------------
+struct RowGrad {
+    float lse2;  // log-sum-exp of the row in base-2 units
+    float g, ng;
+    float tparam;
+    __device__ __forceinline__ RowGrad(float lse, float g_, float tparam_) : lse2(lse * kLog2e), g(g_), ng(-g_), tparam(tparam_) {}
+};
+
+template <int DT, int TEMP> __device__ __forceinline__ float grad_finish(float d, float tparam) {
+    if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), tparam);
+    if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * tparam;
+    return d;
+}
+
+template <int DT, int TEMP> __device__ __forceinline__ float grad_elem(float x, bool is_target, const RowGrad& rg) {
+    const float p = fast_exp2(__builtin_fmaf(scale_logit<DT, TEMP>(x, rg.tparam), kLog2e, -rg.lse2));
+    return grad_finish<DT, TEMP>(is_target ? (1.f - p) * rg.g : p * rg.ng, rg.tparam);
+}
+
+// one 16-byte vector; tsub is the target's place in it, or -1
+template <int DT, int TEMP> __device__ __forceinline__ u32x4 grad_vec(const u32x4& raw, int tsub, const RowGrad& rg) {
+    constexpr int EPV = Row<DT>::EPV;
+    float d[EPV];
+    Row<DT>::decode(raw, d);
+#pragma unroll
+    for (int k = 0; k < EPV; ++k) {
+        const float p = fast_exp2(__builtin_fmaf(scale_logit<DT, TEMP>(d[k], rg.tparam), kLog2e, -rg.lse2));
+        d[k] = grad_finish<DT, TEMP>(p * rg.ng, rg.tparam);
+    }
+    if (tsub >= 0) {  // at most one lane of one vector per row
+        float t[EPV];
+        Row<DT>::decode(raw, t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k)
+            if (k == tsub) d[k] = grad_elem<DT, TEMP>(t[k], true, rg);
+    }
+    return Row<DT>::encode(d);
 }
 
 }  // namespace nrl

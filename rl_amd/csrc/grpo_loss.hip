@@ -312,123 +312,158 @@ __global__ __launch_bounds__(kLossBlock) void grpo_seq_stats_kernel(FusedArgs a)
     }
 }
 
+// Persistent workgroups: workgroup w walks rows w, w + gridDim.x, ...  While the gradient of one row
+// is being stored, the same slots (registers, or a staging register for the LDS slice) are refilled
+// with the next row this workgroup evaluates, and the online (max, sum) of that row is advanced a few
+// vectors behind the loads, so reads, writes and the exponentials all overlap and only the
+// cross-wave merge and the one-thread loss evaluation sit between two rows.
+// Slot order q = 0 .. kFusedVec-1: the LDS slots come first (vector kFusedRegVec + q), then the
+// register slots (vector q - kFusedLdsVec).
+constexpr int kFusedLag = 6;  // slots between issuing a load and folding it into the running sum
+
 template <int DT, int TEMP>
-__global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArgs a) {
+__global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArgs a, int64_t n_rows) {
     constexpr int EPV = Row<DT>::EPV;
     __shared__ u32x4 stash[kFusedLdsVec * kFusedBlock];
-    __shared__ float sm_f[kFusedWaves];
+    __shared__ Lse sm_l[kFusedWaves];
     __shared__ float sh_g, sh_lse;
     const nrl_grpo_cfg& c = a.cfg;
     const nrl_grpo_inputs& in = a.in;
     const int tid = threadIdx.x;
-    const int64_t r = blockIdx.x;
-    const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
-    u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(a.dlogits) + (o * a.ds_outer + i * a.ds_inner) * Row<DT>::BYTES);
-    const int64_t nvec = a.vocab / EPV;
+    const int nvec = static_cast<int>(a.vocab / EPV);
+    const int64_t step = gridDim.x;
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    float tm = 0.f, smv = 0.f;
-    if (i < a.n_inner) {
-        tm = in.token_mask[o * in.token_mask_stride + i];
-        smv = in.sample_mask[o];
-    }
-    const int64_t tok = o * a.n_inner + i;
-    if (tm * smv == 0.f) {  // dropped position or masked token
-        for (int64_t v = tid; v < nvec; v += kFusedBlock) __builtin_nontemporal_store(zero, ov + v);
-        if (i < a.n_inner && tid < T_COUNT) a.terms[tok * T_COUNT + tid] = 0.f;
-        if (i < a.n_inner && tid == 0) a.lp_out[tok] = 0.f;
-        return;
-    }
-    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
-    const u32x4* xv = reinterpret_cast<const u32x4*>(row);
-    u32x4 regs[kFusedRegVec];
-#pragma unroll
-    for (int j = 0; j < kFusedRegVec; ++j) {
-        const int64_t v = tid + static_cast<int64_t>(j) * kFusedBlock;
-        regs[j] = v < nvec ? __builtin_nontemporal_load(xv + v) : zero;
-    }
-#pragma unroll
-    for (int j = 0; j < kFusedLdsVec; ++j) {
-        const int64_t v = tid + static_cast<int64_t>(kFusedRegVec + j) * kFusedBlock;
-        if (v < nvec) stash[j * kFusedBlock + tid] = __builtin_nontemporal_load(xv + v);
-    }
-    // every lane only ever touches its own stash slots, so no barrier is needed around them
-    auto fetch = [&](int j) -> u32x4 { return j < kFusedRegVec ? regs[j] : stash[(j - kFusedRegVec) * kFusedBlock + tid]; };
+    const uint32_t lane_off = static_cast<uint32_t>(tid) * 16u;  // uniform base + 32-bit lane offset addressing
 
-    // row maximum, then the sum of exponentials (the data are on chip: no online rescaling needed)
-    float mx = -FLT_MAX;
-#pragma unroll
-    for (int j = 0; j < kFusedVec; ++j) {
-        if (tid + static_cast<int64_t>(j) * kFusedBlock < nvec) {
-            float t[EPV];
-            Row<DT>::decode(fetch(j), t);
-#pragma unroll
-            for (int k = 0; k < EPV; ++k) mx = fmaxf(mx, scale_logit<DT, TEMP>(t[k], a.tparam));
-        }
-    }
-    const float m = block_max<kFusedWaves>(mx, sm_f);
-    float part = 0.f;
-#pragma unroll
-    for (int j = 0; j < kFusedVec; ++j) {
-        if (tid + static_cast<int64_t>(j) * kFusedBlock < nvec) {
-            float t[EPV];
-            Row<DT>::decode(fetch(j), t);
-#pragma unroll
-            for (int k = 0; k < EPV; ++k) part += fast_exp2((scale_logit<DT, TEMP>(t[k], a.tparam) - m) * kLog2e);
-        }
-    }
-    const float ssum = block_sum<float, kFusedWaves>(part, sm_f);
-    const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
-    const int64_t tloc = (tg >= a.vstart && tg < a.vend) ? tg - a.vstart : -1;
-    if (tid == 0) {
-        const float log_s = logf(ssum);
-        float lp = 0.f;
-        if (tloc >= 0) lp = (scale_logit<DT, TEMP>(Row<DT>::load1(row, tloc), a.tparam) - m) - log_s;
-        SeqStats st;
-        st.seq_den = a.seq_stats[o * 3]; st.seq_ratio = 1.f; st.seq_w = a.seq_stats[o * 3 + 1]; st.seq_keep = a.seq_stats[o * 3 + 2];
-        TokenIn ti;
-        ti.lp = lp; ti.lpu = lp;
-        ti.prev = c.force_on_policy_ratio ? lp : in.prev[o * in.prev_stride + i];
-        ti.gen = in.gen[o * in.gen_stride + i];
-        ti.ref = c.has_kl ? in.ref[o * in.ref_stride + i] : 0.f;
-        ti.adv = in.adv[o * in.adv_stride + i];
-        ti.tm = tm; ti.smv = smv; ti.correct = 0.f;
-        ti.den_s = in.global_valid[0] + 1e-8f;
-        ti.den_t = in.global_valid[1] + 1e-8f;
-        const TokenOut out = token_eval<false>(c, st, ti);
-        float* rec = a.terms + tok * T_COUNT;
-#pragma unroll
-        for (int k = 0; k < P_SAMPLE_MASK; ++k) rec[k] = out.term[k];
-        rec[T_RATIO] = out.ratio;
-        rec[T_RATIO_CL] = out.ratio_cl;
-        rec[T_SELECTED] = out.selected ? 1.f : 0.f;
-        a.lp_out[tok] = lp;
-        sh_g = (out.d_actor + out.d_lpu) * a.loss_scale;
-        sh_lse = m + log_s;
-    }
-    __syncthreads();
-    const float g = sh_g, lse = sh_lse;
-    if (g == 0.f) {
-        for (int64_t v = tid; v < nvec; v += kFusedBlock) __builtin_nontemporal_store(zero, ov + v);
-        return;
-    }
-    const int64_t tvec = tloc >= 0 ? tloc / EPV : -1;
-    const int tsub = tloc >= 0 ? static_cast<int>(tloc % EPV) : -1;
-#pragma unroll
-    for (int j = 0; j < kFusedVec; ++j) {
-        const int64_t v = tid + static_cast<int64_t>(j) * kFusedBlock;
-        if (v < nvec) {
-            float t[EPV];
-            Row<DT>::decode(fetch(j), t);
-#pragma unroll
-            for (int k = 0; k < EPV; ++k) {
-                const float p = fast_exp2((scale_logit<DT, TEMP>(t[k], a.tparam) - lse) * kLog2e);
-                float d = (((v == tvec && k == tsub) ? 1.f : 0.f) - p) * g;
-                if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
-                if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
-                t[k] = d;
+    auto out_row = [&](int64_t r) -> char* {
+        const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+        return static_cast<char*>(a.dlogits) + (o * a.ds_outer + i * a.ds_inner) * Row<DT>::BYTES;
+    };
+    auto vec_at = [&](const char* base, int q) -> const u32x4* {  // this lane's vector of slot q
+        const int vi = q < kFusedLdsVec ? kFusedRegVec + q : q - kFusedLdsVec;
+        return reinterpret_cast<const u32x4*>(base + static_cast<size_t>(vi) * kFusedBlock * 16 + lane_off);
+    };
+    auto in_row = [&](int64_t r) -> const char* {
+        const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+        return static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+    };
+    // First row at or after r (in this workgroup's walk) whose token takes part in the loss.  Rows passed
+    // over are dropped positions or masked tokens: zero gradient, logprob reported as 0, nothing read.
+    auto advance = [&](int64_t r) -> int64_t {
+        for (; r < n_rows; r += step) {
+            const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+            float w = 0.f;
+            if (i < a.n_inner) w = in.token_mask[o * in.token_mask_stride + i] * in.sample_mask[o];
+            if (w != 0.f) break;
+            u32x4* ov = reinterpret_cast<u32x4*>(out_row(r));
+            for (int v = tid; v < nvec; v += kFusedBlock) __builtin_nontemporal_store(zero, ov + v);
+            if (i < a.n_inner) {
+                const int64_t tok = o * a.n_inner + i;
+                if (tid < T_COUNT) a.terms[tok * T_COUNT + tid] = 0.f;
+                if (tid == 0) a.lp_out[tok] = 0.f;
             }
-            __builtin_nontemporal_store(Row<DT>::encode(t), ov + v);
         }
+        return r;
+    };
+    auto slot_vec = [&](int q) -> int { return tid + (q < kFusedLdsVec ? kFusedRegVec + q : q - kFusedLdsVec) * kFusedBlock; };
+
+    u32x4 regs[kFusedRegVec], stage[kFusedLdsVec];
+    Lse acc;
+    auto fold = [&](int q) {  // slot q of the incoming row -> running sum (and its LDS place)
+        if (slot_vec(q) < nvec) {
+            const u32x4 raw = q < kFusedLdsVec ? stage[q < kFusedLdsVec ? q : 0] : regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec];
+            float t[EPV];
+            Row<DT>::decode(raw, t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+            lse_push<EPV>(acc, t);
+            if (q < kFusedLdsVec) stash[q * kFusedBlock + tid] = raw;  // only this lane ever touches the slot
+        }
+    };
+
+    int64_t r = advance(blockIdx.x);
+    if (r < n_rows) {
+        const char* xv = in_row(r);
+#pragma unroll
+        for (int q = 0; q < kFusedVec; ++q) {
+            const u32x4 x = slot_vec(q) < nvec ? __builtin_nontemporal_load(vec_at(xv, q)) : zero;
+            if (q < kFusedLdsVec) stage[q < kFusedLdsVec ? q : 0] = x;
+            else regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec] = x;
+        }
+        acc.m = -FLT_MAX;
+        acc.s = 0.f;
+#pragma unroll
+        for (int q = 0; q < kFusedVec; ++q) fold(q);
+    }
+    while (r < n_rows) {
+        const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+        const int64_t tok = o * a.n_inner + i;
+        const char* row = in_row(r);
+        char* ov = out_row(r);
+        const Lse tot = block_lse<kFusedWaves>(acc, sm_l);
+        const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
+        const int64_t tloc = (tg >= a.vstart && tg < a.vend) ? tg - a.vstart : -1;
+        if (tid == 0) {
+            const float log_s = logf(tot.s);
+            float lp = 0.f;
+            if (tloc >= 0) lp = (scale_logit<DT, TEMP>(Row<DT>::load1(row, tloc), a.tparam) - tot.m) - log_s;
+            SeqStats st;
+            st.seq_den = a.seq_stats[o * 3]; st.seq_ratio = 1.f; st.seq_w = a.seq_stats[o * 3 + 1]; st.seq_keep = a.seq_stats[o * 3 + 2];
+            TokenIn ti;
+            ti.lp = lp; ti.lpu = lp;
+            ti.prev = c.force_on_policy_ratio ? lp : in.prev[o * in.prev_stride + i];
+            ti.gen = in.gen[o * in.gen_stride + i];
+            ti.ref = c.has_kl ? in.ref[o * in.ref_stride + i] : 0.f;
+            ti.adv = in.adv[o * in.adv_stride + i];
+            ti.tm = in.token_mask[o * in.token_mask_stride + i];
+            ti.smv = in.sample_mask[o];
+            ti.correct = 0.f;
+            ti.den_s = in.global_valid[0] + 1e-8f;
+            ti.den_t = in.global_valid[1] + 1e-8f;
+            const TokenOut out = token_eval<false>(c, st, ti);
+            float* rec = a.terms + tok * T_COUNT;
+#pragma unroll
+            for (int k = 0; k < P_SAMPLE_MASK; ++k) rec[k] = out.term[k];
+            rec[T_RATIO] = out.ratio;
+            rec[T_RATIO_CL] = out.ratio_cl;
+            rec[T_SELECTED] = out.selected ? 1.f : 0.f;
+            a.lp_out[tok] = lp;
+            sh_g = (out.d_actor + out.d_lpu) * a.loss_scale;
+            sh_lse = tot.m + log_s;
+        }
+        __syncthreads();
+        const float g = sh_g, lse = sh_lse;
+        const int64_t rn = advance(r + step);
+        const bool more = rn < n_rows;
+        const char* nx = more ? in_row(rn) : row;
+        const int tvec = tloc >= 0 ? static_cast<int>(tloc / EPV) : -1;
+        const int tsub = tloc >= 0 ? static_cast<int>(tloc % EPV) : -1;
+        const RowGrad rg(lse, g, a.tparam);
+        acc.m = -FLT_MAX;
+        acc.s = 0.f;
+#pragma unroll
+        for (int q = 0; q < kFusedVec; ++q) {
+            const int v = slot_vec(q);
+            if (v < nvec) {
+                const u32x4 cur = q < kFusedLdsVec ? stash[(q < kFusedLdsVec ? q : 0) * kFusedBlock + tid]
+                                                   : regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec];
+                const u32x4 d = g == 0.f ? zero : grad_vec<DT, TEMP>(cur, v == tvec ? tsub : -1, rg);
+                __builtin_nontemporal_store(d, const_cast<u32x4*>(vec_at(ov, q)));
+                if (more) {
+                    const u32x4 x = __builtin_nontemporal_load(vec_at(nx, q));
+                    if (q < kFusedLdsVec) stage[q < kFusedLdsVec ? q : 0] = x;
+                    else regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec] = x;
+                }
+            }
+            if (more && q >= kFusedLag) fold(q - kFusedLag);
+        }
+        if (more) {
+#pragma unroll
+            for (int q = kFusedVec - kFusedLag; q < kFusedVec; ++q) fold(q);
+        }
+        // sh_g / sh_lse are rewritten only after the next block_lse, whose barriers every thread passes
+        // after reading them above
+        r = rn;
     }
 }
 
@@ -595,17 +630,21 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     const unsigned nb = static_cast<unsigned>(rows->n_outer);
     if (nb > 0) grpo_seq_stats_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);
     if (n_rows > 0) {
-        const dim3 grid((unsigned)n_rows), block(kFusedBlock);
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+            return fail(NRL_E_LAUNCH, "cannot read the device's compute-unit count");
+        // one resident workgroup per compute unit (64 KiB of LDS and 1024 threads each)
+        const dim3 grid((unsigned)(n_rows < cus ? n_rows : cus)), block(kFusedBlock);
         switch (rows->dtype * 3 + tc) {
-            case NRL_F32 * 3 + 0: fused_logits_loss_kernel<NRL_F32, 0><<<grid, block, 0, s>>>(a); break;
-            case NRL_F32 * 3 + 1: fused_logits_loss_kernel<NRL_F32, 1><<<grid, block, 0, s>>>(a); break;
-            case NRL_F32 * 3 + 2: fused_logits_loss_kernel<NRL_F32, 2><<<grid, block, 0, s>>>(a); break;
-            case NRL_BF16 * 3 + 0: fused_logits_loss_kernel<NRL_BF16, 0><<<grid, block, 0, s>>>(a); break;
-            case NRL_BF16 * 3 + 1: fused_logits_loss_kernel<NRL_BF16, 1><<<grid, block, 0, s>>>(a); break;
-            case NRL_BF16 * 3 + 2: fused_logits_loss_kernel<NRL_BF16, 2><<<grid, block, 0, s>>>(a); break;
-            case NRL_F16 * 3 + 0: fused_logits_loss_kernel<NRL_F16, 0><<<grid, block, 0, s>>>(a); break;
-            case NRL_F16 * 3 + 1: fused_logits_loss_kernel<NRL_F16, 1><<<grid, block, 0, s>>>(a); break;
-            default: fused_logits_loss_kernel<NRL_F16, 2><<<grid, block, 0, s>>>(a); break;
+            case NRL_F32 * 3 + 0: fused_logits_loss_kernel<NRL_F32, 0><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_F32 * 3 + 1: fused_logits_loss_kernel<NRL_F32, 1><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_F32 * 3 + 2: fused_logits_loss_kernel<NRL_F32, 2><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_BF16 * 3 + 0: fused_logits_loss_kernel<NRL_BF16, 0><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_BF16 * 3 + 1: fused_logits_loss_kernel<NRL_BF16, 1><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_BF16 * 3 + 2: fused_logits_loss_kernel<NRL_BF16, 2><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_F16 * 3 + 0: fused_logits_loss_kernel<NRL_F16, 0><<<grid, block, 0, s>>>(a, n_rows); break;
+            case NRL_F16 * 3 + 1: fused_logits_loss_kernel<NRL_F16, 1><<<grid, block, 0, s>>>(a, n_rows); break;
+            default: fused_logits_loss_kernel<NRL_F16, 2><<<grid, block, 0, s>>>(a, n_rows); break;
         }
     }
     if (nb > 0) grpo_terms_reduce_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);

@@ -17,39 +17,35 @@
 
 namespace nrl {
 
-constexpr int kBlock = 256;
+#ifndef NRL_ROW_BLOCK
+#define NRL_ROW_BLOCK 256
+#endif
+#ifndef NRL_ROW_UNROLL
+#define NRL_ROW_UNROLL 4
+#endif
+#ifndef NRL_K2_NT_STORE
+#define NRL_K2_NT_STORE 1
+#endif
+#ifndef NRL_K2_NT_LOAD
+#define NRL_K2_NT_LOAD 1
+#endif
+constexpr int kBlock = NRL_ROW_BLOCK;
 constexpr int kWaves = kBlock / kWave;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = NRL_ROW_UNROLL;
 
-struct Lse {
-    float m;  // running maximum
-    float s;  // sum of exp(x - m)
-};
-
-__device__ __forceinline__ Lse lse_merge(Lse a, Lse b) {
-    const float m = fmaxf(a.m, b.m);
-    Lse r;
-    r.m = m;
-    r.s = a.s * fast_exp2((a.m - m) * kLog2e) + b.s * fast_exp2((b.m - m) * kLog2e);
-    return r;
+template <typename P> __device__ __forceinline__ u32x4 k2_load(const P* p) {
+#if NRL_K2_NT_LOAD
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
 }
-
-template <int N> __device__ __forceinline__ void lse_push(Lse& acc, const float (&v)[N]) {
-    float vm = v[0];
-#pragma unroll
-    for (int k = 1; k < N; ++k) vm = fmaxf(vm, v[k]);
-    const float mn = fmaxf(acc.m, vm);
-    float part = 0.f;
-#pragma unroll
-    for (int k = 0; k < N; ++k) part += fast_exp2((v[k] - mn) * kLog2e);
-    acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + part;
-    acc.m = mn;
-}
-
-__device__ __forceinline__ void lse_push1(Lse& acc, float x) {
-    const float mn = fmaxf(acc.m, x);
-    acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((x - mn) * kLog2e);
-    acc.m = mn;
+template <typename P> __device__ __forceinline__ void k2_store(u32x4 v, P* p) {
+#if NRL_K2_NT_STORE
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
 }
 
 // number of leading elements before the first 16-byte boundary of a row
@@ -99,21 +95,7 @@ __device__ __forceinline__ Lse row_online_lse(const void* row, int64_t vocab, fl
     const int64_t tail0 = head + nvec * EPV;
     if (tail0 + tid < vocab) lse_push1(acc, scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), tparam));
 
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        Lse o;
-        o.m = __shfl_xor(acc.m, off, kWave);
-        o.s = __shfl_xor(acc.s, off, kWave);
-        acc = lse_merge(acc, o);
-    }
-    const int lane = tid & (kWave - 1), w = tid / kWave;
-    __syncthreads();
-    if (lane == 0) smem[w] = acc;
-    __syncthreads();
-    Lse tot = smem[0];
-#pragma unroll
-    for (int i = 1; i < kWaves; ++i) tot = lse_merge(tot, smem[i]);
-    return tot;
+    return block_lse<kWaves>(acc, smem);
 }
 
 template <int DT> __device__ __forceinline__ void row_zero(void* row, int64_t vocab) {
@@ -129,27 +111,17 @@ template <int DT> __device__ __forceinline__ void row_zero(void* row, int64_t vo
     if (tail0 + tid < vocab) Row<DT>::store1(row, tail0 + tid, 0.f);
 }
 
-// gradient of one element: g * (onehot - softmax), narrowed once to the row dtype; with a fused
-// temperature the chain rule through the in-place divide rounds a second time, as autograd does.
-template <int DT, int TEMP>
-__device__ __forceinline__ float grad_elem(float x, bool is_target, float lse, float g, float tparam) {
-    const float p = fast_exp2((scale_logit<DT, TEMP>(x, tparam) - lse) * kLog2e);
-    float d = ((is_target ? 1.f : 0.f) - p) * g;
-    if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), tparam);
-    if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * tparam;
-    return d;
-}
-
 template <int DT, int TEMP>
 __device__ __forceinline__ void row_write_grad(const void* row, void* out, int64_t vocab, float lse, float g,
                                                int64_t tgt, float tparam) {
     constexpr int EPV = Row<DT>::EPV;
     const int tid = threadIdx.x;
+    const RowGrad rg(lse, g, tparam);
     const int64_t head = row_head<DT>(row, vocab);
     if (row_head<DT>(out, vocab) != head) {
         // input and output rows are not congruent modulo 16 bytes: element-wise path
         for (int64_t i = tid; i < vocab; i += kBlock)
-            Row<DT>::store1(out, i, grad_elem<DT, TEMP>(Row<DT>::load1(row, i), i == tgt, lse, g, tparam));
+            Row<DT>::store1(out, i, grad_elem<DT, TEMP>(Row<DT>::load1(row, i), i == tgt, rg));
         return;
     }
     const int64_t nvec = (vocab - head) / EPV;
@@ -162,29 +134,20 @@ __device__ __forceinline__ void row_write_grad(const void* row, void* out, int64
     for (; base + kUnroll * kBlock <= nvec; base += kUnroll * kBlock) {
         u32x4 r[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) r[u] = __builtin_nontemporal_load(xv + base + u * kBlock + tid);
+        for (int u = 0; u < kUnroll; ++u) r[u] = k2_load(xv + base + u * kBlock + tid);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int64_t vi = base + u * kBlock + tid;
-            float t[EPV];
-            Row<DT>::decode(r[u], t);
-#pragma unroll
-            for (int k = 0; k < EPV; ++k) t[k] = grad_elem<DT, TEMP>(t[k], vi == tvec && k == tsub, lse, g, tparam);
-            __builtin_nontemporal_store(Row<DT>::encode(t), ov + vi);
+            k2_store(grad_vec<DT, TEMP>(r[u], vi == tvec ? tsub : -1, rg), ov + vi);
         }
     }
-    for (int64_t vi = base + tid; vi < nvec; vi += kBlock) {
-        float t[EPV];
-        Row<DT>::decode(__builtin_nontemporal_load(xv + vi), t);
-#pragma unroll
-        for (int k = 0; k < EPV; ++k) t[k] = grad_elem<DT, TEMP>(t[k], vi == tvec && k == tsub, lse, g, tparam);
-        __builtin_nontemporal_store(Row<DT>::encode(t), ov + vi);
-    }
-    if (tid < head) Row<DT>::store1(out, tid, grad_elem<DT, TEMP>(Row<DT>::load1(row, tid), tid == tgt, lse, g, tparam));
+    for (int64_t vi = base + tid; vi < nvec; vi += kBlock)
+        k2_store(grad_vec<DT, TEMP>(k2_load(xv + vi), vi == tvec ? tsub : -1, rg), ov + vi);
+    if (tid < head) Row<DT>::store1(out, tid, grad_elem<DT, TEMP>(Row<DT>::load1(row, tid), tid == tgt, rg));
     const int64_t tail0 = head + nvec * EPV;
     if (tail0 + tid < vocab) {
         const int64_t i = tail0 + tid;
-        Row<DT>::store1(out, i, grad_elem<DT, TEMP>(Row<DT>::load1(row, i), i == tgt, lse, g, tparam));
+        Row<DT>::store1(out, i, grad_elem<DT, TEMP>(Row<DT>::load1(row, i), i == tgt, rg));
     }
 }
 

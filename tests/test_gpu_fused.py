@@ -97,7 +97,9 @@ def test_fused_matches_oracle_and_unfused(cfg, dtype, vocab):
     gf, gu = xg.grad.float().cpu(), xu.grad.float().cpu()
     if dtype == torch.float32:
         assert (gf - xo.grad).abs().max().item() <= 1e-4 * scale
-        assert (gf - gu).abs().max().item() <= 1e-5 * scale
+        # the two paths sum the exponentials in different orders; d loss / d logprob amplifies that
+        # ulp-level logprob difference wherever the KL term nearly cancels
+        assert (gf - gu).abs().max().item() <= 1e-4 * scale
     else:
         ulp = 2.0 ** -8
         assert bool(((gf - xo.grad).abs() <= xo.grad.abs() * (ulp + 1e-4) + 1e-4 * scale * ulp + 1e-30).all())
