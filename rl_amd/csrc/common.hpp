@@ -71,6 +71,7 @@ template <int DT> struct Row;
 template <> struct Row<NRL_F32> {
     static constexpr int EPV = 4;
     static constexpr int BYTES = 4;
+    static constexpr uint32_t NEG_INF_WORD = 0xff800000u;  // -inf in every element of a 32-bit word
     __device__ static __forceinline__ float round_self(float v) { return v; }
     __device__ static __forceinline__ void decode(const u32x4& r, float (&v)[4]) {
         v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y);
@@ -89,6 +90,7 @@ template <> struct Row<NRL_F32> {
 template <> struct Row<NRL_BF16> {
     static constexpr int EPV = 8;
     static constexpr int BYTES = 2;
+    static constexpr uint32_t NEG_INF_WORD = 0xff80ff80u;
     __device__ static __forceinline__ float round_self(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
     __device__ static __forceinline__ void decode(const u32x4& r, float (&v)[8]) {
         v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
@@ -115,6 +117,7 @@ template <> struct Row<NRL_BF16> {
 template <> struct Row<NRL_F16> {
     static constexpr int EPV = 8;
     static constexpr int BYTES = 2;
+    static constexpr uint32_t NEG_INF_WORD = 0xfc00fc00u;
     __device__ static __forceinline__ float round_self(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
     __device__ static __forceinline__ void decode(const u32x4& r, float (&v)[8]) {
         v[0] = f16_bits_to_f32(r.x & 0xffffu); v[1] = f16_bits_to_f32(r.x >> 16);
@@ -220,7 +223,7 @@ template <int N> __device__ __forceinline__ void lse_push(Lse& acc, const float 
 #pragma unroll
     for (int k = 1; k < N; ++k) vm = fmaxf(vm, v[k]);
     const float mn = fmaxf(acc.m, vm);
-    const float mn2 = mn * kLog2e;
+    const float mn2 = fmaxf(mn, -1e30f) * kLog2e;  // stays finite while no finite element has been seen
     float part = 0.f;
 #pragma unroll
     for (int k = 0; k < N; ++k) part += fast_exp2(__builtin_fmaf(v[k], kLog2e, -mn2));

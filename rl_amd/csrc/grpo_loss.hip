@@ -313,8 +313,8 @@ __global__ __launch_bounds__(kLossBlock) void grpo_seq_stats_kernel(FusedArgs a)
 }
 
 // Persistent workgroups: workgroup w walks rows w, w + gridDim.x, ...  While the gradient of one row
-// is being stored, the same slots (registers, or a staging register for the LDS slice) are refilled
-// with the next row this workgroup evaluates, and the online (max, sum) of that row is advanced a few
+// is being stored, the same slots (registers, and the LDS slice through direct global-to-LDS loads) are
+// refilled with the next row this workgroup evaluates, and the online (max, sum) of that row is advanced a few
 // vectors behind the loads, so reads, writes and the exponentials all overlap and only the
 // cross-wave merge and the one-thread loss evaluation sit between two rows.
 // Slot order q = 0 .. kFusedVec-1: the LDS slots come first (vector kFusedRegVec + q), then the
@@ -333,19 +333,29 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
     const int nvec = static_cast<int>(a.vocab / EPV);
     const int64_t step = gridDim.x;
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    const uint32_t lane_off = static_cast<uint32_t>(tid) * 16u;  // uniform base + 32-bit lane offset addressing
 
     auto out_row = [&](int64_t r) -> char* {
         const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
         return static_cast<char*>(a.dlogits) + (o * a.ds_outer + i * a.ds_inner) * Row<DT>::BYTES;
     };
-    auto vec_at = [&](const char* base, int q) -> const u32x4* {  // this lane's vector of slot q
-        const int vi = q < kFusedLdsVec ? kFusedRegVec + q : q - kFusedLdsVec;
-        return reinterpret_cast<const u32x4*>(base + static_cast<size_t>(vi) * kFusedBlock * 16 + lane_off);
-    };
     auto in_row = [&](int64_t r) -> const char* {
         const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
         return static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+    };
+    // Slot q holds vector slot_vec(q) of the row.  Lanes past the end of the row are pointed at the
+    // row's last vector instead: they load, compute and store exactly what that vector's own lane does
+    // (harmless duplicates), so the slot loop has no divergent branch around its memory operations and
+    // the loads of the next row stay in flight behind the stores.
+    auto slot_vec = [&](int q) -> int { return tid + (q < kFusedLdsVec ? kFusedRegVec + q : q - kFusedLdsVec) * kFusedBlock; };
+    // (recomputed at every use from an opaque copy of the lane index: twenty precomputed offsets would
+    // not fit in the register file next to the row)
+    auto slot_cl = [&](int q) -> int {
+        int t = tid;
+        asm volatile("" : "+v"(t));
+        return min(t + (q < kFusedLdsVec ? kFusedRegVec + q : q - kFusedLdsVec) * kFusedBlock, nvec - 1);
+    };
+    auto vec_at = [&](const char* base, int vc) -> const u32x4* {  // uniform base + 32-bit lane offset
+        return reinterpret_cast<const u32x4*>(base + static_cast<uint32_t>(vc) * 16u);
     };
     // First row at or after r (in this workgroup's walk) whose token takes part in the loss.  Rows passed
     // over are dropped positions or masked tokens: zero gradient, logprob reported as 0, nothing read.
@@ -365,35 +375,43 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
         }
         return r;
     };
-    auto slot_vec = [&](int q) -> int { return tid + (q < kFusedLdsVec ? kFusedRegVec + q : q - kFusedLdsVec) * kFusedBlock; };
-
-    u32x4 regs[kFusedRegVec], stage[kFusedLdsVec];
+    u32x4 regs[kFusedRegVec];
     Lse acc;
-    auto fold = [&](int q) {  // slot q of the incoming row -> running sum (and its LDS place)
-        if (slot_vec(q) < nvec) {
-            const u32x4 raw = q < kFusedLdsVec ? stage[q < kFusedLdsVec ? q : 0] : regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec];
-            float t[EPV];
-            Row<DT>::decode(raw, t);
-#pragma unroll
-            for (int k = 0; k < EPV; ++k) t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
-            lse_push<EPV>(acc, t);
-            if (q < kFusedLdsVec) stash[q * kFusedBlock + tid] = raw;  // only this lane ever touches the slot
-        }
+    // LDS slot q of the incoming row: global memory -> LDS without passing through registers; each wave
+    // fills the 1 KiB of the slot that its own lanes read back
+    auto lds_fill = [&](const char* base, int q) {
+        u32x4* dst = stash + q * kFusedBlock + (tid & ~(kWave - 1));
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const __attribute__((address_space(1))) void*>(
+                                             reinterpret_cast<uintptr_t>(vec_at(base, slot_cl(q)))),
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
     };
+    auto fold = [&](int q) {  // slot q of the incoming row -> running sum; lanes past the row add nothing
+        u32x4 raw = q < kFusedLdsVec ? stash[(q < kFusedLdsVec ? q : 0) * kFusedBlock + tid] : regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec];
+        if (slot_vec(q) >= nvec) raw = u32x4{Row<DT>::NEG_INF_WORD, Row<DT>::NEG_INF_WORD, Row<DT>::NEG_INF_WORD, Row<DT>::NEG_INF_WORD};
+        float t[EPV];
+        Row<DT>::decode(raw, t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+        lse_push<EPV>(acc, t);
+    };
+    // the direct-to-LDS loads are not tracked against later LDS reads by the compiler: wait for them
+    // (and everything older) by hand before the first read of a refilled LDS slot
+    auto wait_lds_fill = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
     int64_t r = advance(blockIdx.x);
     if (r < n_rows) {
         const char* xv = in_row(r);
 #pragma unroll
-        for (int q = 0; q < kFusedVec; ++q) {
-            const u32x4 x = slot_vec(q) < nvec ? __builtin_nontemporal_load(vec_at(xv, q)) : zero;
-            if (q < kFusedLdsVec) stage[q < kFusedLdsVec ? q : 0] = x;
-            else regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec] = x;
-        }
+        for (int q = 0; q < kFusedLdsVec; ++q) lds_fill(xv, q);
+#pragma unroll
+        for (int q = kFusedLdsVec; q < kFusedVec; ++q) regs[q - kFusedLdsVec] = __builtin_nontemporal_load(vec_at(xv, slot_cl(q)));
         acc.m = -FLT_MAX;
         acc.s = 0.f;
 #pragma unroll
-        for (int q = 0; q < kFusedVec; ++q) fold(q);
+        for (int q = kFusedLdsVec; q < kFusedVec; ++q) fold(q);
+        wait_lds_fill();
+#pragma unroll
+        for (int q = 0; q < kFusedLdsVec; ++q) fold(q);
     }
     while (r < n_rows) {
         const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
@@ -434,33 +452,40 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
         __syncthreads();
         const float g = sh_g, lse = sh_lse;
         const int64_t rn = advance(r + step);
-        const bool more = rn < n_rows;
-        const char* nx = more ? in_row(rn) : row;
+        const char* nx = rn < n_rows ? in_row(rn) : row;
         const int tvec = tloc >= 0 ? static_cast<int>(tloc / EPV) : -1;
         const int tsub = tloc >= 0 ? static_cast<int>(tloc % EPV) : -1;
         const RowGrad rg(lse, g, a.tparam);
         acc.m = -FLT_MAX;
         acc.s = 0.f;
+        // The LDS slots first: once all of them are consumed they are refilled for the next row (after
+        // the last row the refills and loads re-read the current row and are ignored).
 #pragma unroll
-        for (int q = 0; q < kFusedVec; ++q) {
-            const int v = slot_vec(q);
-            if (v < nvec) {
-                const u32x4 cur = q < kFusedLdsVec ? stash[(q < kFusedLdsVec ? q : 0) * kFusedBlock + tid]
-                                                   : regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec];
-                const u32x4 d = g == 0.f ? zero : grad_vec<DT, TEMP>(cur, v == tvec ? tsub : -1, rg);
-                __builtin_nontemporal_store(d, const_cast<u32x4*>(vec_at(ov, q)));
-                if (more) {
-                    const u32x4 x = __builtin_nontemporal_load(vec_at(nx, q));
-                    if (q < kFusedLdsVec) stage[q < kFusedLdsVec ? q : 0] = x;
-                    else regs[q < kFusedLdsVec ? 0 : q - kFusedLdsVec] = x;
-                }
+        for (int q = 0; q < kFusedLdsVec; ++q) {
+            const int vc = slot_cl(q);
+            const u32x4 d = grad_vec<DT, TEMP>(stash[q * kFusedBlock + tid], vc == tvec ? tsub : -1, rg);
+            __builtin_nontemporal_store(d, const_cast<u32x4*>(vec_at(ov, vc)));
+        }
+#pragma unroll
+        for (int q = 0; q < kFusedLdsVec; ++q) lds_fill(nx, q);
+#pragma unroll
+        for (int q = kFusedLdsVec; q < kFusedVec; ++q) {
+            const int vc = slot_cl(q);
+            const u32x4 d = grad_vec<DT, TEMP>(regs[q - kFusedLdsVec], vc == tvec ? tsub : -1, rg);
+            __builtin_nontemporal_store(d, const_cast<u32x4*>(vec_at(ov, vc)));
+            regs[q - kFusedLdsVec] = __builtin_nontemporal_load(vec_at(nx, vc));
+            __builtin_amdgcn_sched_barrier(0);  // keep the fold behind this slot's memory operations ...
+            if (q >= kFusedLdsVec + kFusedLag) {
+                fold(q - kFusedLag);
+                asm volatile("" : "+v"(acc.m), "+v"(acc.s));  // a use right here, so the fold is not sunk past the loop
             }
-            if (more && q >= kFusedLag) fold(q - kFusedLag);
+            __builtin_amdgcn_sched_barrier(0);  // ... and ahead of the next slot's
         }
-        if (more) {
 #pragma unroll
-            for (int q = kFusedVec - kFusedLag; q < kFusedVec; ++q) fold(q);
-        }
+        for (int q = kFusedVec - kFusedLag; q < kFusedVec; ++q) fold(q);
+        wait_lds_fill();
+#pragma unroll
+        for (int q = 0; q < kFusedLdsVec; ++q) fold(q);
         // sh_g / sh_lse are rewritten only after the next block_lse, whose barriers every thread passes
         // after reading them above
         r = rn;

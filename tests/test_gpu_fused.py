@@ -109,6 +109,31 @@ def test_fused_matches_oracle_and_unfused(cfg, dtype, vocab):
     assert torch.all(gf[:, :-1][~mask] == 0) and torch.all(gf[:, -1] == 0)
 
 
+def test_fused_rows_with_masked_vocabulary_runs():
+    """-inf runs in the logits (start of the row included) leave the single pass finite and equal to
+    the three-pass path."""
+    logits, data, gs, gt = _batch(3, 17, 6144, torch.bfloat16, seed=77)
+    logits[..., :2048] = float("-inf")
+    logits[..., 5000:5100] = float("-inf")
+    data["input_ids"] = data["input_ids"] % 2000 + 2100
+    cur = torch.cat([torch.zeros(3, 1), OL.next_token_logprobs(data["input_ids"], logits.float())], 1)
+    for k in ("prev_logprobs", "generation_logprobs", "reference_policy_logprobs"):
+        data[k] = cur + 0.03
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    xg = logits.to(DEV).requires_grad_(True)
+    got, _ = fused_logits_clipped_pg_loss(xg, ddev, fn, gs.to(DEV), gt.to(DEV))
+    got.backward()
+    xu = logits.to(DEV).requires_grad_(True)
+    loss_input, d2 = prepare_loss_input(xu, dict(ddev), fn)
+    un, _ = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    un.backward()
+    assert torch.isfinite(got) and torch.isfinite(xg.grad).all()
+    assert _close(got.item(), un.item(), rel=1e-5)
+    assert (xg.grad[..., :2048] == 0).all()
+    assert (xg.grad.float() == xu.grad.float()).float().mean().item() > 0.995
+
+
 def test_fused_in_place_and_loss_scale():
     logits, data, gs, gt = _batch(3, 16, 1024, torch.bfloat16, seed=5)
     fn = ClippedPGLossFn(ClippedPGLossConfig())

@@ -71,6 +71,30 @@ def test_spiked_logits_times_100_stay_finite():
     torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fill", ["-inf", "min"])
+def test_masked_vocabulary_runs_contribute_nothing(dtype, fill):
+    """Long runs of -inf (or the dtype's most negative value) in a row, including at its start where a
+    lane sees nothing finite first, must not disturb the log-sum-exp or the gradient."""
+    g = torch.Generator().manual_seed(15)
+    vocab = 6144
+    logits = torch.randn(2, 5, vocab, generator=g).to(dtype)
+    val = float("-inf") if fill == "-inf" else torch.finfo(dtype).min
+    logits[..., :2048] = val
+    logits[..., 4000:4100] = val
+    ids = torch.randint(2048, 4000, (2, 5), generator=g)
+    up = torch.randn(2, 4, generator=g)
+    want_lp, want_grad = _oracle_fwd_bwd(logits, ids, up)
+    x = logits.to(DEV).requires_grad_(True)
+    got = MU.from_parallel_logits_to_logprobs(x, ids.to(DEV), 0, vocab, None)
+    (got * up.to(DEV)).sum().backward()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.cpu(), want_lp, rtol=0, atol=1e-5 if dtype == torch.float32 else 2e-3)
+    assert torch.isfinite(x.grad).all()
+    assert (x.grad[..., :2048] == 0).all() and (x.grad[..., 4000:4100] == 0).all()
+    _check_grad(x.grad[:, :-1], want_grad[:, :-1], dtype)
+
+
 def test_out_of_shard_targets():
     g = torch.Generator().manual_seed(6)
     logits = torch.randn(1, 5, 16, generator=g)
