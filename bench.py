@@ -27,7 +27,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (scaled by the same counters on a 4 GiB copy), valid for one microbatch of the named workload
-MEASURED_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}
+MEASURED_TRAFFIC_BYTES = {"c2": 16.90e9 + 19.95e9}  # fused_logits_loss_kernel
+THREE_PASS_BWD_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}  # logprob_bwd_kernel
 
 WORKLOADS = {
     # name: (sequences, seq_len, vocab, dtype, sequences per microbatch, logit std, spike p)
@@ -257,7 +258,20 @@ def main():
     tot_toks = sum((m["data"]["token_mask"][:, 1:].sum() for m in mbs)) * (n_mb / n_buf)
     tot_toks = tot_toks.float()
 
+    from rl_amd.algorithms.loss import wrap_loss_fn_with_input_preparation
+
     def step():
+        # the drop-in call: logits + batch -> loss; dispatches to the single-pass kernel when the loss
+        # configuration allows it (this one does), and autograd hands back d loss / d logits
+        for i in range(n_mb):
+            m = mbs[i % n_buf]
+            logits = m["logits"].requires_grad_(True)
+            loss, _metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare_loss_input)
+            (dlogits,) = torch.autograd.grad(loss, logits)
+            del dlogits, loss
+
+    def three_pass_step():
+        # the reference's call structure spelled out: logprobs (pass 1), loss on logprobs, backward (passes 2+3)
         for i in range(n_mb):
             m = mbs[i % n_buf]
             logits = m["logits"].requires_grad_(True)
@@ -266,26 +280,28 @@ def main():
             (dlogits,) = torch.autograd.grad(loss, logits)
             del dlogits, loss, loss_input
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    timer = EventTimer(torch)
-    ops.KERNEL_TIMER = timer
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ops.KERNEL_TIMER = None
-    kernels = timer.summary()
+    def timed(fn_step):
+        for _ in range(args.warmup):
+            fn_step()
+        torch.cuda.synchronize()
+        timer = EventTimer(torch)
+        ops.KERNEL_TIMER = timer
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn_step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ops.KERNEL_TIMER = None
+        return dt, timer.summary()
 
+    elapsed, kernels = timed(step)
     tokens_per_step = w["seqs"] * w["seq_len"]
     rows_per_launch = w["mb_seqs"] * w["seq_len"]
     row_bytes = w["vocab"] * elt
-    bwd = kernels.get("logprob_bwd", dict(avg_ms=float("nan")))
-    fwd = kernels.get("logprob_fwd", dict(avg_ms=float("nan")))
-    bwd_gbs = 2 * row_bytes * rows_per_launch / (bwd["avg_ms"] * 1e-3) / 1e9
-    fwd_gbs = row_bytes * w["mb_seqs"] * (w["seq_len"] - 1) / (fwd["avg_ms"] * 1e-3) / 1e9
+    nan = dict(avg_ms=float("nan"))
+    fk = kernels.get("fused_logits_loss", nan)
+    alg_launch = 2 * row_bytes * rows_per_launch  # every logit read once, every gradient element written once
+    f_gbs = alg_launch / (fk["avg_ms"] * 1e-3) / 1e9
     result = {
         "metric": "GRPO logprob+loss fwd/bwd tokens/s at V=151936; % of HBM peak",
         "value": tokens_per_step * args.steps / elapsed,
@@ -301,47 +317,35 @@ def main():
         "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
-                   "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level"},
-        "hbm_frac_end_to_end": 3 * row_bytes * tokens_per_step * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "kernel": "logprob_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
+                   "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level",
+                   "api": "wrap_loss_fn_with_input_preparation(logits, batch, ...) + autograd.grad -> "
+                          "nrl_fused_logits_grpo_loss (seq stats + single pass + term reduce + finish)"},
+        "algorithmic_bytes_per_token": 2 * row_bytes,
+        "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel", "achieved": f_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": f_gbs / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if not args.seqs else None,
-                     "avg_launch_ms": bwd["avg_ms"], "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
-        "roofline_fwd": {"bound": "hbm", "kernel": "logprob_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
+                     "avg_launch_ms": fk["avg_ms"], "algorithmic_bytes_per_launch": alg_launch},
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
     }
-    # ---- the single-pass path (its own row: 2 * V * sizeof per token, gradient emitted by the forward launch) ----
-    from rl_amd.algorithms.loss import wrap_loss_fn_with_input_preparation
-
-    def fused_step():
-        for i in range(n_mb):
-            m = mbs[i % n_buf]
-            logits = m["logits"].requires_grad_(True)
-            loss, _metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare_loss_input)
-            (dlogits,) = torch.autograd.grad(loss, logits)
-            del dlogits, loss
-
-    for _ in range(args.warmup):
-        fused_step()
-    torch.cuda.synchronize()
-    ftimer = EventTimer(torch)
-    ops.KERNEL_TIMER = ftimer
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        fused_step()
-    torch.cuda.synchronize()
-    f_elapsed = time.perf_counter() - t0
-    ops.KERNEL_TIMER = None
-    fk = ftimer.summary().get("fused_logits_loss", dict(avg_ms=float("nan")))
-    f_gbs = 2 * row_bytes * rows_per_launch / (fk["avg_ms"] * 1e-3) / 1e9
-    result["fused_single_pass"] = {
-        "value": tokens_per_step * args.steps / f_elapsed, "unit": "tokens/s", "ms_per_step": f_elapsed / args.steps * 1e3,
-        "api": "wrap_loss_fn_with_input_preparation -> fused_logits_grpo_loss (seq stats + fused pass + term reduce + finish)",
-        "algorithmic_bytes_per_token": 2 * row_bytes,
-        "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel", "achieved": f_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": f_gbs / HBM_PEAK_GBS, "avg_launch_ms": fk["avg_ms"],
-                     "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
+    # ---- the three-pass path (its own row: 3 * V * sizeof per token) ----
+    t_elapsed, t_kernels = timed(three_pass_step)
+    bwd = t_kernels.get("logprob_bwd", nan)
+    fwd = t_kernels.get("logprob_fwd", nan)
+    bwd_gbs = 2 * row_bytes * rows_per_launch / (bwd["avg_ms"] * 1e-3) / 1e9
+    fwd_gbs = row_bytes * w["mb_seqs"] * (w["seq_len"] - 1) / (fwd["avg_ms"] * 1e-3) / 1e9
+    result["three_pass"] = {
+        "value": tokens_per_step * args.steps / t_elapsed, "unit": "tokens/s", "ms_per_step": t_elapsed / args.steps * 1e3,
+        "api": "prepare_loss_input -> nrl_logprob_fwd; ClippedPGLossFn -> nrl_grpo_loss_fwd_bwd; backward -> nrl_logprob_bwd",
+        "algorithmic_bytes_per_token": 3 * row_bytes,
+        "hbm_frac_end_to_end": 3 * row_bytes * tokens_per_step * args.steps / t_elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline_bwd": {"bound": "hbm", "kernel": "logprob_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": bwd["avg_ms"],
+                         "traffic": THREE_PASS_BWD_TRAFFIC_BYTES.get(args.workload) if not args.seqs else None,
+                         "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
+        "roofline_fwd": {"bound": "hbm", "kernel": "logprob_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
+        "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in t_kernels.items()},
     }
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)  # 4 GiB
