@@ -259,9 +259,9 @@ __global__ __launch_bounds__(kLossBlock) void nll_finish_kernel(nrl_grpo_inputs 
 // ---------------------------------------------------------------------------------------------
 constexpr int kFusedBlock = 1024;
 constexpr int kFusedWaves = kFusedBlock / kWave;
-constexpr int kFusedRegVec = 16;  // 16-byte vectors per lane held in registers ...
-constexpr int kFusedLdsVec = 4;   // ... and in LDS (64 KiB per workgroup)
-constexpr int kFusedVec = kFusedRegVec + kFusedLdsVec;
+constexpr int kFusedMaxRegVec = 16;  // at most 16 16-byte vectors per lane held in registers ...
+constexpr int kFusedLdsVec = 4;      // ... and 4 in LDS (64 KiB per workgroup)
+constexpr int kFusedMaxVec = kFusedMaxRegVec + kFusedLdsVec;
 constexpr int T_RATIO = P_SAMPLE_MASK, T_RATIO_CL = P_SAMPLE_MASK + 1, T_SELECTED = P_SAMPLE_MASK + 2, T_COUNT = 20;
 static_assert(P_SAMPLE_MASK + 3 <= T_COUNT, "token term record too small");
 
@@ -319,11 +319,13 @@ __global__ __launch_bounds__(kLossBlock) void grpo_seq_stats_kernel(FusedArgs a)
 // cross-wave merge and the one-thread loss evaluation sit between two rows.
 // Slot order q = 0 .. kFusedVec-1: the LDS slots come first (vector kFusedRegVec + q), then the
 // register slots (vector q - kFusedLdsVec).
-constexpr int kFusedLag = 6;  // slots between issuing a load and folding it into the running sum
-
-template <int DT, int TEMP>
+// NREG is the number of register slots the instantiation carries (the row must fit NREG + kFusedLdsVec
+// slots); shorter rows take a smaller instantiation instead of idling through unused slots.
+template <int DT, int TEMP, int NREG>
 __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArgs a, int64_t n_rows) {
     constexpr int EPV = Row<DT>::EPV;
+    constexpr int kFusedRegVec = NREG, kFusedVec = NREG + kFusedLdsVec;
+    constexpr int kFusedLag = NREG / 2 < 6 ? NREG / 2 : 6;  // slots between issuing a load and folding it into the running sum
     __shared__ u32x4 stash[kFusedLdsVec * kFusedBlock];
     __shared__ Lse sm_l[kFusedWaves];
     __shared__ float sh_g, sh_lse;
@@ -613,7 +615,7 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     if (seq_weights && rows->n_outer * rows->n_inner > 0 && !in->prev) return fail(NRL_E_INVALID, "prev_logprobs is NULL");
     if (cfg->kl_type < 1 || cfg->kl_type > 3 || cfg->tis_type < 0 || cfg->tis_type > 3) return fail(NRL_E_INVALID, "bad kl_type or tis_type");
     const int bytes = rows->dtype == NRL_F32 ? 4 : 2, epv = 16 / bytes;
-    if (rows->vocab % epv || rows->vocab / epv > static_cast<int64_t>(kFusedVec) * kFusedBlock)
+    if (rows->vocab % epv || rows->vocab / epv > static_cast<int64_t>(kFusedMaxVec) * kFusedBlock)
         return fail(NRL_E_UNSUPPORTED, "row does not fit the on-chip path (vocab %lld)", (long long)rows->vocab);
     if ((reinterpret_cast<uintptr_t>(rows->logits) & 15) || (reinterpret_cast<uintptr_t>(dlogits) & 15) ||
         (rows->stride_outer * bytes) % 16 || (rows->stride_inner * bytes) % 16 || (d_stride_outer * bytes) % 16 ||
@@ -660,17 +662,22 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
             return fail(NRL_E_LAUNCH, "cannot read the device's compute-unit count");
         // one resident workgroup per compute unit (64 KiB of LDS and 1024 threads each)
         const dim3 grid((unsigned)(n_rows < cus ? n_rows : cus)), block(kFusedBlock);
+        const int64_t slots = (rows->vocab / epv + kFusedBlock - 1) / kFusedBlock;
+        const int nreg = slots <= 8 ? 4 : slots <= 12 ? 8 : slots <= 16 ? 12 : 16;
+#define NRL_FUSED_CASE(DT_, TC_)                                                                                  \
+    case DT_ * 3 + TC_:                                                                                           \
+        if (nreg == 4) fused_logits_loss_kernel<DT_, TC_, 4><<<grid, block, 0, s>>>(a, n_rows);                   \
+        else if (nreg == 8) fused_logits_loss_kernel<DT_, TC_, 8><<<grid, block, 0, s>>>(a, n_rows);              \
+        else if (nreg == 12) fused_logits_loss_kernel<DT_, TC_, 12><<<grid, block, 0, s>>>(a, n_rows);            \
+        else fused_logits_loss_kernel<DT_, TC_, 16><<<grid, block, 0, s>>>(a, n_rows);                            \
+        break;
         switch (rows->dtype * 3 + tc) {
-            case NRL_F32 * 3 + 0: fused_logits_loss_kernel<NRL_F32, 0><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_F32 * 3 + 1: fused_logits_loss_kernel<NRL_F32, 1><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_F32 * 3 + 2: fused_logits_loss_kernel<NRL_F32, 2><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_BF16 * 3 + 0: fused_logits_loss_kernel<NRL_BF16, 0><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_BF16 * 3 + 1: fused_logits_loss_kernel<NRL_BF16, 1><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_BF16 * 3 + 2: fused_logits_loss_kernel<NRL_BF16, 2><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_F16 * 3 + 0: fused_logits_loss_kernel<NRL_F16, 0><<<grid, block, 0, s>>>(a, n_rows); break;
-            case NRL_F16 * 3 + 1: fused_logits_loss_kernel<NRL_F16, 1><<<grid, block, 0, s>>>(a, n_rows); break;
-            default: fused_logits_loss_kernel<NRL_F16, 2><<<grid, block, 0, s>>>(a, n_rows); break;
+            NRL_FUSED_CASE(NRL_F32, 0) NRL_FUSED_CASE(NRL_F32, 1) NRL_FUSED_CASE(NRL_F32, 2)
+            NRL_FUSED_CASE(NRL_BF16, 0) NRL_FUSED_CASE(NRL_BF16, 1) NRL_FUSED_CASE(NRL_BF16, 2)
+            NRL_FUSED_CASE(NRL_F16, 0) NRL_FUSED_CASE(NRL_F16, 1) NRL_FUSED_CASE(NRL_F16, 2)
+            default: return fail(NRL_E_INVALID, "unknown logits dtype");
         }
+#undef NRL_FUSED_CASE
     }
     if (nb > 0) grpo_terms_reduce_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);
     GrpoArgs fa;
