@@ -1,17 +1,19 @@
 // K6: fused lm_head -> token logprob (hidden @ W^T, never materialising the full logits) and its
 // backward (dH, dW), on the gfx950 matrix cores.
 //
-// One bf16 MFMA GEMM core, C[M,N] = A[M,K] * B[N,K]^T with fp32 accumulation, serves every product:
-//   * 256 x 128 output tile per workgroup (4 wave64 in a 2 x 2 grid, 128 x 64 per wave = 4 x 2
-//     v_mfma_f32_32x32x16_bf16 tiles, 128 accumulator registers per lane);
-//   * K is walked in 64-wide slabs: 16-byte global loads into registers for slab k+1 while slab k is
-//     consumed from LDS (rows padded to 72 elements so the 16-byte fragment reads of 32 different
-//     rows do not land on the same banks).
+// Two bf16 MFMA GEMM cores, C[M,N] = A[M,K] * B[N,K]^T with fp32 accumulation (v_mfma_f32_32x32x16_bf16,
+// 4 wave64 in a 2 x 2 grid), serve every product:
+//   * core B, the fast one (K a multiple of 64): 256 x 256 tile, 128 x 128 per wave (256 accumulator
+//     registers, one wave per SIMD), operands double-buffered in LDS by direct global-to-LDS loads;
+//   * core A, the general one (K a multiple of 8): 256 x 128 tile, operands staged through registers
+//     into one padded LDS buffer.
+// Workgroups are numbered so that the 32 that share an XCD (and its L2) cover a 4 x 8 patch of tiles.
 // Epilogues:
-//   LSE    forward: the tile's logits are rounded to bf16 (the reference's matmul returns bf16) and
-//          folded into a running (max, sum-exp) per row kept in registers while the workgroup walks
-//          its vocabulary tiles; the target's logit is captured on the way.  Only [rows] sized partials
-//          leave the chip.
+//   LSE    forward, computed as logits^T = W hidden^T so that the vocabulary runs along the accumulator
+//          rows a lane owns: the tile's logits are rounded to bf16 (the reference's matmul returns
+//          bf16) and folded into a running (max, sum-exp) per token column without any cross-lane
+//          traffic while the workgroup walks its vocabulary tiles; the target's logit is captured on the
+//          way.  Only [tokens] sized partials leave the chip.
 //   GRAD   backward: recomputed tile -> g * (onehot - exp(x - lse)) written as bf16 both row-major
 //          (for dH = G W) and transposed (for dW = G^T hidden) for one token chunk at a time.
 //   STORE / ACCUM  plain fp32 C = or C += for dH and dW.
@@ -19,6 +21,7 @@
 // chunk x V bf16 for G and G^T (1.2 GB each at chunk 4096, V 151936) instead of N x V.
 
 #include <float.h>
+#include <type_traits>
 #include <math.h>
 
 #include "common.hpp"
@@ -28,10 +31,7 @@ namespace nrl {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int GB_M = 256, GB_N = 128, GB_K = 64, GB_LD = GB_K + 8;  // LDS row stride (elements)
-constexpr int GB_THREADS = 256;
-constexpr int GB_A_LOADS = GB_M * GB_K / 8 / GB_THREADS;  // 8
-constexpr int GB_B_LOADS = GB_N * GB_K / 8 / GB_THREADS;  // 4
+constexpr int GB_THREADS = 256;  // 4 wave64 in a 2 x 2 grid, whatever the core
 
 struct GemmOperands {
     const uint16_t* a;  // [M, K] row stride lda
@@ -42,184 +42,369 @@ struct GemmOperands {
 // accumulator element e (0..15) of lane l in a 32x32 tile: column l % 32, row 8*(e/4) + 4*(l/32) + e%4
 __device__ __forceinline__ int acc_row(int e, int lane) { return 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3); }
 
-struct GemmRegs {
-    u32x4 a[GB_A_LOADS];
-    u32x4 b[GB_B_LOADS];
+// ---------------------------------------------------------------------------------------------
+// Core A: 256 x 128 tile (wave tile 128 x 64), any K multiple of 8.  Slab k+1 travels through
+// registers while slab k is consumed from one padded LDS buffer (row stride 72 elements).
+// ---------------------------------------------------------------------------------------------
+struct CoreA {
+    static constexpr int BM = 256, BN = 128, NI = 4, NJ = 2, BK = 64, LD = BK + 8;
+    static constexpr int LDS_BYTES = (BM + BN) * LD * 2;
+    static constexpr int A_LOADS = BM * BK / 8 / GB_THREADS, B_LOADS = BN * BK / 8 / GB_THREADS;
+    struct Regs {
+        u32x4 a[A_LOADS];
+        u32x4 b[B_LOADS];
+    };
+
+    __device__ static __forceinline__ void load_slab(const GemmOperands& op, int64_t row0, int64_t col0, int64_t k0, Regs& r) {
+        const int tid = threadIdx.x;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) {
+            const int c = tid + GB_THREADS * j;
+            const int rr = c >> 3, kc = c & 7;
+            int64_t grow = row0 + rr;
+            grow = grow < op.m ? grow : op.m - 1;
+            const int64_t kk = k0 + kc * 8;
+            r.a[j] = kk < op.k ? *reinterpret_cast<const u32x4*>(op.a + grow * op.lda + kk) : zero;
+        }
+#pragma unroll
+        for (int j = 0; j < B_LOADS; ++j) {
+            const int c = tid + GB_THREADS * j;
+            const int rr = c >> 3, kc = c & 7;
+            int64_t grow = col0 + rr;
+            grow = grow < op.n ? grow : op.n - 1;
+            const int64_t kk = k0 + kc * 8;
+            r.b[j] = kk < op.k ? *reinterpret_cast<const u32x4*>(op.b + grow * op.ldb + kk) : zero;
+        }
+    }
+
+    __device__ static __forceinline__ void store_slab(const Regs& r, uint16_t* As, uint16_t* Bs) {
+        const int tid = threadIdx.x;
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) {
+            const int c = tid + GB_THREADS * j;
+            *reinterpret_cast<u32x4*>(As + (c >> 3) * LD + (c & 7) * 8) = r.a[j];
+        }
+#pragma unroll
+        for (int j = 0; j < B_LOADS; ++j) {
+            const int c = tid + GB_THREADS * j;
+            *reinterpret_cast<u32x4*>(Bs + (c >> 3) * LD + (c & 7) * 8) = r.b[j];
+        }
+    }
+
+    // acc[i][j] += A[row0.., :] * B[col0.., :]^T for the workgroup's tile
+    __device__ static __forceinline__ void tile(const GemmOperands& op, int64_t row0, int64_t col0, f32x16 (&acc)[NI][NJ],
+                                                unsigned char* lds) {
+        uint16_t* As = reinterpret_cast<uint16_t*>(lds);
+        uint16_t* Bs = As + BM * LD;
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int wm = wave >> 1, wn = wave & 1;
+        const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+        Regs regs;
+        const int64_t nk = (op.k + BK - 1) / BK;
+        load_slab(op, row0, col0, 0, regs);
+        __syncthreads();  // previous users of the LDS tiles are done
+        store_slab(regs, As, Bs);
+        __syncthreads();
+        for (int64_t kt = 0; kt < nk; ++kt) {
+            if (kt + 1 < nk) load_slab(op, row0, col0, (kt + 1) * BK, regs);
+#pragma unroll
+            for (int ks = 0; ks < BK / 16; ++ks) {
+                bf16x8 af[NI], bfr[NJ];
+#pragma unroll
+                for (int i = 0; i < NI; ++i)
+                    af[i] = *reinterpret_cast<const bf16x8*>(As + (wm * 128 + i * 32 + frag_row) * LD + ks * 16 + frag_k);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+                    bfr[j] = *reinterpret_cast<const bf16x8*>(Bs + (wn * 64 + j * 32 + frag_row) * LD + ks * 16 + frag_k);
+#pragma unroll
+                for (int i = 0; i < NI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+            }
+            __syncthreads();
+            if (kt + 1 < nk) {
+                store_slab(regs, As, Bs);
+                __syncthreads();
+            }
+        }
+    }
 };
 
-__device__ __forceinline__ void gemm_load_slab(const GemmOperands& op, int64_t row0, int64_t col0, int64_t k0, GemmRegs& r) {
-    const int tid = threadIdx.x;
-    const u32x4 zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int j = 0; j < GB_A_LOADS; ++j) {
-        const int c = tid + GB_THREADS * j;
-        const int rr = c >> 3, kc = c & 7;
-        int64_t grow = row0 + rr;
-        grow = grow < op.m ? grow : op.m - 1;
-        const int64_t kk = k0 + kc * 8;
-        r.a[j] = kk < op.k ? *reinterpret_cast<const u32x4*>(op.a + grow * op.lda + kk) : zero;
-    }
-#pragma unroll
-    for (int j = 0; j < GB_B_LOADS; ++j) {
-        const int c = tid + GB_THREADS * j;
-        const int rr = c >> 3, kc = c & 7;
-        int64_t grow = col0 + rr;
-        grow = grow < op.n ? grow : op.n - 1;
-        const int64_t kk = k0 + kc * 8;
-        r.b[j] = kk < op.k ? *reinterpret_cast<const u32x4*>(op.b + grow * op.ldb + kk) : zero;
-    }
-}
+// ---------------------------------------------------------------------------------------------
+// Core B: 256 x 256 tile (wave tile 128 x 128: 16 MFMA tiles, 256 accumulator registers, one wave per
+// SIMD), K a multiple of 64.  Two LDS buffers per operand (4 x 32 KiB); slab k+1 is fetched by direct
+// global-to-LDS loads while slab k is consumed, one barrier per slab.  A 64-element row is 8 chunks
+// of 16 bytes; chunk c of row r sits at chunk position c ^ ((r >> 1) & 7), which keeps the rows unpadded
+// (a wave's direct load fills 1 KiB contiguously) and the wave's 16-byte fragment reads (32 rows x 2
+// chunks) free of bank conflicts: measured 8.7 cycles per ds_read_b128, the same as a contiguous read,
+// against 12.6 with the key r & 7 and 32 without swizzling.  Per 16-wide k step a wave issues 8 fragment reads for 16 MFMAs.
+// ---------------------------------------------------------------------------------------------
+struct CoreB {
+    static constexpr int BM = 256, BN = 256, NI = 4, NJ = 4, BK = 64;
+    static constexpr int TILE_BYTES = 256 * BK * 2;  // one operand, one buffer
+    static constexpr int LDS_BYTES = 4 * TILE_BYTES;  // A0 A1 B0 B1
+    static constexpr int ROUNDS = 256 * BK / 8 / GB_THREADS;  // direct loads per lane, operand and slab: 8
 
-__device__ __forceinline__ void gemm_store_slab(const GemmRegs& r, uint16_t* As, uint16_t* Bs) {
-    const int tid = threadIdx.x;
-#pragma unroll
-    for (int j = 0; j < GB_A_LOADS; ++j) {
-        const int c = tid + GB_THREADS * j;
-        *reinterpret_cast<u32x4*>(As + (c >> 3) * GB_LD + (c & 7) * 8) = r.a[j];
-    }
-#pragma unroll
-    for (int j = 0; j < GB_B_LOADS; ++j) {
-        const int c = tid + GB_THREADS * j;
-        *reinterpret_cast<u32x4*>(Bs + (c >> 3) * GB_LD + (c & 7) * 8) = r.b[j];
-    }
-}
+    struct Ctx {
+        const char* pa;  // first row of the tile, bytes
+        const char* pb;
+        uint32_t voa[ROUNDS], vob[ROUNDS];  // lane's source offset in each round (rows past the end clamped)
+        uint32_t aoff[BK / 16], boff[BK / 16];  // lane's fragment address for each k step (buffer 0, tile 0)
+        int wave;                               // wave index, held in a scalar register
+    };
 
-// acc[i][j] += A[row0.., :] * B[col0.., :]^T for the workgroup's 256 x 128 tile
-__device__ __forceinline__ void gemm_tile(const GemmOperands& op, int64_t row0, int64_t col0, f32x16 (&acc)[4][2],
-                                          uint16_t* As, uint16_t* Bs) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-    GemmRegs regs;
-    const int64_t nk = (op.k + GB_K - 1) / GB_K;
-    gemm_load_slab(op, row0, col0, 0, regs);
-    __syncthreads();  // previous users of the LDS tiles are done
-    gemm_store_slab(regs, As, Bs);
-    __syncthreads();
-    for (int64_t kt = 0; kt < nk; ++kt) {
-        if (kt + 1 < nk) gemm_load_slab(op, row0, col0, (kt + 1) * GB_K, regs);
+    // direct load number d (0..7: operand A rounds, 8..15: operand B rounds) of slab k0 into buffer buf
+    __device__ static __forceinline__ void issue_one(const Ctx& c, unsigned char* lds, int buf, int64_t k0, int d) {
+        const int op = d / ROUNDS, j = d % ROUNDS;
+        unsigned char* dst = lds + (2 * op + buf) * TILE_BYTES + (j * GB_THREADS + c.wave * 64) * 16;
+        const char* src = (op ? c.pb : c.pa) + k0 * 2 + (op ? c.vob[j] : c.voa[j]);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const __attribute__((address_space(1))) void*>(reinterpret_cast<uintptr_t>(src)),
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+    __device__ static __forceinline__ void issue(const Ctx& c, unsigned char* lds, int buf, int64_t k0) {
 #pragma unroll
-        for (int ks = 0; ks < GB_K / 16; ++ks) {
-            bf16x8 af[4], bfr[2];
+        for (int d = 0; d < 2 * ROUNDS; ++d) issue_one(c, lds, buf, k0, d);
+    }
+
+    // Consume slab buffer BUF while the direct loads of slab k_next go into the other buffer.  One wave per
+    // SIMD: nothing else hides latencies, so the order is fixed by hand -- one direct load behind each of
+    // the first 16 MFMAs (their address arithmetic runs in the shadow of the matrix pipe), and the
+    // fragments of k step ks + 1 requested half-way through the MFMAs of step ks.  (While direct-to-LDS
+    // loads are in flight the compiler drains every LDS read at each wait, so the reads must be issued
+    // half a step ahead of the wait that precedes their first use.)
+    template <int BUF>
+    __device__ static __forceinline__ void compute(const Ctx& c, unsigned char* lds, f32x16 (&acc)[NI][NJ], int64_t k_next) {
+        bf16x8 af[2][NI], bfr[2][NJ];
+        auto frags = [&](int ks, int set) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                af[i] = *reinterpret_cast<const bf16x8*>(As + (wm * 128 + i * 32 + frag_row) * GB_LD + ks * 16 + frag_k);
+            for (int i = 0; i < NI; ++i)
+                af[set][i] = *reinterpret_cast<const bf16x8*>(lds + c.aoff[ks] + BUF * TILE_BYTES + i * 32 * BK * 2);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                bfr[j] = *reinterpret_cast<const bf16x8*>(Bs + (wn * 64 + j * 32 + frag_row) * GB_LD + ks * 16 + frag_k);
+            for (int j = 0; j < NJ; ++j)
+                bfr[set][j] = *reinterpret_cast<const bf16x8*>(lds + c.boff[ks] + BUF * TILE_BYTES + j * 32 * BK * 2);
+        };
+        frags(0, 0);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+        for (int ks = 0; ks < BK / 16; ++ks) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+            for (int i = 0; i < NI; ++i) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+                    if (ks * NI * NJ + i * NJ + j < 2 * ROUNDS) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(c, lds, BUF ^ 1, k_next, ks * NI * NJ + i * NJ + j);
+                    }
+                }
+                if (i == NI / 2 - 1 && ks + 1 < BK / 16) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags(ks + 1, (ks + 1) & 1);
+                }
+            }
         }
-        __syncthreads();
-        if (kt + 1 < nk) {
-            gemm_store_slab(regs, As, Bs);
-            __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // End of a slab: the direct loads must have landed in LDS and every wave must be done reading the
+    // buffer they will overwrite next.  The compiler does not track direct loads against LDS reads, so the
+    // wait is written by hand.
+    __device__ static __forceinline__ void slab_barrier() {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+
+    __device__ static __forceinline__ void tile(const GemmOperands& op, int64_t row0, int64_t col0, f32x16 (&acc)[NI][NJ],
+                                                unsigned char* lds) {
+        const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wm = wave >> 1, wn = wave & 1;
+        Ctx c;
+        c.wave = wave;
+        c.pa = reinterpret_cast<const char*>(op.a + row0 * op.lda);
+        c.pb = reinterpret_cast<const char*>(op.b + col0 * op.ldb);
+        const int lr = tid >> 3, cg = (tid & 7) ^ ((lr >> 1) & 7);
+        const int last_a = static_cast<int>(op.m - 1 - row0 < 255 ? op.m - 1 - row0 : 255);
+        const int last_b = static_cast<int>(op.n - 1 - col0 < 255 ? op.n - 1 - col0 : 255);
+#pragma unroll
+        for (int j = 0; j < ROUNDS; ++j) {
+            const int r = j * 32 + lr;
+            c.voa[j] = static_cast<uint32_t>((r < last_a ? r : last_a) * op.lda + cg * 8) * 2u;
+            c.vob[j] = static_cast<uint32_t>((r < last_b ? r : last_b) * op.ldb + cg * 8) * 2u;
+        }
+        const int fr = lane & 31, fh = lane >> 5;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            const uint32_t sw = static_cast<uint32_t>(((ks * 2 + fh) ^ ((fr >> 1) & 7)) * 16);
+            c.aoff[ks] = static_cast<uint32_t>((wm * 128 + fr) * BK * 2) + sw;
+            c.boff[ks] = static_cast<uint32_t>(2 * TILE_BYTES + (wn * 128 + fr) * BK * 2) + sw;
+        }
+        const int64_t nk = op.k / BK;
+        const int64_t k_last = (nk - 1) * BK;
+        // every wave has passed the barrier that ended the previous tile's last slab, so buffer 0 is free
+        issue(c, lds, 0, 0);
+        slab_barrier();
+        // after the last slab the loads re-fetch it into the idle buffer (no branch in the slab body)
+        for (int64_t kt = 0; kt + 1 < nk; kt += 2) {
+            compute<0>(c, lds, acc, (kt + 1) * BK);
+            slab_barrier();
+            compute<1>(c, lds, acc, kt + 2 < nk ? (kt + 2) * BK : k_last);
+            slab_barrier();
+        }
+        if (nk & 1) {
+            compute<0>(c, lds, acc, k_last);
+            slab_barrier();
         }
     }
-}
+};
 
-__device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][2]) {
+template <class Core> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[Core::NI][Core::NJ]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < Core::NI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < Core::NJ; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 }
 
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
+// Tile coordinates of workgroup w of a 1-D launch over an nbx x nby tile grid.  Workgroups go to the
+// 8 XCDs (each with its own L2) round-robin by index, so index w runs on XCD w % 8 as that XCD's
+// (w / 8)-th workgroup; an XCD's 32 compute units hold one 4 x 8 patch of tiles at a time, which share
+// 4 A panels and 8 B panels through that L2.  Patches past the grid yield false.
+__device__ __forceinline__ bool patch_tile(uint32_t w, int64_t nbx, int64_t nby, int64_t& bx, int64_t& by) {
+    const uint32_t xcd = w & 7, s = w >> 3;
+    const uint32_t patch = (s >> 5) * 8 + xcd, t = s & 31;
+    const uint32_t ppy = static_cast<uint32_t>((nby + 7) >> 3);  // patches along y
+    const uint32_t px = patch / ppy, py = patch - px * ppy;
+    // the division runs on the vector unit; hand the (uniform) results back to scalar registers
+    bx = __builtin_amdgcn_readfirstlane(static_cast<int>(px * 4 + (t >> 3)));
+    by = __builtin_amdgcn_readfirstlane(static_cast<int>(py * 8 + (t & 7)));
+    return bx < nbx && by < nby;
+}
+static int64_t patch_grid(int64_t nbx, int64_t nby) {
+    const int64_t patches = ((nbx + 3) / 4) * ((nby + 7) / 8);
+    return (patches + 7) / 8 * 8 * 32;
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward: running log-sum-exp over the vocabulary tiles of one split
 // ---------------------------------------------------------------------------------------------
+// The product is taken as logits^T = W hidden^T: in the 32 x 32 accumulator tile a lane owns one column
+// and 16 rows, so with the vocabulary along the rows the whole log-sum-exp reduction of a tile stays
+// inside the lane (NJ token columns per lane, 2 registers of running state each) and no cross-lane
+// traffic happens until the very end.
 struct LmFwdArgs {
-    GemmOperands op;           // a = hidden [N,H], b = W [V,H]
+    GemmOperands op;           // a = W [V,H] (m = V), b = hidden [N,H] (n = N)
     const int64_t* targets;    // [N]
-    int64_t vocab_start;       // target ids are global; columns are local
+    int64_t vocab_start;       // target ids are global; rows of W are local
     int n_splits;
     float* part_m;             // [n_splits, N]
     float* part_s;             // [n_splits, N]
     float* xt;                 // [N] target logit (written by the tile that holds it)
 };
 
+template <class Core>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[GB_M * GB_LD];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_N * GB_LD];
-    __shared__ int tgt_local[GB_M];
-    __shared__ float comb_m[2][GB_M], comb_s[2][GB_M];
+    constexpr int NI = Core::NI, NJ = Core::NJ, BV = Core::BM, BT = Core::BN;  // vocabulary rows x token columns
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
+    __shared__ float comb_m[2][BT], comb_s[2][BT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * GB_M;
-    const int split = blockIdx.y;
-    const int64_t n_tiles = (a.op.n + GB_N - 1) / GB_N;
-    {
-        const int64_t grow = row0 + tid;
+    int64_t bx, by;
+    if (!patch_tile(blockIdx.x, (a.op.n + BT - 1) / BT, a.n_splits, bx, by)) return;
+    const int64_t tok0 = bx * BT;
+    const int split = static_cast<int>(by);
+    const int64_t n_tiles = (a.op.m + BV - 1) / BV;
+    // this lane's token columns and their (local) target rows
+    int64_t tok[NJ];
+    int tgt[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        tok[j] = tok0 + wn * (NJ * 32) + j * 32 + (lane & 31);
         int64_t t = -1;
-        if (grow < a.op.m) t = a.targets[grow] - a.vocab_start;
-        tgt_local[tid] = (t >= 0 && t < a.op.n) ? static_cast<int>(t) : -1;
+        if (tok[j] < a.op.n) t = a.targets[tok[j]] - a.vocab_start;
+        tgt[j] = (t >= 0 && t < a.op.m) ? static_cast<int>(t) : -1;
     }
-    float run_m[4][16], run_s[4][16];
+    float run_m[NJ], run_s[NJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) { run_m[i][e] = -FLT_MAX; run_s[i][e] = 0.f; }
+    for (int j = 0; j < NJ; ++j) { run_m[j] = -1e30f; run_s[j] = 0.f; }
 
     for (int64_t tile = split; tile < n_tiles; tile += a.n_splits) {
-        const int64_t col0 = tile * GB_N;
-        f32x16 acc[4][2];
-        zero_acc(acc);
-        gemm_tile(a.op, row0, col0, acc, As, Bs);
-        const int64_t c0 = col0 + wn * 64 + (lane & 31), c1 = c0 + 32;
-        const bool ok0 = c0 < a.op.n, ok1 = c1 < a.op.n;
+        const int64_t v0 = tile * BV;
+        f32x16 acc[NI][NJ];
+        zero_acc<Core>(acc);
+        Core::tile(a.op, v0, tok0, acc, lds);
+        // Accumulator element e of tile i is row `off` = i * 32 + 8 * (e / 4) + e % 4 (a compile-time constant)
+        // below this lane's first row vb.  Only the last vocabulary tile needs the rows-past-the-end mask.
+        const int vb = static_cast<int>(v0) + wm * 128 + 4 * (lane >> 5);
+        const int limit = static_cast<int>(a.op.m) - vb;  // rows with off < limit exist
+        auto fold_tile = [&](auto masked_tag) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+            for (int j = 0; j < NJ; ++j) {
+                __builtin_amdgcn_sched_barrier(0);
+                const int toff = tgt[j] - vb;  // the target's row as an offset, if it is in this lane at all
+                // The logits count as rounded to bf16 (the matmul output dtype).  Rounding is monotone, so the
+                // maximum is taken over the raw accumulators and rounded once.
+                float raw = -INFINITY;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int rl = wm * 128 + i * 32 + acc_row(e, lane);
-                const float x0 = ok0 ? round_bf16(acc[i][0][e]) : -INFINITY;
-                const float x1 = ok1 ? round_bf16(acc[i][1][e]) : -INFINITY;
-                const float mn = fmaxf(run_m[i][e], fmaxf(x0, x1));
-                run_s[i][e] = run_s[i][e] * fast_exp2((run_m[i][e] - mn) * kLog2e) + fast_exp2((x0 - mn) * kLog2e) +
-                              fast_exp2((x1 - mn) * kLog2e);
-                run_m[i][e] = mn;
-                const int tg = tgt_local[rl];
-                if (tg == c0) a.xt[row0 + rl] = x0;
-                if (tg == c1) a.xt[row0 + rl] = x1;
+                for (int i = 0; i < NI; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int off = i * 32 + 8 * (e >> 2) + (e & 3);
+                        raw = fmaxf(raw, (!MASKED || off < limit) ? acc[i][j][e] : -INFINITY);
+                    }
+                const float mx = fmaxf(run_m[j], round_bf16(raw));
+                const float mx2 = mx * kLog2e;
+                // (the subtraction is exact where an FMA against the rounded mx2 would leave a huge residual
+                // while both maxima are still the -1e30 start value)
+                float sx = run_s[j] * fast_exp2((run_m[j] - mx) * kLog2e);
+#pragma unroll
+                for (int i = 0; i < NI; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int off = i * 32 + 8 * (e >> 2) + (e & 3);
+                        const float p = fast_exp2(__builtin_fmaf(round_bf16(acc[i][j][e]), kLog2e, -mx2));
+                        sx += (!MASKED || off < limit) ? p : 0.f;
+                    }
+                run_m[j] = mx;
+                run_s[j] = sx;
+                if (toff >= 0 && toff < 128 && (toff & 4) == 0) {  // rare: the target's row is one of this lane's
+                    float xt = 0.f;
+#pragma unroll
+                    for (int i = 0; i < NI; ++i)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) xt = toff == i * 32 + 8 * (e >> 2) + (e & 3) ? acc[i][j][e] : xt;
+                    a.xt[tok[j]] = round_bf16(xt);
+                }
             }
-        }
+        };
+        if (v0 + BV <= a.op.m) fold_tile(std::false_type{});
+        else fold_tile(std::true_type{});
     }
-    // combine the 32 lanes that share a row, then the two column halves of the workgroup
+    // merge the two half-waves (rows 4 apart), then the two waves that share these token columns
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            float m = run_m[i][e], s = run_s[i][e];
-#pragma unroll
-            for (int off = 16; off > 0; off >>= 1) {
-                const float om = __shfl_xor(m, off, kWave), os = __shfl_xor(s, off, kWave);
-                const float mn = fmaxf(m, om);
-                s = s * fast_exp2((m - mn) * kLog2e) + os * fast_exp2((om - mn) * kLog2e);
-                m = mn;
-            }
-            if ((lane & 31) == 0) {
-                const int rl = wm * 128 + i * 32 + acc_row(e, lane);
-                comb_m[wn][rl] = m;
-                comb_s[wn][rl] = s;
-            }
+    for (int j = 0; j < NJ; ++j) {
+        const float om = __shfl_xor(run_m[j], 32, kWave), os = __shfl_xor(run_s[j], 32, kWave);
+        const float mn = fmaxf(run_m[j], om);
+        run_s[j] = run_s[j] * fast_exp2((run_m[j] - mn) * kLog2e) + os * fast_exp2((om - mn) * kLog2e);
+        run_m[j] = mn;
+        if (lane < 32) {
+            comb_m[wm][wn * (NJ * 32) + j * 32 + lane] = run_m[j];
+            comb_s[wm][wn * (NJ * 32) + j * 32 + lane] = run_s[j];
         }
     }
     __syncthreads();
-    {
-        const int64_t grow = row0 + tid;
-        if (grow < a.op.m) {
+    if (tid < BT) {
+        const int64_t t = tok0 + tid;
+        if (t < a.op.n) {
             const float m0 = comb_m[0][tid], m1 = comb_m[1][tid];
             const float mn = fmaxf(m0, m1);
-            const float s = comb_s[0][tid] * fast_exp2((m0 - mn) * kLog2e) + comb_s[1][tid] * fast_exp2((m1 - mn) * kLog2e);
-            a.part_m[static_cast<int64_t>(split) * a.op.m + grow] = mn;
-            a.part_s[static_cast<int64_t>(split) * a.op.m + grow] = s;
+            const float sv = comb_s[0][tid] * fast_exp2((m0 - mn) * kLog2e) + comb_s[1][tid] * fast_exp2((m1 - mn) * kLog2e);
+            a.part_m[static_cast<int64_t>(split) * a.op.n + t] = mn;
+            a.part_s[static_cast<int64_t>(split) * a.op.n + t] = sv;
         }
     }
 }
@@ -257,55 +442,65 @@ struct LmGradArgs {
     int64_t ldgt;
 };
 
+template <class Core>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[GB_M * GB_LD];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_N * GB_LD];
-    __shared__ int tgt_local[GB_M];
-    __shared__ float lse_l[GB_M], g_l[GB_M];
+    constexpr int NI = Core::NI, NJ = Core::NJ, BM = Core::BM, BN = Core::BN;
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
+    __shared__ int tgt_local[BM];
+    __shared__ float lse_l[BM], g_l[BM];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * GB_M;
-    const int64_t col0 = static_cast<int64_t>(blockIdx.y) * GB_N;
+    int64_t bx, by;
+    if (!patch_tile(blockIdx.x, (a.op.m + BM - 1) / BM, (a.op.n + BN - 1) / BN, bx, by)) return;
+    const int64_t row0 = bx * BM, col0 = by * BN;
     {
         const int64_t grow = row0 + tid;
         int64_t t = -1;
         float l = 0.f, g = 0.f;
         if (grow < a.op.m) { t = a.targets[grow] - a.vocab_start; l = a.lse[grow]; g = a.grad[grow]; }
         tgt_local[tid] = (t >= 0 && t < a.op.n) ? static_cast<int>(t) : -1;
-        lse_l[tid] = l;
+        lse_l[tid] = l * kLog2e;
         g_l[tid] = g;
     }
-    f32x16 acc[4][2];
-    zero_acc(acc);
-    gemm_tile(a.op, row0, col0, acc, As, Bs);
+    __syncthreads();
+    f32x16 acc[NI][NJ];
+    zero_acc<Core>(acc);
+    Core::tile(a.op, row0, col0, acc, lds);
+    const int64_t m_pad = ((a.op.m + 63) / 64) * 64;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int64_t c = col0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < NJ; ++j) {
+        const int64_t c = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
         const bool col_ok = c < a.op.n;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NI; ++i) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {  // four groups of four consecutive rows
-                uint32_t packed[4];
+                float gv[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int e = q * 4 + u;
                     const int rl = wm * 128 + i * 32 + acc_row(e, lane);
                     const bool row_ok = row0 + rl < a.op.m;
-                    float gv = 0.f;
+                    gv[u] = 0.f;
                     if (row_ok && col_ok) {
                         const float x = round_bf16(acc[i][j][e]);
-                        const float p = fast_exp2((x - lse_l[rl]) * kLog2e);
-                        gv = ((tgt_local[rl] == c ? 1.f : 0.f) - p) * g_l[rl];
+                        const float p = fast_exp2(__builtin_fmaf(x, kLog2e, -lse_l[rl]));
+                        gv[u] = ((tgt_local[rl] == c ? 1.f : 0.f) - p) * g_l[rl];
                     }
-                    packed[u] = f32_to_bf16_bits(gv);
-                    if (c < a.ldg && row0 + rl < ((a.op.m + 63) / 64) * 64) a.g[(row0 + rl) * a.ldg + c] = static_cast<uint16_t>(packed[u]);
                 }
+                const uint32_t p01 = pack_bf16x2(gv[0], gv[1]), p23 = pack_bf16x2(gv[2], gv[3]);
                 const int64_t r_first = row0 + wm * 128 + i * 32 + acc_row(q * 4, lane);
+                if (c < a.ldg) {
+                    uint16_t* gp = a.g + r_first * a.ldg + c;
+                    if (r_first + 0 < m_pad) gp[0] = static_cast<uint16_t>(p01);
+                    if (r_first + 1 < m_pad) gp[a.ldg] = static_cast<uint16_t>(p01 >> 16);
+                    if (r_first + 2 < m_pad) gp[2 * a.ldg] = static_cast<uint16_t>(p23);
+                    if (r_first + 3 < m_pad) gp[3 * a.ldg] = static_cast<uint16_t>(p23 >> 16);
+                }
                 if (col_ok && r_first < a.ldgt) {
                     uint2 v;
-                    v.x = packed[0] | (packed[1] << 16);
-                    v.y = packed[2] | (packed[3] << 16);
+                    v.x = p01;
+                    v.y = p23;
                     *reinterpret_cast<uint2*>(a.gt + c * a.ldgt + r_first) = v;
                 }
             }
@@ -316,22 +511,23 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
 // ---------------------------------------------------------------------------------------------
 // plain GEMM with fp32 output: C = A B^T or C += A B^T
 // ---------------------------------------------------------------------------------------------
-template <bool ACCUM>
+template <class Core, bool ACCUM>
 __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, float* c, int64_t ldc) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[GB_M * GB_LD];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[GB_N * GB_LD];
+    constexpr int NI = Core::NI, NJ = Core::NJ, BM = Core::BM, BN = Core::BN;
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * GB_M;
-    const int64_t col0 = static_cast<int64_t>(blockIdx.y) * GB_N;
-    f32x16 acc[4][2];
-    zero_acc(acc);
-    gemm_tile(op, row0, col0, acc, As, Bs);
+    int64_t bx, by;
+    if (!patch_tile(blockIdx.x, (op.m + BM - 1) / BM, (op.n + BN - 1) / BN, bx, by)) return;
+    const int64_t row0 = bx * BM, col0 = by * BN;
+    f32x16 acc[NI][NJ];
+    zero_acc<Core>(acc);
+    Core::tile(op, row0, col0, acc, lds);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t col = col0 + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < NJ; ++j) {
+            const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int64_t row = row0 + wm * 128 + i * 32 + acc_row(e, lane);
@@ -389,17 +585,43 @@ static int check_lmhead(const void* hidden, int64_t n, int64_t h, int64_t ldh, c
 
 using namespace nrl;
 
-static int fwd_splits(int64_t n, int64_t v) {
-    const int64_t row_blocks = (n + GB_M - 1) / GB_M, tiles = (v + GB_N - 1) / GB_N;
-    int64_t s = (512 + row_blocks - 1) / row_blocks;  // aim at two workgroups per CU
-    if (s > tiles) s = tiles;
+// Vocabulary splits of the forward: enough workgroups for every compute unit, in multiples of the
+// 8-wide patch side, never more than there are vocabulary tiles.
+template <class Core> static int fwd_splits(int64_t n, int64_t v) {
+    const int64_t row_blocks = (n + Core::BN - 1) / Core::BN, tiles = (v + Core::BM - 1) / Core::BM;  // token blocks, vocabulary tiles
+    int64_t s = (256 + row_blocks - 1) / row_blocks;
+    s = (s + 7) / 8 * 8;
     if (s > 64) s = 64;
+    if (s > tiles) s = tiles;
     return static_cast<int>(s < 1 ? 1 : s);
 }
 
 extern "C" int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab) {
     const int64_t n = n_tokens < 1 ? 1 : n_tokens;
-    return (2 * fwd_splits(n, vocab) + 1) * n * static_cast<int64_t>(sizeof(float));
+    const int sa = fwd_splits<CoreA>(n, vocab), sb = fwd_splits<CoreB>(n, vocab);
+    return (2 * (sa > sb ? sa : sb) + 1) * n * static_cast<int64_t>(sizeof(float));
+}
+
+template <class Core> static void launch_fwd(LmFwdArgs& a, float* ws, hipStream_t s) {
+    const int64_t n = a.op.n;
+    a.n_splits = fwd_splits<Core>(n, a.op.m);
+    a.part_m = ws; a.part_s = ws + static_cast<int64_t>(a.n_splits) * n; a.xt = ws + 2 * static_cast<int64_t>(a.n_splits) * n;
+    fill_zero_u32<<<dim3(256), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(a.xt), n);
+    lmhead_fwd_kernel<Core><<<dim3((unsigned)patch_grid((n + Core::BN - 1) / Core::BN, a.n_splits)), dim3(GB_THREADS), 0, s>>>(a);
+}
+
+template <class Core> static void launch_grad(const LmGradArgs& a, hipStream_t s) {
+    lmhead_grad_kernel<Core><<<dim3((unsigned)patch_grid((a.op.m + Core::BM - 1) / Core::BM, (a.op.n + Core::BN - 1) / Core::BN)),
+                               dim3(GB_THREADS), 0, s>>>(a);
+}
+
+template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, int64_t ldc, hipStream_t s) {
+    if (op.k % CoreB::BK == 0 && op.k > 0)
+        gemm_f32_kernel<CoreB, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreB::BM - 1) / CoreB::BM, (op.n + CoreB::BN - 1) / CoreB::BN)),
+                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc);
+    else
+        gemm_f32_kernel<CoreA, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreA::BM - 1) / CoreA::BM, (op.n + CoreA::BN - 1) / CoreA::BN)),
+                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc);
 }
 
 extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
@@ -411,18 +633,16 @@ extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int6
     if (n_tokens == 0) return NRL_OK;
     if (!logprob_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
     if (workspace_bytes < nrl_lmhead_fwd_workspace_bytes(n_tokens, vocab)) return fail(NRL_E_WORKSPACE, "workspace too small");
-    const int splits = fwd_splits(n_tokens, vocab);
     float* ws = static_cast<float*>(workspace);
     LmFwdArgs a;
-    a.op.a = static_cast<const uint16_t*>(hidden); a.op.b = static_cast<const uint16_t*>(weight);
-    a.op.lda = ldh; a.op.ldb = ldw; a.op.m = n_tokens; a.op.n = vocab; a.op.k = hidden_size;
-    a.targets = targets; a.vocab_start = vocab_start; a.n_splits = splits;
-    a.part_m = ws; a.part_s = ws + static_cast<int64_t>(splits) * n_tokens; a.xt = ws + 2 * static_cast<int64_t>(splits) * n_tokens;
+    a.op.a = static_cast<const uint16_t*>(weight); a.op.b = static_cast<const uint16_t*>(hidden);
+    a.op.lda = ldw; a.op.ldb = ldh; a.op.m = vocab; a.op.n = n_tokens; a.op.k = hidden_size;
+    a.targets = targets; a.vocab_start = vocab_start;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int64_t row_blocks = (n_tokens + GB_M - 1) / GB_M;
-    if (row_blocks >= (1ll << 31)) return fail(NRL_E_INVALID, "too many tokens");
-    fill_zero_u32<<<dim3(256), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(a.xt), n_tokens);
-    lmhead_fwd_kernel<<<dim3((unsigned)row_blocks, (unsigned)splits), dim3(GB_THREADS), 0, s>>>(a);
+    if ((n_tokens + 255) / 256 >= (1ll << 24)) return fail(NRL_E_INVALID, "too many tokens");
+    if (hidden_size % CoreB::BK == 0) launch_fwd<CoreB>(a, ws, s);
+    else launch_fwd<CoreA>(a, ws, s);
+    const int splits = a.n_splits;
     lmhead_fwd_finish_kernel<<<dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, s>>>(
         n_tokens, splits, a.part_m, a.part_s, a.xt, targets, vocab_start, vocab_end, logprob_out, lse_out);
     return check_launch("lmhead_logprob_fwd");
@@ -476,19 +696,18 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         ga.targets = targets + t0; ga.vocab_start = vocab_start; ga.lse = lse + t0; ga.grad = grad + t0;
         ga.g = g; ga.ldg = vp; ga.gt = gt; ga.ldgt = chunk;
         if (rows_pad < chunk) fill_zero_u32<<<dim3(2048), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(gt), vocab * chunk / 2);
-        lmhead_grad_kernel<<<dim3((unsigned)((rows + GB_M - 1) / GB_M), (unsigned)((vocab + GB_N - 1) / GB_N)), dim3(GB_THREADS), 0, s>>>(ga);
+        if (h % CoreB::BK == 0) launch_grad<CoreB>(ga, s);
+        else launch_grad<CoreA>(ga, s);
         // dH[chunk] = G [rows, V] * (W^T [H, V])^T
         GemmOperands dh;
         dh.a = g; dh.lda = vp; dh.b = wt; dh.ldb = vp; dh.m = rows; dh.n = h; dh.k = vp;
-        gemm_f32_kernel<false><<<dim3((unsigned)((rows + GB_M - 1) / GB_M), (unsigned)((h + GB_N - 1) / GB_N)), dim3(GB_THREADS), 0, s>>>(
-            dh, dhidden_out + t0 * ld_dh, ld_dh);
+        launch_gemm<false>(dh, dhidden_out + t0 * ld_dh, ld_dh, s);
         // dW += G^T [V, rows] * (hidden^T [H, rows])^T
         transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((rows_pad + 63) / 64)), dim3(256), 0, s>>>(
             hid + t0 * ldh, rows, h, ldh, ht, chunk, rows_pad);
         GemmOperands dwo;
         dwo.a = gt; dwo.lda = chunk; dwo.b = ht; dwo.ldb = chunk; dwo.m = vocab; dwo.n = h; dwo.k = rows_pad;
-        gemm_f32_kernel<true><<<dim3((unsigned)((vocab + GB_M - 1) / GB_M), (unsigned)((h + GB_N - 1) / GB_N)), dim3(GB_THREADS), 0, s>>>(
-            dwo, dw, h);
+        launch_gemm<true>(dwo, dw, h, s);
     }
     // narrow dW once
     {
