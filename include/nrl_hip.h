@@ -240,7 +240,7 @@ int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int64_t prompt
  * shifted.  The logits of a tile are rounded to bf16 before the softmax, as the reference's bf16
  * matmul does.  logprob_out / lse_out: fp32 [N] (lse_out may be NULL).
  * Backward: grad fp32 [N] -> dhidden_out fp32 [N, H] (row stride ld_dh) and dweight_out bf16 [V, H]
- * (row stride ld_dw), accumulated in fp32 and narrowed once.  Tokens are processed in chunks of 4096:
+ * (row stride ld_dw), accumulated in fp32 and narrowed once.  Tokens are processed in chunks of 16384:
  * per chunk the gradient of the logits exists as bf16 [chunk, V] (twice, one transposed).
  * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
  * ------------------------------------------------------------------------------------------ */

@@ -18,7 +18,7 @@
 //          (for dH = G W) and transposed (for dW = G^T hidden) for one token chunk at a time.
 //   STORE / ACCUM  plain fp32 C = or C += for dH and dW.
 // The vocabulary is walked in tiles while the token chunk bounds what is materialised:
-// chunk x V bf16 for G and G^T (1.2 GB each at chunk 4096, V 151936) instead of N x V.
+// chunk x V bf16 for G and G^T (5 GB each at chunk 16384, V 151936) instead of N x V.
 
 #include <float.h>
 #include <type_traits>
@@ -467,41 +467,111 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     zero_acc<Core>(acc);
     Core::tile(a.op, row0, col0, acc, lds);
     const int64_t m_pad = ((a.op.m + 63) / 64) * 64;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
+    // gradient of the lane's 4 consecutive tokens (accumulator rows) of tile (i, j), group q, as two bf16 pairs
+    auto grad4 = [&](int i, int j, int q, uint32_t& p01, uint32_t& p23) {
         const int64_t c = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
         const bool col_ok = c < a.op.n;
+        float gv[4];
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int u = 0; u < 4; ++u) {
+            const int e = q * 4 + u;
+            const int rl = wm * 128 + i * 32 + acc_row(e, lane);
+            const bool row_ok = row0 + rl < a.op.m;
+            gv[u] = 0.f;
+            if (row_ok && col_ok) {
+                const float x = round_bf16(acc[i][j][e]);
+                const float p = fast_exp2(__builtin_fmaf(x, kLog2e, -lse_l[rl]));
+                gv[u] = ((tgt_local[rl] == c ? 1.f : 0.f) - p) * g_l[rl];
+            }
+        }
+        p01 = pack_bf16x2(gv[0], gv[1]);
+        p23 = pack_bf16x2(gv[2], gv[3]);
+    };
+    if constexpr (Core::LDS_BYTES >= BM * BN * 2) {
+        // Both layouts leave through LDS so that every global store is a 16-byte piece of a 512-byte run.
+        // Pass 1, [vocab][token]: a lane's 4 tokens are one 8-byte unit; unit U of row v sits at U ^ (v & 63).
+        // Pass 2, [token][vocab]: 2-byte writes; the 16-byte chunk C of row t sits at C ^ ((t >> 2) & 7).
+        constexpr int RV = BN / 8;  // 16-byte pieces per token row of the tile
+        uint32_t p01[NI][NJ][4], p23[NI][NJ][4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {  // four groups of four consecutive rows
-                float gv[4];
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int e = q * 4 + u;
-                    const int rl = wm * 128 + i * 32 + acc_row(e, lane);
-                    const bool row_ok = row0 + rl < a.op.m;
-                    gv[u] = 0.f;
-                    if (row_ok && col_ok) {
-                        const float x = round_bf16(acc[i][j][e]);
-                        const float p = fast_exp2(__builtin_fmaf(x, kLog2e, -lse_l[rl]));
-                        gv[u] = ((tgt_local[rl] == c ? 1.f : 0.f) - p) * g_l[rl];
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) grad4(i, j, q, p01[i][j][q], p23[i][j][q]);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int v = wn * (NJ * 32) + j * 32 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int t0 = wm * 128 + i * 32 + acc_row(q * 4, lane);
+                    const int unit = (t0 >> 2) ^ (v & 63);
+                    *reinterpret_cast<uint2*>(lds + v * (BM * 2) + unit * 8) = uint2{p01[i][j][q], p23[i][j][q]};
+                }
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int it = 0; it < BN * 32 / GB_THREADS; ++it) {
+            const int idx = it * GB_THREADS + tid, v = idx >> 5, m = idx & 31;
+            const uint2 lo = *reinterpret_cast<const uint2*>(lds + v * (BM * 2) + (((2 * m) ^ (v & 63)) * 8));
+            const uint2 hi = *reinterpret_cast<const uint2*>(lds + v * (BM * 2) + (((2 * m + 1) ^ (v & 63)) * 8));
+            const int64_t c = col0 + v, r = row0 + 8 * m;
+            if (c < a.op.n && r < a.ldgt) *reinterpret_cast<u32x4*>(a.gt + c * a.ldgt + r) = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int v = wn * (NJ * 32) + j * 32 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int t0 = wm * 128 + i * 32 + acc_row(q * 4, lane);
+                    const uint32_t w[2] = {p01[i][j][q], p23[i][j][q]};
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int t = t0 + u;
+                        const int chunk = (v >> 3) ^ ((t >> 2) & 7);
+                        *reinterpret_cast<uint16_t*>(lds + t * (BN * 2) + chunk * 16 + (v & 7) * 2) =
+                            static_cast<uint16_t>(w[u >> 1] >> ((u & 1) * 16));
                     }
                 }
-                const uint32_t p01 = pack_bf16x2(gv[0], gv[1]), p23 = pack_bf16x2(gv[2], gv[3]);
-                const int64_t r_first = row0 + wm * 128 + i * 32 + acc_row(q * 4, lane);
-                if (c < a.ldg) {
-                    uint16_t* gp = a.g + r_first * a.ldg + c;
-                    if (r_first + 0 < m_pad) gp[0] = static_cast<uint16_t>(p01);
-                    if (r_first + 1 < m_pad) gp[a.ldg] = static_cast<uint16_t>(p01 >> 16);
-                    if (r_first + 2 < m_pad) gp[2 * a.ldg] = static_cast<uint16_t>(p23);
-                    if (r_first + 3 < m_pad) gp[3 * a.ldg] = static_cast<uint16_t>(p23 >> 16);
-                }
-                if (col_ok && r_first < a.ldgt) {
-                    uint2 v;
-                    v.x = p01;
-                    v.y = p23;
-                    *reinterpret_cast<uint2*>(a.gt + c * a.ldgt + r_first) = v;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int it = 0; it < BM * RV / GB_THREADS; ++it) {
+            const int idx = it * GB_THREADS + tid, t = idx / RV, m = idx % RV;
+            const u32x4 x = *reinterpret_cast<const u32x4*>(lds + t * (BN * 2) + ((m ^ ((t >> 2) & 7)) * 16));
+            const int64_t r = row0 + t, c = col0 + 8 * m;
+            if (r < m_pad && c < a.ldg) *reinterpret_cast<u32x4*>(a.g + r * a.ldg + c) = x;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int64_t c = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+            const bool col_ok = c < a.op.n;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {  // four groups of four consecutive rows
+                    uint32_t p01, p23;
+                    grad4(i, j, q, p01, p23);
+                    const int64_t r_first = row0 + wm * 128 + i * 32 + acc_row(q * 4, lane);
+                    if (c < a.ldg) {
+                        uint16_t* gp = a.g + r_first * a.ldg + c;
+                        if (r_first + 0 < m_pad) gp[0] = static_cast<uint16_t>(p01);
+                        if (r_first + 1 < m_pad) gp[a.ldg] = static_cast<uint16_t>(p01 >> 16);
+                        if (r_first + 2 < m_pad) gp[2 * a.ldg] = static_cast<uint16_t>(p23);
+                        if (r_first + 3 < m_pad) gp[3 * a.ldg] = static_cast<uint16_t>(p23 >> 16);
+                    }
+                    if (col_ok && r_first < a.ldgt) {
+                        uint2 v;
+                        v.x = p01;
+                        v.y = p23;
+                        *reinterpret_cast<uint2*>(a.gt + c * a.ldgt + r_first) = v;
+                    }
                 }
             }
         }
@@ -648,7 +718,9 @@ extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int6
     return check_launch("lmhead_logprob_fwd");
 }
 
-static int64_t bwd_chunk(int64_t n) { return n < 4096 ? round_up(n < 1 ? 1 : n, 64) : 4096; }
+// tokens per backward chunk: long enough that the dW product (K = chunk) amortises its fp32 read-modify-write
+static constexpr int64_t kBwdChunk = 16384;
+static int64_t bwd_chunk(int64_t n) { return n < kBwdChunk ? round_up(n < 1 ? 1 : n, 64) : kBwdChunk; }
 
 extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab) {
     const int64_t chunk = bwd_chunk(n_tokens), vp = round_up(vocab, 64);
