@@ -1,0 +1,216 @@
+"""GPU checks at the full shapes of the benchmark configurations.
+
+The CPU oracle cannot run these sizes whole, so each test combines (a) size-independent properties that
+hold for every row (softmax gradients sum to zero, masked rows are exactly zero, filtered rows keep at
+most k entries, a launch is bit-identical to the same rows launched alone) with (b) oracle parity on a
+random sample of rows of the very same tensors.  Tolerances as everywhere: logprobs 2e-3 for bf16 logits,
+gradients within the bf16 narrowing of the fp32 oracle gradient plus 1e-4."""
+
+import pytest
+import torch
+
+from oracle import logprob as OL
+from oracle import loss as O
+from rl_amd.algorithms.logits_sampling_utils import TrainingSamplingParams
+from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn, prepare_loss_input, wrap_loss_fn_with_input_preparation
+from rl_amd.distributed import model_utils as MU
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+V_QWEN = 151936
+
+
+def _randn_bf16(shape, std, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    out = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+    for i in range(shape[0]):  # one sequence at a time keeps the fp32 temporary small
+        out[i] = (torch.randn(shape[1:], generator=g, device=DEV) * std).to(torch.bfloat16)
+    return out
+
+
+def _grad_close_bf16(got, want_f32):
+    scale = want_f32.abs().max().item() + 1e-30
+    bound = want_f32.abs() * (2.0 ** -8 + 1e-4) + 1e-4 * scale * 2.0 ** -8 + 1e-30
+    return bool(((got.float() - want_f32).abs() <= bound).all())
+
+
+def test_config2_microbatch_full_shape():
+    """One microbatch of BASELINE config 2: 16 x 4096 tokens, V = 151936, bf16, prompt prefix U[256,1024]."""
+    b, s, v = 16, 4096, V_QWEN
+    g = torch.Generator().manual_seed(2002)
+    logits = _randn_bf16((b, s, v), 3.0, 2002)
+    ids = torch.randint(0, v, (b, s), generator=g)
+    spike = torch.rand(b, s - 1, generator=g) < 0.3
+    rows = spike.nonzero()
+    logits[rows[:, 0].to(DEV), rows[:, 1].to(DEV), ids[:, 1:][spike].to(DEV)] += 8.0
+    prefix = torch.randint(256, 1025, (b,), generator=g)
+    tm = (torch.arange(s)[None, :] >= prefix[:, None]).long()
+    sm = torch.ones(b, dtype=torch.long)
+    ids_d = ids.to(DEV)
+
+    # three passes: logprobs, then loss, then the gradient
+    x3 = logits.detach().requires_grad_(True)
+    cur = MU.from_parallel_logits_to_logprobs(x3.detach(), ids_d, 0, v, None)
+    assert cur.shape == (b, s - 1) and bool(torch.isfinite(cur).all()) and bool((cur <= 0).all())
+    pad = lambda t: torch.cat([torch.zeros(b, 1, device=DEV), t], 1)  # noqa: E731
+    gn = torch.Generator(device=DEV).manual_seed(7)
+    data = {"input_ids": ids_d, "token_mask": tm.to(DEV), "sample_mask": sm.to(DEV),
+            "advantages": torch.randn(b, 1, generator=gn, device=DEV).expand(b, s).contiguous(),
+            "prev_logprobs": pad(cur + 0.05 * torch.randn(b, s - 1, generator=gn, device=DEV)),
+            "generation_logprobs": pad(cur + 0.05 * torch.randn(b, s - 1, generator=gn, device=DEV)),
+            "reference_policy_logprobs": pad(cur + 0.05 * torch.randn(b, s - 1, generator=gn, device=DEV))}
+    gs = sm.sum().float().to(DEV)
+    gt = (tm[:, 1:] * sm[:, None]).sum().float().to(DEV)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    loss_input, d2 = prepare_loss_input(x3, dict(data), fn)
+    loss3, m3 = fn(data=d2, global_valid_seqs=gs, global_valid_toks=gt, **loss_input)
+    g3, dlp = torch.autograd.grad(loss3, [x3, loss_input["next_token_logprobs"]])
+
+    # batch invariance: rows launched alone are bit-identical to the same rows of the big launch
+    for bi in (0, 9):
+        alone = MU.from_parallel_logits_to_logprobs(logits[bi : bi + 1, 1000:1100], ids_d[bi : bi + 1, 1000:1100], 0, v, None)
+        assert torch.equal(alone[0], cur[bi, 1000:1099])
+
+    # properties of every gradient row
+    masked = (tm[:, 1:] == 0).to(DEV)
+    assert bool((g3[:, :-1][masked] == 0).all()) and bool((g3[:, -1] == 0).all())
+    live_rows = g3[:, :-1][~masked].float()
+    row_sum = live_rows.sum(-1).abs()
+    row_abs = live_rows.abs().sum(-1)
+    assert bool((row_sum <= 2e-2 * row_abs + 1e-12).all())  # softmax - onehot sums to zero up to the bf16 narrowing
+    del live_rows
+
+    # the single pass gives the same loss and (almost everywhere bit-identical) gradient
+    x1 = logits.detach().requires_grad_(True)
+    loss1, m1 = wrap_loss_fn_with_input_preparation(x1, data, gs, gt, fn, prepare_loss_input)
+    (g1,) = torch.autograd.grad(loss1, x1)
+    assert abs(loss1.item() - loss3.item()) <= 1e-5 * abs(loss3.item()) + 1e-9
+    for k in m3:
+        assert abs(float(m1[k]) - float(m3[k])) <= 1e-4 * abs(float(m3[k])) + 1e-6, k
+    same = 0.0
+    for bi in range(b):
+        same += (g1[bi] == g3[bi]).float().mean().item() / b
+    assert same > 0.995, same
+    assert bool((g1[:, :-1][masked] == 0).all()) and bool((g1[:, -1] == 0).all())
+
+    # oracle parity on sampled rows of the same tensors: logprob, and the gradient row for the upstream
+    # d loss / d logprob the loss kernel produced
+    picks = [(0, 1500), (3, 4094), (7, 2047), (12, 1024), (15, 3000), (5, 100)]
+    rows = torch.stack([logits[bi, si].float().cpu() for bi, si in picks])
+    tgt = torch.stack([ids[bi, si + 1] for bi, si in picks])
+    xo = rows.clone().requires_grad_(True)
+    want_lp = OL.rows_logprob(xo, tgt)
+    got_lp = torch.stack([cur[bi, si] for bi, si in picks]).cpu()
+    assert (got_lp - want_lp.detach()).abs().max().item() <= 2e-3
+    up = torch.stack([dlp[bi, si] for bi, si in picks]).cpu()
+    assert (up != 0).any() and (up == 0).any()  # live and masked rows are both in the sample
+    (want_lp * up).sum().backward()
+    got_g = torch.stack([g3[bi, si].float().cpu() for bi, si in picks])
+    assert _grad_close_bf16(got_g, xo.grad)
+
+
+def test_config4_microbatch_topk_topp_full_vocab():
+    """BASELINE config 4 rows (8192-token sequences, V = 151936 bf16, T = 0.7, top_k 50, top_p 0.95), two sequences."""
+    b, s, v = 2, 8192, V_QWEN
+    g = torch.Generator().manual_seed(4004)
+    logits = _randn_bf16((b, s, v), 3.0, 4004)
+    scaled = (logits.float() * (1.0 / torch.tensor(0.7, device=DEV))).to(torch.bfloat16)  # logits.div_(T) on the GPU
+    del logits
+    ids = torch.randint(0, v, (b, s), generator=g)
+    top = torch.stack([scaled[bi].float().argmax(-1) for bi in range(b)]).cpu()
+    ids[:, 1:] = torch.where(torch.rand(b, s - 1, generator=g) < 0.8, top[:, :-1], ids[:, 1:])
+    params = TrainingSamplingParams(top_k=50, top_p=0.95)
+    x = scaled.detach().requires_grad_(True)
+    lp = MU.from_parallel_logits_to_logprobs(x, ids.to(DEV), 0, v, None, sampling_params=params)
+    fin = torch.isfinite(lp)
+    assert fin.float().mean().item() > 0.7 and bool((lp[fin] <= 0).all())
+    assert bool((lp[~fin] == float("-inf")).all())  # a target outside the kept set
+    up = torch.randn(b, s - 1, generator=torch.Generator(device=DEV).manual_seed(1), device=DEV)
+    up = torch.where(fin, up, torch.zeros_like(up))
+    (torch.where(fin, lp, torch.zeros_like(lp)) * up).sum().backward()
+    gx = x.grad
+    nz = (gx[:, :-1] != 0).sum(-1)
+    assert bool((gx[:, -1] == 0).all())
+    # at most k entries survive, plus values tied with the k-th one (bf16 logits tie often; the filter keeps ties)
+    sample = x.detach()[0, 100:356].float()
+    kth = sample.topk(50, dim=-1).values[:, -1:]
+    assert bool(((gx[0, 100:356] != 0) <= (sample >= kth)).all())
+    assert int(nz.max()) <= 50 + int((sample >= kth).sum(-1).max() - 50) + 8
+    assert bool((nz[~fin] == 0).all())
+    live = gx[:, :-1][fin].float()
+    assert bool((live.sum(-1).abs() <= 2e-2 * live.abs().sum(-1) + 1e-12).all())
+    # oracle on sampled rows
+    picks = [(0, 0), (0, 4095), (1, 17), (1, 8190), (1, 5000)]
+    rows = torch.stack([scaled[bi, si].float().cpu() for bi, si in picks])
+    tgt = torch.stack([ids[bi, si + 1] for bi, si in picks])
+    xo = rows.clone().requires_grad_(True)
+    want = OL.rows_logprob_sampled(xo, tgt, 50, 0.95)
+    got = torch.stack([lp[bi, si] for bi, si in picks]).detach().cpu()
+    wf = torch.isfinite(want)
+    assert torch.equal(torch.isfinite(got), wf)
+    assert (got[wf] - want.detach()[wf]).abs().max().item() <= 2e-3
+    upr = torch.stack([up[bi, si] for bi, si in picks]).cpu()
+    (torch.where(wf, want, torch.zeros_like(want)) * upr).sum().backward()
+    got_g = torch.stack([gx[bi, si].float().cpu() for bi, si in picks])
+    assert _grad_close_bf16(got_g, xo.grad)
+
+
+def test_config5_packed_row_full_shape():
+    """BASELINE config 5: one packed row of 131072 tokens (lengths U[2048, 32768]), V = 131072 bf16."""
+    v, total = 131072, 131072
+    g = torch.Generator().manual_seed(5005)
+    lens = []
+    while sum(lens) < total:
+        n = int(torch.randint(2048, 32769, (1,), generator=g))
+        lens.append(min(n, total - sum(lens)))
+    nseq, smax = len(lens), max(lens)
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+    ids = torch.zeros(nseq, smax, dtype=torch.int64)
+    for i, n in enumerate(lens):
+        ids[i, :n] = torch.randint(0, v, (n,), generator=g)
+    targets = OL.pack_input_ids(ids, cu, cu)
+    logits = _randn_bf16((1, total, v), 3.0, 5005)
+    x = logits.detach().requires_grad_(True)
+    lp = MU.from_parallel_logits_to_logprobs_packed_sequences(x, targets.to(DEV), cu.to(DEV), smax, 0, v, None)
+    assert lp.shape == (nseq, smax - 1) and bool(torch.isfinite(lp).all()) and bool((lp <= 0).all())
+    valid = (torch.arange(smax - 1)[None, :] < (torch.tensor(lens)[:, None] - 1)).to(DEV)
+    assert bool((lp[~valid] == 0).all())
+    # packed == the same sequence launched on its own
+    for i in (0, nseq - 1):
+        a, e = int(cu[i]), int(cu[i + 1])
+        own = MU.from_parallel_logits_to_logprobs(logits[:, a:e], ids[i : i + 1, : e - a].to(DEV), 0, v, None)
+        assert torch.equal(own[0], lp[i, : e - a - 1])
+    # sequence-level-normalised loss with KL 0.001, forward + backward
+    cur = lp.detach()
+    pad = lambda t: torch.cat([torch.zeros(nseq, 1, device=DEV), t], 1)  # noqa: E731
+    gn = torch.Generator(device=DEV).manual_seed(9)
+    tm = torch.cat([torch.zeros(nseq, 1, device=DEV), valid.float()], 1)
+    tm[:, 1:200] = 0
+    data = {"token_mask": tm, "sample_mask": torch.ones(nseq, device=DEV),
+            "advantages": torch.randn(nseq, 1, generator=gn, device=DEV).expand(nseq, smax).contiguous(),
+            "prev_logprobs": pad(cur + 0.05 * torch.randn(nseq, smax - 1, generator=gn, device=DEV)),
+            "generation_logprobs": pad(cur + 0.05 * torch.randn(nseq, smax - 1, generator=gn, device=DEV)),
+            "reference_policy_logprobs": pad(cur + 0.05 * torch.randn(nseq, smax - 1, generator=gn, device=DEV))}
+    fn = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, reference_policy_kl_penalty=0.001))
+    gs = torch.tensor(float(nseq), device=DEV)
+    gt = (tm[:, 1:]).sum()
+    loss, metrics = fn(next_token_logprobs=lp, data=data, global_valid_seqs=gs, global_valid_toks=gt)
+    loss.backward()
+    want, wm = O.clipped_pg_loss(O.LossConfig(token_level_loss=False, reference_policy_kl_penalty=0.001), cur.cpu(),
+                                 {k: t.cpu() for k, t in data.items()}, gs.cpu(), gt.cpu())
+    assert abs(loss.item() - want.item()) <= 1e-4 * abs(want.item()) + 1e-7
+    gx = x.grad[0]
+    live_tok = torch.zeros(total, dtype=torch.bool, device=DEV)
+    for i, n in enumerate(lens):
+        live_tok[int(cu[i]) : int(cu[i]) + n - 1] = tm[i, 1:n] > 0
+    assert bool((gx[~live_tok] == 0).all())
+    rows = gx[live_tok][::97].float()
+    assert bool((rows.sum(-1).abs() <= 2e-2 * rows.abs().sum(-1) + 1e-12).all())
+    # oracle logprobs on sampled packed positions
+    picks = [0, int(cu[1]) - 2, int(cu[1]), total // 2, total - 2]
+    rows = torch.stack([logits[0, p].float().cpu() for p in picks])
+    seq_of = [int(torch.searchsorted(cu[1:], torch.tensor(p), right=True)) for p in picks]
+    tgt = torch.stack([ids[si, p - int(cu[si]) + 1] for p, si in zip(picks, seq_of)])
+    want_lp = OL.rows_logprob(rows, tgt)
+    got_lp = torch.stack([lp[si, p - int(cu[si])] for p, si in zip(picks, seq_of)]).detach().cpu()
+    assert (got_lp - want_lp).abs().max().item() <= 2e-3
