@@ -64,6 +64,14 @@ typedef struct nrl_rows {
  * logprob_out, lse_out: fp32 [n_outer * n_inner]; lse_out may be NULL (inference_only). */
 int nrl_logprob_fwd(const nrl_rows* rows, float* logprob_out, float* lse_out, void* stream);
 
+/* Forward-only logprobs in the shape a policy worker returns for prev_logprobs / reference_policy_logprobs.
+ * Replaces LogprobsPostProcessor.__call__ for right-padded batches at TP = CP = 1
+ * (nemo_rl/models/automodel/train.py:689-806: _compute_local_logprobs, the prepended zero column and the
+ * input_lengths mask): out[b, 0] = 0, out[b, i] = logprob(row i-1 -> target i-1) for 1 <= i < lengths[b],
+ * 0 for i >= lengths[b].  rows describes the n_inner = S-1 rows per sequence exactly as for nrl_logprob_fwd;
+ * lengths: int64 [n_outer] device; out: fp32 [n_outer, n_inner + 1].  Padding rows are never read. */
+int nrl_logprob_post_fwd(const nrl_rows* rows, const int64_t* lengths, float* out, void* stream);
+
 /* K2  dlogits = g * (onehot(target) - exp(x - lse)), written once in the logits' dtype.
  * Replaces DistributedLogprob.backward / ChunkedDistributedLogprob.backward (:167-207, 333-380).
  * grad: fp32 upstream gradient of the logprobs, element (o, i) at

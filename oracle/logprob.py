@@ -202,3 +202,27 @@ def mask_out_neg_inf_logprobs(logprobs, mask):
     positions that are masked out or hold +-inf become 0."""
     keep = mask * (~torch.isinf(logprobs)).float()
     return torch.where(keep.bool(), logprobs, 0.0)
+
+
+def logprobs_post_process(logits, input_ids, input_lengths, cu_seqlens=None, original_batch_size=None,
+                          original_seq_len=None, top_k=None, top_p: float = 1.0):
+    """``LogprobsPostProcessor.__call__`` without TP / CP (``models/automodel/train.py:689-806``):
+    fp32 log-softmax + gather of the next token (``_compute_local_logprobs`` ``:808-864``), a zero
+    prepended for the first token (``:759-762``), then either the per-sequence unpack of a packed row
+    (``:764-778``) or the right-padding mask from ``input_lengths`` (``:779-791``).  Pinned by the
+    textbook identity it is written in (``log_softmax`` + ``gather``) and by brute force on tiny
+    inputs in ``tests/test_oracle_logprob.py``."""
+    nxt = input_ids[:, 1:]
+    x = logits[:, : nxt.shape[1]].to(torch.float32)
+    if top_k is not None or top_p < 1.0:
+        x, _ = sampling.apply_top_k_top_p(x, top_k, top_p)
+    lp = torch.log_softmax(x, dim=-1).gather(-1, nxt.unsqueeze(-1)).squeeze(-1)
+    lp = torch.cat([torch.zeros_like(lp[:, :1]), lp], dim=1)
+    if cu_seqlens is not None:
+        out = torch.zeros(original_batch_size, original_seq_len, dtype=lp.dtype)
+        for i in range(original_batch_size):
+            start, end = int(cu_seqlens[i]) + 1, int(cu_seqlens[i + 1])
+            out[i, 1 : int(input_lengths[i])] = lp[0, start:end]
+        return out
+    mask = torch.arange(lp.shape[1])[None, :] < torch.as_tensor(input_lengths).reshape(-1, 1)
+    return lp * mask

@@ -68,6 +68,7 @@ SIGNATURES = {
     "nrl_version": (C.c_int, []),
     "nrl_last_error": (C.c_char_p, []),
     "nrl_logprob_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P]),
+    "nrl_logprob_post_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P]),
     "nrl_logprob_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _I64, _I64, _P, _I64, _I64, _I64, _P]),
     "nrl_logprob_packed_fwd": (C.c_int, [_P, _I32, _I64, _I64, _I64, _P, _I32, _P, _I64, _I64, _I64, _I64, _F, _I32, _P, _P, _P]),
     "nrl_logprob_packed_bwd": (C.c_int, [_P, _I32, _I64, _I64, _I64, _P, _I32, _P, _I64, _I64, _I64, _I64, _F, _I32, _P, _P, _P, _I64, _P]),

@@ -2,7 +2,8 @@
 
 ``install()`` either registers ``nemo_rl.distributed.model_utils``, ``nemo_rl.algorithms.loss`` (and
 its sub-modules), ``nemo_rl.algorithms.loss_functions``, ``nemo_rl.algorithms.utils``,
-``nemo_rl.algorithms.logits_sampling_utils`` and ``nemo_rl.algorithms.advantage_estimator`` as
+``nemo_rl.algorithms.logits_sampling_utils``, ``nemo_rl.algorithms.advantage_estimator`` and
+``nemo_rl.models.automodel.train`` (its ``LogprobsPostProcessor``) as
 aliases of the ``rl_amd`` modules (when NeMo-RL is not importable), or replaces the hot-path
 attributes of an existing NeMo-RL install in place.
 """
@@ -24,6 +25,7 @@ _ALIASES = {
     "nemo_rl.algorithms.loss.utils": "rl_amd.algorithms.loss.utils",
     "nemo_rl.algorithms.loss.wrapper": "rl_amd.algorithms.loss.wrapper",
     "nemo_rl.algorithms.loss_functions": "rl_amd.algorithms.loss_functions",
+    "nemo_rl.models.automodel.train": "rl_amd.models.automodel.train",
 }
 
 # attributes replaced on a real NeMo-RL install (module -> names)
@@ -38,6 +40,7 @@ _PATCHED = {
     "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],
     "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
+    "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }
 
@@ -61,7 +64,7 @@ def install(force_alias: bool = False) -> str:
             for name in names:
                 setattr(dst, name, getattr(src, name))
         return "patched"
-    for parent in ("nemo_rl", "nemo_rl.distributed", "nemo_rl.algorithms"):
+    for parent in ("nemo_rl", "nemo_rl.distributed", "nemo_rl.algorithms", "nemo_rl.models", "nemo_rl.models.automodel"):
         if parent not in sys.modules:
             pkg = types.ModuleType(parent)
             pkg.__path__ = []  # a package, so sub-module imports resolve through sys.modules

@@ -183,6 +183,33 @@ __global__ __launch_bounds__(kBlock) void logprob_fwd_kernel(RowArgs a, float* _
     }
 }
 
+// Forward-only logprobs in the [n_outer, n_inner + 1] shape handed to the driver: column 0 is zero, column i
+// is the logprob of row i - 1, and everything at or past the sequence's length is zero; rows that only
+// produce zeros are never read.
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kBlock) void logprob_post_fwd_kernel(RowArgs a, const int64_t* __restrict__ lengths,
+                                                                  float* __restrict__ out) {
+    __shared__ Lse smem[kWaves];
+    const int64_t r = blockIdx.x, cols = a.n_inner + 1;
+    const int64_t o = r / cols, c = r - o * cols;
+    if (c == 0 || c >= lengths[o]) {
+        if (threadIdx.x == 0) out[r] = 0.f;
+        return;
+    }
+    const int64_t i = c - 1;
+    const char* row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+    const Lse t = row_online_lse<DT, TEMP>(row, a.vocab, a.tparam, smem);
+    if (threadIdx.x == 0) {
+        const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
+        float lp = 0.f;
+        if (tg >= a.vstart && tg < a.vend) {
+            const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(row, tg - a.vstart), a.tparam);
+            lp = (xt - t.m) - logf(t.s);
+        }
+        out[r] = lp;
+    }
+}
+
 struct GradArgs {
     const float* lse;
     const float* grad;
@@ -379,6 +406,20 @@ extern "C" int nrl_logprob_fwd(const nrl_rows* rows, float* logprob_out, float* 
     hipStream_t s = static_cast<hipStream_t>(stream);
     NRL_DISPATCH(rows->dtype, tc, logprob_fwd_kernel<DT, TEMP><<<dim3((unsigned)n), dim3(kBlock), 0, s>>>(a, logprob_out, lse_out));
     return check_launch("logprob_fwd");
+}
+
+extern "C" int nrl_logprob_post_fwd(const nrl_rows* rows, const int64_t* lengths, float* out, void* stream) {
+    if (int e = check_rows(rows)) return e;
+    const int64_t n = rows->n_outer * (rows->n_inner + 1);
+    if (rows->n_outer == 0) return NRL_OK;
+    if (!lengths || !out) return fail(NRL_E_INVALID, "lengths or out is NULL");
+    if (n >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 positions in one launch");
+    float tparam;
+    const int tc = temp_code(rows->temperature, rows->temp_mode, &tparam);
+    const RowArgs a = make_row_args(rows, tparam);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(rows->dtype, tc, logprob_post_fwd_kernel<DT, TEMP><<<dim3((unsigned)n), dim3(kBlock), 0, s>>>(a, lengths, out));
+    return check_launch("logprob_post_fwd");
 }
 
 extern "C" int nrl_logprob_bwd(const nrl_rows* rows, const float* lse, const float* grad, int64_t grad_stride_outer,

@@ -1,0 +1,94 @@
+"""``LogprobsPostProcessor`` (``nemo_rl/models/automodel/train.py:655-864``) on the HIP kernels.
+
+The policy worker runs this forward-only pass twice per step (``prev_logprobs`` and
+``reference_policy_logprobs``) on the same logits shapes as training.  Here one launch emits the
+``[B, S]`` result directly: the logprob of every next token, the zero column in front and the
+zeros from ``input_lengths`` on, without reading the logits of padding positions and without the
+fp32 ``[B, S, V]`` log-softmax the reference materialises.  One GPU: ``cp_size`` must be 1 and the
+logits a plain tensor (no DTensor / TP mesh).
+"""
+
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+
+from .. import _need_single_gpu
+from ... import ops  # noqa: F401  (registers torch.ops.rl_amd)
+from ..._lib import NRL_TEMP_RCP
+from ...algorithms.logits_sampling_utils import TrainingSamplingParams, need_top_k_or_top_p_filtering
+from ...algorithms.loss.utils import mask_out_neg_inf_logprobs
+from ...distributed import model_utils as MU
+
+
+class LogprobsPostProcessor:
+    """Same constructor and call signature as the reference class."""
+
+    def __init__(
+        self,
+        cfg: Any,
+        device_mesh: Any,
+        cp_mesh: Any,
+        tp_mesh: Any,
+        cp_size: int,
+        enable_seq_packing: bool = False,
+        sampling_params: Optional[TrainingSamplingParams] = None,
+    ):
+        self.cfg = cfg
+        self.device_mesh = device_mesh
+        self.cp_mesh = cp_mesh
+        self.tp_mesh = tp_mesh
+        self.cp_size = cp_size
+        self.enable_seq_packing = enable_seq_packing
+        self.sampling_params = sampling_params
+        self.logprob_chunk_size = cfg.get("logprob_chunk_size", None) if hasattr(cfg, "get") else None
+        _need_single_gpu(cp_size, "LogprobsPostProcessor")
+
+    def __call__(
+        self,
+        logits: torch.Tensor,
+        data_dict: Any,
+        processed_inputs: Any,
+        original_batch_size: int,
+        original_seq_len: int,
+        sequence_dim: int = 1,
+    ) -> torch.Tensor:
+        """``[batch, seq]`` fp32 token logprobs (``train.py:689-806``)."""
+        if type(logits).__name__ == "DTensor":
+            raise NotImplementedError("LogprobsPostProcessor: vocabulary-parallel (DTensor) logits need more than one GPU")
+        seq_len = processed_inputs.seq_len
+        input_ids = processed_inputs.input_ids.to(logits.device)
+        filtering = need_top_k_or_top_p_filtering(self.sampling_params)
+        with torch.no_grad():
+            if self.enable_seq_packing:
+                token_logprobs = self._unpack(logits, input_ids, processed_inputs, data_dict, original_batch_size,
+                                              original_seq_len, filtering)
+            elif filtering:
+                lp = MU.from_parallel_logits_to_logprobs(logits, input_ids, 0, logits.shape[-1], None, inference_only=True,
+                                                         sampling_params=self.sampling_params)
+                token_logprobs = torch.cat([torch.zeros_like(lp[:, :1]), lp], dim=1)
+                lengths = torch.as_tensor(data_dict["input_lengths"], device=lp.device).reshape(-1, 1)
+                token_logprobs = token_logprobs * (torch.arange(seq_len, device=lp.device)[None, :] < lengths)
+            else:
+                lengths = torch.as_tensor(data_dict["input_lengths"]).to(device=logits.device, dtype=torch.int64).contiguous()
+                x = logits if logits.stride(-1) == 1 else logits.contiguous()
+                token_logprobs = torch.ops.rl_amd.logprob_post_fwd(
+                    x, input_ids[:, 1:], lengths, input_ids.shape[1] - 1, 0, x.shape[-1], 1.0, NRL_TEMP_RCP)
+        if filtering:  # ``train.py:799-804``
+            mask = data_dict["token_mask"] * data_dict["sample_mask"].unsqueeze(-1)
+            token_logprobs = mask_out_neg_inf_logprobs(token_logprobs, mask.to(token_logprobs.device), "prev_logprobs")
+        return token_logprobs
+
+    def _unpack(self, logits, input_ids, processed_inputs, data_dict, batch, seq_len, filtering):
+        """Packed ``[1, T, V]`` logits -> ``[batch, seq_len]`` (``train.py:764-778``): sequence ``i`` occupies
+        ``cu_seqlens[i] .. cu_seqlens[i+1]``, its first token gets 0 and so does everything past its length."""
+        cu = processed_inputs.flash_attn_kwargs.cu_seqlens_q
+        cu = torch.as_tensor(cu).to(device=logits.device, dtype=torch.int32)
+        lengths = torch.as_tensor(data_dict["input_lengths"]).to(cu.device)
+        if cu.numel() != batch + 1 or not bool(((cu[1:] - cu[:-1]) == lengths.to(cu.dtype)).all()):
+            raise ValueError("cu_seqlens_q must delimit exactly the input_lengths of the microbatch")
+        lp = MU.from_parallel_logits_to_logprobs_packed_sequences(
+            logits, input_ids.reshape(-1), cu, seq_len, 0, logits.shape[-1], None, inference_only=True,
+            sampling_params=self.sampling_params if filtering else None)
+        return torch.cat([torch.zeros_like(lp[:, :1]), lp], dim=1)

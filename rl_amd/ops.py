@@ -136,7 +136,29 @@ def _logprob_bwd_inplace(logits, targets, lse, grad, n_inner, vocab_start, vocab
     _logprob_bwd(logits, targets, lse, grad, n_inner, vocab_start, vocab_end, temperature, temp_mode, in_place=True)
 
 
-for _name, _fn in (("logprob_fwd", _logprob_fwd), ("logprob_bwd", _logprob_bwd), ("logprob_bwd_", _logprob_bwd_inplace)):
+_LIB.define(
+    "logprob_post_fwd(Tensor logits, Tensor targets, Tensor lengths, int n_inner, int vocab_start, int vocab_end, "
+    "float temperature, int temp_mode) -> Tensor"
+)
+
+
+def _logprob_post_fwd(logits, targets, lengths, n_inner, vocab_start, vocab_end, temperature, temp_mode):
+    """[B, n_inner + 1] forward-only logprobs: zero column in front, zeros from each sequence's length on."""
+    _need_gpu(logits, targets, lengths)
+    rows = _rows(logits, targets, n_inner, vocab_start, vocab_end, temperature, temp_mode)
+    b = logits.shape[0]
+    if lengths.dtype != torch.int64 or tuple(lengths.shape) != (b,) or not lengths.is_contiguous():
+        raise ValueError("lengths must be a contiguous int64 [B] tensor")
+    with torch.cuda.device(logits.device):
+        out = torch.empty((b, n_inner + 1), dtype=torch.float32, device=logits.device)
+        with _timed("logprob_post_fwd"):
+            code = _lib.load().nrl_logprob_post_fwd(C.byref(rows), _ptr(lengths), _ptr(out), _stream())
+    _lib.check(code, "nrl_logprob_post_fwd")
+    return out
+
+
+for _name, _fn in (("logprob_fwd", _logprob_fwd), ("logprob_bwd", _logprob_bwd), ("logprob_bwd_", _logprob_bwd_inplace),
+                   ("logprob_post_fwd", _logprob_post_fwd)):
     _LIB.impl(_name, _fn, "CUDA")
     _LIB.impl(_name, _fn, "CPU")  # raises: there is no CPU path
 

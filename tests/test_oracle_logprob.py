@@ -203,3 +203,28 @@ def test_lmhead_equals_unfused_and_autograd():
     d_h, d_w = H.hidden_to_logprobs_backward(hid, w, rolled, g, chunk_size=4)
     torch.testing.assert_close(d_h, hid_g.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(d_w, w_g.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_logprobs_post_process_brute_force():
+    """The forward-only post-processor restatement against plain Python loops on a tiny input."""
+    g = torch.Generator().manual_seed(3)
+    b, s, v = 3, 6, 5
+    logits = torch.randn(b, s, v, generator=g)
+    ids = torch.randint(0, v, (b, s), generator=g)
+    lengths = [6, 3, 1]
+    got = L.logprobs_post_process(logits, ids, torch.tensor(lengths))
+    for i in range(b):
+        for t in range(s):
+            if t == 0 or t >= lengths[i]:
+                assert got[i, t] == 0
+            else:
+                row = logits[i, t - 1].tolist()
+                lse = math.log(sum(math.exp(x) for x in row))
+                assert abs(got[i, t].item() - (row[int(ids[i, t])] - lse)) < 1e-5
+    # packed: the same sequences laid end to end give the same rows
+    cu = torch.tensor([0, 6, 9, 10], dtype=torch.int32)
+    packed_logits = torch.cat([logits[i, : lengths[i]] for i in range(b)])[None]
+    packed_ids = torch.cat([ids[i, : lengths[i]] for i in range(b)])[None]
+    unpacked = L.logprobs_post_process(packed_logits, packed_ids, torch.tensor(lengths), cu_seqlens=cu,
+                                        original_batch_size=b, original_seq_len=s)
+    assert torch.allclose(unpacked, got, atol=1e-6)
