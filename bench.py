@@ -36,6 +36,9 @@ WORKLOADS = {
                desc="BASELINE config 2: 16 prompts x 8 = 128 seq x 4096 tok, V=151936 bf16, fwd+bwd to dlogits"),
     "c3": dict(seqs=16, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=0.0, spike_p=0.0, hidden=4096,
                desc="BASELINE config 3: fused lm_head + logprob, hidden [65536,4096] bf16, W [151936,4096] bf16, fwd+bwd (dH, dW)"),
+    "c4": dict(seqs=64, seq_len=8192, vocab=151936, dtype="bf16", mb_seqs=8, std=3.0, spike_p=0.0, temperature=0.7,
+               top_k=50, top_p=0.95,
+               desc="BASELINE config 4: 64 seq x 8192 tok, V=151936 bf16, T=0.7, top_k=50, top_p=0.95, DAPO clip-higher, no KL"),
     "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
                desc="BASELINE config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
 }
@@ -159,6 +162,88 @@ def cpu_baseline(torch, w, seconds):
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
 
 
+def bench_topk(args, torch, w):
+    """Config 4: top-k / top-p filtered training logprobs -> DAPO loss -> dlogits (K3 forward + backward)."""
+    from rl_amd import ops
+    from rl_amd.algorithms.logits_sampling_utils import TrainingSamplingParams
+    from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn, prepare_loss_input
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.seqs:
+        w["seqs"] = args.seqs
+        w["mb_seqs"] = min(w["mb_seqs"], args.seqs)
+    n_mb = (w["seqs"] + w["mb_seqs"] - 1) // w["mb_seqs"]
+    mb_bytes = w["mb_seqs"] * w["seq_len"] * w["vocab"] * 2
+    free, _ = torch.cuda.mem_get_info()
+    n_buf = max(1, min(n_mb, int((free * 0.9 - mb_bytes * 1.5) // mb_bytes)))
+    params = TrainingSamplingParams(top_k=w["top_k"], top_p=w["top_p"])
+    fn = ClippedPGLossFn(ClippedPGLossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0))
+    mbs = []
+    for i in range(n_buf):
+        m = make_microbatch(torch, dict(w, spike_p=0.0), w["mb_seqs"], 4004 + i, dev)
+        # logits.div_(T) in bf16, as the worker does before the loss; targets mostly the argmax so that they survive the filter
+        m["logits"].mul_(1.0 / w["temperature"])
+        top = torch.stack([m["logits"][b].float().argmax(-1) for b in range(w["mb_seqs"])])
+        keep = torch.rand(top[:, :-1].shape, device=dev) < 0.8
+        m["data"]["input_ids"][:, 1:] = torch.where(keep, top[:, :-1], m["data"]["input_ids"][:, 1:])
+        with torch.no_grad():
+            from rl_amd.distributed.model_utils import get_next_token_logprobs_from_logits
+            cur = get_next_token_logprobs_from_logits(m["data"]["input_ids"], m["logits"], sampling_params=params)
+        cur = torch.cat([torch.zeros((w["mb_seqs"], 1), device=dev), torch.nan_to_num(cur, neginf=0.0)], dim=1)
+        for k in ("prev_logprobs", "generation_logprobs"):
+            m["data"][k] = cur + 0.05 * torch.randn_like(cur)
+        m["data"].pop("reference_policy_logprobs", None)
+        mbs.append(m)
+    tot_seqs = torch.tensor(float(w["seqs"]), device=dev)
+    tot_toks = (sum(m["data"]["token_mask"][:, 1:].sum() for m in mbs) * (n_mb / n_buf)).float()
+
+    def step():
+        for i in range(n_mb):
+            m = mbs[i % n_buf]
+            logits = m["logits"].requires_grad_(True)
+            loss_input, data = prepare_loss_input(logits, m["data"], fn, sampling_params=params)
+            loss, _ = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+            (d,) = torch.autograd.grad(loss, logits)
+            del d, loss, loss_input
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = EventTimer(torch)
+    ops.KERNEL_TIMER = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    k = timer.summary()
+    nan = dict(avg_ms=float("nan"))
+    fwd, bwd = k.get("topk_topp_fwd", nan), k.get("topk_topp_bwd", nan)
+    rows = w["mb_seqs"] * w["seq_len"]
+    row_bytes = w["vocab"] * 2
+    tokens = w["seqs"] * w["seq_len"]
+    fwd_gbs = row_bytes * w["mb_seqs"] * (w["seq_len"] - 1) / (fwd["avg_ms"] * 1e-3) / 1e9
+    bwd_gbs = 2 * row_bytes * rows / (bwd["avg_ms"] * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "top-k/top-p filtered logprob + DAPO loss fwd/bwd tokens/s at V=151936; % of HBM peak",
+        "value": tokens * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
+                   "microbatches": n_mb, "resident_logit_buffers": n_buf},
+        "algorithmic_bytes_per_token": 3 * row_bytes,
+        "hbm_frac_end_to_end": 3 * row_bytes * tokens * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "topk_topp_stream_kernel (backward)", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": bwd["avg_ms"],
+                     "algorithmic_bytes_per_launch": 2 * row_bytes * rows},
+        "roofline_fwd": {"bound": "hbm", "kernel": "topk_topp_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
+        "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
+    }))
+
+
 def bench_lmhead(args, torch, w):
     """Config 3: hidden states -> logprobs -> loss -> (dH, dW) through the fused MFMA path."""
     from rl_amd import ops
@@ -238,6 +323,8 @@ def main():
     w = dict(WORKLOADS[args.workload])
     if args.workload == "c3":
         return bench_lmhead(args, torch, w)
+    if args.workload == "c4":
+        return bench_topk(args, torch, w)
     if args.seqs:
         w["seqs"] = args.seqs
         w["mb_seqs"] = min(w["mb_seqs"], args.seqs)

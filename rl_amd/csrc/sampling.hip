@@ -30,7 +30,9 @@ constexpr int kSelBlock = 512;
 constexpr int kSelWaves = kSelBlock / kWave;
 constexpr int kSub = 4;                      // chunk maxima per thread
 constexpr int kChunks = kSelBlock * kSub;    // 2048
-constexpr int kCap = 4096;                   // candidate capacity (LDS)
+constexpr int kCap = 4096;                   // candidate capacity (LDS); rows under a small top-k use kCapSmall
+constexpr int kCapSmall = 2048;              // ... which lets four workgroups share a compute unit instead of three
+constexpr int kSmallTopK = 512;
 
 struct Lse2 {
     float m, s;
@@ -58,15 +60,12 @@ template <int DT> __device__ __forceinline__ int64_t sel_row_head(const void* ro
     return h < vocab ? h : vocab;
 }
 
-struct SelShared {
-    uint32_t maxima[kChunks];
-    unsigned long long cand[kCap];
-    float expv[kCap];
-    uint32_t hist[256];
+template <int CAP> struct SelShared {
+    unsigned long long cand[CAP];
+    float expv[CAP];
+    int sel_cnt[2][kSelWaves * 3];
     Lse2 lse_w[kSelWaves];
     int count;
-    uint32_t sel_prefix;
-    int sel_k;
     float bound;
     float thr;
     int tie;
@@ -74,40 +73,79 @@ struct SelShared {
     int n_keep;
 };
 
-// k-th largest (1-based) of the kChunks keys in sh.maxima; every thread returns it
-__device__ __forceinline__ uint32_t select_kth_largest(SelShared& sh, int k) {
-    const int tid = threadIdx.x;
-    if (tid == 0) { sh.sel_prefix = 0u; sh.sel_k = k; }
-    uint32_t mask = 0u;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        if (tid < 256) sh.hist[tid] = 0u;
-        __syncthreads();
-        const uint32_t prefix = sh.sel_prefix;
-        for (int i = tid; i < kChunks; i += kSelBlock) {
-            const uint32_t key = sh.maxima[i];
-            if ((key & mask) == prefix) atomicAdd(&sh.hist[(key >> shift) & 255u], 1u);
+// k-th largest (1-based) of the workgroup's kChunks keys (kSub per thread, in registers); every thread
+// returns it.  Two bits at a time from the top: the answer is the largest v with at least k keys >= v.  A
+// round costs 3 * kSub ballots per wave, three LDS words per wave and one barrier (the buffers alternate), with
+// no atomics -- chunk maxima share their high bits, so a histogram would serialise on one bin.
+template <int CAP>
+__device__ __forceinline__ uint32_t select_kth_largest(SelShared<CAP>& sh, const uint32_t (&keys)[kSub], int k) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    uint32_t v = 0u;
+    for (int bit = 30; bit >= 0; bit -= 2) {  // two bits per round: three trial values, one barrier
+        int cnt[3] = {0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            const uint32_t cand = v | (static_cast<uint32_t>(c + 1) << bit);
+#pragma unroll
+            for (int u = 0; u < kSub; ++u) cnt[c] += __popcll(__ballot(keys[u] >= cand));
         }
+        const int par = (bit >> 1) & 1;
+        if (lane < 3) sh.sel_cnt[par][wave * 3 + lane] = lane == 0 ? cnt[0] : lane == 1 ? cnt[1] : cnt[2];
         __syncthreads();
-        if (tid == 0) {
-            int need = sh.sel_k;
-            int b = 255;
-            for (; b > 0; --b) {
-                const int c = static_cast<int>(sh.hist[b]);
-                if (c >= need) break;
-                need -= c;
-            }
-            sh.sel_prefix = prefix | (static_cast<uint32_t>(b) << shift);
-            sh.sel_k = need;
-        }
-        mask |= 0xffu << shift;
-        __syncthreads();
+        int tot[3] = {0, 0, 0};
+#pragma unroll
+        for (int w = 0; w < kSelWaves; ++w)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) tot[c] += sh.sel_cnt[par][w * 3 + c];
+        // counts fall as the trial value rises: take the largest trial that still has k keys at or above it
+        const uint32_t step = tot[2] >= k ? 3u : tot[1] >= k ? 2u : tot[0] >= k ? 1u : 0u;
+        v |= step << bit;
     }
-    return sh.sel_prefix;
+    return v;
+}
+
+// sum of e[n-1], e[n-2], ..., e[0] in exactly that order; called by every lane of one wave, which all
+// return the same value (64 elements per LDS read, then lane-to-scalar moves instead of one dependent
+// LDS round trip per element)
+__device__ __forceinline__ float wave_seq_sum_desc(const float* e, int n) {
+    const int lane = threadIdx.x & (kWave - 1);
+    float s = 0.f;
+    for (int blk = (n - 1) / kWave; blk >= 0; --blk) {
+        const int idx = blk * kWave + lane;
+        const float v = idx < n ? e[idx] : 0.f;
+        const int top = n - 1 - blk * kWave < kWave - 1 ? n - 1 - blk * kWave : kWave - 1;
+        for (int i = top; i >= 0; --i) s += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), i));
+    }
+    return s;
 }
 
 // descending bitonic sort of sh.cand[0 .. n_pad)
-__device__ __forceinline__ void sort_candidates_desc(SelShared& sh, int n_pad) {
+template <int CAP> __device__ __forceinline__ void sort_candidates_desc(SelShared<CAP>& sh, int n_pad) {
     const int tid = threadIdx.x;
+    if (n_pad <= 2 * kWave) {
+        // short lists (the usual case under top-k) are sorted by one wave alone: its LDS operations execute
+        // in order, so the compare-exchange steps need no workgroup barrier
+        __syncthreads();
+        if (tid < kWave) {
+            for (int size = 2; size <= n_pad; size <<= 1) {
+                for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                    const int i = tid;
+                    if (i < (n_pad >> 1)) {
+                        const int lo = ((i / stride) * (stride << 1)) + (i % stride);
+                        const int hi = lo + stride;
+                        const bool desc = ((lo & size) == 0);
+                        const unsigned long long a = sh.cand[lo], b = sh.cand[hi];
+                        if ((a < b) == desc) { sh.cand[lo] = b; sh.cand[hi] = a; }
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                }
+            }
+        }
+        __syncthreads();
+        return;
+    }
     for (int size = 2; size <= n_pad; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             __syncthreads();
@@ -140,9 +178,9 @@ struct SelArgs {
     int32_t* overflow;   // device flag
 };
 
-template <int DT, int TEMP, bool FULL_LSE>
+template <int DT, int TEMP, bool FULL_LSE, int CAP>
 __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
-    __shared__ SelShared sh;
+    __shared__ SelShared<CAP> sh;
     constexpr int EPV = Row<DT>::EPV;
     const int tid = threadIdx.x;
     const int64_t r = blockIdx.x;
@@ -165,7 +203,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     for (; base + kSub * kSelBlock <= nvec; base += kSub * kSelBlock) {
         u32x4 q[kSub];
 #pragma unroll
-        for (int u = 0; u < kSub; ++u) q[u] = xv[base + u * kSelBlock + tid];
+        for (int u = 0; u < kSub; ++u) q[u] = __builtin_nontemporal_load(xv + base + u * kSelBlock + tid);
         float v[kSub * EPV];
 #pragma unroll
         for (int u = 0; u < kSub; ++u) {
@@ -219,8 +257,9 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             }
         }
     }
+    uint32_t mx_key[kSub];
 #pragma unroll
-    for (int u = 0; u < kSub; ++u) sh.maxima[u * kSelBlock + tid] = order_key(mx[u]);
+    for (int u = 0; u < kSub; ++u) mx_key[u] = order_key(mx[u]);
     float lse_full = 0.f;
     if (FULL_LSE) {
 #pragma unroll
@@ -246,7 +285,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     const bool use_p = a.top_p < 1.0f;
     uint32_t bound_key = 0u;
     if (use_k) {
-        if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, a.top_k);
+        if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, mx_key, a.top_k);
     } else {
         // top-p alone: elements with probability <= (1-p)/V sum to at most 1-p and are the smallest
         const float b = lse_full + logf((1.0f - a.top_p) / static_cast<float>(vocab));
@@ -254,34 +293,47 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     }
 
     // ---- pass 2: collect candidates ----
-    for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
-        float t[EPV];
-        Row<DT>::decode(xv[vi], t);
-#pragma unroll
-        for (int k = 0; k < EPV; ++k) {
-            const uint32_t key = order_key(scale_logit<DT, TEMP>(t[k], a.tparam));
-            if (key >= bound_key) {
-                const int pos = atomicAdd(&sh.count, 1);
-                if (pos < kCap)
-                    sh.cand[pos] = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(head + vi * EPV + k);
-            }
-        }
-    }
-    for (int w = 0; w < 2; ++w) {
-        const int64_t e = w == 0 ? (tid < head ? tid : -1) : (tail0 + tid < vocab ? tail0 + tid : -1);
-        if (e < 0) continue;
-        const uint32_t key = order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, e), a.tparam));
+    // Only the chunks whose maximum reaches the bound can hold candidates; a thread re-reads just those
+    // of its own chunks (with top-k that is about k of the 2048 chunks, a few percent of the row).
+    auto push = [&](uint32_t key, int64_t index) {
         if (key >= bound_key) {
             const int pos = atomicAdd(&sh.count, 1);
-            if (pos < kCap) sh.cand[pos] = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(e);
+            if (pos < CAP) sh.cand[pos] = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(index);
+        }
+    };
+    auto push_raw = [&](const u32x4& q, int64_t vi) {
+        float t[EPV];
+        Row<DT>::decode(q, t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) push(order_key(scale_logit<DT, TEMP>(t[k], a.tparam)), head + vi * EPV + k);
+    };
+    constexpr int kBatch = 8;  // loads of one chunk in flight together (a chunk of a 152k row is 9-10 vectors)
+    const int64_t n_full = nvec / (kSub * kSelBlock);  // vectors every chunk got in the main loop of pass 1
+#pragma unroll
+    for (int u = 0; u < kSub; ++u) {
+        if (mx_key[u] < bound_key) continue;
+        for (int64_t b0 = 0; b0 < n_full; b0 += kBatch) {
+            u32x4 q[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                if (b0 + j < n_full) q[j] = xv[(b0 + j) * (kSub * kSelBlock) + u * kSelBlock + tid];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                if (b0 + j < n_full) push_raw(q[j], (b0 + j) * (kSub * kSelBlock) + u * kSelBlock + tid);
+        }
+        if (u == 0) {  // chunk 0 also took the ragged end of the row and the unaligned head / tail elements
+            for (int64_t vi = base + tid; vi < nvec; vi += kSelBlock) push_raw(xv[vi], vi);
+            if (tid < head) push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam)), tid);
+            if (tail0 + tid < vocab)
+                push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam)), tail0 + tid);
         }
     }
     __syncthreads();
     const int n = sh.count;
-    if (n > kCap || n == 0) {
+    if (n > CAP || n == 0) {
         // the kept set does not fit the candidate list (or the row holds no finite value)
         if (tid == 0) {
-            if (n > kCap) atomicExch(a.overflow, 1);
+            if (n > CAP) atomicExch(a.overflow, 1);
             a.thr[r] = __builtin_nanf("");
             a.tie[r] = 0;
             a.lse_kept[r] = __builtin_nanf("");
@@ -310,11 +362,10 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     for (int i = tid; i < n_k; i += kSelBlock)
         sh.expv[i] = expf(key_value(static_cast<uint32_t>(sh.cand[i] >> 32)) - m);
     __syncthreads();
-    if (tid == 0) {
+    if (tid < kWave) {  // one wave; every lane computes the same scalars, lane 0 writes them
         int n_keep = n_k;
         if (use_p) {
-            float s_k = 0.f;
-            for (int i = n_k - 1; i >= 0; --i) s_k += sh.expv[i];
+            float s_k = wave_seq_sum_desc(sh.expv, n_k);
             // ascending cumulative probability, smallest kept value first; keep while it exceeds 1 - p
             const float cut = 1.0f - a.top_p;
             float cum = 0.f;
@@ -326,36 +377,41 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                 s_k = s_full;
             }
             n_keep = 1;
-            for (int i = n_k - 1; i >= 1; --i) {
-                cum += sh.expv[i] / s_k;
-                if (cum > cut) { n_keep = i + 1; break; }
+            bool done = false;
+            for (int blk = (n_k - 1) / kWave; blk >= 0 && !done; --blk) {
+                const int idx = blk * kWave + tid;
+                const float v = idx < n_k ? sh.expv[idx] : 0.f;
+                const int top = n_k - 1 - blk * kWave < kWave - 1 ? n_k - 1 - blk * kWave : kWave - 1;
+                for (int i = top; i >= 0; --i) {
+                    if (blk * kWave + i < 1) break;  // index 0 is always kept
+                    cum += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), i)) / s_k;
+                    if (cum > cut) { n_keep = blk * kWave + i + 1; done = true; break; }
+                }
             }
         }
-        float s = 0.f;
-        for (int i = n_keep - 1; i >= 0; --i) s += sh.expv[i];
+        const float s = wave_seq_sum_desc(sh.expv, n_keep);
         const unsigned long long last = sh.cand[n_keep - 1];
         const uint32_t last_key = static_cast<uint32_t>(last >> 32);
         int tie = 0;
         if (n_keep < n && static_cast<uint32_t>(sh.cand[n_keep] >> 32) == last_key) tie = static_cast<int>(last & 0xffffffffu);
-        sh.thr = key_value(last_key);
-        sh.tie = tie;
-        sh.lse_kept = m + logf(s);
-        sh.n_keep = n_keep;
-        a.thr[r] = sh.thr;
-        a.tie[r] = tie;
-        a.lse_kept[r] = sh.lse_kept;
-        if (a.lse_full) a.lse_full[r] = lse_full;
-        if (a.targets && a.logprob) {
-            const int64_t tg = a.targets[o * a.ts_outer + i_in * a.ts_inner];
-            float lp = -INFINITY, lpf = 0.f;
-            if (tg >= 0 && tg < vocab) {
-                const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(row, tg), a.tparam);
-                const bool kept = xt > sh.thr || (xt == sh.thr && tg >= tie);
-                if (kept) lp = xt - sh.lse_kept;
-                lpf = xt - lse_full;
+        const float thr = key_value(last_key), lse_kept = m + logf(s);
+        if (tid == 0) {
+            a.thr[r] = thr;
+            a.tie[r] = tie;
+            a.lse_kept[r] = lse_kept;
+            if (a.lse_full) a.lse_full[r] = lse_full;
+            if (a.targets && a.logprob) {
+                const int64_t tg = a.targets[o * a.ts_outer + i_in * a.ts_inner];
+                float lp = -INFINITY, lpf = 0.f;
+                if (tg >= 0 && tg < vocab) {
+                    const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(row, tg), a.tparam);
+                    const bool kept = xt > thr || (xt == thr && tg >= tie);
+                    if (kept) lp = xt - lse_kept;
+                    lpf = xt - lse_full;
+                }
+                a.logprob[r] = lp;
+                if (a.logprob_full) a.logprob_full[r] = lpf;
             }
-            a.logprob[r] = lp;
-            if (a.logprob_full) a.logprob_full[r] = lpf;
         }
     }
 }
@@ -505,10 +561,15 @@ extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, fl
     const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
     const bool full = !use_k || logprob_unfiltered_out != nullptr || lse_full_out != nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (full) {
-        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    const bool small = use_k && a.top_k <= kSmallTopK;
+    if (full && small) {
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true, kCapSmall><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    } else if (full) {
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true, kCap><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    } else if (small) {
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, false, kCapSmall><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
     } else {
-        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, false><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, false, kCap><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
     }
     return check_launch("topk_topp_logprob_fwd");
 }
