@@ -239,6 +239,21 @@ int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int64_t prompt
                            float* baseline_out, float* std_out, float* adv_out, int32_t* group_out,
                            void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Per-sequence multiplicative logprob error and the mask that drops sequences above a threshold.
+ * Replaces compute_and_apply_seq_logprob_error_masking (nemo_rl/algorithms/grpo.py:2513-2640):
+ * err[b] = sum_t exp(|gen - prev| * m) * m / max(sum_t m, 1) over t >= 1 with m = token_mask[b,t] * sample_mask[b]
+ * (0 for a sequence without unmasked tokens); with a threshold sample_mask_out[b] = (err[b] <= threshold) *
+ * sample_mask[b], otherwise a copy of sample_mask.
+ * All tensors fp32; prev / gen / token_mask [B, S] with their row strides; rewards [B] or NULL.
+ * record_out (fp32 [8]): max, mean, min error over sequences with unmasked tokens; the same three over the
+ * sequences that stay; number of newly masked sequences; fraction of those with reward == 1.
+ * workspace: B floats. */
+int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* gen, int64_t gen_stride,
+                          const float* token_mask, int64_t token_mask_stride, const float* sample_mask,
+                          const float* rewards, int64_t batch, int64_t seq_len, int32_t has_threshold,
+                          float threshold, float* seq_err_out, float* sample_mask_out, float* record_out,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * K6  Fused lm_head -> token logprob on the bf16 matrix cores (MFMA), never materialising the
  * [N, V] logits.  Replaces ChunkedDistributedHiddenStatesToLogprobs

@@ -34,6 +34,10 @@ Pinning status (what fixes each function besides its own text):
                            from the source text and checked against
                            independent float64 formulas only.
 * ``advantage.*``          pinned: golden vectors of the reference's unit tests.
+* ``advantage.seq_logprob_error_masking``  pinned by brute-force loops on tiny
+                           inputs (the reference's tests only mock it).
+* ``logprob.logprobs_post_process``  pinned: ``log_softmax`` + ``gather``
+                           identity and brute-force loops on tiny inputs.
 * ``lmhead.*``             PARITY UNPINNED against the reference (its only test
                            needs Megatron, two GPUs and a model download);
                            pinned here to ``logprob(hidden @ W.T)`` in fp32.

@@ -79,3 +79,38 @@ def clip_advantages(adv, low=None, high=None):
     if low is None and high is None:
         return adv
     return torch.clamp(adv, min=low, max=high)
+
+
+def seq_logprob_error_masking(prev_logprobs, generation_logprobs, token_mask, sample_mask, rewards, threshold):
+    """``compute_and_apply_seq_logprob_error_masking`` (``nemo_rl/algorithms/grpo.py:2513-2640``)
+    restated: returns ``(metrics dict, new sample_mask)``.  The reference's tests only mock this
+    function, so it is pinned by brute-force loops on tiny inputs (``tests/test_oracle_advantage.py``)."""
+    tm = token_mask[:, 1:].float()
+    sm = sample_mask.float()
+    lp_error = (generation_logprobs[:, 1:] - prev_logprobs[:, 1:]).abs()
+    mask = tm * sm.unsqueeze(-1)
+    denom = mask.sum(-1)
+    valid = denom > 0
+    err = torch.zeros_like(denom)
+    stats = [0.0, 0.0, 0.0]
+    if valid.any():
+        num = (torch.exp(lp_error * mask) * mask).sum(-1)
+        err[valid] = num[valid] / denom[valid].clamp(min=1)
+        v = err[valid]
+        stats = [v.max().item(), v.mean().item(), v.min().item()]
+    after = list(stats)
+    n_masked, pct, new_mask = 0, 0.0, sample_mask
+    if threshold is not None:
+        new_mask = (err <= threshold).float() * sm
+        diff = sm - new_mask
+        n_masked = int(diff.sum().item())
+        if n_masked > 0:
+            pct = int((rewards.view(-1)[diff.bool()] == 1).sum().item()) / n_masked
+        kept = new_mask.bool() & valid
+        after = [err[kept].max().item(), err[kept].mean().item(), err[kept].min().item()] if kept.sum() > 0 else [0.0, 0.0, 0.0]
+    keys = ["max_seq_mult_prob_error", "mean_seq_mult_prob_error", "min_seq_mult_prob_error",
+            "max_seq_mult_prob_error_after_mask", "mean_seq_mult_prob_error_after_mask", "min_seq_mult_prob_error_after_mask"]
+    out = dict(zip(keys, stats + after))
+    out["num_masked_seqs"] = n_masked
+    out["masked_correct_pct"] = pct
+    return out, new_mask

@@ -26,6 +26,7 @@ _ALIASES = {
     "nemo_rl.algorithms.loss.wrapper": "rl_amd.algorithms.loss.wrapper",
     "nemo_rl.algorithms.loss_functions": "rl_amd.algorithms.loss_functions",
     "nemo_rl.models.automodel.train": "rl_amd.models.automodel.train",
+    "nemo_rl.algorithms.grpo": "rl_amd.algorithms.grpo",
 }
 
 # attributes replaced on a real NeMo-RL install (module -> names)
@@ -41,6 +42,7 @@ _PATCHED = {
     "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
+    "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }
 

@@ -91,6 +91,86 @@ __global__ void group_stats_kernel(const int32_t* group, int64_t batch, const fl
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Per-sequence multiplicative logprob error between the generation engine and the policy, and the mask
+// that drops sequences above a threshold.  Launch 1: one workgroup per sequence.  Launch 2: one workgroup
+// reduces the sequences in a fixed order into an 8-float record.
+// ---------------------------------------------------------------------------------------------
+struct SeqErrArgs {
+    const float* prev;   // [B, S] row stride prev_stride; column 0 is skipped
+    const float* gen;
+    const float* token_mask;
+    const float* sample_mask;  // [B]
+    const float* rewards;      // [B] or NULL
+    int64_t batch, seq_len, prev_stride, gen_stride, tm_stride;
+    int has_threshold;
+    float threshold;
+    float* seq_err;          // [B]
+    float* valid;            // [B] 1 if the sequence has any unmasked token
+    float* sample_mask_out;  // [B] (= sample_mask when no threshold)
+    float* record;           // [8]
+};
+
+__global__ __launch_bounds__(kAdvBlock) void seq_err_rows_kernel(SeqErrArgs a) {
+    __shared__ float sm[kAdvWaves];
+    const int64_t b = blockIdx.x;
+    const float smv = a.sample_mask[b];
+    float num = 0.f, den = 0.f;
+    for (int64_t t = 1 + threadIdx.x; t < a.seq_len; t += kAdvBlock) {
+        const float m = a.token_mask[b * a.tm_stride + t] * smv;
+        const float e = fabsf(a.gen[b * a.gen_stride + t] - a.prev[b * a.prev_stride + t]);
+        num += expf(e * m) * m;
+        den += m;
+    }
+    num = block_sum<float, kAdvWaves>(num, sm);
+    den = block_sum<float, kAdvWaves>(den, sm);
+    if (threadIdx.x == 0) {
+        const bool valid = den > 0.f;
+        const float err = valid ? num / fmaxf(den, 1.f) : 0.f;
+        a.seq_err[b] = err;
+        a.valid[b] = valid ? 1.f : 0.f;
+        a.sample_mask_out[b] = a.has_threshold ? ((err <= a.threshold) ? 1.f : 0.f) * smv : smv;
+    }
+}
+
+__global__ __launch_bounds__(kAdvBlock) void seq_err_finish_kernel(SeqErrArgs a) {
+    __shared__ float sm[kAdvWaves];
+    float mx = -FLT_MAX, mn = FLT_MAX, sum = 0.f, cnt = 0.f;
+    float mx2 = -FLT_MAX, mn2 = FLT_MAX, sum2 = 0.f, cnt2 = 0.f, n_masked = 0.f, n_correct = 0.f;
+    for (int64_t b = threadIdx.x; b < a.batch; b += kAdvBlock) {
+        const float e = a.seq_err[b];
+        const bool valid = a.valid[b] != 0.f;
+        if (valid) { mx = fmaxf(mx, e); mn = fminf(mn, e); sum += e; cnt += 1.f; }
+        if (a.has_threshold) {
+            const float kept = a.sample_mask_out[b], diff = a.sample_mask[b] - kept;
+            n_masked += diff;
+            if (diff != 0.f && a.rewards && a.rewards[b] == 1.f) n_correct += 1.f;
+            if (kept != 0.f && valid) { mx2 = fmaxf(mx2, e); mn2 = fminf(mn2, e); sum2 += e; cnt2 += 1.f; }
+        }
+    }
+    mx = block_max<kAdvWaves>(mx, sm); mn = block_min<kAdvWaves>(mn, sm);
+    sum = block_sum<float, kAdvWaves>(sum, sm); cnt = block_sum<float, kAdvWaves>(cnt, sm);
+    mx2 = block_max<kAdvWaves>(mx2, sm); mn2 = block_min<kAdvWaves>(mn2, sm);
+    sum2 = block_sum<float, kAdvWaves>(sum2, sm); cnt2 = block_sum<float, kAdvWaves>(cnt2, sm);
+    n_masked = block_sum<float, kAdvWaves>(n_masked, sm); n_correct = block_sum<float, kAdvWaves>(n_correct, sm);
+    if (threadIdx.x == 0) {
+        float* r = a.record;
+        r[0] = cnt > 0.f ? mx : 0.f;
+        r[1] = cnt > 0.f ? sum / cnt : 0.f;
+        r[2] = cnt > 0.f ? mn : 0.f;
+        if (a.has_threshold) {
+            r[3] = cnt2 > 0.f ? mx2 : 0.f;
+            r[4] = cnt2 > 0.f ? sum2 / cnt2 : 0.f;
+            r[5] = cnt2 > 0.f ? mn2 : 0.f;
+        } else {
+            r[3] = r[0]; r[4] = r[1]; r[5] = r[2];
+        }
+        const int masked = static_cast<int>(n_masked);  // the reference truncates the float sum the same way
+        r[6] = static_cast<float>(masked);
+        r[7] = masked > 0 ? n_correct / static_cast<float>(masked) : 0.f;
+    }
+}
+
 }  // namespace nrl
 
 using namespace nrl;
@@ -120,4 +200,26 @@ extern "C" int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int
     group_stats_kernel<<<dim3((unsigned)((batch + 127) / 128)), dim3(128), 0, s>>>(
         group, batch, rewards, valid, std_rewards, leave_one_out, normalize, baseline_out, std_out, adv_out);
     return check_launch("group_baseline_std");
+}
+
+extern "C" int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* gen, int64_t gen_stride,
+                                     const float* token_mask, int64_t token_mask_stride, const float* sample_mask,
+                                     const float* rewards, int64_t batch, int64_t seq_len, int32_t has_threshold,
+                                     float threshold, float* seq_err_out, float* sample_mask_out, float* record_out,
+                                     void* workspace, int64_t workspace_bytes, void* stream) {
+    if (batch < 0 || seq_len < 0) return fail(NRL_E_INVALID, "bad shape");
+    if (!record_out) return fail(NRL_E_INVALID, "record_out is NULL");
+    if (batch > 0 && (!prev || !gen || !token_mask || !sample_mask || !seq_err_out || !sample_mask_out || !workspace))
+        return fail(NRL_E_INVALID, "null argument");
+    if (workspace_bytes < batch * static_cast<int64_t>(sizeof(float))) return fail(NRL_E_WORKSPACE, "workspace too small");
+    if (batch >= (1ll << 31)) return fail(NRL_E_INVALID, "too many sequences");
+    SeqErrArgs a;
+    a.prev = prev; a.gen = gen; a.token_mask = token_mask; a.sample_mask = sample_mask; a.rewards = rewards;
+    a.batch = batch; a.seq_len = seq_len; a.prev_stride = prev_stride; a.gen_stride = gen_stride; a.tm_stride = token_mask_stride;
+    a.has_threshold = has_threshold; a.threshold = threshold;
+    a.seq_err = seq_err_out; a.valid = static_cast<float*>(workspace); a.sample_mask_out = sample_mask_out; a.record = record_out;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (batch > 0) seq_err_rows_kernel<<<dim3((unsigned)batch), dim3(kAdvBlock), 0, s>>>(a);
+    seq_err_finish_kernel<<<dim3(1), dim3(kAdvBlock), 0, s>>>(a);
+    return check_launch("seq_logprob_error");
 }

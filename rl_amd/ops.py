@@ -531,6 +531,48 @@ def _group_baseline_std(prompts, rewards, valid, std_rewards, leave_one_out, nor
 _LIB.impl("group_baseline_std", _group_baseline_std, "CUDA")
 _LIB.impl("group_baseline_std", _group_baseline_std, "CPU")
 
+_LIB.define(
+    "seq_logprob_error(Tensor prev, Tensor gen, Tensor token_mask, Tensor sample_mask, Tensor? rewards, "
+    "float? threshold) -> (Tensor, Tensor, Tensor)"
+)
+
+
+def _seq_logprob_error(prev, gen, token_mask, sample_mask, rewards, threshold):
+    """-> (per-sequence error [B], sample mask after the threshold [B], 8-float record)."""
+    _need_gpu(prev, gen, token_mask, sample_mask, rewards)
+    if prev.dim() != 2 or gen.shape != prev.shape or token_mask.shape != prev.shape:
+        raise ValueError("prev_logprobs, generation_logprobs and token_mask must share one [B, S] shape")
+    b, s = prev.shape
+
+    def rows(t, name):
+        t = t.to(torch.float32)
+        if s > 1 and t.stride(1) != 1:
+            t = t.contiguous()
+        return t
+
+    prev, gen, token_mask = rows(prev, "prev"), rows(gen, "gen"), rows(token_mask, "token_mask")
+    sample_mask = _vec(sample_mask, b, "sample_mask")
+    rewards = _vec(rewards, b, "rewards") if rewards is not None else None
+    lib = _lib.load()
+    dev = prev.device
+    with torch.cuda.device(dev):
+        err = torch.empty((b,), dtype=torch.float32, device=dev)
+        mask_out = torch.empty((b,), dtype=torch.float32, device=dev)
+        record = torch.empty((8,), dtype=torch.float32, device=dev)
+        ws = torch.empty((max(b, 1),), dtype=torch.float32, device=dev)
+        code = lib.nrl_seq_logprob_error(
+            _ptr(prev), prev.stride(0) if b > 1 else s, _ptr(gen), gen.stride(0) if b > 1 else s,
+            _ptr(token_mask), token_mask.stride(0) if b > 1 else s, _ptr(sample_mask), _ptr(rewards), b, s,
+            int(threshold is not None), float(threshold) if threshold is not None else 0.0,
+            _ptr(err), _ptr(mask_out), _ptr(record), _ptr(ws), ws.numel() * 4, _stream(),
+        )
+    _lib.check(code, "nrl_seq_logprob_error")
+    return err, mask_out, record
+
+
+_LIB.impl("seq_logprob_error", _seq_logprob_error, "CUDA")
+_LIB.impl("seq_logprob_error", _seq_logprob_error, "CPU")
+
 
 # ------------------------------------------------------------------------------------------------
 # K6: fused lm_head

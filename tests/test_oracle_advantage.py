@@ -78,3 +78,39 @@ def test_grpo_advantage_golden(case):
         assert torch.allclose(out[0], -out[2], rtol=1e-5)
     else:
         assert abs(out.mean()) < 1e-5
+
+
+def test_seq_logprob_error_masking_brute_force():
+    """The restatement against plain Python loops (the reference's tests only mock this function)."""
+    import math
+
+    g = torch.Generator().manual_seed(21)
+    b, s = 6, 9
+    prev = torch.randn(b, s, generator=g)
+    gen = prev + 0.3 * torch.randn(b, s, generator=g)
+    tm = (torch.rand(b, s, generator=g) < 0.7).long()
+    tm[2] = 0  # a sequence without unmasked tokens must not touch the statistics
+    sm = torch.tensor([1, 1, 1, 0, 1, 1])
+    rewards = torch.tensor([1.0, 0.0, 1.0, 1.0, 1.0, 0.0])
+    errs = []
+    for i in range(b):
+        m = [float(tm[i, t]) * float(sm[i]) for t in range(1, s)]
+        den = sum(m)
+        num = sum(math.exp(abs(float(gen[i, t + 1] - prev[i, t + 1])) * m[t]) * m[t] for t in range(s - 1))
+        errs.append(num / max(den, 1.0) if den > 0 else None)
+    valid = [e for e in errs if e is not None]
+    got, new_mask = A.seq_logprob_error_masking(prev, gen, tm, sm, rewards, None)
+    assert abs(got["max_seq_mult_prob_error"] - max(valid)) < 1e-5
+    assert abs(got["mean_seq_mult_prob_error"] - sum(valid) / len(valid)) < 1e-5
+    assert abs(got["min_seq_mult_prob_error"] - min(valid)) < 1e-5
+    assert got["num_masked_seqs"] == 0 and new_mask is sm
+    thr = sorted(valid)[len(valid) // 2]  # masks the sequences strictly above the median
+    got, new_mask = A.seq_logprob_error_masking(prev, gen, tm, sm, rewards, thr + 1e-6)
+    want_mask = [float(sm[i]) * (1.0 if (errs[i] if errs[i] is not None else 0.0) <= thr + 1e-6 else 0.0) for i in range(b)]
+    assert new_mask.tolist() == want_mask
+    dropped = [i for i in range(b) if float(sm[i]) - want_mask[i] != 0]
+    assert got["num_masked_seqs"] == len(dropped) > 0
+    assert abs(got["masked_correct_pct"] - sum(1 for i in dropped if rewards[i] == 1) / len(dropped)) < 1e-6
+    kept = [errs[i] for i in range(b) if want_mask[i] and errs[i] is not None]
+    assert abs(got["max_seq_mult_prob_error_after_mask"] - max(kept)) < 1e-5
+    assert abs(got["min_seq_mult_prob_error_after_mask"] - min(kept)) < 1e-5
