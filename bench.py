@@ -6,7 +6,7 @@ microbatch, logits -> token logprobs (K1), clipped-PG loss forward+backward (K4)
 through the public API (``prepare_loss_input`` -> ``ClippedPGLossFn`` -> autograd).  Inputs are
 resident in HBM before the timed region.  Prints ONE JSON line.
 
-Default workload (BASELINE config 2): 16 prompts x 8 generations = 128 sequences x 4096 tokens,
+Default workload (benchmark config 2): 16 prompts x 8 generations = 128 sequences x 4096 tokens,
 V = 151936, bf16 logits ~ N(0,3) with a +8 spike at the target id with p = 0.3, prompt prefix
 U[256,1024] masked out; run as microbatches of 16 sequences (19.9 GB of logits each).
 """
@@ -33,14 +33,14 @@ THREE_PASS_BWD_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}  # logprob_bwd_kernel
 WORKLOADS = {
     # name: (sequences, seq_len, vocab, dtype, sequences per microbatch, logit std, spike p)
     "c2": dict(seqs=128, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=3.0, spike_p=0.3,
-               desc="BASELINE config 2: 16 prompts x 8 = 128 seq x 4096 tok, V=151936 bf16, fwd+bwd to dlogits"),
+               desc="benchmark config 2: 16 prompts x 8 = 128 seq x 4096 tok, V=151936 bf16, fwd+bwd to dlogits"),
     "c3": dict(seqs=16, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=0.0, spike_p=0.0, hidden=4096,
-               desc="BASELINE config 3: fused lm_head + logprob, hidden [65536,4096] bf16, W [151936,4096] bf16, fwd+bwd (dH, dW)"),
+               desc="benchmark config 3: fused lm_head + logprob, hidden [65536,4096] bf16, W [151936,4096] bf16, fwd+bwd (dH, dW)"),
     "c4": dict(seqs=64, seq_len=8192, vocab=151936, dtype="bf16", mb_seqs=8, std=3.0, spike_p=0.0, temperature=0.7,
                top_k=50, top_p=0.95,
-               desc="BASELINE config 4: 64 seq x 8192 tok, V=151936 bf16, T=0.7, top_k=50, top_p=0.95, DAPO clip-higher, no KL"),
+               desc="benchmark config 4: 64 seq x 8192 tok, V=151936 bf16, T=0.7, top_k=50, top_p=0.95, DAPO clip-higher, no KL"),
     "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
-               desc="BASELINE config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
+               desc="benchmark config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
 }
 
 

@@ -5,9 +5,11 @@
 //   pass 1 (HBM)   streams the row keeping 2048 chunk maxima in registers (and, when the caller
 //                  wants the unfiltered logprob too, the online log-sum-exp of the full row);
 //   select         the k-th largest chunk maximum is a lower bound of the k-th largest element
-//                  (radix select over the 2048 maxima in LDS); for top-p alone the bound is
-//                  lse + log((1-p)/V): everything below it is dropped whatever the order;
-//   pass 2 (cache) re-reads the row and appends the few elements above the bound to an LDS list;
+//                  (found two bits per round with wave ballots, the maxima staying in registers);
+//                  for top-p alone the bound is lse + log((1-p)/V): everything below it is dropped
+//                  whatever the order;
+//   pass 2         re-reads only the chunks whose maximum reaches the bound (about k of 2048) and
+//                  appends the elements above the bound to an LDS list;
 //   finish         bitonic sort of the list by (value, index), top-k threshold with ties kept,
 //                  softmax over the kept values, ascending cumulative mass > 1 - top_p, the
 //                  renormalised log-sum-exp, the target's logprob (-inf when it was filtered).
@@ -66,11 +68,6 @@ template <int CAP> struct SelShared {
     int sel_cnt[2][kSelWaves * 3];
     Lse2 lse_w[kSelWaves];
     int count;
-    float bound;
-    float thr;
-    int tie;
-    float lse_kept;
-    int n_keep;
 };
 
 // k-th largest (1-based) of the workgroup's kChunks keys (kSub per thread, in registers); every thread

@@ -1,5 +1,5 @@
 """Shared builders for the parity tests (golden cases -> tensors, synthetic
-BASELINE-style workloads)."""
+benchmark-style workloads)."""
 
 from __future__ import annotations
 
@@ -77,7 +77,7 @@ def exact_logits_for_logprobs(target_lp, input_ids, vocab):
 
 def synthetic_grpo_batch(n_prompts, group, seq, vocab, seed, logits_dtype=torch.float32,
                          logit_std=2.0, min_resp=None, spike_p=0.0, spike=8.0):
-    """BASELINE-style synthetic step input on the CPU (fp32 generated, then cast)."""
+    """benchmark-style synthetic step input on the CPU (fp32 generated, then cast)."""
     g = torch.Generator().manual_seed(seed)
     b = n_prompts * group
     logits = (torch.randn(b, seq, vocab, generator=g) * logit_std)

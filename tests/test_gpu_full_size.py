@@ -35,7 +35,7 @@ def _grad_close_bf16(got, want_f32):
 
 
 def test_config2_microbatch_full_shape():
-    """One microbatch of BASELINE config 2: 16 x 4096 tokens, V = 151936, bf16, prompt prefix U[256,1024]."""
+    """One microbatch of benchmark config 2: 16 x 4096 tokens, V = 151936, bf16, prompt prefix U[256,1024]."""
     b, s, v = 16, 4096, V_QWEN
     g = torch.Generator().manual_seed(2002)
     logits = _randn_bf16((b, s, v), 3.0, 2002)
@@ -110,7 +110,7 @@ def test_config2_microbatch_full_shape():
 
 
 def test_config4_microbatch_topk_topp_full_vocab():
-    """BASELINE config 4 rows (8192-token sequences, V = 151936 bf16, T = 0.7, top_k 50, top_p 0.95), two sequences."""
+    """benchmark config 4 rows (8192-token sequences, V = 151936 bf16, T = 0.7, top_k 50, top_p 0.95), two sequences."""
     b, s, v = 2, 8192, V_QWEN
     g = torch.Generator().manual_seed(4004)
     logits = _randn_bf16((b, s, v), 3.0, 4004)
@@ -156,7 +156,7 @@ def test_config4_microbatch_topk_topp_full_vocab():
 
 
 def test_config5_packed_row_full_shape():
-    """BASELINE config 5: one packed row of 131072 tokens (lengths U[2048, 32768]), V = 131072 bf16."""
+    """benchmark config 5: one packed row of 131072 tokens (lengths U[2048, 32768]), V = 131072 bf16."""
     v, total = 131072, 131072
     g = torch.Generator().manual_seed(5005)
     lens = []

@@ -284,7 +284,7 @@ def test_grpo_advantage_golden(case):
 
 @pytest.mark.parametrize("loo", [True, False])
 def test_groups_and_advantages_match_oracle_bit_exact_decisions(loo):
-    """Random prompts with duplicates, shuffled; Bernoulli rewards (the BASELINE workload): group
+    """Random prompts with duplicates, shuffled; Bernoulli rewards (the benchmark workload): group
     indices, std > 0 decisions and values must agree with the oracle."""
     g = torch.Generator().manual_seed(12)
     n_prompts, group, plen = 37, 8, 33
@@ -313,7 +313,7 @@ def test_groups_and_advantages_match_oracle_bit_exact_decisions(loo):
 
 
 def test_config1_end_to_end_small():
-    """BASELINE config 1 at reduced size: advantages -> logprobs -> loss -> dlogits, fp32 logits."""
+    """benchmark config 1 at reduced size: advantages -> logprobs -> loss -> dlogits, fp32 logits."""
     w = synthetic_grpo_batch(4, 4, 64, 2048, seed=1001)
     ids, logits = w["input_ids"], w["logits"]
     adv = OA.grpo_advantages(w["prompt_ids"], w["rewards"], w["token_mask"])

@@ -99,7 +99,7 @@ def test_ties_at_the_boundaries():
 
 
 def test_c4_slice_bf16_temperature_topk_topp():
-    """BASELINE config 4 at reduced rows: V=151936 bf16, T=0.7 (divide in bf16), top_k=50, top_p=0.95."""
+    """benchmark config 4 at reduced rows: V=151936 bf16, T=0.7 (divide in bf16), top_k=50, top_p=0.95."""
     g = torch.Generator().manual_seed(1004)
     vocab, b, s = 151936, 2, 6
     logits = (torch.randn(b, s, vocab, generator=g) * 3).to(torch.bfloat16)
