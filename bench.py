@@ -39,6 +39,8 @@ WORKLOADS = {
     "c4": dict(seqs=64, seq_len=8192, vocab=151936, dtype="bf16", mb_seqs=8, std=3.0, spike_p=0.0, temperature=0.7,
                top_k=50, top_p=0.95,
                desc="benchmark config 4: 64 seq x 8192 tok, V=151936 bf16, T=0.7, top_k=50, top_p=0.95, DAPO clip-higher, no KL"),
+    "distill": dict(seqs=8, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=8, std=3.0, spike_p=0.0, topk=64,
+                    desc="distillation reductions on 8 x 4096 rows, V=151936 bf16: negative entropy, 64 gathered logprobs, soft cross entropy"),
     "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
                desc="benchmark config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
 }
@@ -244,6 +246,61 @@ def bench_topk(args, torch, w):
     }))
 
 
+def bench_distill(args, torch, w):
+    """Negative entropy, gathered logprobs and soft-target cross entropy, forward + backward each."""
+    from rl_amd import ops
+    from rl_amd.distributed import model_utils as MU
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    b, s, v, k = w["seqs"], w["seq_len"], w["vocab"], w["topk"]
+    g = torch.Generator(device=dev).manual_seed(6006)
+    student = torch.empty((b, s, v), dtype=torch.bfloat16, device=dev).normal_(0.0, w["std"], generator=g)
+    teacher = torch.empty((b, s, v), dtype=torch.bfloat16, device=dev).normal_(0.0, w["std"], generator=g)
+    idx = torch.randint(0, v, (b, s, k), generator=g, device=dev)
+    up2 = torch.randn((b, s), generator=g, device=dev)
+    up3 = torch.randn((b, s, k), generator=g, device=dev)
+
+    def step():
+        x = student.requires_grad_(True)
+        (d,) = torch.autograd.grad((MU.ChunkedDistributedEntropy.apply(x, s, None) * up2).sum(), x)
+        del d
+        (d,) = torch.autograd.grad((MU.ChunkedDistributedGatherLogprob.apply(x, idx, 0, v, s, None) * up3).sum(), x)
+        del d
+        (d,) = torch.autograd.grad((MU.DistributedCrossEntropy.apply(x, teacher, None) * up2).sum(), x)
+        del d
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = EventTimer(torch)
+    ops.KERNEL_TIMER = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    km = timer.summary()
+    tensor_bytes = b * s * v * 2
+    passes = {"neg_entropy_fwd": 1, "neg_entropy_bwd": 2, "gather_logprob_fwd": 1, "gather_logprob_bwd": 2,
+              "soft_cross_entropy_fwd": 2, "soft_cross_entropy_bwd": 3}
+    kernels = {n: {"avg_launch_ms": round(km[n]["avg_ms"], 4), "algorithmic_bytes_per_launch": passes[n] * tensor_bytes,
+                   "achieved_GBps": passes[n] * tensor_bytes / (km[n]["avg_ms"] * 1e-3) / 1e9,
+                   "frac_of_hbm_peak": passes[n] * tensor_bytes / (km[n]["avg_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+               for n in passes if n in km}
+    worst = min(kernels, key=lambda n: kernels[n]["frac_of_hbm_peak"])
+    print(json.dumps({
+        "metric": "distillation reductions fwd/bwd tokens/s at V=151936 (three losses per token); % of HBM peak",
+        "value": 3 * b * s * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": w["desc"]},
+        "roofline": {"bound": "hbm", "kernel": worst, "achieved": kernels[worst]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": kernels[worst]["frac_of_hbm_peak"], "traffic": None},
+        "kernels": kernels,
+    }))
+
+
 def bench_lmhead(args, torch, w):
     """Config 3: hidden states -> logprobs -> loss -> (dH, dW) through the fused MFMA path."""
     from rl_amd import ops
@@ -325,6 +382,8 @@ def main():
         return bench_lmhead(args, torch, w)
     if args.workload == "c4":
         return bench_topk(args, torch, w)
+    if args.workload == "distill":
+        return bench_distill(args, torch, w)
     if args.seqs:
         w["seqs"] = args.seqs
         w["mb_seqs"] = min(w["mb_seqs"], args.seqs)

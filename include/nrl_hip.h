@@ -239,6 +239,36 @@ int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int64_t prompt
                            float* baseline_out, float* std_out, float* adv_out, int32_t* group_out,
                            void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Full-vocabulary reductions of the distillation losses, on the K1 / K2 streaming core (TP = 1).
+ * `rows` describes the logits as for nrl_logprob_fwd; its `targets` / temperature fields are not used.
+ * Gradients are written in the logits' dtype (one narrowing of the fp32 value); dlogits must not alias
+ * the logits.
+ *
+ * nrl_neg_entropy_*: ChunkedDistributedEntropy (nemo_rl/distributed/model_utils.py:2023-2103):
+ *   h_out[r] = sum_v p_v log p_v, lse_out[r]; backward g * p_v * (log p_v - h).
+ * nrl_gather_logprob_*: ChunkedDistributedGatherLogprob (model_utils.py:722-836): out[r, k] = log p at
+ *   indices[r, k] (int64 [rows, K], global ids; 0 outside [vocab_start, vocab_end)); backward
+ *   -p_v * sum_k g_k + sum over the k with indices[r, k] == v of g_k.
+ * nrl_soft_cross_entropy_*: DistributedCrossEntropy (model_utils.py:209-264): ce_out[r] =
+ *   -sum_v softmax(teacher)_v * log_softmax(student)_v; backward g * (softmax(student) - softmax(teacher)).
+ *   teacher: same dtype and [n_outer, n_inner, vocab] shape as the student, with its own row strides.
+ * ------------------------------------------------------------------------------------------ */
+int nrl_neg_entropy_fwd(const nrl_rows* rows, float* h_out, float* lse_out, void* stream);
+int nrl_neg_entropy_bwd(const nrl_rows* rows, const float* lse, const float* h, const float* grad, void* dlogits,
+                        int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
+int nrl_gather_logprob_fwd(const nrl_rows* rows, const int64_t* indices, int64_t k, float* out, float* lse_out,
+                           void* stream);
+int nrl_gather_logprob_bwd(const nrl_rows* rows, const int64_t* indices, int64_t k, const float* lse, const float* grad,
+                           void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
+int nrl_soft_cross_entropy_fwd(const nrl_rows* student, const void* teacher, int64_t t_stride_outer,
+                               int64_t t_stride_inner, float* ce_out, float* lse_student_out, float* lse_teacher_out,
+                               void* stream);
+int nrl_soft_cross_entropy_bwd(const nrl_rows* student, const void* teacher, int64_t t_stride_outer,
+                               int64_t t_stride_inner, const float* lse_student, const float* lse_teacher,
+                               const float* grad, void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner,
+                               void* stream);
+
 /* Per-sequence multiplicative logprob error and the mask that drops sequences above a threshold.
  * Replaces compute_and_apply_seq_logprob_error_masking (nemo_rl/algorithms/grpo.py:2513-2640):
  * err[b] = sum_t exp(|gen - prev| * m) * m / max(sum_t m, 1) over t >= 1 with m = token_mask[b,t] * sample_mask[b]

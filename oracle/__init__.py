@@ -38,6 +38,9 @@ Pinning status (what fixes each function besides its own text):
                            inputs (the reference's tests only mock it).
 * ``logprob.logprobs_post_process``  pinned: ``log_softmax`` + ``gather``
                            identity and brute-force loops on tiny inputs.
+* ``distill.*``            pinned: closed forms (uniform / one-hot rows, H(p,q) =
+                           H(p) + KL), the reference's stated backward formulas
+                           and brute force (``tests/test_oracle_distill.py``).
 * ``lmhead.*``             PARITY UNPINNED against the reference (its only test
                            needs Megatron, two GPUs and a model download);
                            pinned here to ``logprob(hidden @ W.T)`` in fp32.

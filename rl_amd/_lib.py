@@ -81,6 +81,12 @@ SIGNATURES = {
     "nrl_fused_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _F, _P, _I64,
                                              _I64, _I64, _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _I64, _P]),
+    "nrl_neg_entropy_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P]),
+    "nrl_neg_entropy_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P, _P, _I64, _I64, _P]),
+    "nrl_gather_logprob_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P, _P]),
+    "nrl_gather_logprob_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P, _P, _I64, _I64, _P]),
+    "nrl_soft_cross_entropy_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _I64, _P, _P, _P, _P]),
+    "nrl_soft_cross_entropy_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _I64, _P, _P, _P, _P, _I64, _I64, _P]),
     "nrl_seq_logprob_error": (C.c_int, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _I64, C.c_int32, C.c_float, _P, _P, _P, _P, _I64, _P]),
     "nrl_lmhead_fwd_workspace_bytes": (_I64, [_I64, _I64]),
     "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P]),

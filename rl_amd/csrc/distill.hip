@@ -1,0 +1,434 @@
+// Full-vocabulary reductions that distillation losses need, on the same one-pass-per-row streaming core as
+// the token logprob kernels (one 256-thread workgroup per row, 16-byte loads, online rescaling):
+//   * sum_v p_v log p_v (the negative entropy) and its gradient,
+//   * log-probabilities gathered at K given vocabulary indices per row and their gradient,
+//   * soft-target cross entropy H(p_teacher, q_student) of two logit tensors and its gradient.
+// Rows whose start is not 16-byte aligned (or whose length is not a whole number of vectors) take an
+// element-wise path; nothing is ever materialised at [rows, V] in fp32.
+
+#include <float.h>
+#include <math.h>
+
+#include "common.hpp"
+
+namespace nrl {
+
+constexpr int kDBlock = 256;
+constexpr int kDWaves = kDBlock / kWave;
+constexpr int kDUnroll = 4;
+
+struct RowsView {
+    const void* p;
+    int64_t n_inner, vocab, stride_outer, stride_inner;
+};
+
+template <int DT> __device__ __forceinline__ const char* row_ptr(const RowsView& v, int64_t r) {
+    const int64_t o = r / v.n_inner, i = r - o * v.n_inner;
+    return static_cast<const char*>(v.p) + (o * v.stride_outer + i * v.stride_inner) * Row<DT>::BYTES;
+}
+
+template <int DT> __device__ __forceinline__ bool vec_ok(const void* row, int64_t vocab) {
+    return (reinterpret_cast<uintptr_t>(row) & 15) == 0 && vocab % Row<DT>::EPV == 0;
+}
+
+// fv(values of one 16-byte vector) / f1(one element) over the row, each thread taking a strided share
+template <int DT, class FV, class F1> __device__ __forceinline__ void row_for_each_vec(const void* row, int64_t vocab, FV fv, F1 f1) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    if (!vec_ok<DT>(row, vocab)) {
+        for (int64_t i = tid; i < vocab; i += kDBlock) f1(Row<DT>::load1(row, i));
+        return;
+    }
+    const u32x4* xv = static_cast<const u32x4*>(row);
+    const int64_t nvec = vocab / EPV;
+    int64_t base = 0;
+    for (; base + kDUnroll * kDBlock <= nvec; base += kDUnroll * kDBlock) {
+        u32x4 q[kDUnroll];
+#pragma unroll
+        for (int u = 0; u < kDUnroll; ++u) q[u] = __builtin_nontemporal_load(xv + base + u * kDBlock + tid);
+#pragma unroll
+        for (int u = 0; u < kDUnroll; ++u) {
+            float t[EPV];
+            Row<DT>::decode(q[u], t);
+            fv(t);
+        }
+    }
+    for (int64_t vi = base + tid; vi < nvec; vi += kDBlock) {
+        float t[EPV];
+        Row<DT>::decode(__builtin_nontemporal_load(xv + vi), t);
+        fv(t);
+    }
+}
+
+// f(x) for every element of the row
+template <int DT, class F> __device__ __forceinline__ void row_for_each(const void* row, int64_t vocab, F f) {
+    constexpr int EPV = Row<DT>::EPV;
+    row_for_each_vec<DT>(
+        row, vocab,
+        [&](const float(&t)[EPV]) {
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) f(t[k]);
+        },
+        f);
+}
+
+// out[i] = f(x[i], y[i], i) over one row; y may be NULL (then f receives 0 for it)
+template <int DT, class F>
+__device__ __forceinline__ void row_map(const void* xrow, const void* yrow, void* out, int64_t vocab, F f) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const bool vec = vec_ok<DT>(xrow, vocab) && vec_ok<DT>(out, vocab) && (!yrow || vec_ok<DT>(yrow, vocab));
+    if (!vec) {
+        for (int64_t i = tid; i < vocab; i += kDBlock)
+            Row<DT>::store1(out, i, f(Row<DT>::load1(xrow, i), yrow ? Row<DT>::load1(yrow, i) : 0.f, i));
+        return;
+    }
+    const u32x4* xv = static_cast<const u32x4*>(xrow);
+    const u32x4* yv = static_cast<const u32x4*>(yrow);
+    u32x4* ov = static_cast<u32x4*>(out);
+    const int64_t nvec = vocab / EPV;
+    for (int64_t vi = tid; vi < nvec; vi += kDBlock) {
+        float a[EPV], b[EPV], d[EPV];
+        Row<DT>::decode(__builtin_nontemporal_load(xv + vi), a);
+        if (yrow) Row<DT>::decode(__builtin_nontemporal_load(yv + vi), b);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) d[k] = f(a[k], yrow ? b[k] : 0.f, vi * EPV + k);
+        __builtin_nontemporal_store(Row<DT>::encode(d), ov + vi);
+    }
+}
+
+template <int DT> __device__ __forceinline__ void row_fill_zero(void* out, int64_t vocab) {
+    row_map<DT>(out, nullptr, out, vocab, [](float, float, int64_t) { return 0.f; });
+}
+
+// online (max, sum exp, sum exp * (x - max)): enough for the log-sum-exp and for sum_v p_v x_v
+struct Ent {
+    float m, s, t;
+};
+__device__ __forceinline__ void ent_push(Ent& a, float x) {
+    if (x > a.m) {
+        const float d = a.m - x, e = fast_exp2(d * kLog2e);
+        a.t = e * (a.t + d * a.s);
+        a.s = e * a.s;
+        a.m = x;
+    }
+    const float d = x - a.m, p = fast_exp2(d * kLog2e);
+    a.s += p;
+    a.t += p > 0.f ? p * d : 0.f;  // a -inf logit has probability 0 and adds nothing
+}
+__device__ __forceinline__ Ent ent_merge(Ent a, Ent b) {
+    const float m = fmaxf(a.m, b.m), da = a.m - m, db = b.m - m;
+    const float ea = fast_exp2(da * kLog2e), eb = fast_exp2(db * kLog2e);
+    Ent r;
+    r.m = m;
+    r.s = a.s * ea + b.s * eb;
+    r.t = ea * (a.t + da * a.s) + eb * (b.t + db * b.s);
+    return r;
+}
+__device__ __forceinline__ Ent ent_block(Ent a, Ent* smem) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        Ent o;
+        o.m = __shfl_xor(a.m, off, kWave);
+        o.s = __shfl_xor(a.s, off, kWave);
+        o.t = __shfl_xor(a.t, off, kWave);
+        a = ent_merge(a, o);
+    }
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = a;
+    __syncthreads();
+    Ent tot = smem[0];
+#pragma unroll
+    for (int i = 1; i < kDWaves; ++i) tot = ent_merge(tot, smem[i]);
+    return tot;
+}
+
+// ---------------------------------------------------------------------------------------------
+// sum_v p_v log p_v
+// ---------------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void neg_entropy_fwd_kernel(RowsView x, float* __restrict__ h_out, float* __restrict__ lse_out) {
+    __shared__ Ent smem[kDWaves];
+    const int64_t r = blockIdx.x;
+    const char* row = row_ptr<DT>(x, r);
+    Ent acc{-1e30f, 0.f, 0.f};
+    row_for_each<DT>(row, x.vocab, [&](float v) { ent_push(acc, v); });
+    const Ent tot = ent_block(acc, smem);
+    if (threadIdx.x == 0) {
+        const float log_s = logf(tot.s);
+        h_out[r] = tot.t / tot.s - log_s;  // sum p (x - m) - log s
+        lse_out[r] = tot.m + log_s;
+    }
+}
+
+// d / dz of sum_v p_v log p_v, times the upstream gradient: g * p_v * (log p_v - H)
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void neg_entropy_bwd_kernel(RowsView x, const float* __restrict__ lse, const float* __restrict__ h,
+                                                                  const float* __restrict__ grad, RowsView d) {
+    const int64_t r = blockIdx.x;
+    void* out = const_cast<char*>(row_ptr<DT>(d, r));
+    const float g = grad[r];
+    if (g == 0.f) { row_fill_zero<DT>(out, x.vocab); return; }
+    const float l = lse[r], hh = h[r];
+    row_map<DT>(row_ptr<DT>(x, r), nullptr, out, x.vocab, [&](float v, float, int64_t) {
+        const float lp = v - l, p = fast_exp2(lp * kLog2e);
+        return p > 0.f ? g * p * (lp - hh) : 0.f;
+    });
+}
+
+// ---------------------------------------------------------------------------------------------
+// log-probabilities at K given indices per row
+// ---------------------------------------------------------------------------------------------
+struct GatherArgs {
+    const int64_t* idx;  // [rows, K]
+    int64_t k, vstart, vend;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void gather_logprob_fwd_kernel(RowsView x, GatherArgs ga, float* __restrict__ out,
+                                                                     float* __restrict__ lse_out) {
+    __shared__ Lse smem[kDWaves];
+    const int64_t r = blockIdx.x;
+    const char* row = row_ptr<DT>(x, r);
+    Lse acc{-FLT_MAX, 0.f};
+    row_for_each_vec<DT>(
+        row, x.vocab, [&](const float(&t)[Row<DT>::EPV]) { lse_push<Row<DT>::EPV>(acc, t); }, [&](float v) { lse_push1(acc, v); });
+    const Lse tot = block_lse<kDWaves>(acc, smem);
+    const float lse = tot.m + logf(tot.s);
+    if (threadIdx.x == 0 && lse_out) lse_out[r] = lse;
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) {
+        const int64_t gi = ga.idx[r * ga.k + j];
+        out[r * ga.k + j] = (gi >= ga.vstart && gi < ga.vend) ? Row<DT>::load1(row, gi - ga.vstart) - lse : 0.f;
+    }
+}
+
+// dz_v = -p_v * sum_k g_k + sum_{k: idx_k = v} g_k; the K touched elements are rewritten after the streaming
+// pass with their complete value (every duplicate of an index computes and writes the same number)
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void gather_logprob_bwd_kernel(RowsView x, GatherArgs ga, const float* __restrict__ lse,
+                                                                     const float* __restrict__ grad, RowsView d) {
+    __shared__ float sm[kDWaves];
+    const int64_t r = blockIdx.x;
+    const char* row = row_ptr<DT>(x, r);
+    void* out = const_cast<char*>(row_ptr<DT>(d, r));
+    float part = 0.f;
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) part += grad[r * ga.k + j];
+    const float gsum = block_sum<float, kDWaves>(part, sm);
+    const float l = lse[r];
+    row_map<DT>(row, nullptr, out, x.vocab, [&](float v, float, int64_t) { return -fast_exp2((v - l) * kLog2e) * gsum; });
+    __syncthreads();  // the streaming stores of this workgroup are visible to it before the patches land
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) {
+        const int64_t gi = ga.idx[r * ga.k + j];
+        if (gi < ga.vstart || gi >= ga.vend) continue;
+        float add = 0.f;
+        for (int64_t q = 0; q < ga.k; ++q) add += ga.idx[r * ga.k + q] == gi ? grad[r * ga.k + q] : 0.f;
+        const float v = Row<DT>::load1(row, gi - ga.vstart);
+        Row<DT>::store1(out, gi - ga.vstart, -fast_exp2((v - l) * kLog2e) * gsum + add);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// soft-target cross entropy  -sum_v softmax(y)_v * log_softmax(x)_v  = lse(x) - sum_v softmax(y)_v x_v
+// ---------------------------------------------------------------------------------------------
+struct Ce {
+    float m, s, u;  // teacher max, sum exp(y - m), sum exp(y - m) * x
+};
+__device__ __forceinline__ void ce_push(Ce& a, float y, float x) {
+    if (y > a.m) {
+        const float e = fast_exp2((a.m - y) * kLog2e);
+        a.s *= e;
+        a.u *= e;
+        a.m = y;
+    }
+    const float p = fast_exp2((y - a.m) * kLog2e);
+    a.s += p;
+    a.u += p > 0.f ? p * x : 0.f;
+}
+__device__ __forceinline__ Ce ce_merge(Ce a, Ce b) {
+    const float m = fmaxf(a.m, b.m);
+    const float ea = fast_exp2((a.m - m) * kLog2e), eb = fast_exp2((b.m - m) * kLog2e);
+    return Ce{m, a.s * ea + b.s * eb, a.u * ea + b.u * eb};
+}
+
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void soft_ce_fwd_kernel(RowsView x, RowsView y, float* __restrict__ ce_out,
+                                                              float* __restrict__ lse_x_out, float* __restrict__ lse_y_out) {
+    constexpr int EPV = Row<DT>::EPV;
+    __shared__ Lse smem[kDWaves];
+    __shared__ Ce smem_c[kDWaves];
+    const int64_t r = blockIdx.x;
+    const char* xr = row_ptr<DT>(x, r);
+    const char* yr = row_ptr<DT>(y, r);
+    const int tid = threadIdx.x;
+    Lse ax{-FLT_MAX, 0.f};
+    Ce ay{-1e30f, 0.f, 0.f};
+    if (vec_ok<DT>(xr, x.vocab) && vec_ok<DT>(yr, x.vocab)) {
+        const u32x4* xv = reinterpret_cast<const u32x4*>(xr);
+        const u32x4* yv = reinterpret_cast<const u32x4*>(yr);
+        const int64_t nvec = x.vocab / EPV;
+        auto fold = [&](const u32x4& qx, const u32x4& qy) {
+            float a[EPV], b[EPV];
+            Row<DT>::decode(qx, a);
+            Row<DT>::decode(qy, b);
+            lse_push<EPV>(ax, a);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) ce_push(ay, b[k], a[k]);
+        };
+        int64_t base = 0;
+        for (; base + kDUnroll * kDBlock <= nvec; base += kDUnroll * kDBlock) {
+            u32x4 qx[kDUnroll], qy[kDUnroll];
+#pragma unroll
+            for (int u = 0; u < kDUnroll; ++u) {
+                qx[u] = __builtin_nontemporal_load(xv + base + u * kDBlock + tid);
+                qy[u] = __builtin_nontemporal_load(yv + base + u * kDBlock + tid);
+            }
+#pragma unroll
+            for (int u = 0; u < kDUnroll; ++u) fold(qx[u], qy[u]);
+        }
+        for (int64_t vi = base + tid; vi < nvec; vi += kDBlock) fold(__builtin_nontemporal_load(xv + vi), __builtin_nontemporal_load(yv + vi));
+    } else {
+        for (int64_t i = tid; i < x.vocab; i += kDBlock) {
+            const float a = Row<DT>::load1(xr, i), b = Row<DT>::load1(yr, i);
+            lse_push1(ax, a);
+            ce_push(ay, b, a);
+        }
+    }
+    const Lse tx = block_lse<kDWaves>(ax, smem);
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        Ce o{__shfl_xor(ay.m, off, kWave), __shfl_xor(ay.s, off, kWave), __shfl_xor(ay.u, off, kWave)};
+        ay = ce_merge(ay, o);
+    }
+    if ((tid & (kWave - 1)) == 0) smem_c[tid / kWave] = ay;
+    __syncthreads();
+    if (tid == 0) {
+        Ce ty = smem_c[0];
+#pragma unroll
+        for (int i = 1; i < kDWaves; ++i) ty = ce_merge(ty, smem_c[i]);
+        const float lse_x = tx.m + logf(tx.s);
+        ce_out[r] = lse_x - ty.u / ty.s;
+        lse_x_out[r] = lse_x;
+        lse_y_out[r] = ty.m + logf(ty.s);
+    }
+}
+
+// d H(p, q) / d student logits = g * (q_v - p_v)
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void soft_ce_bwd_kernel(RowsView x, RowsView y, const float* __restrict__ lse_x,
+                                                              const float* __restrict__ lse_y, const float* __restrict__ grad, RowsView d) {
+    const int64_t r = blockIdx.x;
+    void* out = const_cast<char*>(row_ptr<DT>(d, r));
+    const float g = grad[r];
+    if (g == 0.f) { row_fill_zero<DT>(out, x.vocab); return; }
+    const float lx = lse_x[r], ly = lse_y[r];
+    row_map<DT>(row_ptr<DT>(x, r), row_ptr<DT>(y, r), out, x.vocab, [&](float a, float b, int64_t) {
+        return g * (fast_exp2((a - lx) * kLog2e) - fast_exp2((b - ly) * kLog2e));
+    });
+}
+
+static int check_view(const nrl_rows* r) {
+    if (!r) return fail(NRL_E_INVALID, "rows is NULL");
+    if (r->dtype != NRL_F32 && r->dtype != NRL_BF16 && r->dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype %d", r->dtype);
+    if (r->n_outer < 0 || r->n_inner < 0 || r->vocab <= 0) return fail(NRL_E_INVALID, "bad shape");
+    if (r->n_outer * r->n_inner > 0 && !r->logits) return fail(NRL_E_INVALID, "null logits");
+    if (r->n_outer * r->n_inner >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    return NRL_OK;
+}
+
+static RowsView view_of(const nrl_rows* r) { return RowsView{r->logits, r->n_inner, r->vocab, r->stride_outer, r->stride_inner}; }
+static RowsView view_of(const nrl_rows* r, const void* p, int64_t so, int64_t si) { return RowsView{p, r->n_inner, r->vocab, so, si}; }
+
+}  // namespace nrl
+
+using namespace nrl;
+
+#define NRL_DT_DISPATCH(DTV, ...)                                   \
+    switch (DTV) {                                                  \
+        case NRL_F32: { constexpr int DT = NRL_F32; __VA_ARGS__; break; }  \
+        case NRL_BF16: { constexpr int DT = NRL_BF16; __VA_ARGS__; break; } \
+        default: { constexpr int DT = NRL_F16; __VA_ARGS__; break; }        \
+    }
+
+extern "C" int nrl_neg_entropy_fwd(const nrl_rows* rows, float* h_out, float* lse_out, void* stream) {
+    if (int e = check_view(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!h_out || !lse_out) return fail(NRL_E_INVALID, "null output");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsView x = view_of(rows);
+    NRL_DT_DISPATCH(rows->dtype, neg_entropy_fwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, h_out, lse_out));
+    return check_launch("neg_entropy_fwd");
+}
+
+extern "C" int nrl_neg_entropy_bwd(const nrl_rows* rows, const float* lse, const float* h, const float* grad, void* dlogits,
+                                   int64_t d_stride_outer, int64_t d_stride_inner, void* stream) {
+    if (int e = check_view(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!lse || !h || !grad || !dlogits) return fail(NRL_E_INVALID, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsView x = view_of(rows), d = view_of(rows, dlogits, d_stride_outer, d_stride_inner);
+    NRL_DT_DISPATCH(rows->dtype, neg_entropy_bwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, lse, h, grad, d));
+    return check_launch("neg_entropy_bwd");
+}
+
+extern "C" int nrl_gather_logprob_fwd(const nrl_rows* rows, const int64_t* indices, int64_t k, float* out, float* lse_out,
+                                      void* stream) {
+    if (int e = check_view(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (k < 0) return fail(NRL_E_INVALID, "negative K");
+    if (n == 0 || k == 0) return NRL_OK;
+    if (!indices || !out) return fail(NRL_E_INVALID, "null argument");
+    if (rows->vocab_end - rows->vocab_start != rows->vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsView x = view_of(rows);
+    const GatherArgs ga{indices, k, rows->vocab_start, rows->vocab_end};
+    NRL_DT_DISPATCH(rows->dtype, gather_logprob_fwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, ga, out, lse_out));
+    return check_launch("gather_logprob_fwd");
+}
+
+extern "C" int nrl_gather_logprob_bwd(const nrl_rows* rows, const int64_t* indices, int64_t k, const float* lse, const float* grad,
+                                      void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner, void* stream) {
+    if (int e = check_view(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (k < 0) return fail(NRL_E_INVALID, "negative K");
+    if (n == 0) return NRL_OK;
+    if (!lse || !dlogits || (k > 0 && (!indices || !grad))) return fail(NRL_E_INVALID, "null argument");
+    if (rows->vocab_end - rows->vocab_start != rows->vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsView x = view_of(rows), d = view_of(rows, dlogits, d_stride_outer, d_stride_inner);
+    const GatherArgs ga{indices, k, rows->vocab_start, rows->vocab_end};
+    NRL_DT_DISPATCH(rows->dtype, gather_logprob_bwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, ga, lse, grad, d));
+    return check_launch("gather_logprob_bwd");
+}
+
+extern "C" int nrl_soft_cross_entropy_fwd(const nrl_rows* student, const void* teacher, int64_t t_stride_outer,
+                                          int64_t t_stride_inner, float* ce_out, float* lse_student_out, float* lse_teacher_out,
+                                          void* stream) {
+    if (int e = check_view(student)) return e;
+    const int64_t n = student->n_outer * student->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!teacher || !ce_out || !lse_student_out || !lse_teacher_out) return fail(NRL_E_INVALID, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsView x = view_of(student), y = view_of(student, teacher, t_stride_outer, t_stride_inner);
+    NRL_DT_DISPATCH(student->dtype,
+                    soft_ce_fwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, y, ce_out, lse_student_out, lse_teacher_out));
+    return check_launch("soft_cross_entropy_fwd");
+}
+
+extern "C" int nrl_soft_cross_entropy_bwd(const nrl_rows* student, const void* teacher, int64_t t_stride_outer,
+                                          int64_t t_stride_inner, const float* lse_student, const float* lse_teacher,
+                                          const float* grad, void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner,
+                                          void* stream) {
+    if (int e = check_view(student)) return e;
+    const int64_t n = student->n_outer * student->n_inner;
+    if (n == 0) return NRL_OK;
+    if (!teacher || !lse_student || !lse_teacher || !grad || !dlogits) return fail(NRL_E_INVALID, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsView x = view_of(student), y = view_of(student, teacher, t_stride_outer, t_stride_inner);
+    const RowsView d = view_of(student, dlogits, d_stride_outer, d_stride_inner);
+    NRL_DT_DISPATCH(student->dtype,
+                    soft_ce_bwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, y, lse_student, lse_teacher, grad, d));
+    return check_launch("soft_cross_entropy_bwd");
+}

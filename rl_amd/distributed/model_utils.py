@@ -395,3 +395,81 @@ def from_parallel_hidden_states_to_logprobs(
         tp_group, inference_only,
     )
     return logprobs[:, :-1]
+
+
+
+# ------------------------------------------------------------------------------------------------
+# distillation reductions on the same streaming core (TP = 1)
+# ------------------------------------------------------------------------------------------------
+class ChunkedDistributedEntropy(torch.autograd.Function):
+    """``model_utils.py:2023-2103``: ``H_all[b, s] = sum_v p_v log p_v``.  ``chunk_size`` is accepted for
+    signature compatibility; a row never leaves the chip, so nothing needs chunking."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, chunk_size, tp_group, inference_only=False):
+        _require_single_rank(tp_group, "ChunkedDistributedEntropy")
+        x = vocab_parallel_logits if vocab_parallel_logits.stride(-1) == 1 else vocab_parallel_logits.contiguous()
+        h, lse = torch.ops.rl_amd.neg_entropy_fwd(x)
+        if not inference_only:
+            ctx.save_for_backward(x, lse, h)
+        return h
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        x, lse, h = ctx.saved_tensors
+        g = grad_outputs[0].to(torch.float32).contiguous()
+        return torch.ops.rl_amd.neg_entropy_bwd(x, lse, h, g), None, None, None
+
+
+class ChunkedDistributedGatherLogprob(torch.autograd.Function):
+    """``model_utils.py:722-836``: log-softmax once, gathered at ``global_indices [B, S, K]``."""
+
+    @staticmethod
+    def forward(ctx, vocab_parallel_logits, global_indices, vocab_start_index, vocab_end_index, chunk_size, tp_group,
+                inference_only=False):
+        _require_single_rank(tp_group, "ChunkedDistributedGatherLogprob")
+        x = vocab_parallel_logits if vocab_parallel_logits.stride(-1) == 1 else vocab_parallel_logits.contiguous()
+        idx = _to_device(global_indices, x).long().contiguous()
+        out, lse = torch.ops.rl_amd.gather_logprob_fwd(x, idx, int(vocab_start_index), int(vocab_end_index))
+        if not inference_only:
+            ctx.save_for_backward(x, idx, lse)
+            ctx.vocab_range = (int(vocab_start_index), int(vocab_end_index))
+        return out
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        x, idx, lse = ctx.saved_tensors
+        g = grad_outputs[0].to(torch.float32).contiguous()
+        d = torch.ops.rl_amd.gather_logprob_bwd(x, idx, ctx.vocab_range[0], ctx.vocab_range[1], lse, g)
+        return d, None, None, None, None, None, None
+
+
+class DistributedCrossEntropy(torch.autograd.Function):
+    """``model_utils.py:209-264``: soft-target cross entropy ``H(p_target, q_student)``; the gradient
+    flows to the student logits only."""
+
+    @staticmethod
+    def forward(ctx, student_logits, target_logits, group, inference_only=False):
+        if student_logits.shape != target_logits.shape:
+            raise ValueError(
+                "student_logits and target_logits must have the same shape, "
+                f"got {student_logits.shape} and {target_logits.shape}."
+            )
+        _require_single_rank(group, "DistributedCrossEntropy")
+        lead = student_logits.shape[:-1]
+        x = student_logits.reshape(1, -1, student_logits.shape[-1]) if student_logits.dim() != 3 else student_logits
+        y = target_logits.reshape(x.shape) if target_logits.dim() != 3 else target_logits
+        x = x if x.stride(-1) == 1 else x.contiguous()
+        y = _to_device(y, x)
+        ce, lx, ly = torch.ops.rl_amd.soft_cross_entropy_fwd(x, y)
+        if not inference_only:
+            ctx.save_for_backward(x, y, lx, ly)
+            ctx.in_shape = student_logits.shape
+        return ce.reshape(lead)
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        x, y, lx, ly = ctx.saved_tensors
+        g = grad_outputs[0].to(torch.float32).reshape(lx.shape).contiguous()
+        d = torch.ops.rl_amd.soft_cross_entropy_bwd(x, y, lx, ly, g)
+        return d.reshape(ctx.in_shape), None, None, None

@@ -575,6 +575,153 @@ _LIB.impl("seq_logprob_error", _seq_logprob_error, "CPU")
 
 
 # ------------------------------------------------------------------------------------------------
+# distillation reductions (negative entropy, gathered logprobs, soft-target cross entropy)
+# ------------------------------------------------------------------------------------------------
+_LIB.define("neg_entropy_fwd(Tensor logits) -> (Tensor, Tensor)")
+_LIB.define("neg_entropy_bwd(Tensor logits, Tensor lse, Tensor h, Tensor grad) -> Tensor")
+_LIB.define("gather_logprob_fwd(Tensor logits, Tensor indices, int vocab_start, int vocab_end) -> (Tensor, Tensor)")
+_LIB.define("gather_logprob_bwd(Tensor logits, Tensor indices, int vocab_start, int vocab_end, Tensor lse, Tensor grad) -> Tensor")
+_LIB.define("soft_cross_entropy_fwd(Tensor student, Tensor teacher) -> (Tensor, Tensor, Tensor)")
+_LIB.define("soft_cross_entropy_bwd(Tensor student, Tensor teacher, Tensor lse_student, Tensor lse_teacher, Tensor grad) -> Tensor")
+
+
+def _plain_rows(logits, vocab_start=0, vocab_end=None):
+    """nrl_rows for kernels that take no targets: logits [B, S, V] with a contiguous vocabulary axis."""
+    if logits.dim() != 3:
+        raise ValueError(f"expected logits [B, S, V], got {tuple(logits.shape)}")
+    if logits.stride(2) != 1 and logits.shape[2] > 1:
+        raise ValueError("the vocabulary axis of the logits must be contiguous")
+    b, s, v = logits.shape
+    r = _lib.NrlRows()
+    r.logits = logits.data_ptr()
+    r.dtype = _dtype_code(logits)
+    r.n_outer, r.n_inner, r.vocab = b, s, v
+    r.stride_outer, r.stride_inner = logits.stride(0), logits.stride(1)
+    r.targets = None
+    r.tgt_stride_outer = r.tgt_stride_inner = 0
+    r.vocab_start, r.vocab_end = vocab_start, (vocab_start + v if vocab_end is None else vocab_end)
+    r.temperature, r.temp_mode = 1.0, _lib.NRL_TEMP_RCP
+    return r
+
+
+def _row_scalar(t, b, s, name):
+    if t.dtype != torch.float32 or tuple(t.shape) != (b, s):
+        raise ValueError(f"{name} must be fp32 [{b}, {s}], got {t.dtype} {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def _neg_entropy_fwd(logits):
+    _need_gpu(logits)
+    rows = _plain_rows(logits)
+    b, s, _ = logits.shape
+    with torch.cuda.device(logits.device):
+        h = torch.empty((b, s), dtype=torch.float32, device=logits.device)
+        lse = torch.empty((b, s), dtype=torch.float32, device=logits.device)
+        with _timed("neg_entropy_fwd"):
+            code = _lib.load().nrl_neg_entropy_fwd(C.byref(rows), _ptr(h), _ptr(lse), _stream())
+    _lib.check(code, "nrl_neg_entropy_fwd")
+    return h, lse
+
+
+def _neg_entropy_bwd(logits, lse, h, grad):
+    _need_gpu(logits, lse, h, grad)
+    rows = _plain_rows(logits)
+    b, s, _ = logits.shape
+    lse, h, grad = _row_scalar(lse, b, s, "lse"), _row_scalar(h, b, s, "h"), _row_scalar(grad, b, s, "grad")
+    with torch.cuda.device(logits.device):
+        d = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+        with _timed("neg_entropy_bwd"):
+            code = _lib.load().nrl_neg_entropy_bwd(C.byref(rows), _ptr(lse), _ptr(h), _ptr(grad), _ptr(d), d.stride(0), d.stride(1), _stream())
+    _lib.check(code, "nrl_neg_entropy_bwd")
+    return d
+
+
+def _gather_indices(logits, indices):
+    b, s, _ = logits.shape
+    if indices.dtype != torch.int64 or indices.dim() != 3 or tuple(indices.shape[:2]) != (b, s):
+        raise ValueError(f"indices must be int64 [{b}, {s}, K], got {indices.dtype} {tuple(indices.shape)}")
+    return indices.contiguous()
+
+
+def _gather_logprob_fwd(logits, indices, vocab_start, vocab_end):
+    _need_gpu(logits, indices)
+    rows = _plain_rows(logits, vocab_start, vocab_end)
+    indices = _gather_indices(logits, indices)
+    b, s, k = indices.shape
+    with torch.cuda.device(logits.device):
+        out = torch.empty((b, s, k), dtype=torch.float32, device=logits.device)
+        lse = torch.empty((b, s), dtype=torch.float32, device=logits.device)
+        with _timed("gather_logprob_fwd"):
+            code = _lib.load().nrl_gather_logprob_fwd(C.byref(rows), _ptr(indices), k, _ptr(out), _ptr(lse), _stream())
+    _lib.check(code, "nrl_gather_logprob_fwd")
+    return out, lse
+
+
+def _gather_logprob_bwd(logits, indices, vocab_start, vocab_end, lse, grad):
+    _need_gpu(logits, indices, lse, grad)
+    rows = _plain_rows(logits, vocab_start, vocab_end)
+    indices = _gather_indices(logits, indices)
+    b, s, k = indices.shape
+    lse = _row_scalar(lse, b, s, "lse")
+    if grad.dtype != torch.float32 or tuple(grad.shape) != (b, s, k):
+        raise ValueError(f"grad must be fp32 [{b}, {s}, {k}], got {grad.dtype} {tuple(grad.shape)}")
+    grad = grad.contiguous()
+    with torch.cuda.device(logits.device):
+        d = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+        with _timed("gather_logprob_bwd"):
+            code = _lib.load().nrl_gather_logprob_bwd(C.byref(rows), _ptr(indices), k, _ptr(lse), _ptr(grad), _ptr(d),
+                                                      d.stride(0), d.stride(1), _stream())
+    _lib.check(code, "nrl_gather_logprob_bwd")
+    return d
+
+
+def _teacher_like(student, teacher):
+    if teacher.shape != student.shape:
+        raise ValueError(f"student_logits and target_logits must have the same shape, got {tuple(student.shape)} and {tuple(teacher.shape)}.")
+    if teacher.dtype != student.dtype:
+        teacher = teacher.to(student.dtype)
+    if teacher.stride(2) != 1 and teacher.shape[2] > 1:
+        teacher = teacher.contiguous()
+    return teacher
+
+
+def _soft_cross_entropy_fwd(student, teacher):
+    _need_gpu(student, teacher)
+    rows = _plain_rows(student)
+    teacher = _teacher_like(student, teacher)
+    b, s, _ = student.shape
+    with torch.cuda.device(student.device):
+        ce, lx, ly = (torch.empty((b, s), dtype=torch.float32, device=student.device) for _ in range(3))
+        with _timed("soft_cross_entropy_fwd"):
+            code = _lib.load().nrl_soft_cross_entropy_fwd(C.byref(rows), _ptr(teacher), teacher.stride(0), teacher.stride(1),
+                                                          _ptr(ce), _ptr(lx), _ptr(ly), _stream())
+    _lib.check(code, "nrl_soft_cross_entropy_fwd")
+    return ce, lx, ly
+
+
+def _soft_cross_entropy_bwd(student, teacher, lse_student, lse_teacher, grad):
+    _need_gpu(student, teacher, lse_student, lse_teacher, grad)
+    rows = _plain_rows(student)
+    teacher = _teacher_like(student, teacher)
+    b, s, _ = student.shape
+    lx, ly, grad = _row_scalar(lse_student, b, s, "lse_student"), _row_scalar(lse_teacher, b, s, "lse_teacher"), _row_scalar(grad, b, s, "grad")
+    with torch.cuda.device(student.device):
+        d = torch.empty(student.shape, dtype=student.dtype, device=student.device)
+        with _timed("soft_cross_entropy_bwd"):
+            code = _lib.load().nrl_soft_cross_entropy_bwd(C.byref(rows), _ptr(teacher), teacher.stride(0), teacher.stride(1),
+                                                          _ptr(lx), _ptr(ly), _ptr(grad), _ptr(d), d.stride(0), d.stride(1), _stream())
+    _lib.check(code, "nrl_soft_cross_entropy_bwd")
+    return d
+
+
+for _name, _fn in (("neg_entropy_fwd", _neg_entropy_fwd), ("neg_entropy_bwd", _neg_entropy_bwd),
+                   ("gather_logprob_fwd", _gather_logprob_fwd), ("gather_logprob_bwd", _gather_logprob_bwd),
+                   ("soft_cross_entropy_fwd", _soft_cross_entropy_fwd), ("soft_cross_entropy_bwd", _soft_cross_entropy_bwd)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
+# ------------------------------------------------------------------------------------------------
 # K6: fused lm_head
 # ------------------------------------------------------------------------------------------------
 _LIB.define(
