@@ -77,7 +77,9 @@ class _FusedLogitsLoss(torch.autograd.Function):
         (dlogits,) = ctx.saved_tensors
         factor = float(grad_loss) / ctx.loss_scale
         if factor != 1.0:
-            dlogits = (dlogits.float() * factor).to(dlogits.dtype)
+            # the stored gradient was final for the announced loss_scale; any other upstream factor costs one
+            # more pass (computed in fp32 per element, no fp32 copy of the tensor)
+            dlogits = dlogits * factor
         return (dlogits,) + (None,) * 13
 
 
