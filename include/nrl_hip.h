@@ -218,6 +218,21 @@ int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_cfg* cfg, co
                                int64_t d_stride_inner, float* logprob_out, float* loss_out,
                                float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same single pass over a packed microbatch: `rows` describes the one packed row (n_outer 1,
+ * n_inner = total positions, stride_inner = row stride, targets = packed ids [total] with stride 1),
+ * sequence s occupies positions [cu_seqlens[s], cu_seqlens[s+1]) and the loss inputs are [n_seq, in->sm1]
+ * with in->sm1 = unpacked_seqlen - 1.  Replaces SequencePackingFusionLossWrapper.__call__ =
+ * prepare_packed_loss_input + ClippedPGLossFn + backward (nemo_rl/algorithms/loss/wrapper.py:169-228,
+ * loss/utils.py:214-385) at CP = 1.  Position p of a sequence uses target cu[s] + p + 1 (cu[s] + p when
+ * the targets are pre-rolled); the last position of every sequence, positions past unpacked_seqlen - 1 and
+ * positions outside every sequence get a zero gradient row.  dlogits: [total, vocab] rows of d_row_stride.
+ * workspace: nrl_fused_workspace_bytes(n_seq, in->sm1). */
+int nrl_fused_packed_logits_grpo_loss(const nrl_rows* rows, int32_t target_is_pre_rolled, const int32_t* cu_seqlens,
+                                      int64_t n_seq, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
+                                      float loss_scale, void* dlogits, int64_t d_row_stride, float* logprob_out,
+                                      float* loss_out, float* metrics_out, void* workspace, int64_t workspace_bytes,
+                                      void* stream);
+
 /* NLLLossFn scalar branch (loss_functions.py:818-842): loss = -sum(lp*mask)/(Gt+1e-8);
  * metrics_out[0..2] = {loss, num_unmasked_tokens, num_valid_samples}; dlp_out = -mask/(Gt+1e-8). */
 int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,

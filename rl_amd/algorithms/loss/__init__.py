@@ -1,6 +1,11 @@
 """Loss functions of the GRPO hot path (counterpart of ``nemo_rl/algorithms/loss/__init__.py``)."""
 
-from .fused import fused_logits_clipped_pg_loss, why_not_fusable
+from .fused import (
+    fused_logits_clipped_pg_loss,
+    fused_packed_logits_clipped_pg_loss,
+    why_not_fusable,
+    why_not_fusable_packed,
+)
 from .interfaces import LossFunction, LossInputType, LossType, MetricNormalizer
 from .loss_functions import ClippedPGLossConfig, ClippedPGLossFn, NLLLossFn
 from .utils import prepare_loss_input, prepare_packed_loss_input
@@ -11,7 +16,8 @@ from .wrapper import (
 )
 
 __all__ = [
-    "fused_logits_clipped_pg_loss", "why_not_fusable", "ClippedPGLossConfig", "ClippedPGLossFn", "NLLLossFn", "LossFunction", "LossInputType", "LossType",
+    "fused_logits_clipped_pg_loss", "fused_packed_logits_clipped_pg_loss", "why_not_fusable", "why_not_fusable_packed",
+    "ClippedPGLossConfig", "ClippedPGLossFn", "NLLLossFn", "LossFunction", "LossInputType", "LossType",
     "MetricNormalizer", "prepare_loss_input", "prepare_packed_loss_input", "SequencePackingFusionLossWrapper",
     "SequencePackingLossWrapper", "wrap_loss_fn_with_input_preparation",
 ]

@@ -55,6 +55,33 @@ def why_not_fusable(loss_fn, logits, data, sampling_params=None) -> Optional[str
     return None
 
 
+def _metrics_dict(metrics, loss_fn, sample_mask_in):
+    beta = loss_fn.reference_policy_kl_penalty
+    m = metrics.cpu().tolist()
+    get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
+    n_valid = get("num_valid_samples")
+    out = {
+        "loss": get("loss"),
+        "probs_ratio": get("probs_ratio"),
+        "probs_ratio_clamped": get("probs_ratio_clamped"),
+        "probs_ratio_min": get("probs_ratio_min"),
+        "probs_ratio_max": get("probs_ratio_max"),
+        "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
+        "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
+        "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
+        "token_mult_prob_error": get("token_mult_prob_error"),
+        "gen_kl_error": get("gen_kl_error"),
+        "policy_kl_error": get("policy_kl_error"),
+        "js_divergence_error": get("js_divergence_error"),
+        "sampling_importance_ratio": get("sampling_importance_ratio"),
+        "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
+        "approx_entropy": get("approx_entropy"),
+    }
+    if loss_fn.truncated_importance_sampling_ratio is not None:
+        out["is_oob_ratio"] = get("is_oob_ratio")
+    out["positive_nll_loss"] = get("positive_nll_loss")
+    return out
+
 class _FusedLogitsLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams,
@@ -119,27 +146,66 @@ def fused_logits_clipped_pg_loss(
         _f32(data["advantages"][:, 1:], dev), _f32(data["token_mask"][:, 1:], dev), _f32(sample_mask_in, dev),
         _global_valid(global_valid_seqs, global_valid_toks, dev), iflags, fparams, float(loss_scale), bool(in_place),
     )
-    m = metrics.cpu().tolist()
-    get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
-    n_valid = get("num_valid_samples")
-    out = {
-        "loss": get("loss"),
-        "probs_ratio": get("probs_ratio"),
-        "probs_ratio_clamped": get("probs_ratio_clamped"),
-        "probs_ratio_min": get("probs_ratio_min"),
-        "probs_ratio_max": get("probs_ratio_max"),
-        "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
-        "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
-        "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
-        "token_mult_prob_error": get("token_mult_prob_error"),
-        "gen_kl_error": get("gen_kl_error"),
-        "policy_kl_error": get("policy_kl_error"),
-        "js_divergence_error": get("js_divergence_error"),
-        "sampling_importance_ratio": get("sampling_importance_ratio"),
-        "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
-        "approx_entropy": get("approx_entropy"),
-    }
-    if loss_fn.truncated_importance_sampling_ratio is not None:
-        out["is_oob_ratio"] = get("is_oob_ratio")
-    out["positive_nll_loss"] = get("positive_nll_loss")
-    return loss, out
+    return loss, _metrics_dict(metrics, loss_fn, sample_mask_in)
+
+
+
+class _FusedPackedLogitsLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits2d, targets, cu, unpacked_seqlen, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags,
+                fparams, loss_scale):
+        loss, dlogits, lp, metrics = _OPS.fused_packed_logits_grpo_loss(
+            logits2d.detach(), targets, True, cu, unpacked_seqlen, prev, gen, ref, adv, token_mask, sample_mask, global_valid,
+            iflags, fparams, loss_scale)
+        ctx.save_for_backward(dlogits)
+        ctx.loss_scale = loss_scale
+        ctx.mark_non_differentiable(lp, metrics)
+        return loss, lp, metrics
+
+    @staticmethod
+    def backward(ctx, grad_loss, _g_lp, _g_metrics):
+        (dlogits,) = ctx.saved_tensors
+        factor = float(grad_loss) / ctx.loss_scale
+        if factor != 1.0:
+            dlogits = dlogits * factor
+        return (dlogits,) + (None,) * 13
+
+
+def why_not_fusable_packed(loss_fn, logits, data, sampling_params=None) -> Optional[str]:
+    """As ``why_not_fusable`` for a packed ``[1, T, V]`` microbatch."""
+    if not isinstance(logits, torch.Tensor) or logits.dim() != 3 or logits.shape[0] != 1:
+        return "logits are not a packed [1, T, V] tensor"
+    probe = dict(data)
+    probe["input_ids"] = data["input_ids"][:, :1]  # the shape test of the unpacked path does not apply
+    return why_not_fusable(loss_fn, logits, probe, sampling_params)
+
+
+def fused_packed_logits_clipped_pg_loss(logits, data, loss_fn, cu_seqlens_q, cu_seqlens_q_padded, global_valid_seqs,
+                                        global_valid_toks, *, loss_scale: float = 1.0):
+    """``SequencePackingFusionLossWrapper.__call__`` (``loss/wrapper.py:169-228``) in one pass over the packed
+    logits: ``prepare_packed_loss_input`` + ``ClippedPGLossFn`` + the backward of the packed logprob op."""
+    from .utils import _pack_input_ids, _pad_to
+
+    reason = why_not_fusable_packed(loss_fn, logits, data)
+    if reason is not None:
+        raise NotImplementedError(f"fused packed logits->loss path: {reason}")
+    from ...distributed.model_utils import _checked_cu_seqlens
+
+    dev = logits.device
+    input_ids = data["input_ids"]
+    x = logits.squeeze(0)
+    targets = _pad_to(_pack_input_ids(input_ids, cu_seqlens_q, cu_seqlens_q_padded, roll_shift=-1), x.shape[0])
+    targets = targets.to(dev).reshape(-1).long().contiguous()
+    cu = _checked_cu_seqlens(cu_seqlens_q_padded, x.shape[0], targets.shape[0], dev)
+    beta = loss_fn.reference_policy_kl_penalty
+    sample_mask_in = data["sample_mask"]
+    prev = None if loss_fn.force_on_policy_ratio else _f32(data["prev_logprobs"][:, 1:], dev)
+    ref = _f32(data["reference_policy_logprobs"][:, 1:], dev) if beta != 0 else None
+    iflags, fparams = loss_fn._kernel_config(False)
+    loss, _lp, metrics = _FusedPackedLogitsLoss.apply(
+        x, targets, cu, input_ids.shape[1], prev,
+        _f32(data["generation_logprobs"][:, 1:], dev), ref, _f32(data["advantages"][:, 1:], dev),
+        _f32(data["token_mask"][:, 1:], dev), _f32(sample_mask_in, dev),
+        _global_valid(global_valid_seqs, global_valid_toks, dev), iflags, fparams, float(loss_scale),
+    )
+    return loss, _metrics_dict(metrics, loss_fn, sample_mask_in)

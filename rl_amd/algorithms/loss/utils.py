@@ -95,6 +95,12 @@ def _pack_input_ids(
     return packed.unsqueeze(0)
 
 
+def _pad_to(packed_ids: torch.Tensor, total: int) -> torch.Tensor:
+    """Zero ids for packed positions behind the last sequence (a row padded past ``cu_seqlens_padded[-1]``)."""
+    short = total - packed_ids.shape[1]
+    return torch.nn.functional.pad(packed_ids, (0, short)) if short > 0 else packed_ids
+
+
 def prepare_packed_loss_input(
     logits: torch.Tensor,
     data: Any,
@@ -117,7 +123,7 @@ def prepare_packed_loss_input(
     input_ids = data["input_ids"]
     rank = vocab_parallel_rank or 0
     vocab = logits.shape[-1]
-    targets = _pack_input_ids(input_ids, cu_seqlens_q, cu_seqlens_q_padded, roll_shift=-1)
+    targets = _pad_to(_pack_input_ids(input_ids, cu_seqlens_q, cu_seqlens_q_padded, roll_shift=-1), logits.shape[1])
 
     def logprobs_with(params):
         return from_parallel_logits_to_logprobs_packed_sequences(

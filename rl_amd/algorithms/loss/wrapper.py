@@ -90,6 +90,20 @@ class SequencePackingFusionLossWrapper:
         self.context_parallel_group = context_parallel_group
 
     def __call__(self, next_token_logits, data, global_valid_seqs, global_valid_toks):
+        from .fused import fused_packed_logits_clipped_pg_loss, why_not_fusable_packed
+        from .utils import prepare_packed_loss_input
+
+        # a ClippedPGLossFn whose token gradient needs no other token's logprob: logits -> loss -> gradient
+        # in one pass over the packed row, as in wrap_loss_fn_with_input_preparation
+        if (self.prepare_fn is prepare_packed_loss_input and torch.is_grad_enabled()
+                and isinstance(next_token_logits, torch.Tensor) and next_token_logits.requires_grad
+                and why_not_fusable_packed(self.loss_fn, next_token_logits, data) is None):
+            from ...distributed.model_utils import _group_size
+
+            if _group_size(self.vocab_parallel_group) == 1 and _group_size(self.context_parallel_group) == 1:
+                return fused_packed_logits_clipped_pg_loss(
+                    next_token_logits, data, self.loss_fn, self.cu_seqlens_q, self.cu_seqlens_q_padded,
+                    global_valid_seqs, global_valid_toks)
         loss_input, prepared = self.prepare_fn(
             logits=next_token_logits, data=data, loss_fn=self.loss_fn, cu_seqlens_q=self.cu_seqlens_q,
             cu_seqlens_q_padded=self.cu_seqlens_q_padded, vocab_parallel_rank=self.vocab_parallel_rank,

@@ -279,7 +279,44 @@ struct FusedArgs {
     float* seq_stats;  // [B, 3]: seq_den, seq_w, seq_keep
     float* terms;      // [B * n_inner, T_COUNT]
     double* parts;     // [B, P_COUNT]
+    // packed mode (cu != NULL): the logits are one row of `total` positions, sequence s occupies
+    // [cu[s], cu[s+1]); the loss inputs stay [n_seq, n_inner]
+    const int32_t* cu;
+    int64_t n_seq;
+    int pre_rolled;
 };
+
+// where a logits row sits in the loss inputs: sequence o, position i (i >= n_inner: the row feeds no token),
+// and the index of its target id
+struct FusedPos {
+    int64_t o, i, tgt;
+};
+template <bool PACKED>
+__device__ __forceinline__ FusedPos fused_where(const FusedArgs& a, int64_t r) {
+    FusedPos q;
+    if (!PACKED) {
+        q.o = r / a.d_n_inner;
+        q.i = r - q.o * a.d_n_inner;
+        q.tgt = q.o * a.ts_outer + q.i * a.ts_inner;
+        return q;
+    }
+    const int64_t seq = find_seq(a.cu, a.n_seq, r);
+    q.o = seq < 0 ? 0 : seq;
+    q.i = a.n_inner;
+    q.tgt = 0;
+    if (seq >= 0) {
+        const int64_t start = a.cu[seq], len = a.cu[seq + 1] - start, pos = r - start;
+        if (pos + 1 < len && pos < a.n_inner) q.i = pos;  // the last position of a sequence predicts nothing
+        q.tgt = start + (a.pre_rolled ? pos : (pos + 1 < len ? pos + 1 : 0));
+    }
+    return q;
+}
+template <bool PACKED>
+__device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& a, int64_t r, int64_t so, int64_t si) {
+    if (PACKED) return r * si;
+    const int64_t o = r / a.d_n_inner;
+    return o * so + (r - o * a.d_n_inner) * si;
+}
 
 __global__ __launch_bounds__(kLossBlock) void grpo_seq_stats_kernel(FusedArgs a) {
     __shared__ double sm_d[kLossWaves];
@@ -321,7 +358,12 @@ __global__ __launch_bounds__(kLossBlock) void grpo_seq_stats_kernel(FusedArgs a)
 // register slots (vector q - kFusedLdsVec).
 // NREG is the number of register slots the instantiation carries (the row must fit NREG + kFusedLdsVec
 // slots); shorter rows take a smaller instantiation instead of idling through unused slots.
-template <int DT, int TEMP, int NREG>
+__global__ void fused_fill_zero_kernel(float* p, int64_t n) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+        p[i] = 0.f;
+}
+
+template <int DT, int TEMP, int NREG, bool PACKED>
 __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArgs a, int64_t n_rows) {
     constexpr int EPV = Row<DT>::EPV;
     constexpr int kFusedRegVec = NREG, kFusedVec = NREG + kFusedLdsVec;
@@ -337,12 +379,10 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
     const u32x4 zero = {0u, 0u, 0u, 0u};
 
     auto out_row = [&](int64_t r) -> char* {
-        const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
-        return static_cast<char*>(a.dlogits) + (o * a.ds_outer + i * a.ds_inner) * Row<DT>::BYTES;
+        return static_cast<char*>(a.dlogits) + fused_row_offset<PACKED>(a, r, a.ds_outer, a.ds_inner) * Row<DT>::BYTES;
     };
     auto in_row = [&](int64_t r) -> const char* {
-        const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
-        return static_cast<const char*>(a.logits) + (o * a.stride_outer + i * a.stride_inner) * Row<DT>::BYTES;
+        return static_cast<const char*>(a.logits) + fused_row_offset<PACKED>(a, r, a.stride_outer, a.stride_inner) * Row<DT>::BYTES;
     };
     // Slot q holds vector slot_vec(q) of the row.  Lanes past the end of the row are pointed at the
     // row's last vector instead: they load, compute and store exactly what that vector's own lane does
@@ -363,7 +403,8 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
     // over are dropped positions or masked tokens: zero gradient, logprob reported as 0, nothing read.
     auto advance = [&](int64_t r) -> int64_t {
         for (; r < n_rows; r += step) {
-            const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+            const FusedPos q = fused_where<PACKED>(a, r);
+            const int64_t o = q.o, i = q.i;
             float w = 0.f;
             if (i < a.n_inner) w = in.token_mask[o * in.token_mask_stride + i] * in.sample_mask[o];
             if (w != 0.f) break;
@@ -416,12 +457,13 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
         for (int q = 0; q < kFusedLdsVec; ++q) fold(q);
     }
     while (r < n_rows) {
-        const int64_t o = r / a.d_n_inner, i = r - o * a.d_n_inner;
+        const FusedPos where = fused_where<PACKED>(a, r);
+        const int64_t o = where.o, i = where.i;
         const int64_t tok = o * a.n_inner + i;
         const char* row = in_row(r);
         char* ov = out_row(r);
         const Lse tot = block_lse<kFusedWaves>(acc, sm_l);
-        const int64_t tg = a.targets[o * a.ts_outer + i * a.ts_inner];
+        const int64_t tg = a.targets[where.tgt];
         const int64_t tloc = (tg >= a.vstart && tg < a.vend) ? tg - a.vstart : -1;
         if (tid == 0) {
             const float log_s = logf(tot.s);
@@ -594,14 +636,17 @@ extern "C" int64_t nrl_fused_workspace_bytes(int64_t batch, int64_t n_inner) {
     return align8(b * 3 * 4) + align8(b * n * T_COUNT * 4) + b * P_COUNT * 8;
 }
 
-extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
-                                          float loss_scale, void* dlogits, int64_t d_n_inner, int64_t d_stride_outer,
-                                          int64_t d_stride_inner, float* logprob_out, float* loss_out, float* metrics_out,
-                                          void* workspace, int64_t workspace_bytes, void* stream) {
+// rows describes the logits; with cu != NULL it is one packed row of rows->n_inner positions (n_outer 1) and
+// the loss inputs are [n_seq, in->sm1]
+static int fused_impl(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float loss_scale, void* dlogits,
+                      int64_t d_n_inner, int64_t d_stride_outer, int64_t d_stride_inner, float* logprob_out, float* loss_out,
+                      float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream, const int32_t* cu,
+                      int64_t n_seq, int pre_rolled) {
     if (!rows || !cfg || !in) return fail(NRL_E_INVALID, "null argument");
     if (rows->dtype != NRL_F32 && rows->dtype != NRL_BF16 && rows->dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype");
     if (rows->n_outer < 0 || rows->n_inner < 0 || rows->vocab <= 0 || d_n_inner < rows->n_inner) return fail(NRL_E_INVALID, "bad shape");
-    if (in->batch != rows->n_outer || in->sm1 != rows->n_inner) return fail(NRL_E_INVALID, "loss inputs and logits rows disagree");
+    if (!cu && (in->batch != rows->n_outer || in->sm1 != rows->n_inner)) return fail(NRL_E_INVALID, "loss inputs and logits rows disagree");
+    if (cu && (in->batch != n_seq || rows->n_outer != 1 || n_seq < 0)) return fail(NRL_E_INVALID, "packed loss inputs and cu_seqlens disagree");
     if (rows->vocab_end - rows->vocab_start != rows->vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
     if (!(rows->temperature > 0.f)) return fail(NRL_E_INVALID, "temperature must be positive");
     const bool gspo = cfg->sequence_level_importance_ratios && !cfg->disable_ppo_ratio && !cfg->force_on_policy_ratio;
@@ -612,7 +657,7 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     const bool seq_weights = cfg->sequence_level_importance_ratios || cfg->tis_type == NRL_TIS_SEQ_MASK;
     if (seq_weights && cfg->force_on_policy_ratio)
         return fail(NRL_E_UNSUPPORTED, "sequence-level importance weights with force_on_policy_ratio depend on the current logprobs");
-    if (seq_weights && rows->n_outer * rows->n_inner > 0 && !in->prev) return fail(NRL_E_INVALID, "prev_logprobs is NULL");
+    if (seq_weights && in->batch * in->sm1 > 0 && !in->prev) return fail(NRL_E_INVALID, "prev_logprobs is NULL");
     if (cfg->kl_type < 1 || cfg->kl_type > 3 || cfg->tis_type < 0 || cfg->tis_type > 3) return fail(NRL_E_INVALID, "bad kl_type or tis_type");
     const int bytes = rows->dtype == NRL_F32 ? 4 : 2, epv = 16 / bytes;
     if (rows->vocab % epv || rows->vocab / epv > static_cast<int64_t>(kFusedMaxVec) * kFusedBlock)
@@ -624,7 +669,7 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     const int64_t n_rows = rows->n_outer * d_n_inner;
     if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
     if (!loss_out || !metrics_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
-    if (workspace_bytes < nrl_fused_workspace_bytes(rows->n_outer, rows->n_inner)) return fail(NRL_E_WORKSPACE, "workspace too small");
+    if (workspace_bytes < nrl_fused_workspace_bytes(in->batch, in->sm1)) return fail(NRL_E_WORKSPACE, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 7) return fail(NRL_E_INVALID, "workspace must be 8-byte aligned");
     if (n_rows > 0) {
         if (!rows->logits || !rows->targets || !dlogits || !logprob_out) return fail(NRL_E_INVALID, "null logits, targets or output");
@@ -636,7 +681,8 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     a.cfg = *cfg;
     a.in = *in;
     a.in.lp = nullptr; a.in.lpu = nullptr;
-    a.logits = rows->logits; a.n_inner = rows->n_inner; a.d_n_inner = d_n_inner; a.vocab = rows->vocab;
+    a.cu = cu; a.n_seq = n_seq; a.pre_rolled = pre_rolled;
+    a.logits = rows->logits; a.n_inner = in->sm1; a.d_n_inner = d_n_inner; a.vocab = rows->vocab;
     a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
     a.targets = rows->targets; a.ts_outer = rows->tgt_stride_outer; a.ts_inner = rows->tgt_stride_inner;
     a.vstart = rows->vocab_start; a.vend = rows->vocab_end;
@@ -644,8 +690,8 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     a.dlogits = dlogits; a.ds_outer = d_stride_outer; a.ds_inner = d_stride_inner;
     a.lp_out = logprob_out;
     char* ws = static_cast<char*>(workspace);
-    a.seq_stats = reinterpret_cast<float*>(ws); ws += align8(rows->n_outer * 3 * 4);
-    a.terms = reinterpret_cast<float*>(ws); ws += align8(rows->n_outer * (rows->n_inner < 1 ? 1 : rows->n_inner) * T_COUNT * 4);
+    a.seq_stats = reinterpret_cast<float*>(ws); ws += align8(in->batch * 3 * 4);
+    a.terms = reinterpret_cast<float*>(ws); ws += align8(in->batch * (in->sm1 < 1 ? 1 : in->sm1) * T_COUNT * 4);
     a.parts = reinterpret_cast<double*>(ws);
     int tc = 0;
     a.tparam = 1.f;
@@ -654,8 +700,13 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
         else { tc = 2; a.tparam = 1.0f / rows->temperature; }
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const unsigned nb = static_cast<unsigned>(rows->n_outer);
+    const unsigned nb = static_cast<unsigned>(in->batch);
     if (nb > 0) grpo_seq_stats_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);
+    if (cu && in->batch * in->sm1 > 0) {
+        // positions past a sequence's end have no packed row: their records and logprobs start at zero
+        fused_fill_zero_kernel<<<dim3(1024), dim3(256), 0, s>>>(a.terms, in->batch * in->sm1 * T_COUNT);
+        fused_fill_zero_kernel<<<dim3(256), dim3(256), 0, s>>>(a.lp_out, in->batch * in->sm1);
+    }
     if (n_rows > 0) {
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
@@ -664,12 +715,15 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
         const dim3 grid((unsigned)(n_rows < cus ? n_rows : cus)), block(kFusedBlock);
         const int64_t slots = (rows->vocab / epv + kFusedBlock - 1) / kFusedBlock;
         const int nreg = slots <= 8 ? 4 : slots <= 12 ? 8 : slots <= 16 ? 12 : 16;
+#define NRL_FUSED_LAUNCH(DT_, TC_, NR_)                                                                           \
+    if (cu) fused_logits_loss_kernel<DT_, TC_, NR_, true><<<grid, block, 0, s>>>(a, n_rows);                      \
+    else fused_logits_loss_kernel<DT_, TC_, NR_, false><<<grid, block, 0, s>>>(a, n_rows)
 #define NRL_FUSED_CASE(DT_, TC_)                                                                                  \
     case DT_ * 3 + TC_:                                                                                           \
-        if (nreg == 4) fused_logits_loss_kernel<DT_, TC_, 4><<<grid, block, 0, s>>>(a, n_rows);                   \
-        else if (nreg == 8) fused_logits_loss_kernel<DT_, TC_, 8><<<grid, block, 0, s>>>(a, n_rows);              \
-        else if (nreg == 12) fused_logits_loss_kernel<DT_, TC_, 12><<<grid, block, 0, s>>>(a, n_rows);            \
-        else fused_logits_loss_kernel<DT_, TC_, 16><<<grid, block, 0, s>>>(a, n_rows);                            \
+        if (nreg == 4) { NRL_FUSED_LAUNCH(DT_, TC_, 4); }                                                         \
+        else if (nreg == 8) { NRL_FUSED_LAUNCH(DT_, TC_, 8); }                                                    \
+        else if (nreg == 12) { NRL_FUSED_LAUNCH(DT_, TC_, 12); }                                                  \
+        else { NRL_FUSED_LAUNCH(DT_, TC_, 16); }                                                                  \
         break;
         switch (rows->dtype * 3 + tc) {
             NRL_FUSED_CASE(NRL_F32, 0) NRL_FUSED_CASE(NRL_F32, 1) NRL_FUSED_CASE(NRL_F32, 2)
@@ -678,6 +732,7 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
             default: return fail(NRL_E_INVALID, "unknown logits dtype");
         }
 #undef NRL_FUSED_CASE
+#undef NRL_FUSED_LAUNCH
     }
     if (nb > 0) grpo_terms_reduce_kernel<<<dim3(nb), dim3(kLossBlock), 0, s>>>(a);
     GrpoArgs fa;
@@ -687,4 +742,23 @@ extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_c
     fa.parts = a.parts;
     grpo_finish_kernel<<<dim3(1), dim3(kLossBlock), 0, s>>>(fa, loss_out, metrics_out);
     return check_launch("fused_logits_grpo_loss");
+}
+
+extern "C" int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
+                                          float loss_scale, void* dlogits, int64_t d_n_inner, int64_t d_stride_outer,
+                                          int64_t d_stride_inner, float* logprob_out, float* loss_out, float* metrics_out,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
+    return fused_impl(rows, cfg, in, loss_scale, dlogits, d_n_inner, d_stride_outer, d_stride_inner, logprob_out, loss_out,
+                      metrics_out, workspace, workspace_bytes, stream, nullptr, 0, 0);
+}
+
+extern "C" int nrl_fused_packed_logits_grpo_loss(const nrl_rows* rows, int32_t target_is_pre_rolled, const int32_t* cu_seqlens,
+                                                 int64_t n_seq, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
+                                                 float loss_scale, void* dlogits, int64_t d_row_stride, float* logprob_out,
+                                                 float* loss_out, float* metrics_out, void* workspace, int64_t workspace_bytes,
+                                                 void* stream) {
+    if (!cu_seqlens) return fail(NRL_E_INVALID, "cu_seqlens is NULL");
+    if (rows && rows->tgt_stride_inner != 1) return fail(NRL_E_INVALID, "packed targets must be contiguous");
+    return fused_impl(rows, cfg, in, loss_scale, dlogits, rows ? rows->n_inner : 0, 0, d_row_stride, logprob_out, loss_out,
+                      metrics_out, workspace, workspace_bytes, stream, cu_seqlens, n_seq, target_is_pre_rolled);
 }

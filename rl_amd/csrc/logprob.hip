@@ -248,16 +248,6 @@ struct PackedArgs {
     float tparam;
 };
 
-// sequence index of packed position p, or -1 if p lies outside every sequence
-__device__ __forceinline__ int64_t find_seq(const int32_t* cu, int64_t n_seq, int64_t p) {
-    if (n_seq <= 0 || p < cu[0] || p >= cu[n_seq]) return -1;
-    int64_t lo = 0, hi = n_seq;  // invariant: cu[lo] <= p < cu[hi]
-    while (hi - lo > 1) {
-        const int64_t mid = (lo + hi) >> 1;
-        if (cu[mid] <= p) lo = mid; else hi = mid;
-    }
-    return lo;
-}
 
 struct PackedPos {
     int64_t seq, pos, len, start;

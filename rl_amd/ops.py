@@ -469,6 +469,60 @@ for _name, _fn in (("fused_logits_grpo_loss", _fused_logits_grpo_loss), ("fused_
     _LIB.impl(_name, _fn, "CUDA")
     _LIB.impl(_name, _fn, "CPU")
 
+_LIB.define(
+    "fused_packed_logits_grpo_loss(Tensor logits, Tensor targets, bool pre_rolled, Tensor cu_seqlens, int unpacked_seqlen, "
+    "Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, Tensor token_mask, Tensor sample_mask, Tensor global_valid, "
+    "int[] iflags, float[] fparams, float loss_scale) -> (Tensor, Tensor, Tensor, Tensor)"
+)
+
+
+def _fused_packed_logits_grpo_loss(logits, targets, pre_rolled, cu_seqlens, unpacked_seqlen, prev, gen, ref, adv, token_mask,
+                                   sample_mask, global_valid, iflags, fparams, loss_scale):
+    """Packed [T, V] logits -> (loss, dlogits [T, V], logprobs [n_seq, unpacked_seqlen - 1], metrics)."""
+    if len(iflags) != len(_CFG_INT) or len(fparams) != len(_CFG_FLT):
+        raise ValueError("malformed loss configuration")
+    _check_packed(logits, targets, cu_seqlens, unpacked_seqlen)
+    t, v = logits.shape
+    n_seq, n_inner = cu_seqlens.shape[0] - 1, unpacked_seqlen - 1
+    rows = _lib.NrlRows()
+    rows.logits = logits.data_ptr()
+    rows.dtype = _dtype_code(logits)
+    rows.n_outer, rows.n_inner, rows.vocab = 1, t, v
+    rows.stride_outer, rows.stride_inner = 0, logits.stride(0)
+    rows.targets = targets.data_ptr()
+    rows.tgt_stride_outer, rows.tgt_stride_inner = 0, 1
+    rows.vocab_start, rows.vocab_end = 0, v
+    rows.temperature, rows.temp_mode = 1.0, _lib.NRL_TEMP_RCP
+    dev = logits.device
+    lp = torch.empty((n_seq, n_inner), dtype=torch.float32, device=dev)
+    inp, keep, _, _ = _grpo_inputs(lp, None, prev, gen, ref, adv, token_mask, sample_mask, None, global_valid)
+    cfg = _lib.NrlGrpoCfg()
+    for name, val in zip(_CFG_INT, iflags):
+        setattr(cfg, name, int(val))
+    for name, val in zip(_CFG_FLT, fparams):
+        setattr(cfg, name, float(val))
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        metrics = torch.empty((_lib.NRL_GRPO_N_METRICS,), dtype=torch.float32, device=dev)
+        d = torch.empty((t, v), dtype=logits.dtype, device=dev)
+        ws_bytes = lib.nrl_fused_workspace_bytes(n_seq, n_inner)
+        ws = torch.empty(((ws_bytes + 7) // 8,), dtype=torch.float64, device=dev)
+        with _timed("fused_packed_logits_loss"):
+            code = lib.nrl_fused_packed_logits_grpo_loss(
+                C.byref(rows), int(pre_rolled), _ptr(cu_seqlens), n_seq, C.byref(cfg), C.byref(inp), float(loss_scale),
+                _ptr(d), d.stride(0), _ptr(lp), _ptr(loss), _ptr(metrics), _ptr(ws), ws.numel() * 8, _stream(),
+            )
+    if code == -2:
+        raise NotImplementedError(lib.nrl_last_error().decode(errors="replace"))
+    _lib.check(code, "nrl_fused_packed_logits_grpo_loss")
+    del keep
+    return loss, d, lp, metrics
+
+
+_LIB.impl("fused_packed_logits_grpo_loss", _fused_packed_logits_grpo_loss, "CUDA")
+_LIB.impl("fused_packed_logits_grpo_loss", _fused_packed_logits_grpo_loss, "CPU")
+
 
 def _nll_loss(lp, token_mask, sample_mask, global_valid):
     inp, keep, b, n = _grpo_inputs(lp, None, None, None, None, None, token_mask, sample_mask, None, global_valid)

@@ -214,3 +214,142 @@ def test_fused_row_lengths(dtype, vocab):
         assert err.max().item() <= 1e-4 * scale
     else:  # one narrowing to bf16 on top of the 1e-4
         assert bool((err <= xo.grad.abs() * (2.0 ** -8 + 1e-4) + 1e-4 * scale * 2.0 ** -8 + 1e-30).all())
+
+
+def _packed_case(lens, pads, width, vocab, dtype, seed, tail=0):
+    """Unpacked ``[B, width]`` loss data plus the packed ``[1, T, V]`` logits of the same sequences:
+    sequence i holds ``lens[i]`` tokens inside a span of ``lens[i] + pads[i]`` packed positions,
+    ``tail`` unused positions follow the last span."""
+    b = len(lens)
+    g = torch.Generator().manual_seed(seed)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    cup = torch.tensor([0] + list((torch.tensor(lens) + torch.tensor(pads)).cumsum(0)), dtype=torch.int32)
+    total = int(cup[-1]) + tail
+    logits = (torch.randn(1, total, vocab, generator=g) * 2.5).to(dtype)
+    ids = torch.zeros(b, width, dtype=torch.int64)
+    tm = torch.zeros(b, width, dtype=torch.int64)
+    for i, n in enumerate(lens):
+        ids[i, :n] = torch.randint(0, vocab, (n,), generator=g)
+        if n > 2:
+            tm[i, int(torch.randint(1, n - 1, (1,), generator=g)):n] = 1
+    sm = torch.ones(b, dtype=torch.int64)
+    if b > 2:
+        sm[1] = 0
+    targets = OL.pack_input_ids(ids, cu, cup, roll_shift=-1)
+    cur = OL.packed_logits_to_logprobs(logits.float()[:, : int(cup[-1])], targets, cup, width, target_is_pre_rolled=True)
+    pad = lambda t: torch.cat([torch.zeros(b, 1), t], 1)  # noqa: E731
+    noise = lambda: 0.05 * torch.randn(b, width - 1, generator=g)  # noqa: E731
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm,
+            "advantages": torch.randn(b, 1, generator=g).expand(b, width).contiguous(),
+            "prev_logprobs": pad(cur + noise()), "generation_logprobs": pad(cur + noise()),
+            "reference_policy_logprobs": pad(cur + noise())}
+    gs = sm.sum()
+    gt = (tm[:, 1:] * sm.unsqueeze(-1)).sum()
+    return logits, data, cu, cup, gs, gt
+
+
+PACKED_SHAPES = [
+    dict(lens=[9, 5, 12, 7], pads=[0, 0, 0, 0], width=12),
+    dict(lens=[9, 5, 12, 7], pads=[3, 1, 0, 5], width=14, tail=6),
+    dict(lens=[6, 0, 10, 1, 8], pads=[2, 4, 0, 3, 0], width=10),   # an empty and a one-token sequence
+]
+
+
+@pytest.mark.parametrize("cfg", [FUSABLE[0], FUSABLE[2], FUSABLE[3], FUSABLE[7], FUSABLE[9], FUSABLE[10]],
+                         ids=["0", "2", "3", "7", "9", "10"])
+@pytest.mark.parametrize("shape", PACKED_SHAPES, ids=["tight", "padded", "ragged"])
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 2000), (torch.bfloat16, 4096)])
+def test_fused_packed_matches_oracle_and_three_pass(cfg, shape, dtype, vocab):
+    from rl_amd.algorithms.loss import SequencePackingFusionLossWrapper, prepare_packed_loss_input
+    from rl_amd.algorithms.loss.fused import fused_packed_logits_clipped_pg_loss, why_not_fusable_packed
+
+    logits, data, cu, cup, gs, gt = _packed_case(vocab=vocab, dtype=dtype, seed=31 + len(cfg) + vocab, **shape)
+    width = data["input_ids"].shape[1]
+    xo = logits.to(torch.float32, copy=True).requires_grad_(True)
+    targets = OL.pack_input_ids(data["input_ids"], cu, cup, roll_shift=-1)
+    lp = OL.packed_logits_to_logprobs(xo[:, : int(cup[-1])], targets, cup, width, target_is_pre_rolled=True)
+    want, wm = O.clipped_pg_loss(O.LossConfig(**cfg), lp, data, gs, gt)
+    want.backward()
+
+    fn = ClippedPGLossFn(ClippedPGLossConfig(**cfg))
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    xg = logits.to(DEV).requires_grad_(True)
+    assert why_not_fusable_packed(fn, xg, ddev) is None
+    got, gm = fused_packed_logits_clipped_pg_loss(xg, ddev, fn, cu.to(DEV), cup.to(DEV), gs.to(DEV), gt.to(DEV))
+    got.backward()
+    assert _close(got.item(), want.item()), (got.item(), want.item())
+    assert set(gm) == set(wm)
+    for k in wm:
+        assert _close(float(gm[k]), float(wm[k]), rel=1e-4, abs_=1e-6), (k, gm[k], wm[k])
+
+    # the three-pass packed path on the same inputs; the wrapper itself takes the single pass
+    xu = logits.to(DEV).requires_grad_(True)
+    loss_input, d2 = prepare_packed_loss_input(xu, dict(ddev), fn, cu.to(DEV), cup.to(DEV))
+    un, _ = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    un.backward()
+    xw = logits.to(DEV).requires_grad_(True)
+    wrapped = SequencePackingFusionLossWrapper(fn, prepare_packed_loss_input, cu.to(DEV), cup.to(DEV))
+    lw, mw = wrapped(xw, dict(ddev), gs.to(DEV), gt.to(DEV))
+    lw.backward()
+    assert lw.item() == got.item() and torch.equal(xw.grad, xg.grad) and set(mw) == set(wm)
+    assert _close(got.item(), un.item(), rel=1e-5)
+
+    scale = xo.grad.abs().max().item() + 1e-30
+    gf, gu = xg.grad.float().cpu(), xu.grad.float().cpu()
+    if dtype == torch.float32:
+        assert (gf - xo.grad).abs().max().item() <= 1e-4 * scale
+        assert (gf - gu).abs().max().item() <= 1e-4 * scale
+    else:
+        ulp = 2.0 ** -8
+        assert bool(((gf - xo.grad).abs() <= xo.grad.abs() * (ulp + 1e-4) + 1e-4 * scale * ulp + 1e-30).all())
+        assert (gf == gu).float().mean().item() > 0.995
+    # rows that feed no token (padding inside a span, every sequence's last position, the unused tail,
+    # masked tokens) receive exactly zero
+    live = torch.zeros(logits.shape[1], dtype=torch.bool)
+    w = data["token_mask"][:, 1:] * data["sample_mask"].unsqueeze(-1)
+    for i in range(len(cup) - 1):
+        n = min(max(int(cup[i + 1] - cup[i]) - 1, 0), width - 1)
+        live[int(cup[i]) : int(cup[i]) + n] = w[i, :n] != 0
+    assert torch.all(gf[0][~live] == 0)
+
+
+def test_fused_packed_full_rows():
+    """A packed microbatch at a real vocabulary (19 on-chip slots) with more live rows than workgroups."""
+    from rl_amd.algorithms.loss import prepare_packed_loss_input
+    from rl_amd.algorithms.loss.fused import fused_packed_logits_clipped_pg_loss
+
+    lens = [70, 33, 120, 64, 90, 17, 101, 55]
+    logits, data, cu, cup, gs, gt = _packed_case(lens, [2, 7, 0, 0, 6, 7, 3, 1], 128, 151936, torch.bfloat16, seed=8)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    xg = logits.to(DEV).requires_grad_(True)
+    got, gm = fused_packed_logits_clipped_pg_loss(xg, ddev, fn, cu.to(DEV), cup.to(DEV), gs.to(DEV), gt.to(DEV))
+    got.backward()
+    xu = logits.to(DEV).requires_grad_(True)
+    loss_input, d2 = prepare_packed_loss_input(xu, dict(ddev), fn, cu.to(DEV), cup.to(DEV))
+    un, um = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    un.backward()
+    assert _close(got.item(), un.item(), rel=1e-5)
+    for k in um:
+        if k not in ("probs_ratio_min", "probs_ratio_max", "probs_ratio_clamped_min", "probs_ratio_clamped_max"):
+            assert _close(float(gm[k]), float(um[k]), rel=1e-4, abs_=1e-6), (k, gm[k], um[k])
+    assert (xg.grad.float() == xu.grad.float()).float().mean().item() > 0.995
+    lp_want = OL.packed_logits_to_logprobs(logits.float(), OL.pack_input_ids(data["input_ids"], cu, cup, roll_shift=-1),
+                                           cup, 128, target_is_pre_rolled=True)
+    got_lp = loss_input["next_token_logprobs"].detach().float().cpu()
+    assert (got_lp - lp_want).abs().max().item() <= 2e-3
+
+
+def test_fused_packed_rejects_what_it_cannot_take():
+    from rl_amd.algorithms.loss.fused import fused_packed_logits_clipped_pg_loss, why_not_fusable_packed
+
+    logits, data, cu, cup, gs, gt = _packed_case([5, 6], [0, 0], 8, 512, torch.float32, seed=3)
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    gspo = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, sequence_level_importance_ratios=True))
+    assert why_not_fusable_packed(gspo, logits.to(DEV), ddev) is not None
+    with pytest.raises(NotImplementedError):
+        fused_packed_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, gspo, cu, cup, gs, gt)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    with pytest.raises(ValueError):   # boundaries that leave the packed row
+        fused_packed_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, fn, cu,
+                                            torch.tensor([0, 5, 40], dtype=torch.int32), gs, gt)
