@@ -41,6 +41,9 @@ WORKLOADS = {
                desc="benchmark config 4: 64 seq x 8192 tok, V=151936 bf16, T=0.7, top_k=50, top_p=0.95, DAPO clip-higher, no KL"),
     "distill": dict(seqs=8, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=8, std=3.0, spike_p=0.0, topk=64,
                     desc="distillation reductions on 8 x 4096 rows, V=151936 bf16: negative entropy, 64 gathered logprobs, soft cross entropy"),
+    "c5": dict(seqs=0, seq_len=131072, vocab=131072, dtype="bf16", mb_seqs=0, std=3.0, spike_p=0.0,
+               desc="benchmark config 5: sequences of U[2048,32768] tokens packed into one 131072-token row, V=131072 bf16, "
+                    "sequence-level-normalised loss, k3 KL beta=0.001, fwd+bwd to dlogits"),
     "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
                desc="benchmark config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
 }
@@ -301,6 +304,100 @@ def bench_distill(args, torch, w):
     }))
 
 
+def bench_packed(args, torch, w):
+    """One packed row through SequencePackingFusionLossWrapper (single pass), then the three-pass packed path."""
+    from rl_amd import ops
+    from rl_amd.algorithms.loss import (ClippedPGLossConfig, ClippedPGLossFn, SequencePackingFusionLossWrapper,
+                                        prepare_packed_loss_input)
+    from rl_amd.distributed.model_utils import from_parallel_logits_to_logprobs_packed_sequences
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    total, v = w["seq_len"], w["vocab"]
+    g = torch.Generator(device=dev).manual_seed(5005)
+    lens = []
+    while sum(lens) < total:
+        lens.append(min(int(torch.randint(2048, 32769, (1,), generator=g, device=dev)), total - sum(lens)))
+    nseq, smax = len(lens), max(lens)
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+    logits = torch.empty((1, total, v), dtype=torch.bfloat16, device=dev).normal_(0.0, w["std"], generator=g)
+    ids = torch.randint(0, v, (nseq, smax), generator=g, device=dev)
+    in_seq = torch.arange(smax, device=dev).unsqueeze(0) < torch.tensor(lens, device=dev).unsqueeze(-1)
+    ids = ids * in_seq
+    prefix = torch.randint(256, 1025, (nseq, 1), generator=g, device=dev)
+    token_mask = ((torch.arange(smax, device=dev).unsqueeze(0) >= prefix) & in_seq).to(torch.int64)
+    fn = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, reference_policy_kl_penalty=0.001))
+    with torch.no_grad():
+        targets = torch.cat([ids[i, : lens[i]].roll(-1) for i in range(nseq)]).unsqueeze(0)
+        cur = from_parallel_logits_to_logprobs_packed_sequences(logits, targets, cu, smax, 0, v, None,
+                                                                target_is_pre_rolled=True)
+    cur = torch.cat([torch.zeros((nseq, 1), device=dev), cur], dim=1)
+    noise = lambda: cur + 0.05 * torch.randn((nseq, smax), generator=g, device=dev)  # noqa: E731
+    prev = noise()
+    data = {"input_ids": ids, "token_mask": token_mask, "sample_mask": torch.ones(nseq, device=dev),
+            "advantages": torch.randn((nseq, 1), generator=g, device=dev).expand(nseq, smax).contiguous(),
+            "prev_logprobs": prev, "generation_logprobs": prev, "reference_policy_logprobs": noise()}
+    gs = torch.tensor(float(nseq), device=dev)
+    gt = token_mask[:, 1:].sum().float()
+    live_rows = int(gt.item())
+    wrapped = SequencePackingFusionLossWrapper(fn, prepare_packed_loss_input, cu, cu)
+
+    def step():
+        x = logits.requires_grad_(True)
+        loss, _m = wrapped(x, data, gs, gt)
+        (d,) = torch.autograd.grad(loss, x)
+        del d, loss
+
+    def three_pass_step():
+        x = logits.requires_grad_(True)
+        loss_input, prepared = prepare_packed_loss_input(x, data, fn, cu, cu)
+        loss, _m = fn(data=prepared, global_valid_seqs=gs, global_valid_toks=gt, **loss_input)
+        (d,) = torch.autograd.grad(loss, x)
+        del d, loss, loss_input
+
+    def timed(fn_step):
+        for _ in range(args.warmup):
+            fn_step()
+        torch.cuda.synchronize()
+        timer = EventTimer(torch)
+        ops.KERNEL_TIMER = timer
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn_step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ops.KERNEL_TIMER = None
+        return dt, timer.summary()
+
+    elapsed, km = timed(step)
+    row_bytes = v * 2
+    # a live row is read once and its gradient written once; a row that feeds no token is only zero-filled
+    alg = live_rows * 2 * row_bytes + (total - live_rows) * row_bytes
+    fk = km["fused_packed_logits_loss"]["avg_ms"]
+    gbs = alg / (fk * 1e-3) / 1e9
+    out = {
+        "metric": "GRPO logprob+loss fwd/bwd tokens/s, packed 131072-token row at V=131072; % of HBM peak",
+        "value": total * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["desc"], "sequences": nseq, "packed_tokens": total, "vocab": v, "loss_tokens": live_rows,
+                   "api": "SequencePackingFusionLossWrapper(ClippedPGLossFn, prepare_packed_loss_input)(logits, batch, ...) + "
+                          "autograd.grad -> nrl_fused_packed_logits_grpo_loss"},
+        "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel (packed)", "achieved": gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fk,
+                     "algorithmic_bytes_per_launch": alg},
+        "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in km.items()},
+    }
+    t_elapsed, tk = timed(three_pass_step)
+    out["three_pass"] = {
+        "value": total * args.steps / t_elapsed, "unit": "tokens/s", "ms_per_step": t_elapsed / args.steps * 1e3,
+        "api": "prepare_packed_loss_input -> nrl_logprob_packed_fwd; ClippedPGLossFn -> nrl_grpo_loss_fwd_bwd; "
+               "backward -> nrl_logprob_packed_bwd",
+        "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in tk.items()},
+    }
+    print(json.dumps(out))
+
+
 def bench_lmhead(args, torch, w):
     """Config 3: hidden states -> logprobs -> loss -> (dH, dW) through the fused MFMA path."""
     from rl_amd import ops
@@ -384,6 +481,8 @@ def main():
         return bench_topk(args, torch, w)
     if args.workload == "distill":
         return bench_distill(args, torch, w)
+    if args.workload == "c5":
+        return bench_packed(args, torch, w)
     if args.seqs:
         w["seqs"] = args.seqs
         w["mb_seqs"] = min(w["mb_seqs"], args.seqs)

@@ -226,7 +226,9 @@ int nrl_fused_logits_grpo_loss(const nrl_rows* rows, const nrl_grpo_cfg* cfg, co
  * loss/utils.py:214-385) at CP = 1.  Position p of a sequence uses target cu[s] + p + 1 (cu[s] + p when
  * the targets are pre-rolled); the last position of every sequence, positions past unpacked_seqlen - 1 and
  * positions outside every sequence get a zero gradient row.  dlogits: [total, vocab] rows of d_row_stride.
- * workspace: nrl_fused_workspace_bytes(n_seq, in->sm1). */
+ * workspace: nrl_fused_packed_workspace_bytes(n_seq, in->sm1, total) bytes, 8-byte aligned (it also holds one
+ * 16-byte record per packed position: where the position sits in the loss inputs). */
+int64_t nrl_fused_packed_workspace_bytes(int64_t n_seq, int64_t n_inner, int64_t total);
 int nrl_fused_packed_logits_grpo_loss(const nrl_rows* rows, int32_t target_is_pre_rolled, const int32_t* cu_seqlens,
                                       int64_t n_seq, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in,
                                       float loss_scale, void* dlogits, int64_t d_row_stride, float* logprob_out,

@@ -78,6 +78,7 @@ SIGNATURES = {
     "nrl_grpo_loss_workspace_bytes": (_I64, [_I64]),
     "nrl_grpo_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _P, _I64, _P]),
     "nrl_fused_workspace_bytes": (_I64, [_I64, _I64]),
+    "nrl_fused_packed_workspace_bytes": (_I64, [_I64, _I64, _I64]),
     "nrl_fused_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _F, _P, _I64,
                                              _I64, _I64, _P, _P, _P, _P, _I64, _P]),
     "nrl_fused_packed_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.c_int32, _P, _I64, C.POINTER(NrlGrpoCfg),

@@ -284,6 +284,7 @@ struct FusedArgs {
     const int32_t* cu;
     int64_t n_seq;
     int pre_rolled;
+    int4* row_pos;     // packed mode: [total] (sequence, position or -1, target index, 0), filled before the pass
 };
 
 // where a logits row sits in the loss inputs: sequence o, position i (i >= n_inner: the row feeds no token),
@@ -291,6 +292,27 @@ struct FusedArgs {
 struct FusedPos {
     int64_t o, i, tgt;
 };
+__device__ __forceinline__ FusedPos fused_where_packed(const FusedArgs& a, int64_t r) {
+    FusedPos q;
+    const int64_t seq = find_seq(a.cu, a.n_seq, r);
+    q.o = seq < 0 ? 0 : seq;
+    q.i = -1;
+    q.tgt = 0;
+    if (seq >= 0) {
+        const int64_t start = a.cu[seq], len = a.cu[seq + 1] - start, pos = r - start;
+        if (pos + 1 < len && pos < a.n_inner) q.i = pos;  // the last position of a sequence predicts nothing
+        q.tgt = start + (a.pre_rolled ? pos : (pos + 1 < len ? pos + 1 : 0));
+    }
+    return q;
+}
+// The search through the boundaries is a chain of dependent loads; done once per row ahead of the pass,
+// the persistent kernel finds a row's place with a single load.
+__global__ __launch_bounds__(256) void fused_row_pos_kernel(FusedArgs a, int64_t total) {
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r >= total) return;
+    const FusedPos q = fused_where_packed(a, r);
+    a.row_pos[r] = make_int4(static_cast<int>(q.o), static_cast<int>(q.i), static_cast<int>(q.tgt), 0);
+}
 template <bool PACKED>
 __device__ __forceinline__ FusedPos fused_where(const FusedArgs& a, int64_t r) {
     FusedPos q;
@@ -300,15 +322,10 @@ __device__ __forceinline__ FusedPos fused_where(const FusedArgs& a, int64_t r) {
         q.tgt = q.o * a.ts_outer + q.i * a.ts_inner;
         return q;
     }
-    const int64_t seq = find_seq(a.cu, a.n_seq, r);
-    q.o = seq < 0 ? 0 : seq;
-    q.i = a.n_inner;
-    q.tgt = 0;
-    if (seq >= 0) {
-        const int64_t start = a.cu[seq], len = a.cu[seq + 1] - start, pos = r - start;
-        if (pos + 1 < len && pos < a.n_inner) q.i = pos;  // the last position of a sequence predicts nothing
-        q.tgt = start + (a.pre_rolled ? pos : (pos + 1 < len ? pos + 1 : 0));
-    }
+    const int4 p = a.row_pos[r];
+    q.o = p.x;
+    q.i = p.y < 0 ? a.n_inner : p.y;
+    q.tgt = p.z;
     return q;
 }
 template <bool PACKED>
@@ -636,6 +653,10 @@ extern "C" int64_t nrl_fused_workspace_bytes(int64_t batch, int64_t n_inner) {
     return align8(b * 3 * 4) + align8(b * n * T_COUNT * 4) + b * P_COUNT * 8;
 }
 
+extern "C" int64_t nrl_fused_packed_workspace_bytes(int64_t n_seq, int64_t n_inner, int64_t total) {
+    return nrl_fused_workspace_bytes(n_seq, n_inner) + 16 + (total < 1 ? 1 : total) * 16;
+}
+
 // rows describes the logits; with cu != NULL it is one packed row of rows->n_inner positions (n_outer 1) and
 // the loss inputs are [n_seq, in->sm1]
 static int fused_impl(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float loss_scale, void* dlogits,
@@ -669,7 +690,8 @@ static int fused_impl(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_g
     const int64_t n_rows = rows->n_outer * d_n_inner;
     if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
     if (!loss_out || !metrics_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
-    if (workspace_bytes < nrl_fused_workspace_bytes(in->batch, in->sm1)) return fail(NRL_E_WORKSPACE, "workspace too small");
+    const int64_t need = cu ? nrl_fused_packed_workspace_bytes(in->batch, in->sm1, n_rows) : nrl_fused_workspace_bytes(in->batch, in->sm1);
+    if (workspace_bytes < need) return fail(NRL_E_WORKSPACE, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 7) return fail(NRL_E_INVALID, "workspace must be 8-byte aligned");
     if (n_rows > 0) {
         if (!rows->logits || !rows->targets || !dlogits || !logprob_out) return fail(NRL_E_INVALID, "null logits, targets or output");
@@ -692,7 +714,8 @@ static int fused_impl(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_g
     char* ws = static_cast<char*>(workspace);
     a.seq_stats = reinterpret_cast<float*>(ws); ws += align8(in->batch * 3 * 4);
     a.terms = reinterpret_cast<float*>(ws); ws += align8(in->batch * (in->sm1 < 1 ? 1 : in->sm1) * T_COUNT * 4);
-    a.parts = reinterpret_cast<double*>(ws);
+    a.parts = reinterpret_cast<double*>(ws); ws += in->batch * P_COUNT * 8;
+    a.row_pos = cu ? reinterpret_cast<int4*>(ws + ((16 - (reinterpret_cast<uintptr_t>(ws) & 15)) & 15)) : nullptr;
     int tc = 0;
     a.tparam = 1.f;
     if (rows->temperature != 1.0f) {
@@ -707,6 +730,7 @@ static int fused_impl(const nrl_rows* rows, const nrl_grpo_cfg* cfg, const nrl_g
         fused_fill_zero_kernel<<<dim3(1024), dim3(256), 0, s>>>(a.terms, in->batch * in->sm1 * T_COUNT);
         fused_fill_zero_kernel<<<dim3(256), dim3(256), 0, s>>>(a.lp_out, in->batch * in->sm1);
     }
+    if (cu && n_rows > 0) fused_row_pos_kernel<<<dim3((unsigned)((n_rows + 255) / 256)), dim3(256), 0, s>>>(a, n_rows);
     if (n_rows > 0) {
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)

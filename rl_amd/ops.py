@@ -198,11 +198,13 @@ def _logprob_packed_fwd(logits, targets, pre_rolled, cu_seqlens, unpacked_seqlen
     with torch.cuda.device(logits.device):
         out = torch.empty((n_seq, unpacked_seqlen - 1), dtype=torch.float32, device=logits.device)
         lse = torch.empty((t,) if save_lse else (0,), dtype=torch.float32, device=logits.device)
-        code = _lib.load().nrl_logprob_packed_fwd(
-            _ptr(logits), _dtype_code(logits), t, v, logits.stride(0), _ptr(targets), int(pre_rolled),
-            _ptr(cu_seqlens), n_seq, unpacked_seqlen, vocab_start, vocab_end, temperature, temp_mode,
-            _ptr(out), _ptr(lse if save_lse else None), _stream(),
-        )
+        lib = _lib.load()
+        with _timed("logprob_packed_fwd"):
+            code = lib.nrl_logprob_packed_fwd(
+                _ptr(logits), _dtype_code(logits), t, v, logits.stride(0), _ptr(targets), int(pre_rolled),
+                _ptr(cu_seqlens), n_seq, unpacked_seqlen, vocab_start, vocab_end, temperature, temp_mode,
+                _ptr(out), _ptr(lse if save_lse else None), _stream(),
+            )
     _lib.check(code, "nrl_logprob_packed_fwd")
     return out, lse
 
@@ -220,11 +222,13 @@ def _logprob_packed_bwd(logits, targets, pre_rolled, cu_seqlens, unpacked_seqlen
     grad = grad.contiguous()
     with torch.cuda.device(logits.device):
         d = torch.empty((t, v), dtype=logits.dtype, device=logits.device)
-        code = _lib.load().nrl_logprob_packed_bwd(
-            _ptr(logits), _dtype_code(logits), t, v, logits.stride(0), _ptr(targets), int(pre_rolled),
-            _ptr(cu_seqlens), n_seq, unpacked_seqlen, vocab_start, vocab_end, temperature, temp_mode,
-            _ptr(lse), _ptr(grad), _ptr(d), d.stride(0), _stream(),
-        )
+        lib = _lib.load()
+        with _timed("logprob_packed_bwd"):
+            code = lib.nrl_logprob_packed_bwd(
+                _ptr(logits), _dtype_code(logits), t, v, logits.stride(0), _ptr(targets), int(pre_rolled),
+                _ptr(cu_seqlens), n_seq, unpacked_seqlen, vocab_start, vocab_end, temperature, temp_mode,
+                _ptr(lse), _ptr(grad), _ptr(d), d.stride(0), _stream(),
+            )
     _lib.check(code, "nrl_logprob_packed_bwd")
     return d
 
@@ -506,7 +510,7 @@ def _fused_packed_logits_grpo_loss(logits, targets, pre_rolled, cu_seqlens, unpa
         loss = torch.empty((), dtype=torch.float32, device=dev)
         metrics = torch.empty((_lib.NRL_GRPO_N_METRICS,), dtype=torch.float32, device=dev)
         d = torch.empty((t, v), dtype=logits.dtype, device=dev)
-        ws_bytes = lib.nrl_fused_workspace_bytes(n_seq, n_inner)
+        ws_bytes = lib.nrl_fused_packed_workspace_bytes(n_seq, n_inner, t)
         ws = torch.empty(((ws_bytes + 7) // 8,), dtype=torch.float64, device=dev)
         with _timed("fused_packed_logits_loss"):
             code = lib.nrl_fused_packed_logits_grpo_loss(
