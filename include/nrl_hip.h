@@ -240,6 +240,44 @@ int nrl_fused_packed_logits_grpo_loss(const nrl_rows* rows, int32_t target_is_pr
 int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,
                          float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* NLLLossFn per-sample branch (dpo_loss=True, loss_functions.py:823-829): loss_rows_out[b] =
+ * -sum_t lp[b,t] * token_mask[b,t] * sample_mask[b], divided by max(sum_t mask, 1) with
+ * average_log_probs; den_out[b] is that divisor (1 without averaging); totals_out[0..1] =
+ * {num_unmasked_tokens, num_valid_samples}.  workspace: B floats.  _bwd: dlp_out[b,t] =
+ * -token_mask * sample_mask[b] / den[b] * grad_rows[b], contiguous [B, n]. */
+int nrl_nll_rows_fwd(const float* lp, int64_t lp_stride, const float* token_mask, int64_t token_mask_stride,
+                     const float* sample_mask, int64_t batch, int64_t n, int32_t average_log_probs,
+                     float* loss_rows_out, float* den_out, float* totals_out, void* workspace,
+                     int64_t workspace_bytes, void* stream);
+int nrl_nll_rows_bwd(const float* grad_rows, const float* token_mask, int64_t token_mask_stride,
+                     const float* sample_mask, const float* den, int64_t batch, int64_t n, float* dlp_out,
+                     void* stream);
+
+/* DPOLossFn (loss_functions.py:1025-1106) on token logprobs, forward and gradient in one call.  Rows
+ * alternate chosen / rejected (batch must be even).  reward[b] = sum_t (lp - ref) * token_mask (/ max(sum_t
+ * token_mask, 1) with preference_average_log_probs); preference = sum_p -logsigmoid(beta * (reward_c -
+ * reward_r)) * sample_mask_c^2 / (Gs/2 + 1e-8) with Gs = global_valid[0]; the SFT term (weight > 0) is the
+ * chosen rows' per-sample NLL, masked-mean over the pairs in the same way.  ref may be NULL (zeros); the
+ * caller passes it already aligned with lp (the reference reads reference_policy_logprobs[:, :-1]).
+ * metrics_out[0..6] = {loss, sft_loss, preference_loss, accuracy, rewards_chosen_mean,
+ * rewards_rejected_mean, num_valid_samples}; dlp_out: contiguous fp32 [B, n].
+ * workspace: nrl_dpo_workspace_bytes(B) bytes. */
+int64_t nrl_dpo_workspace_bytes(int64_t batch);
+int nrl_dpo_loss_fwd_bwd(const float* lp, int64_t lp_stride, const float* ref, int64_t ref_stride,
+                         const float* token_mask, int64_t token_mask_stride, const float* sample_mask,
+                         const float* global_valid, int64_t batch, int64_t n, float beta,
+                         float preference_loss_weight, float sft_loss_weight,
+                         int32_t preference_average_log_probs, int32_t sft_average_log_probs, float* loss_out,
+                         float* dlp_out, float* metrics_out, void* workspace, int64_t workspace_bytes,
+                         void* stream);
+
+/* PreferenceLossFn (loss_functions.py:877-946): rewards [B] from a reward model, beta = 1.
+ * metrics_out[0..4] = {loss, accuracy, rewards_chosen_mean, rewards_rejected_mean, num_valid_samples};
+ * drewards_out: fp32 [B]. */
+int nrl_preference_loss_fwd_bwd(const float* rewards, const float* sample_mask, const float* global_valid,
+                                int64_t batch, float* loss_out, float* drewards_out, float* metrics_out,
+                                void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * K5  calculate_baseline_and_std_per_prompt (nemo_rl/algorithms/utils.py:104-198) and
  * GRPOAdvantageEstimator.compute_advantage (nemo_rl/algorithms/advantage_estimator.py:82-98).

@@ -41,6 +41,11 @@ Pinning status (what fixes each function besides its own text):
 * ``distill.*``            pinned: closed forms (uniform / one-hot rows, H(p,q) =
                            H(p) + KL), the reference's stated backward formulas
                            and brute force (``tests/test_oracle_distill.py``).
+* ``preference.*``         pinned: the closed-form cases of the reference's own
+                           DPO tests (zero logits vs zero reference, SFT term of
+                           the chosen rows, SFT-only == rescaled NLL) and a
+                           loop-per-pair brute force
+                           (``tests/test_oracle_preference.py``).
 * ``lmhead.*``             PARITY UNPINNED against the reference (its only test
                            needs Megatron, two GPUs and a model download);
                            pinned here to ``logprob(hidden @ W.T)`` in fp32.

@@ -7,7 +7,14 @@ from .fused import (
     why_not_fusable_packed,
 )
 from .interfaces import LossFunction, LossInputType, LossType, MetricNormalizer
-from .loss_functions import ClippedPGLossConfig, ClippedPGLossFn, NLLLossFn
+from .loss_functions import (
+    ClippedPGLossConfig,
+    ClippedPGLossFn,
+    DPOLossConfig,
+    DPOLossFn,
+    NLLLossFn,
+    PreferenceLossFn,
+)
 from .utils import prepare_loss_input, prepare_packed_loss_input
 from .wrapper import (
     SequencePackingFusionLossWrapper,
@@ -17,7 +24,7 @@ from .wrapper import (
 
 __all__ = [
     "fused_logits_clipped_pg_loss", "fused_packed_logits_clipped_pg_loss", "why_not_fusable", "why_not_fusable_packed",
-    "ClippedPGLossConfig", "ClippedPGLossFn", "NLLLossFn", "LossFunction", "LossInputType", "LossType",
+    "ClippedPGLossConfig", "ClippedPGLossFn", "DPOLossConfig", "DPOLossFn", "NLLLossFn", "PreferenceLossFn", "LossFunction", "LossInputType", "LossType",
     "MetricNormalizer", "prepare_loss_input", "prepare_packed_loss_input", "SequencePackingFusionLossWrapper",
     "SequencePackingLossWrapper", "wrap_loss_fn_with_input_preparation",
 ]

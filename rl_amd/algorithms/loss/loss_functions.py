@@ -285,7 +285,8 @@ class _FusedNll(torch.autograd.Function):
 
 
 class NLLLossFn(LossFunction):
-    """Negative log-likelihood over the masked tokens (``loss_functions.py:791-842``, scalar branch)."""
+    """Negative log-likelihood over the masked tokens (``loss_functions.py:791-842``): the scalar loss,
+    or with ``dpo_loss=True`` one value per sample."""
 
     loss_type = LossType.TOKEN_LEVEL
     input_type = LossInputType.LOGPROB
@@ -301,7 +302,7 @@ class NLLLossFn(LossFunction):
     def __call__(self, next_token_logprobs, data, global_valid_seqs, global_valid_toks,
                  dpo_loss: bool = False, dpo_average_log_probs: bool = False):
         if dpo_loss:
-            raise NotImplementedError("the per-sample DPO reduction is outside the GRPO hot path")
+            return self._per_sample(next_token_logprobs, data, dpo_average_log_probs)
         home = next_token_logprobs.device
         dev = _gpu_for(next_token_logprobs)
         sample_mask_in, token_mask_in = data["sample_mask"], data["token_mask"]
@@ -318,3 +319,124 @@ class NLLLossFn(LossFunction):
             "num_unmasked_tokens": int(m[1]) if integral else m[1],
             "num_valid_samples": m[2] if sample_mask_in.is_floating_point() else int(m[2]),
         }
+
+
+    def _per_sample(self, next_token_logprobs, data, average_log_probs):
+        """``dpo_loss=True`` (``loss_functions.py:823-829``): ``loss [B]``, summed (or averaged) over each sample's tokens."""
+        home = next_token_logprobs.device
+        dev = _gpu_for(next_token_logprobs)
+        loss, totals = _NllRows.apply(_f32(next_token_logprobs, dev), _f32(data["token_mask"][:, 1:], dev),
+                                      _f32(data["sample_mask"], dev), bool(average_log_probs))
+        if home != dev:
+            loss = loss.to(home)
+        t = totals.cpu().tolist()
+        return loss, {"loss": loss, "num_unmasked_tokens": t[0], "num_valid_samples": t[1]}
+
+
+class _NllRows(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, lp, token_mask, sample_mask, average):
+        rows, den, totals = _OPS.nll_rows_fwd(lp.detach(), token_mask, sample_mask, average)
+        ctx.save_for_backward(token_mask, sample_mask, den)
+        ctx.mark_non_differentiable(totals)
+        return rows, totals
+
+    @staticmethod
+    def backward(ctx, grad_rows, _grad_totals):
+        token_mask, sample_mask, den = ctx.saved_tensors
+        return _OPS.nll_rows_bwd(grad_rows.contiguous().float(), token_mask, sample_mask, den), None, None, None
+
+
+class _Preference(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rewards, sample_mask, global_valid):
+        loss, drewards, metrics = _OPS.preference_loss(rewards.detach(), sample_mask, global_valid)
+        ctx.save_for_backward(drewards)
+        ctx.mark_non_differentiable(metrics)
+        return loss, metrics
+
+    @staticmethod
+    def backward(ctx, grad_loss, _grad_metrics):
+        (drewards,) = ctx.saved_tensors
+        return drewards * grad_loss, None, None
+
+
+class PreferenceLossFn(LossFunction):
+    """Reward-model preference loss ``-E[log sigmoid(r_chosen - r_rejected)]`` over rows that alternate
+    chosen / rejected (``loss_functions.py:853-946``)."""
+
+    loss_type = LossType.SEQUENCE_LEVEL
+    input_type = LossInputType.LOGIT
+
+    def split_output_tensor(self, tensor):
+        return tensor[::2], tensor[1::2]
+
+    def __call__(self, logits, data, global_valid_seqs, global_valid_toks):
+        home = logits.device
+        dev = _gpu_for(logits)
+        loss, metrics = _Preference.apply(_f32(logits.squeeze(-1), dev), _f32(data["sample_mask"], dev),
+                                          _global_valid(global_valid_seqs, 1.0, dev))
+        if home != dev:
+            loss = loss.to(home)
+        m = metrics.cpu().tolist()
+        return loss, {"loss": m[0], "accuracy": m[1], "rewards_chosen_mean": m[2], "rewards_rejected_mean": m[3],
+                      "num_valid_samples": m[4]}
+
+
+class DPOLossConfig(BaseModel, extra="allow"):
+    """Field names and defaults of ``loss_functions.py:949-954``."""
+
+    reference_policy_kl_penalty: float = 0.05
+    preference_loss_weight: float = 1.0
+    sft_loss_weight: float = 0.0
+    preference_average_log_probs: bool = False
+    sft_average_log_probs: bool = False
+
+
+class _Dpo(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, lp, ref, token_mask, sample_mask, global_valid, beta, w_pref, w_sft, avg_pref, avg_sft):
+        loss, dlp, metrics = _OPS.dpo_loss(lp.detach(), ref, token_mask, sample_mask, global_valid, beta, w_pref, w_sft,
+                                           avg_pref, avg_sft)
+        ctx.save_for_backward(dlp)
+        ctx.mark_non_differentiable(metrics)
+        return loss, metrics
+
+    @staticmethod
+    def backward(ctx, grad_loss, _grad_metrics):
+        (dlp,) = ctx.saved_tensors
+        return (dlp * grad_loss,) + (None,) * 9
+
+
+class DPOLossFn(PreferenceLossFn):
+    """Direct preference optimisation on token logprobs (``loss_functions.py:966-1106``): preference
+    term on the summed (or averaged) logprob margins against the reference policy, plus an optional
+    SFT term on the chosen rows.  Rewards, both terms and the gradient come from one fused call."""
+
+    loss_type = LossType.SEQUENCE_LEVEL
+    input_type = LossInputType.LOGPROB
+
+    def __init__(self, cfg, use_fused_linear_logprobs: bool = False):
+        get = cfg.get if isinstance(cfg, dict) else lambda k, d=None: getattr(cfg, k, d)  # noqa: E731
+        defaults = DPOLossConfig()
+        for name in DPOLossConfig.model_fields:
+            setattr(self, name, get(name, getattr(defaults, name)))
+        self.use_fused_linear_logprobs = use_fused_linear_logprobs
+        self.sft_loss = NLLLossFn(use_fused_linear_logprobs=use_fused_linear_logprobs)
+
+    def __call__(self, next_token_logprobs, data, global_valid_seqs, global_valid_toks):
+        if self.sft_loss_weight > 0 and global_valid_toks is None:
+            raise AssertionError("global_valid_toks must be provided for SFT loss")
+        home = next_token_logprobs.device
+        dev = _gpu_for(next_token_logprobs)
+        loss, metrics = _Dpo.apply(
+            _f32(next_token_logprobs, dev), _f32(data["reference_policy_logprobs"][:, :-1], dev),
+            _f32(data["token_mask"][:, 1:], dev), _f32(data["sample_mask"], dev), _global_valid(global_valid_seqs, 1.0, dev),
+            float(self.reference_policy_kl_penalty), float(self.preference_loss_weight), float(self.sft_loss_weight),
+            bool(self.preference_average_log_probs), bool(self.sft_average_log_probs),
+        )
+        if home != dev:
+            loss = loss.to(home)
+        m = metrics.cpu().tolist()
+        return loss, {"loss": m[0], "sft_loss": m[1], "preference_loss": m[2], "accuracy": m[3], "rewards_chosen_mean": m[4],
+                      "rewards_rejected_mean": m[5], "num_valid_samples": m[6]}

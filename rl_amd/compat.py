@@ -40,7 +40,7 @@ _PATCHED = {
     ],
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
     "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],
-    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn"],
+    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
     "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking"],

@@ -550,6 +550,110 @@ for _name, _fn in (("grpo_loss", _grpo_loss), ("nll_loss", _nll_loss)):
 
 
 # ------------------------------------------------------------------------------------------------
+# preference losses (DPO, reward model) and the per-sample NLL rows
+# ------------------------------------------------------------------------------------------------
+_LIB.define("nll_rows_fwd(Tensor lp, Tensor token_mask, Tensor sample_mask, bool average) -> (Tensor, Tensor, Tensor)")
+_LIB.define("nll_rows_bwd(Tensor grad_rows, Tensor token_mask, Tensor sample_mask, Tensor den) -> Tensor")
+_LIB.define(
+    "dpo_loss(Tensor lp, Tensor? ref, Tensor token_mask, Tensor sample_mask, Tensor global_valid, float beta, "
+    "float preference_loss_weight, float sft_loss_weight, bool preference_average_log_probs, bool sft_average_log_probs) "
+    "-> (Tensor, Tensor, Tensor)"
+)
+_LIB.define("preference_loss(Tensor rewards, Tensor sample_mask, Tensor global_valid) -> (Tensor, Tensor, Tensor)")
+
+
+def _lp_and_masks(lp, token_mask, sample_mask):
+    _need_gpu(lp, token_mask, sample_mask)
+    if lp.dim() != 2:
+        raise ValueError(f"logprobs must be [B, S-1], got {tuple(lp.shape)}")
+    b, n = lp.shape
+    lp, lp_stride = _rowmat(lp, b, n, "logprobs")
+    tm, tm_stride = _rowmat(token_mask, b, n, "token_mask")
+    return b, n, lp, lp_stride, tm, tm_stride, _vec(sample_mask, b, "sample_mask")
+
+
+def _nll_rows_fwd(lp, token_mask, sample_mask, average):
+    """-> (per-sample loss [B], divisor [B], (num_unmasked_tokens, num_valid_samples))."""
+    b, n, lp, lp_stride, tm, tm_stride, sm = _lp_and_masks(lp, token_mask, sample_mask)
+    dev = lp.device
+    with torch.cuda.device(dev):
+        rows = torch.empty((b,), dtype=torch.float32, device=dev)
+        den = torch.empty((b,), dtype=torch.float32, device=dev)
+        totals = torch.empty((2,), dtype=torch.float32, device=dev)
+        ws = torch.empty((max(b, 1),), dtype=torch.float32, device=dev)
+        code = _lib.load().nrl_nll_rows_fwd(_ptr(lp), lp_stride, _ptr(tm), tm_stride, _ptr(sm), b, n, int(average), _ptr(rows),
+                                            _ptr(den), _ptr(totals), _ptr(ws), ws.numel() * 4, _stream())
+    _lib.check(code, "nrl_nll_rows_fwd")
+    return rows, den, totals
+
+
+def _nll_rows_bwd(grad_rows, token_mask, sample_mask, den):
+    _need_gpu(grad_rows, token_mask, sample_mask, den)
+    b, n = token_mask.shape
+    tm, tm_stride = _rowmat(token_mask, b, n, "token_mask")
+    g, sm, den = _vec(grad_rows, b, "grad_rows"), _vec(sample_mask, b, "sample_mask"), _vec(den, b, "den")
+    dev = tm.device
+    with torch.cuda.device(dev):
+        dlp = torch.empty((b, n), dtype=torch.float32, device=dev)
+        code = _lib.load().nrl_nll_rows_bwd(_ptr(g), _ptr(tm), tm_stride, _ptr(sm), _ptr(den), b, n, _ptr(dlp), _stream())
+    _lib.check(code, "nrl_nll_rows_bwd")
+    return dlp
+
+
+def _dpo_loss(lp, ref, token_mask, sample_mask, global_valid, beta, preference_loss_weight, sft_loss_weight,
+              preference_average_log_probs, sft_average_log_probs):
+    """-> (loss, d loss / d logprobs [B, n], metrics[7])."""
+    _need_gpu(ref, global_valid)
+    b, n, lp, lp_stride, tm, tm_stride, sm = _lp_and_masks(lp, token_mask, sample_mask)
+    ref, ref_stride = _rowmat(ref, b, n, "reference_policy_logprobs")
+    if global_valid.dtype != torch.float32 or global_valid.numel() < 1:
+        raise ValueError("global_valid must be an fp32 tensor whose first element is the number of valid sequences")
+    gv = global_valid.contiguous()
+    lib = _lib.load()
+    dev = lp.device
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dlp = torch.empty((b, n), dtype=torch.float32, device=dev)
+        metrics = torch.empty((7,), dtype=torch.float32, device=dev)
+        ws_bytes = lib.nrl_dpo_workspace_bytes(b)
+        ws = torch.empty(((ws_bytes + 3) // 4,), dtype=torch.float32, device=dev)
+        code = lib.nrl_dpo_loss_fwd_bwd(
+            _ptr(lp), lp_stride, _ptr(ref), ref_stride, _ptr(tm), tm_stride, _ptr(sm), _ptr(gv), b, n, float(beta),
+            float(preference_loss_weight), float(sft_loss_weight), int(preference_average_log_probs),
+            int(sft_average_log_probs), _ptr(loss), _ptr(dlp), _ptr(metrics), _ptr(ws), ws.numel() * 4, _stream(),
+        )
+    _lib.check(code, "nrl_dpo_loss_fwd_bwd")
+    return loss, dlp, metrics
+
+
+def _preference_loss(rewards, sample_mask, global_valid):
+    """-> (loss, d loss / d rewards [B], metrics[5])."""
+    _need_gpu(rewards, sample_mask, global_valid)
+    if rewards.dim() != 1:
+        raise ValueError(f"rewards must be [B], got {tuple(rewards.shape)}")
+    b = rewards.shape[0]
+    r, sm = _vec(rewards, b, "rewards"), _vec(sample_mask, b, "sample_mask")
+    if global_valid.dtype != torch.float32 or global_valid.numel() < 1:
+        raise ValueError("global_valid must be an fp32 tensor whose first element is the number of valid sequences")
+    gv = global_valid.contiguous()
+    dev = r.device
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dr = torch.zeros((b,), dtype=torch.float32, device=dev)
+        metrics = torch.empty((5,), dtype=torch.float32, device=dev)
+        code = _lib.load().nrl_preference_loss_fwd_bwd(_ptr(r), _ptr(sm), _ptr(gv), b, _ptr(loss), _ptr(dr), _ptr(metrics),
+                                                       _stream())
+    _lib.check(code, "nrl_preference_loss_fwd_bwd")
+    return loss, dr, metrics
+
+
+for _name, _fn in (("nll_rows_fwd", _nll_rows_fwd), ("nll_rows_bwd", _nll_rows_bwd), ("dpo_loss", _dpo_loss),
+                   ("preference_loss", _preference_loss)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
+# ------------------------------------------------------------------------------------------------
 # K5
 # ------------------------------------------------------------------------------------------------
 _LIB.define(
