@@ -151,7 +151,7 @@ struct CoreB {
         const char* pa;  // first row of the tile, bytes
         const char* pb;
         uint32_t voa[ROUNDS], vob[ROUNDS];  // lane's source offset in each round (rows past the end clamped)
-        uint32_t aoff[BK / 16], boff[BK / 16];  // lane's fragment address for each k step (buffer 0, tile 0)
+        uint32_t aoff[BK / 16], boff[BK / 16];  // lane's fragment address in LDS for each k step (buffer 0, tile 0)
         int wave;                               // wave index, held in a scalar register
     };
 
@@ -168,40 +168,57 @@ struct CoreB {
         for (int d = 0; d < 2 * ROUNDS; ++d) issue_one(c, lds, buf, k0, d);
     }
 
+    // Fragment reads are written as inline assembly.  A read the compiler can see is treated as possibly
+    // aliasing every direct-to-LDS load still in flight and gets a vmcnt(0) in front of it, which stalls the
+    // wave for a full memory latency in the middle of the slab; the two never touch the same buffer here
+    // (the slab barrier orders them), so the reads are hidden from that analysis and waited for by hand.
+    __device__ static __forceinline__ bf16x8 lds_read16(uint32_t addr, int imm) {
+        bf16x8 v;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(imm));
+        return v;
+    }
+    // every LDS read issued so far has returned; the operands tie the wait to the fragments it guards
+    __device__ static __forceinline__ void wait_frags(bf16x8 (&a)[NI], bf16x8 (&b)[NJ]) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    }
+
+    static constexpr int DMA_EVERY = 2;  // one direct load behind every second MFMA of the first 32
+
     // Consume slab buffer BUF while the direct loads of slab k_next go into the other buffer.  One wave per
-    // SIMD: nothing else hides latencies, so the order is fixed by hand -- one direct load behind each of
-    // the first 16 MFMAs (their address arithmetic runs in the shadow of the matrix pipe), and the
-    // fragments of k step ks + 1 requested half-way through the MFMAs of step ks.  (While direct-to-LDS
-    // loads are in flight the compiler drains every LDS read at each wait, so the reads must be issued
-    // half a step ahead of the wait that precedes their first use.)
+    // SIMD: nothing else hides latencies, so the order is fixed by hand -- the 16 direct loads go out one
+    // behind every second MFMA of the first half of the slab (their address arithmetic runs in the shadow of
+    // the matrix pipe, and the four waves do not queue up at the load unit), and the 8 fragment reads of k
+    // step ks + 1 follow the first 8 MFMAs of step ks.
     template <int BUF>
     __device__ static __forceinline__ void compute(const Ctx& c, unsigned char* lds, f32x16 (&acc)[NI][NJ], int64_t k_next) {
+        static_assert(NI == 4 && NJ == 4, "wait_frags names four fragments per operand");
         bf16x8 af[2][NI], bfr[2][NJ];
-        auto frags = [&](int ks, int set) {
-#pragma unroll
-            for (int i = 0; i < NI; ++i)
-                af[set][i] = *reinterpret_cast<const bf16x8*>(lds + c.aoff[ks] + BUF * TILE_BYTES + i * 32 * BK * 2);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j)
-                bfr[set][j] = *reinterpret_cast<const bf16x8*>(lds + c.boff[ks] + BUF * TILE_BYTES + j * 32 * BK * 2);
+        // fragment read number f of k step ks: 0..NI-1 operand A, NI..NI+NJ-1 operand B
+        auto frag_one = [&](int ks, int set, int f) {
+            if (f < NI) af[set][f] = lds_read16(c.aoff[ks], BUF * TILE_BYTES + f * 32 * BK * 2);
+            else bfr[set][f - NI] = lds_read16(c.boff[ks], BUF * TILE_BYTES + (f - NI) * 32 * BK * 2);
         };
-        frags(0, 0);
+#pragma unroll
+        for (int f = 0; f < NI + NJ; ++f) frag_one(0, 0, f);
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
+            wait_frags(af[ks & 1], bfr[ks & 1]);
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
+                    const int idx = i * NJ + j, n = ks * NI * NJ + idx;  // MFMA number within the step / the slab
                     __builtin_amdgcn_sched_barrier(0);
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
-                    if (ks * NI * NJ + i * NJ + j < 2 * ROUNDS) {
+                    if (n % DMA_EVERY == 0 && n / DMA_EVERY < 2 * ROUNDS) {
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_one(c, lds, BUF ^ 1, k_next, ks * NI * NJ + i * NJ + j);
+                        issue_one(c, lds, BUF ^ 1, k_next, n / DMA_EVERY);
                     }
-                }
-                if (i == NI / 2 - 1 && ks + 1 < BK / 16) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    frags(ks + 1, (ks + 1) & 1);
+                    if (ks + 1 < BK / 16 && idx < NI + NJ) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        frag_one(ks + 1, (ks + 1) & 1, idx);
+                    }
                 }
             }
         }
@@ -233,11 +250,13 @@ struct CoreB {
             c.vob[j] = static_cast<uint32_t>((r < last_b ? r : last_b) * op.ldb + cg * 8) * 2u;
         }
         const int fr = lane & 31, fh = lane >> 5;
+        // the buffer's address inside LDS (the low half of its generic address)
+        const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
             const uint32_t sw = static_cast<uint32_t>(((ks * 2 + fh) ^ ((fr >> 1) & 7)) * 16);
-            c.aoff[ks] = static_cast<uint32_t>((wm * 128 + fr) * BK * 2) + sw;
-            c.boff[ks] = static_cast<uint32_t>(2 * TILE_BYTES + (wn * 128 + fr) * BK * 2) + sw;
+            c.aoff[ks] = lds_base + static_cast<uint32_t>((wm * 128 + fr) * BK * 2) + sw;
+            c.boff[ks] = lds_base + static_cast<uint32_t>(2 * TILE_BYTES + (wn * 128 + fr) * BK * 2) + sw;
         }
         const int64_t nk = op.k / BK;
         const int64_t k_last = (nk - 1) * BK;
