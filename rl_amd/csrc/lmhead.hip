@@ -612,20 +612,36 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
     f32x16 acc[NI][NJ];
     zero_acc<Core>(acc);
     Core::tile(op, row0, col0, acc, lds);
+    // an interior tile takes the path without per-element bounds (no divergent branch between the loads)
+    const bool interior = row0 + BM <= op.m && col0 + BN <= op.n;
+    auto write_back = [&](auto interior_tag) {
+        constexpr bool INTERIOR = decltype(interior_tag)::value;
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+            for (int j = 0; j < NJ; ++j) {
+                const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+                float* base = c + (row0 + wm * 128 + i * 32) * ldc + col;
+                // all 16 loads of a 32 x 32 block go out before the first is used (one memory latency per
+                // block, not one per element)
+                float prior[16];
+                if (ACCUM) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int64_t row = row0 + wm * 128 + i * 32 + acc_row(e, lane);
-                if (row < op.m && col < op.n) {
-                    float* p = c + row * ldc + col;
-                    *p = ACCUM ? *p + acc[i][j][e] : acc[i][j][e];
+                    for (int e = 0; e < 16; ++e) {
+                        const int r = acc_row(e, lane);
+                        prior[e] = (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n)) ? base[r * ldc] : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int r = acc_row(e, lane);
+                    if (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n))
+                        base[r * ldc] = ACCUM ? prior[e] + acc[i][j][e] : acc[i][j][e];
                 }
             }
-        }
+    };
+    if (interior) write_back(std::true_type{});
+    else write_back(std::false_type{});
 }
 
 // dst[c, r] = src[r, c] for r < rows, c < cols; dst row stride ldd, columns [rows, pad_cols) zero-filled
