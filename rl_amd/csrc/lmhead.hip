@@ -506,18 +506,46 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
         p01 = pack_bf16x2(gv[0], gv[1]);
         p23 = pack_bf16x2(gv[2], gv[3]);
     };
+    // The whole tile's gradients as bf16 pairs.  A group of 4 accumulator rows is the same for every j, so
+    // its per-token values are read from LDS once; out-of-range elements become zero by a select, not a branch.
+    auto grad_all = [&](uint32_t (&p01)[NI][NJ][4], uint32_t (&p23)[NI][NJ][4]) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int rl = wm * 128 + i * 32 + acc_row(q * 4, lane);  // first of the 4 consecutive rows
+                float lse_r[4], g_r[4];
+                int tgt_r[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    lse_r[u] = lse_l[rl + u];
+                    g_r[u] = row0 + rl + u < a.op.m ? g_l[rl + u] : 0.f;
+                    tgt_r[u] = tgt_local[rl + u];
+                }
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int c = static_cast<int>(col0) + wn * (NJ * 32) + j * 32 + (lane & 31);
+                    float gv[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float x = round_bf16(acc[i][j][q * 4 + u]);
+                        const float p = fast_exp2(__builtin_fmaf(x, kLog2e, -lse_r[u]));
+                        const float v = ((tgt_r[u] == c ? 1.f : 0.f) - p) * g_r[u];
+                        gv[u] = (c < a.op.n && g_r[u] != 0.f) ? v : 0.f;  // (also keeps 0 * inf out of the padding)
+                    }
+                    p01[i][j][q] = pack_bf16x2(gv[0], gv[1]);
+                    p23[i][j][q] = pack_bf16x2(gv[2], gv[3]);
+                }
+            }
+        }
+    };
     if constexpr (Core::LDS_BYTES >= BM * BN * 2) {
         // Both layouts leave through LDS so that every global store is a 16-byte piece of a 512-byte run.
         // Pass 1, [vocab][token]: a lane's 4 tokens are one 8-byte unit; unit U of row v sits at U ^ (v & 63).
         // Pass 2, [token][vocab]: 2-byte writes; the 16-byte chunk C of row t sits at C ^ ((t >> 2) & 7).
         constexpr int RV = BN / 8;  // 16-byte pieces per token row of the tile
         uint32_t p01[NI][NJ][4], p23[NI][NJ][4];
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int i = 0; i < NI; ++i)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) grad4(i, j, q, p01[i][j][q], p23[i][j][q]);
+        grad_all(p01, p23);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int v = wn * (NJ * 32) + j * 32 + (lane & 31);
