@@ -3,7 +3,7 @@
 ``install()`` either registers ``nemo_rl.distributed.model_utils``, ``nemo_rl.algorithms.loss`` (and
 its sub-modules), ``nemo_rl.algorithms.loss_functions``, ``nemo_rl.algorithms.utils``,
 ``nemo_rl.algorithms.logits_sampling_utils``, ``nemo_rl.algorithms.advantage_estimator`` and
-``nemo_rl.models.automodel.train`` (its ``LogprobsPostProcessor``) as
+``nemo_rl.models.automodel.train`` / ``nemo_rl.models.megatron.train`` (their ``LogprobsPostProcessor``) as
 aliases of the ``rl_amd`` modules (when NeMo-RL is not importable), or replaces the hot-path
 attributes of an existing NeMo-RL install in place.
 """
@@ -26,6 +26,7 @@ _ALIASES = {
     "nemo_rl.algorithms.loss.wrapper": "rl_amd.algorithms.loss.wrapper",
     "nemo_rl.algorithms.loss_functions": "rl_amd.algorithms.loss_functions",
     "nemo_rl.models.automodel.train": "rl_amd.models.automodel.train",
+    "nemo_rl.models.megatron.train": "rl_amd.models.megatron.train",
     "nemo_rl.algorithms.grpo": "rl_amd.algorithms.grpo",
 }
 
@@ -43,6 +44,7 @@ _PATCHED = {
     "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
+    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor"],
     "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }
@@ -67,7 +69,8 @@ def install(force_alias: bool = False) -> str:
             for name in names:
                 setattr(dst, name, getattr(src, name))
         return "patched"
-    for parent in ("nemo_rl", "nemo_rl.distributed", "nemo_rl.algorithms", "nemo_rl.models", "nemo_rl.models.automodel"):
+    for parent in ("nemo_rl", "nemo_rl.distributed", "nemo_rl.algorithms", "nemo_rl.models", "nemo_rl.models.automodel",
+                   "nemo_rl.models.megatron"):
         if parent not in sys.modules:
             pkg = types.ModuleType(parent)
             pkg.__path__ = []  # a package, so sub-module imports resolve through sys.modules
