@@ -37,6 +37,7 @@ _PATCHED = {
         "ChunkedDistributedLogprobWithSampling", "ChunkedDistributedHiddenStatesToLogprobs",
         "from_parallel_logits_to_logprobs", "from_parallel_logits_to_logprobs_packed_sequences",
         "from_parallel_hidden_states_to_logprobs", "get_next_token_logprobs_from_logits",
+        "dtensor_from_parallel_logits_to_logprobs", "get_logprobs_from_vocab_parallel_logits",
         "ChunkedDistributedEntropy", "ChunkedDistributedGatherLogprob", "DistributedCrossEntropy",
     ],
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],

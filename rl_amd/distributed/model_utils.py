@@ -246,6 +246,62 @@ def get_next_token_logprobs_from_logits(
     )[:, : input_ids.shape[1] - 1]
 
 
+def _mesh_dim_size(mesh, name: str) -> int:
+    names = getattr(mesh, "mesh_dim_names", None)
+    if names is None or name not in names:
+        return 1
+    return int(mesh.shape[names.index(name)])
+
+
+def dtensor_from_parallel_logits_to_logprobs(
+    vocab_parallel_logits: torch.Tensor,
+    target: Any,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    tp_group: Any,
+    inference_only: bool = False,
+    seq_index: Optional[torch.Tensor] = None,
+    chunk_size: Optional[int] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+) -> torch.Tensor:
+    """``model_utils.py:839-944``: the DTensor worker's twin of ``from_parallel_logits_to_logprobs``.  ``target``
+    may be a DTensor; on one GPU its mesh has no context-parallel extent, so the re-ordering by
+    ``seq_index`` (``:880-892``) never applies and the local shard is the whole tensor."""
+    if hasattr(target, "to_local"):
+        if _mesh_dim_size(target.device_mesh, "cp") > 1:
+            raise NotImplementedError("dtensor_from_parallel_logits_to_logprobs: context parallelism needs more than one GPU")
+        target = target.to_local()
+    if seq_index is not None:
+        raise NotImplementedError("seq_index belongs to context-parallel logits (more than one GPU)")
+    return from_parallel_logits_to_logprobs(
+        vocab_parallel_logits, target, vocab_start_index, vocab_end_index, tp_group, inference_only=inference_only,
+        cp_group=None, chunk_size=chunk_size, sampling_params=sampling_params)
+
+
+def get_logprobs_from_vocab_parallel_logits(
+    vocab_parallel_logits: Any,
+    input_ids: Any,
+    seq_index: Optional[torch.Tensor] = None,
+    chunk_size: Optional[int] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+) -> torch.Tensor:
+    """``model_utils.py:1558-1608``: vocabulary-parallel DTensor logits -> ``[B, S-1]`` logprobs.  The rank's
+    vocabulary interval comes from the mesh's ``tp`` group (``:1592-1596``), which has one member here."""
+    mesh = vocab_parallel_logits.device_mesh
+    if seq_index is not None:
+        assert _mesh_dim_size(mesh, "cp") >= 1 and "cp" in (mesh.mesh_dim_names or ()), (
+            "seq_index must be provided for cp sharded logits"
+        )
+    tp_group = mesh.get_group("tp")
+    _require_single_rank(tp_group, "get_logprobs_from_vocab_parallel_logits")
+    tp_rank, tp_size = tp_group.rank(), tp_group.size()
+    per_rank = vocab_parallel_logits.shape[-1] // tp_size
+    return dtensor_from_parallel_logits_to_logprobs(
+        vocab_parallel_logits.to_local(), input_ids, per_rank * tp_rank, (tp_rank + 1) * per_rank, tp_group,
+        inference_only=not torch.is_grad_enabled(), seq_index=seq_index, chunk_size=chunk_size,
+        sampling_params=sampling_params)
+
+
 # ------------------------------------------------------------------------------------------------
 # packed sequences
 # ------------------------------------------------------------------------------------------------
