@@ -1,6 +1,6 @@
 // K3: token logprobs under top-k / top-p (nucleus) filtering, forward and backward, for gfx950.
 //
-// The reference sorts every 151 936-wide row (values + int64 indices).  Here one workgroup of 512
+// The reference sorts every 151 936-wide row (values + int64 indices).  Here one workgroup of 256
 // threads owns a row and never sorts it:
 //   pass 1 (HBM)   streams the row keeping 2048 chunk maxima in registers (and, when the caller
 //                  wants the unfiltered logprob too, the online log-sum-exp of the full row);
@@ -28,12 +28,12 @@
 
 namespace nrl {
 
-constexpr int kSelBlock = 512;
+constexpr int kSelBlock = 256;
 constexpr int kSelWaves = kSelBlock / kWave;
-constexpr int kSub = 4;                      // chunk maxima per thread
+constexpr int kSub = 8;                      // chunk maxima per thread
 constexpr int kChunks = kSelBlock * kSub;    // 2048
 constexpr int kCap = 4096;                   // candidate capacity (LDS); rows under a small top-k use kCapSmall
-constexpr int kCapSmall = 2048;              // ... which lets four workgroups share a compute unit instead of three
+constexpr int kCapSmall = 2048;              // ... which lets six workgroups share a compute unit instead of three
 constexpr int kSmallTopK = 512;
 
 struct Lse2 {
@@ -216,7 +216,9 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             mx[u] = fmaxf(mx[u], vm);
         }
         if (FULL_LSE) {
-            float vm = fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3]));
+            float vm = mx[0];
+#pragma unroll
+            for (int u = 1; u < kSub; ++u) vm = fmaxf(vm, mx[u]);
             const float mn = fmaxf(acc.m, vm);
             float part = 0.f;
 #pragma unroll
@@ -225,13 +227,18 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             acc.m = mn;
         }
     }
-    for (int64_t vi = base + tid; vi < nvec; vi += kSelBlock) {
+    // the ragged end of the row: fewer than kSub vectors per thread, vector u of a thread goes to its chunk u
+    // (so a short row still spreads over many chunks and the k-th largest chunk maximum stays a useful bound)
+#pragma unroll
+    for (int u = 0; u < kSub; ++u) {
+        const int64_t vi = base + u * kSelBlock + tid;
+        if (vi >= nvec) continue;
         float t[EPV];
         Row<DT>::decode(xv[vi], t);
 #pragma unroll
         for (int k = 0; k < EPV; ++k) {
             t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
-            mx[0] = fmaxf(mx[0], t[k]);
+            mx[u] = fmaxf(mx[u], t[k]);
             if (FULL_LSE) {
                 const float mn = fmaxf(acc.m, t[k]);
                 acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((t[k] - mn) * kLog2e);
@@ -318,8 +325,8 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             for (int j = 0; j < kBatch; ++j)
                 if (b0 + j < n_full) push_raw(q[j], (b0 + j) * (kSub * kSelBlock) + u * kSelBlock + tid);
         }
-        if (u == 0) {  // chunk 0 also took the ragged end of the row and the unaligned head / tail elements
-            for (int64_t vi = base + tid; vi < nvec; vi += kSelBlock) push_raw(xv[vi], vi);
+        if (base + u * kSelBlock + tid < nvec) push_raw(xv[base + u * kSelBlock + tid], base + u * kSelBlock + tid);  // ragged end
+        if (u == 0) {  // chunk 0 also took the unaligned head / tail elements
             if (tid < head) push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam)), tid);
             if (tail0 + tid < vocab)
                 push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam)), tail0 + tid);
