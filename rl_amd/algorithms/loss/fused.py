@@ -16,7 +16,6 @@ import torch
 
 from ... import ops as _ops  # noqa: F401
 from ..._lib import METRIC_SLOTS
-from .interfaces import LossType
 from .loss_functions import ClippedPGLossFn, _f32, _global_valid
 
 _OPS = torch.ops.rl_amd
@@ -149,7 +148,6 @@ def fused_logits_clipped_pg_loss(
     return loss, _metrics_dict(metrics, loss_fn, sample_mask_in)
 
 
-
 class _FusedPackedLogitsLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits2d, targets, cu, unpacked_seqlen, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags,
@@ -184,12 +182,12 @@ def fused_packed_logits_clipped_pg_loss(logits, data, loss_fn, cu_seqlens_q, cu_
                                         global_valid_toks, *, loss_scale: float = 1.0):
     """``SequencePackingFusionLossWrapper.__call__`` (``loss/wrapper.py:169-228``) in one pass over the packed
     logits: ``prepare_packed_loss_input`` + ``ClippedPGLossFn`` + the backward of the packed logprob op."""
+    from ...distributed.model_utils import _checked_cu_seqlens
     from .utils import _pack_input_ids, _pad_to
 
     reason = why_not_fusable_packed(loss_fn, logits, data)
     if reason is not None:
         raise NotImplementedError(f"fused packed logits->loss path: {reason}")
-    from ...distributed.model_utils import _checked_cu_seqlens
 
     dev = logits.device
     input_ids = data["input_ids"]
