@@ -324,6 +324,11 @@ int nrl_soft_cross_entropy_bwd(const nrl_rows* student, const void* teacher, int
                                const float* grad, void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner,
                                void* stream);
 
+/* Ascending indices of the non-zero entries of values [n] (NaN counts as non-zero) and their number: the
+ * selection `arange(n)[std != 0.0]` of dynamic_sampling (nemo_rl/algorithms/grpo.py:1752-1758).
+ * indices_out: int32 [n] (the first *count_out entries are written). */
+int nrl_nonzero_indices(const float* values, int64_t n, int32_t* indices_out, int32_t* count_out, void* stream);
+
 /* Per-sequence multiplicative logprob error and the mask that drops sequences above a threshold.
  * Replaces compute_and_apply_seq_logprob_error_masking (nemo_rl/algorithms/grpo.py:2513-2640):
  * err[b] = sum_t exp(|gen - prev| * m) * m / max(sum_t m, 1) over t >= 1 with m = token_mask[b,t] * sample_mask[b]

@@ -114,3 +114,10 @@ def seq_logprob_error_masking(prev_logprobs, generation_logprobs, token_mask, sa
     out["num_masked_seqs"] = n_masked
     out["masked_correct_pct"] = pct
     return out, new_mask
+
+
+def dynamic_sampling_keep_indices(std):
+    """``dynamic_sampling`` (``nemo_rl/algorithms/grpo.py:1752-1758``): the rows whose prompt group has a
+    non-zero reward spread, ``arange(n)[std != 0.0]`` (ascending; NaN counts as non-zero)."""
+    mask = std != 0.0
+    return torch.arange(len(mask))[mask].tolist()

@@ -96,6 +96,7 @@ SIGNATURES = {
     "nrl_gather_logprob_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P, _P, _I64, _I64, _P]),
     "nrl_soft_cross_entropy_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _I64, _P, _P, _P, _P]),
     "nrl_soft_cross_entropy_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _I64, _P, _P, _P, _P, _I64, _I64, _P]),
+    "nrl_nonzero_indices": (C.c_int, [_P, _I64, _P, _P, _P]),
     "nrl_seq_logprob_error": (C.c_int, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _I64, C.c_int32, C.c_float, _P, _P, _P, _P, _I64, _P]),
     "nrl_lmhead_fwd_workspace_bytes": (_I64, [_I64, _I64]),
     "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P]),

@@ -46,7 +46,7 @@ _PATCHED = {
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
     "nemo_rl.models.megatron.train": ["LogprobsPostProcessor"],
-    "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking"],
+    "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking", "dynamic_sampling"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }
 

@@ -171,9 +171,44 @@ __global__ __launch_bounds__(kAdvBlock) void seq_err_finish_kernel(SeqErrArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Indices of the non-zero entries of a vector, ascending: the prompt groups that dynamic sampling keeps
+// (std != 0).  One workgroup walks the vector 256 entries at a time; a wave's ballot and the waves'
+// running counts give every kept entry its output slot, so the order of the input is preserved.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kAdvBlock) void nonzero_indices_kernel(const float* v, int64_t n, int32_t* idx, int32_t* count) {
+    __shared__ int wave_cnt[kAdvWaves];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    int base = 0;
+    for (int64_t i0 = 0; i0 < n; i0 += kAdvBlock) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool keep = i < n && v[i] != 0.0f;  // NaN != 0 is true, as in the reference's `std != 0.0`
+        const unsigned long long ballot = __ballot(keep);
+        if (lane == 0) wave_cnt[wave] = __popcll(ballot);
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kAdvWaves; ++w) {
+            before += w < wave ? wave_cnt[w] : 0;
+            total += wave_cnt[w];
+        }
+        if (keep) idx[base + before + __popcll(ballot & ((1ull << lane) - 1ull))] = static_cast<int32_t>(i);
+        base += total;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *count = base;
+}
+
 }  // namespace nrl
 
 using namespace nrl;
+
+extern "C" int nrl_nonzero_indices(const float* values, int64_t n, int32_t* indices_out, int32_t* count_out, void* stream) {
+    if (n < 0 || n >= (1ll << 31)) return fail(NRL_E_INVALID, "bad length %lld", (long long)n);
+    if (!count_out || (n > 0 && (!values || !indices_out))) return fail(NRL_E_INVALID, "null argument");
+    nonzero_indices_kernel<<<dim3(1), dim3(kAdvBlock), 0, static_cast<hipStream_t>(stream)>>>(values, n, indices_out, count_out);
+    return check_launch("nonzero_indices");
+}
 
 extern "C" int64_t nrl_group_workspace_bytes(int64_t batch) {
     const int64_t b = batch < 1 ? 1 : batch;

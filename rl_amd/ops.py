@@ -549,6 +549,29 @@ for _name, _fn in (("grpo_loss", _grpo_loss), ("nll_loss", _nll_loss)):
     _LIB.impl(_name, _fn, "CPU")
 
 
+_LIB.define("nonzero_indices(Tensor values) -> Tensor")
+
+
+def _nonzero_indices(values):
+    """Ascending int64 indices of the non-zero entries of a 1-D fp32 tensor."""
+    _need_gpu(values)
+    if values.dim() != 1 or values.dtype != torch.float32:
+        raise ValueError(f"values must be fp32 [n], got {values.dtype} {tuple(values.shape)}")
+    v = values.contiguous()
+    n = v.shape[0]
+    dev = v.device
+    with torch.cuda.device(dev):
+        idx = torch.empty((max(n, 1),), dtype=torch.int32, device=dev)
+        count = torch.empty((1,), dtype=torch.int32, device=dev)
+        code = _lib.load().nrl_nonzero_indices(_ptr(v), n, _ptr(idx), _ptr(count), _stream())
+    _lib.check(code, "nrl_nonzero_indices")
+    return idx[: int(count.item())].to(torch.int64)
+
+
+_LIB.impl("nonzero_indices", _nonzero_indices, "CUDA")
+_LIB.impl("nonzero_indices", _nonzero_indices, "CPU")
+
+
 # ------------------------------------------------------------------------------------------------
 # preference losses (DPO, reward model) and the per-sample NLL rows
 # ------------------------------------------------------------------------------------------------

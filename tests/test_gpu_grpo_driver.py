@@ -55,3 +55,92 @@ def test_clip_grpo_advantages():
     assert torch.equal(_clip_grpo_advantages(adv, {"advantage_clip_low": -2.0, "advantage_clip_high": 3.0}).cpu(),
                        torch.tensor([[-2.0, 0.5, 3.0]]))
     assert _clip_grpo_advantages(adv, {"advantage_clip_low": None, "advantage_clip_high": None}) is adv
+
+
+# ---- dynamic sampling (DAPO): scenarios of the reference's tests (tests/unit/algorithms/test_grpo.py:1701-1960) ----
+def _ds_batch(n, rewards):
+    from rl_amd.distributed.batched_data_dict import BatchedDataDict
+
+    logs = [[{"role": "user", "content": f"prompt_{i // 3}"}, {"role": "assistant", "content": f"response_{i}"}] for i in range(n)]
+    return BatchedDataDict({"message_log": logs, "task_name": ["math"] * n, "total_reward": torch.tensor(rewards)})
+
+
+def _ds_config(prompts, gens, max_batches=5, enabled=True):
+    from types import SimpleNamespace
+
+    return SimpleNamespace(grpo=SimpleNamespace(use_dynamic_sampling=enabled, num_prompts_per_step=prompts,
+                                                num_generations_per_prompt=gens, dynamic_sampling_max_gen_batches=max_batches))
+
+
+@pytest.mark.parametrize("n", [0, 1, 63, 64, 65, 256, 257, 5000])
+def test_nonzero_indices_matches_oracle(n):
+    from oracle import advantage as A
+
+    g = torch.Generator().manual_seed(n)
+    v = torch.randn(n, generator=g) * (torch.rand(n, generator=g) < 0.5)
+    if n > 2:
+        v[1] = float("nan")
+        v[2] = -0.0
+    got = torch.ops.rl_amd.nonzero_indices(v.to(DEV))
+    assert got.dtype == torch.int64 and got.tolist() == A.dynamic_sampling_keep_indices(v)
+
+
+def test_dynamic_sampling_keeps_every_group_with_spread():
+    from rl_amd.algorithms.grpo import dynamic_sampling
+
+    batch = _ds_batch(6, [1.0, 0.0, 1.0, 0.5, 0.5, 0.0])
+    std = torch.tensor([0.5, 0.5, 0.5, 0.25, 0.25, 0.25])
+    baseline = torch.tensor([0.67, 0.67, 0.67, 0.33, 0.33, 0.33])
+    out, complete, cache, metrics = dynamic_sampling(batch, std, baseline, 1, _ds_config(2, 3))
+    assert out.size == 6 and complete is True
+    assert torch.allclose(out["std"], std) and torch.allclose(out["baseline"], baseline)
+    assert metrics == {"dynamic_sampling_num_discarded_valid_samples": 0}
+
+
+def test_dynamic_sampling_drops_groups_without_spread():
+    from rl_amd.algorithms.grpo import dynamic_sampling
+
+    batch = _ds_batch(6, [1.0, 1.0, 1.0, 0.5, 0.5, 0.0])
+    std = torch.tensor([0.0, 0.0, 0.0, 0.25, 0.25, 0.25])
+    baseline = torch.tensor([1.0, 1.0, 1.0, 0.33, 0.33, 0.33])
+    out, complete, _cache, _ = dynamic_sampling(batch, std, baseline, 1, _ds_config(1, 3))
+    assert out.size == 3 and complete is True
+    assert torch.allclose(out["std"], torch.tensor([0.25, 0.25, 0.25]))
+    assert torch.allclose(out["baseline"], torch.tensor([0.33, 0.33, 0.33]))
+    assert [out["message_log"][i][0]["content"] for i in range(out.size)] == ["prompt_1"] * 3
+    assert torch.allclose(out["filtered_reward"], torch.tensor([0.5, 0.5, 0.0]))
+
+
+def test_dynamic_sampling_rows_stay_aligned_through_filter_and_cut():
+    from rl_amd.algorithms.grpo import dynamic_sampling
+
+    batch = _ds_batch(9, [1.0, 0.0, 1.0, 0.5, 0.0, 0.5, 0.2, 0.6, 0.9])
+    batch["mask_sample"] = torch.tensor([False, True, False, True, False, True, False, False, True])
+    std = torch.tensor([0.5, 0.5, 0.5, 0.25, 0.25, 0.25, 0.35, 0.35, 0.35])
+    baseline = torch.tensor([0.67, 0.67, 0.67, 0.33, 0.33, 0.33, 0.57, 0.57, 0.57])
+    out, complete, _, metrics = dynamic_sampling(batch, std, baseline, dynamic_sampling_num_gen_batches=1,
+                                                 master_config=_ds_config(2, 3))
+    assert complete is True and out.size == 6
+    assert torch.equal(out["mask_sample"], torch.tensor([False, True, False, True, False, True]))
+    assert metrics["dynamic_sampling_num_discarded_valid_samples"] == 3
+
+
+def test_dynamic_sampling_caches_until_enough_and_gives_up_after_the_limit():
+    from rl_amd.algorithms.grpo import dynamic_sampling
+
+    std = torch.tensor([0.4, 0.4, 0.4])
+    baseline = torch.tensor([0.5, 0.5, 0.5])
+    cfg = _ds_config(2, 3)
+    out, complete, cache, _ = dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 1, cfg)
+    assert out.size == 3 and complete is False and cache is not None and cache == out
+    out, complete, cache, _ = dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 1, cfg, None, cache)
+    assert out.size == 6 and complete is True and cache is not None
+    # nothing kept: the batch is ignored, the cache is left alone
+    out, complete, cache2, _ = dynamic_sampling(_ds_batch(3, [1.0, 1.0, 1.0]), torch.zeros(3), baseline, 2, cfg, None, None)
+    assert out.size == 0 and complete is False and cache2 is None
+    with pytest.raises(ValueError):
+        dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 6, cfg)
+    # switched off: the batch comes back whole, with baseline and std attached
+    batch = _ds_batch(3, [1.0, 1.0, 1.0])
+    out, complete, _, metrics = dynamic_sampling(batch, torch.zeros(3), baseline, 1, _ds_config(2, 3, enabled=False))
+    assert out is batch and complete is True and metrics == {} and torch.equal(out["std"], torch.zeros(3))

@@ -114,3 +114,19 @@ def test_seq_logprob_error_masking_brute_force():
     kept = [errs[i] for i in range(b) if want_mask[i] and errs[i] is not None]
     assert abs(got["max_seq_mult_prob_error_after_mask"] - max(kept)) < 1e-5
     assert abs(got["min_seq_mult_prob_error_after_mask"] - min(kept)) < 1e-5
+
+
+def test_dynamic_sampling_keep_indices_brute_force():
+    """``oracle.advantage.dynamic_sampling_keep_indices`` against a plain loop, and on the std vectors of the
+    reference's tests (``tests/unit/algorithms/test_grpo.py:1733-1736, 1790-1793``)."""
+    from oracle import advantage as A
+
+    g = torch.Generator().manual_seed(0)
+    v = torch.randn(200, generator=g) * (torch.rand(200, generator=g) < 0.6)
+    v[17] = float("nan")
+    v[40] = -0.0
+    want = [i for i in range(200) if not (v[i].item() == 0.0)]
+    assert A.dynamic_sampling_keep_indices(v) == want and 17 in want and 40 not in want
+    assert A.dynamic_sampling_keep_indices(torch.tensor([0.5, 0.5, 0.5, 0.25, 0.25, 0.25])) == [0, 1, 2, 3, 4, 5]
+    assert A.dynamic_sampling_keep_indices(torch.tensor([0.0, 0.0, 0.0, 0.25, 0.25, 0.25])) == [3, 4, 5]
+    assert A.dynamic_sampling_keep_indices(torch.zeros(0)) == []
