@@ -240,6 +240,35 @@ int nrl_fused_packed_logits_grpo_loss(const nrl_rows* rows, int32_t target_is_pr
 int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,
                          float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* log_softmax over the K logits of a row at the given vocabulary indices (the teacher's top-k), the
+ * zero_outside_topk = False branch of get_distillation_topk_logprobs_from_logits
+ * (nemo_rl/distributed/model_utils.py:1981-2005): out[r, j] = x[r, idx[r, j]] - logsumexp_j x[r, idx[r, j]].
+ * indices: int64 [rows, K] global ids (ids outside [vocab_start, vocab_end) count as -inf), or NULL with
+ * K == vocab: plain log_softmax of the row (the teacher's own top-k logits, :2007-2010).  out: fp32 [rows, K].
+ * _bwd: dlogits (layout as in nrl_logprob_bwd) is zero except at the K indices, where it holds
+ * grad[j] - exp(logprobs[j]) * sum_q grad[q] (summed over duplicates of an index). */
+int nrl_topk_logsoftmax_fwd(const nrl_rows* rows, const int64_t* indices, int64_t k, float* out, void* stream);
+int nrl_topk_logsoftmax_bwd(const nrl_rows* rows, const int64_t* indices, int64_t k, const float* logprobs,
+                            const float* grad, void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner,
+                            void* stream);
+
+/* DistillationLossFn (nemo_rl/algorithms/loss/loss_functions.py:1124-1206) on top-k log-probabilities,
+ * forward and gradients in one call.  student / teacher logprobs: contiguous fp32 [B, n, K]; h_all: fp32
+ * [B, n] (sum_v p log p of the student's full rows) or NULL.  kl_type 0 forward sum t_p (t - s), 1 reverse
+ * sum s_p (s - t), 2 mixed with weight mixed_kl_weight on the forward term.  With zero_outside_topk and a
+ * non-forward kl_type the correction (H_all - sum s_p s) - log_infinitesimal * (1 - sum s_p) is added (times
+ * 1 - mixed_kl_weight when mixed).  With token_mask: loss = sum(per_token * token_mask * sample_mask) /
+ * (global_valid_toks[0] + 1e-8); with token_mask == NULL the plain mean over the B * n tokens.
+ * d_student_out: fp32 [B, n, K]; d_h_all_out: fp32 [B, n] (written when the correction applies).
+ * workspace: nrl_distill_topk_loss_workspace_bytes(B, n) bytes, 8-byte aligned. */
+int64_t nrl_distill_topk_loss_workspace_bytes(int64_t batch, int64_t n);
+int nrl_distill_topk_loss_fwd_bwd(const float* student_logprobs, const float* teacher_logprobs, const float* h_all,
+                                  const float* token_mask, int64_t token_mask_stride, const float* sample_mask,
+                                  const float* global_valid_toks, int64_t batch, int64_t n, int64_t k,
+                                  int32_t kl_type, float mixed_kl_weight, int32_t zero_outside_topk,
+                                  float log_infinitesimal, float* loss_out, float* d_student_out, float* d_h_all_out,
+                                  void* workspace, int64_t workspace_bytes, void* stream);
+
 /* NLLLossFn per-sample branch (dpo_loss=True, loss_functions.py:823-829): loss_rows_out[b] =
  * -sum_t lp[b,t] * token_mask[b,t] * sample_mask[b], divided by max(sum_t mask, 1) with
  * average_log_probs; den_out[b] is that divisor (1 without averaging); totals_out[0..1] =

@@ -39,8 +39,10 @@ Pinning status (what fixes each function besides its own text):
 * ``logprob.logprobs_post_process``  pinned: ``log_softmax`` + ``gather``
                            identity and brute-force loops on tiny inputs.
 * ``distill.*``            pinned: closed forms (uniform / one-hot rows, H(p,q) =
-                           H(p) + KL), the reference's stated backward formulas
-                           and brute force (``tests/test_oracle_distill.py``).
+                           H(p) + KL; equal distributions give zero KL; a top-k
+                           spanning the vocabulary gives the textbook KL), the
+                           reference's stated backward formulas and brute force
+                           (``tests/test_oracle_distill.py``).
 * ``preference.*``         pinned: the closed-form cases of the reference's own
                            DPO tests (zero logits vs zero reference, SFT term of
                            the chosen rows, SFT-only == rescaled NLL) and a

@@ -84,6 +84,11 @@ SIGNATURES = {
     "nrl_fused_packed_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.c_int32, _P, _I64, C.POINTER(NrlGrpoCfg),
                                                     C.POINTER(NrlGrpoInputs), _F, _P, _I64, _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _I64, _P]),
+    "nrl_topk_logsoftmax_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P]),
+    "nrl_topk_logsoftmax_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P, _P, _I64, _I64, _P]),
+    "nrl_distill_topk_loss_workspace_bytes": (_I64, [_I64, _I64]),
+    "nrl_distill_topk_loss_fwd_bwd": (C.c_int, [_P, _P, _P, _P, _I64, _P, _P, _I64, _I64, _I64, C.c_int32, _F, C.c_int32, _F,
+                                                _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_rows_fwd": (C.c_int, [_P, _I64, _P, _I64, _P, _I64, _I64, C.c_int32, _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_rows_bwd": (C.c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P]),
     "nrl_dpo_workspace_bytes": (_I64, [_I64]),

@@ -10,6 +10,8 @@ from .interfaces import LossFunction, LossInputType, LossType, MetricNormalizer
 from .loss_functions import (
     ClippedPGLossConfig,
     ClippedPGLossFn,
+    DistillationLossConfig,
+    DistillationLossFn,
     DPOLossConfig,
     DPOLossFn,
     NLLLossFn,
@@ -24,7 +26,7 @@ from .wrapper import (
 
 __all__ = [
     "fused_logits_clipped_pg_loss", "fused_packed_logits_clipped_pg_loss", "why_not_fusable", "why_not_fusable_packed",
-    "ClippedPGLossConfig", "ClippedPGLossFn", "DPOLossConfig", "DPOLossFn", "NLLLossFn", "PreferenceLossFn", "LossFunction", "LossInputType", "LossType",
+    "ClippedPGLossConfig", "ClippedPGLossFn", "DistillationLossConfig", "DistillationLossFn", "DPOLossConfig", "DPOLossFn", "NLLLossFn", "PreferenceLossFn", "LossFunction", "LossInputType", "LossType",
     "MetricNormalizer", "prepare_loss_input", "prepare_packed_loss_input", "SequencePackingFusionLossWrapper",
     "SequencePackingLossWrapper", "wrap_loss_fn_with_input_preparation",
 ]

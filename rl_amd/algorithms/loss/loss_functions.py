@@ -440,3 +440,67 @@ class DPOLossFn(PreferenceLossFn):
         m = metrics.cpu().tolist()
         return loss, {"loss": m[0], "sft_loss": m[1], "preference_loss": m[2], "accuracy": m[3], "rewards_chosen_mean": m[4],
                       "rewards_rejected_mean": m[5], "num_valid_samples": m[6]}
+
+
+class DistillationLossConfig(BaseModel, extra="allow"):
+    """Field names and defaults of ``loss_functions.py:1109-1112``."""
+
+    kl_type: str = "mixed"
+    mixed_kl_weight: float = 0.5
+    zero_outside_topk: bool = False
+
+
+class _DistillTopk(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, student_lp, teacher_lp, h_all, token_mask, sample_mask, global_valid_toks, kl_type, w, zero_outside, log_inf):
+        loss, d_s, d_h = _OPS.distill_topk_loss(student_lp.detach(), teacher_lp.detach(), None if h_all is None else h_all.detach(),
+                                                token_mask, sample_mask, global_valid_toks, kl_type, w, zero_outside, log_inf)
+        ctx.save_for_backward(d_s, d_h)
+        ctx.has_h = h_all is not None and d_h.numel() > 0
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        d_s, d_h = ctx.saved_tensors
+        return (d_s * grad_loss, None, d_h * grad_loss if ctx.has_h else None) + (None,) * 7
+
+
+class DistillationLossFn(LossFunction):
+    """Top-k distillation loss (``loss_functions.py:1124-1206``): forward, reverse or mixed KL between the
+    teacher's and the student's top-k log-probabilities per token, optionally with the correction for the
+    student's mass outside the top-k, masked mean over the tokens.  One fused call returns the loss and
+    the gradients with respect to the student's top-k log-probabilities and ``H_all``."""
+
+    loss_type = LossType.TOKEN_LEVEL
+    input_type = LossInputType.DISTILLATION
+    _KL = {"forward": 0, "reverse": 1, "mixed": 2}
+
+    def __init__(self, cfg):
+        get = cfg.get if isinstance(cfg, dict) else lambda k, d=None: getattr(cfg, k, d)  # noqa: E731
+        defaults = DistillationLossConfig()
+        self.kl_type = get("kl_type", defaults.kl_type)
+        self.mixed_kl_weight = get("mixed_kl_weight", defaults.mixed_kl_weight)
+        self.zero_outside_topk = get("zero_outside_topk", defaults.zero_outside_topk)
+        self.log_infinitesimal = -100
+        assert self.kl_type in ["forward", "reverse", "mixed"], "Invalid KL type"
+        assert self.mixed_kl_weight >= 0 and self.mixed_kl_weight <= 1, (
+            "Invalid mixed KL weight"
+        )
+
+    def __call__(self, student_topk_logprobs, teacher_topk_logprobs, H_all, data, global_valid_seqs, global_valid_toks):
+        home = student_topk_logprobs.device
+        dev = _gpu_for(student_topk_logprobs)
+        token_mask = sample_mask = valid = None
+        if "token_mask" in data and "sample_mask" in data:
+            n = student_topk_logprobs.shape[1]
+            token_mask = _f32(data["token_mask"][:, 1:][:, :n], dev)
+            sample_mask = _f32(data["sample_mask"], dev)
+            valid = _global_valid(1.0, global_valid_toks, dev)[1:]
+        loss = _DistillTopk.apply(
+            _f32(student_topk_logprobs, dev), _f32(teacher_topk_logprobs, dev), None if H_all is None else _f32(H_all, dev),
+            token_mask, sample_mask, valid, self._KL[self.kl_type], float(self.mixed_kl_weight), bool(self.zero_outside_topk),
+            float(self.log_infinitesimal),
+        )
+        if home != dev:
+            loss = loss.to(home)
+        return loss, {"loss": float(loss.item()), "num_valid_samples": data["input_ids"].shape[0]}

@@ -35,6 +35,20 @@ def prepare_loss_input(
     top-p active ``data`` gains ``curr_logprobs_unfiltered`` when the loss has a KL penalty."""
     if loss_fn.input_type == LossInputType.LOGIT:
         return {"logits": logits}, data
+    if loss_fn.input_type == LossInputType.DISTILLATION:  # ``loss/utils.py:122-141``
+        from ...distributed.model_utils import get_distillation_topk_logprobs_from_logits
+
+        student, teacher, h_all = get_distillation_topk_logprobs_from_logits(
+            student_logits=logits,
+            teacher_topk_logits=data["teacher_topk_logits"],
+            teacher_topk_indices=data["teacher_topk_indices"],
+            zero_outside_topk=loss_fn.zero_outside_topk,
+            calculate_entropy=loss_fn.zero_outside_topk and loss_fn.kl_type != "forward",
+            vocab_parallel_rank=vocab_parallel_rank,
+            vocab_parallel_group=vocab_parallel_group,
+            context_parallel_group=context_parallel_group,
+        )
+        return {"student_topk_logprobs": student, "teacher_topk_logprobs": teacher, "H_all": h_all}, data
     if loss_fn.input_type != LossInputType.LOGPROB:
         raise ValueError(f"Unknown loss function input type: {loss_fn.input_type}")
 

@@ -38,11 +38,13 @@ _PATCHED = {
         "from_parallel_logits_to_logprobs", "from_parallel_logits_to_logprobs_packed_sequences",
         "from_parallel_hidden_states_to_logprobs", "get_next_token_logprobs_from_logits",
         "dtensor_from_parallel_logits_to_logprobs", "get_logprobs_from_vocab_parallel_logits",
+        "get_distillation_topk_logprobs_from_logits",
         "ChunkedDistributedEntropy", "ChunkedDistributedGatherLogprob", "DistributedCrossEntropy",
     ],
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
     "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],
-    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn"],
+    "nemo_rl.algorithms.loss.utils": ["prepare_loss_input", "prepare_packed_loss_input"],
+    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
     "nemo_rl.models.megatron.train": ["LogprobsPostProcessor"],

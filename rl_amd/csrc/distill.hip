@@ -327,6 +327,138 @@ __global__ __launch_bounds__(kDBlock) void soft_ce_bwd_kernel(RowsView x, RowsVi
     });
 }
 
+// ---------------------------------------------------------------------------------------------
+// log-softmax over K selected logits of a row: the K given vocabulary indices (the teacher's top-k) or,
+// without indices, the row as it is (K = vocab).  The backward scatters into a zero-filled row.
+// ---------------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void topk_logsoftmax_fwd_kernel(RowsView x, GatherArgs ga, float* __restrict__ out) {
+    __shared__ Lse smem[kDWaves];
+    const int64_t r = blockIdx.x;
+    const char* row = row_ptr<DT>(x, r);
+    auto value = [&](int64_t j) -> float {
+        if (!ga.idx) return Row<DT>::load1(row, j);
+        const int64_t gi = ga.idx[r * ga.k + j];
+        return (gi >= ga.vstart && gi < ga.vend) ? Row<DT>::load1(row, gi - ga.vstart) : -INFINITY;
+    };
+    Lse a{-FLT_MAX, 0.f};
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) lse_push1(a, value(j));
+    const Lse t = block_lse<kDWaves>(a, smem);
+    const float lse = t.m + logf(t.s);
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) out[r * ga.k + j] = value(j) - lse;
+}
+
+// d x[idx_j] = sum over duplicates of (g_j - exp(lp_j) * sum_q g_q); every other element of the row is zero
+template <int DT>
+__global__ __launch_bounds__(kDBlock) void topk_logsoftmax_bwd_kernel(RowsView d, GatherArgs ga, const float* __restrict__ lp,
+                                                                      const float* __restrict__ grad) {
+    __shared__ float sm[kDWaves];
+    const int64_t r = blockIdx.x;
+    void* out = const_cast<char*>(row_ptr<DT>(d, r));
+    float part = 0.f;
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) part += grad[r * ga.k + j];
+    const float gsum = block_sum<float, kDWaves>(part, sm);
+    row_fill_zero<DT>(out, d.vocab);
+    __syncthreads();  // the zero fill of this workgroup is visible to it before the K values land
+    for (int64_t j = threadIdx.x; j < ga.k; j += kDBlock) {
+        const int64_t gi = ga.idx[r * ga.k + j];
+        if (gi < ga.vstart || gi >= ga.vend) continue;
+        float add = 0.f;
+        for (int64_t q = 0; q < ga.k; ++q)
+            add += ga.idx[r * ga.k + q] == gi ? grad[r * ga.k + q] - expf(lp[r * ga.k + q]) * gsum : 0.f;
+        Row<DT>::store1(out, gi - ga.vstart, add);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// distillation loss on top-k log-probabilities: forward / reverse / mixed KL per token over the K entries,
+// plus the correction for the mass outside the top-k, masked mean over the tokens; loss and gradients in
+// one pass.  One wave per token; a workgroup's four token sums go to one partial, the partials are added
+// in index order by the finish kernel.
+// ---------------------------------------------------------------------------------------------
+struct KdArgs {
+    const float* s_lp;         // [tokens, K] student log-probabilities
+    const float* t_lp;         // [tokens, K] teacher log-probabilities
+    const float* h_all;        // [tokens] sum_v p log p of the student's full row, or NULL
+    const float* token_mask;   // [B, n] with row stride, or NULL (plain mean over the tokens)
+    const float* sample_mask;  // [B]
+    const float* global_valid; // [1] = valid tokens (index 1 of the usual pair)
+    int64_t batch, n, k, tm_stride;
+    int kl_type;               // 0 forward, 1 reverse, 2 mixed
+    float w, log_infinitesimal;
+    int correct;               // add the outside-top-k term
+    float* d_s;                // [tokens, K]
+    float* d_h;                // [tokens] or NULL
+    double* parts;             // one per workgroup
+    float* loss;
+};
+
+__global__ __launch_bounds__(kDBlock) void distill_topk_loss_kernel(KdArgs a) {
+    __shared__ double sm[kDWaves];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t tokens = a.batch * a.n;
+    const int64_t tok = static_cast<int64_t>(blockIdx.x) * kDWaves + wave;
+    double contrib = 0.0;
+    if (tok < tokens) {
+        const int64_t b = tok / a.n, t = tok - b * a.n;
+        const float den = a.token_mask ? a.global_valid[0] + 1e-8f : static_cast<float>(tokens);
+        const float mask = a.token_mask ? a.token_mask[b * a.tm_stride + t] * a.sample_mask[b] : 1.f;
+        const float wt = mask / den;  // d loss / d per-token value
+        const float wf = a.kl_type == 0 ? 1.f : a.kl_type == 1 ? 0.f : a.w;  // weight of the forward term
+        const float wr = 1.f - wf;                                            // ... of the reverse term
+        const float c = a.correct ? (a.kl_type == 2 ? 1.f - a.w : 1.f) : 0.f;
+        const float* sl = a.s_lp + tok * a.k;
+        const float* tl = a.t_lp + tok * a.k;
+        float fwd = 0.f, rev = 0.f, sp_slp = 0.f, sp_sum = 0.f;
+        for (int64_t j = lane; j < a.k; j += kWave) {
+            const float s = sl[j], u = tl[j];
+            const float sp = expf(s), tp = expf(u);
+            fwd += tp * (u - s);
+            rev += sp * (s - u);
+            sp_slp += sp * s;
+            sp_sum += sp;
+            float g = wf * -tp + wr * sp * (s - u + 1.f);
+            if (a.correct) g -= c * sp * (s + 1.f - a.log_infinitesimal);
+            a.d_s[tok * a.k + j] = wt * g;
+        }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            fwd += __shfl_xor(fwd, off, kWave);
+            rev += __shfl_xor(rev, off, kWave);
+            sp_slp += __shfl_xor(sp_slp, off, kWave);
+            sp_sum += __shfl_xor(sp_sum, off, kWave);
+        }
+        float per_token = wf * fwd + wr * rev;
+        if (a.correct) {
+            const float h_rest = a.h_all[tok] - sp_slp, p_rest = 1.f - sp_sum;
+            per_token += c * (h_rest - a.log_infinitesimal * p_rest);
+        }
+        if (lane == 0) {
+            if (a.d_h) a.d_h[tok] = wt * c;
+            contrib = static_cast<double>(per_token * mask);
+        }
+    }
+    if (lane == 0) sm[wave] = contrib;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double tot = 0.0;
+#pragma unroll
+        for (int w = 0; w < kDWaves; ++w) tot += sm[w];
+        a.parts[blockIdx.x] = tot;
+    }
+}
+
+__global__ __launch_bounds__(kDBlock) void distill_topk_finish_kernel(KdArgs a, int64_t n_parts) {
+    __shared__ double sm[kDWaves];
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < n_parts; i += kDBlock) acc += a.parts[i];
+    acc = block_sum<double, kDWaves>(acc, sm);
+    if (threadIdx.x == 0) {
+        const float den = a.token_mask ? a.global_valid[0] + 1e-8f : static_cast<float>(a.batch * a.n);
+        *a.loss = static_cast<float>(acc) / den;
+    }
+}
+
 static int check_view(const nrl_rows* r) {
     if (!r) return fail(NRL_E_INVALID, "rows is NULL");
     if (r->dtype != NRL_F32 && r->dtype != NRL_BF16 && r->dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype %d", r->dtype);
@@ -431,4 +563,69 @@ extern "C" int nrl_soft_cross_entropy_bwd(const nrl_rows* student, const void* t
     NRL_DT_DISPATCH(student->dtype,
                     soft_ce_bwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, y, lse_student, lse_teacher, grad, d));
     return check_launch("soft_cross_entropy_bwd");
+}
+
+extern "C" int nrl_topk_logsoftmax_fwd(const nrl_rows* rows, const int64_t* indices, int64_t k, float* out, void* stream) {
+    if (int e = check_view(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (k < 0) return fail(NRL_E_INVALID, "negative K");
+    if (!indices && k != rows->vocab) return fail(NRL_E_INVALID, "without indices K must be the row length");
+    if (n == 0 || k == 0) return NRL_OK;
+    if (!out) return fail(NRL_E_INVALID, "null output");
+    if (rows->vocab_end - rows->vocab_start != rows->vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
+    const RowsView x = view_of(rows);
+    const GatherArgs ga{indices, k, rows->vocab_start, rows->vocab_end};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DT_DISPATCH(rows->dtype, topk_logsoftmax_fwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(x, ga, out));
+    return check_launch("topk_logsoftmax_fwd");
+}
+
+extern "C" int nrl_topk_logsoftmax_bwd(const nrl_rows* rows, const int64_t* indices, int64_t k, const float* logprobs,
+                                       const float* grad, void* dlogits, int64_t d_stride_outer, int64_t d_stride_inner,
+                                       void* stream) {
+    if (int e = check_view(rows)) return e;
+    const int64_t n = rows->n_outer * rows->n_inner;
+    if (k < 0) return fail(NRL_E_INVALID, "negative K");
+    if (n == 0) return NRL_OK;
+    if (!dlogits || (k > 0 && (!indices || !logprobs || !grad))) return fail(NRL_E_INVALID, "null argument");
+    if (rows->vocab_end - rows->vocab_start != rows->vocab) return fail(NRL_E_INVALID, "vocab range does not span the columns");
+    const RowsView d = view_of(rows, dlogits, d_stride_outer, d_stride_inner);
+    const GatherArgs ga{indices, k, rows->vocab_start, rows->vocab_end};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DT_DISPATCH(rows->dtype, topk_logsoftmax_bwd_kernel<DT><<<dim3((unsigned)n), dim3(kDBlock), 0, s>>>(d, ga, logprobs, grad));
+    return check_launch("topk_logsoftmax_bwd");
+}
+
+extern "C" int64_t nrl_distill_topk_loss_workspace_bytes(int64_t batch, int64_t n) {
+    const int64_t tokens = batch * n;
+    return ((tokens + kDWaves - 1) / kDWaves + 1) * static_cast<int64_t>(sizeof(double));
+}
+
+extern "C" int nrl_distill_topk_loss_fwd_bwd(const float* student_logprobs, const float* teacher_logprobs, const float* h_all,
+                                             const float* token_mask, int64_t token_mask_stride, const float* sample_mask,
+                                             const float* global_valid_toks, int64_t batch, int64_t n, int64_t k,
+                                             int32_t kl_type, float mixed_kl_weight, int32_t zero_outside_topk,
+                                             float log_infinitesimal, float* loss_out, float* d_student_out, float* d_h_all_out,
+                                             void* workspace, int64_t workspace_bytes, void* stream) {
+    if (batch < 0 || n < 0 || k < 0) return fail(NRL_E_INVALID, "bad shape [%lld, %lld, %lld]", (long long)batch, (long long)n, (long long)k);
+    if (kl_type < 0 || kl_type > 2) return fail(NRL_E_INVALID, "kl_type must be 0 (forward), 1 (reverse) or 2 (mixed)");
+    if (!loss_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
+    if (workspace_bytes < nrl_distill_topk_loss_workspace_bytes(batch, n)) return fail(NRL_E_WORKSPACE, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7) return fail(NRL_E_INVALID, "workspace must be 8-byte aligned");
+    const int64_t tokens = batch * n;
+    if (tokens >= (1ll << 31) * kDWaves) return fail(NRL_E_INVALID, "too many tokens");
+    const bool correct = zero_outside_topk && kl_type != 0;
+    if (tokens * k > 0 && (!student_logprobs || !teacher_logprobs || !d_student_out)) return fail(NRL_E_INVALID, "null logprobs or gradient output");
+    if (tokens > 0 && correct && !h_all) return fail(NRL_E_INVALID, "H_all is NULL");
+    if (tokens > 0 && token_mask && (!sample_mask || !global_valid_toks)) return fail(NRL_E_INVALID, "null sample_mask or global_valid_toks");
+    KdArgs a;
+    a.s_lp = student_logprobs; a.t_lp = teacher_logprobs; a.h_all = h_all; a.token_mask = token_mask; a.sample_mask = sample_mask;
+    a.global_valid = global_valid_toks; a.batch = batch; a.n = n; a.k = k; a.tm_stride = token_mask_stride;
+    a.kl_type = kl_type; a.w = mixed_kl_weight; a.log_infinitesimal = log_infinitesimal; a.correct = correct;
+    a.d_s = d_student_out; a.d_h = correct ? d_h_all_out : nullptr; a.parts = static_cast<double*>(workspace); a.loss = loss_out;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t n_parts = (tokens + kDWaves - 1) / kDWaves;
+    if (n_parts > 0) distill_topk_loss_kernel<<<dim3((unsigned)n_parts), dim3(kDBlock), 0, s>>>(a);
+    distill_topk_finish_kernel<<<dim3(1), dim3(kDBlock), 0, s>>>(a, n_parts);
+    return check_launch("distill_topk_loss_fwd_bwd");
 }

@@ -529,3 +529,77 @@ class DistributedCrossEntropy(torch.autograd.Function):
         g = grad_outputs[0].to(torch.float32).reshape(lx.shape).contiguous()
         d = torch.ops.rl_amd.soft_cross_entropy_bwd(x, y, lx, ly, g)
         return d.reshape(ctx.in_shape), None, None, None
+
+
+class _TopkLogSoftmax(torch.autograd.Function):
+    """log_softmax over the K logits of every row at the given vocabulary indices."""
+
+    @staticmethod
+    def forward(ctx, logits, indices):
+        out = torch.ops.rl_amd.topk_logsoftmax_fwd(logits.detach(), indices)
+        ctx.save_for_backward(logits, indices, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        logits, indices, out = ctx.saved_tensors
+        return torch.ops.rl_amd.topk_logsoftmax_bwd(logits, indices, out, grad.contiguous().float()), None
+
+
+def get_distillation_topk_logprobs_from_logits(
+    student_logits: torch.Tensor,
+    teacher_topk_logits: torch.Tensor,
+    teacher_topk_indices: torch.Tensor,
+    zero_outside_topk: bool,
+    calculate_entropy: bool,
+    vocab_parallel_rank: Optional[int] = None,
+    vocab_parallel_group: Optional[Any] = None,
+    context_parallel_group: Optional[Any] = None,
+):
+    """``model_utils.py:1856-2020``: the student's log-probabilities at the teacher's top-k ids, the teacher's
+    own top-k log-probabilities and (optionally) ``H_all = sum_v p log p`` of the student rows, all cut to the
+    next-token alignment ``[:, :-1]``.
+
+    ``zero_outside_topk``: the student entries come from the full-vocabulary log-softmax (streaming gather
+    kernel); otherwise from a softmax over just the K gathered logits.  The student's fp32 copy
+    (``:1874``) is not made: the kernels read the logits in their dtype and accumulate in fp32."""
+    if teacher_topk_indices.shape[-1] <= 0:
+        raise ValueError(
+            f"topk must be positive, got {teacher_topk_indices.shape[-1]}. "
+            "topk=0 is not supported as it would result in empty tensor operations."
+        )
+    if vocab_parallel_group is not None:
+        assert vocab_parallel_rank is not None, (
+            "vocab_parallel_rank must be provided when vocab_parallel_group is provided"
+        )
+        _require_single_rank(vocab_parallel_group, "get_distillation_topk_logprobs_from_logits")
+    _require_single_rank(context_parallel_group, "get_distillation_topk_logprobs_from_logits")
+    if hasattr(student_logits, "to_local"):
+        mesh = student_logits.device_mesh
+        _require_single_rank(mesh.get_group("tp"), "get_distillation_topk_logprobs_from_logits")
+        if _mesh_dim_size(mesh, "cp") > 1:
+            raise NotImplementedError("get_distillation_topk_logprobs_from_logits: context parallelism needs more than one GPU")
+        student_logits = student_logits.to_local()
+    indices = teacher_topk_indices.to(student_logits.device)
+    if indices.dtype != torch.int64:
+        indices = indices.long()
+    vocab = student_logits.shape[-1]
+    seq = student_logits.shape[1]
+    H_all = None
+    if zero_outside_topk:
+        student_topk_logprobs = ChunkedDistributedGatherLogprob.apply(student_logits, indices, 0, vocab, seq, None, False)
+        if calculate_entropy:
+            H_all = ChunkedDistributedEntropy.apply(student_logits, seq, None, False)
+    else:
+        student_topk_logprobs = _TopkLogSoftmax.apply(student_logits, indices)
+    teacher = teacher_topk_logits.to(student_topk_logprobs.device)
+    if teacher.dim() != 3:
+        raise ValueError(f"teacher_topk_logits must be [B, S, K], got {tuple(teacher.shape)}")
+    if teacher.stride(2) != 1 and teacher.shape[2] > 1:
+        teacher = teacher.contiguous()
+    teacher_topk_logprobs = torch.ops.rl_amd.topk_logsoftmax_fwd(teacher.detach(), None)
+    teacher_topk_logprobs = teacher_topk_logprobs[:, :-1, :]
+    student_topk_logprobs = student_topk_logprobs[:, :-1, :]
+    if calculate_entropy and H_all is not None:
+        H_all = H_all[:, :-1]
+    return student_topk_logprobs, teacher_topk_logprobs, H_all

@@ -549,6 +549,91 @@ for _name, _fn in (("grpo_loss", _grpo_loss), ("nll_loss", _nll_loss)):
     _LIB.impl(_name, _fn, "CPU")
 
 
+_LIB.define("topk_logsoftmax_fwd(Tensor logits, Tensor? indices) -> Tensor")
+_LIB.define("topk_logsoftmax_bwd(Tensor logits, Tensor indices, Tensor logprobs, Tensor grad) -> Tensor")
+_LIB.define(
+    "distill_topk_loss(Tensor student_logprobs, Tensor teacher_logprobs, Tensor? h_all, Tensor? token_mask, "
+    "Tensor? sample_mask, Tensor? global_valid_toks, int kl_type, float mixed_kl_weight, bool zero_outside_topk, "
+    "float log_infinitesimal) -> (Tensor, Tensor, Tensor)"
+)
+
+
+def _topk_logsoftmax_fwd(logits, indices):
+    """log_softmax over the K logits at ``indices`` [B, S, K] of every row (or over the whole last axis)."""
+    _need_gpu(logits, indices)
+    rows = _plain_rows(logits)
+    b, s, v = logits.shape
+    if indices is not None:
+        indices = _gather_indices(logits, indices)
+    k = v if indices is None else indices.shape[2]
+    with torch.cuda.device(logits.device):
+        out = torch.empty((b, s, k), dtype=torch.float32, device=logits.device)
+        code = _lib.load().nrl_topk_logsoftmax_fwd(C.byref(rows), _ptr(indices), k, _ptr(out), _stream())
+    _lib.check(code, "nrl_topk_logsoftmax_fwd")
+    return out
+
+
+def _topk_logsoftmax_bwd(logits, indices, logprobs, grad):
+    _need_gpu(logits, indices, logprobs, grad)
+    rows = _plain_rows(logits)
+    indices = _gather_indices(logits, indices)
+    b, s, k = indices.shape
+    for name, t in (("logprobs", logprobs), ("grad", grad)):
+        if t.dtype != torch.float32 or tuple(t.shape) != (b, s, k):
+            raise ValueError(f"{name} must be fp32 [{b}, {s}, {k}], got {t.dtype} {tuple(t.shape)}")
+    logprobs, grad = logprobs.contiguous(), grad.contiguous()
+    with torch.cuda.device(logits.device):
+        d = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+        code = _lib.load().nrl_topk_logsoftmax_bwd(C.byref(rows), _ptr(indices), k, _ptr(logprobs), _ptr(grad), _ptr(d),
+                                                   d.stride(0), d.stride(1), _stream())
+    _lib.check(code, "nrl_topk_logsoftmax_bwd")
+    return d
+
+
+def _distill_topk_loss(student_logprobs, teacher_logprobs, h_all, token_mask, sample_mask, global_valid_toks, kl_type,
+                       mixed_kl_weight, zero_outside_topk, log_infinitesimal):
+    """-> (loss, d loss / d student_logprobs [B, n, K], d loss / d h_all [B, n] (empty without the correction))."""
+    _need_gpu(student_logprobs, teacher_logprobs, h_all, token_mask, sample_mask, global_valid_toks)
+    if student_logprobs.dim() != 3 or student_logprobs.shape != teacher_logprobs.shape:
+        raise ValueError(f"student / teacher logprobs must both be [B, n, K], got {tuple(student_logprobs.shape)} and "
+                         f"{tuple(teacher_logprobs.shape)}")
+    if student_logprobs.dtype != torch.float32 or teacher_logprobs.dtype != torch.float32:
+        raise ValueError("top-k logprobs must be fp32")
+    b, n, k = student_logprobs.shape
+    sl, tl = student_logprobs.contiguous(), teacher_logprobs.contiguous()
+    correct = bool(zero_outside_topk) and kl_type != 0
+    if correct:
+        if h_all is None:
+            raise ValueError("H_all is required when zero_outside_topk is set and the KL is not the forward one")
+        h_all = _row_scalar(h_all, b, n, "H_all")
+    tm, tm_stride = (None, 0) if token_mask is None else _rowmat(token_mask, b, n, "token_mask")
+    sm = _vec(sample_mask, b, "sample_mask")
+    if tm is not None and (sm is None or global_valid_toks is None):
+        raise ValueError("token_mask needs sample_mask and global_valid_toks")
+    gv = None if global_valid_toks is None else global_valid_toks.reshape(-1)[:1].to(torch.float32).contiguous()
+    lib = _lib.load()
+    dev = sl.device
+    with torch.cuda.device(dev):
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        d_s = torch.empty((b, n, k), dtype=torch.float32, device=dev)
+        d_h = torch.empty((b, n) if correct else (0,), dtype=torch.float32, device=dev)
+        ws_bytes = lib.nrl_distill_topk_loss_workspace_bytes(b, n)
+        ws = torch.empty(((ws_bytes + 7) // 8,), dtype=torch.float64, device=dev)
+        code = lib.nrl_distill_topk_loss_fwd_bwd(
+            _ptr(sl), _ptr(tl), _ptr(h_all if correct else None), _ptr(tm), tm_stride, _ptr(sm), _ptr(gv), b, n, k, int(kl_type),
+            float(mixed_kl_weight), int(bool(zero_outside_topk)), float(log_infinitesimal), _ptr(loss), _ptr(d_s),
+            _ptr(d_h if correct else None), _ptr(ws), ws.numel() * 8, _stream(),
+        )
+    _lib.check(code, "nrl_distill_topk_loss_fwd_bwd")
+    return loss, d_s, d_h
+
+
+for _name, _fn in (("topk_logsoftmax_fwd", _topk_logsoftmax_fwd), ("topk_logsoftmax_bwd", _topk_logsoftmax_bwd),
+                   ("distill_topk_loss", _distill_topk_loss)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
 _LIB.define("nonzero_indices(Tensor values) -> Tensor")
 
 

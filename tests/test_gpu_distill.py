@@ -99,3 +99,85 @@ def test_strided_views_and_odd_alignment():
     want = OD.neg_entropy(view.cpu())
     got = MU.ChunkedDistributedEntropy.apply(view, 4, None, True)
     assert (got.cpu() - want).abs().max().item() <= 1e-5
+
+
+# ---- top-k distillation path: prepare_loss_input(DISTILLATION) + DistillationLossFn ----
+def _kd_inputs(b, s, v, k, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    student = (torch.randn(b, s, v, generator=g) * 2).to(dtype)
+    teacher_full = torch.randn(b, s, v, generator=g) * 2
+    t_logits, t_idx = torch.topk(teacher_full, k, dim=-1)
+    tm = (torch.rand(b, s, generator=g) < 0.7).float()
+    tm[:, 0] = 0
+    sm = torch.ones(b)
+    if b > 1:
+        sm[1] = 0.5
+    if b > 2:
+        sm[2] = 0
+    data = {"input_ids": torch.zeros(b, s, dtype=torch.long), "token_mask": tm, "sample_mask": sm,
+            "teacher_topk_logits": t_logits, "teacher_topk_indices": t_idx}
+    gt = (tm[:, 1:] * sm.unsqueeze(-1)).sum()
+    return student, data, gt
+
+
+@pytest.mark.parametrize("kl_type,zero_outside", [("forward", False), ("forward", True), ("reverse", False), ("reverse", True),
+                                                  ("mixed", False), ("mixed", True)])
+@pytest.mark.parametrize("dtype,v,k,tol", [(torch.float32, 500, 16, 1e-5), (torch.bfloat16, 4096, 64, 2e-3)])
+def test_distillation_path_matches_oracle(kl_type, zero_outside, dtype, v, k, tol):
+    from oracle import distill as D
+    from rl_amd.algorithms.loss import DistillationLossConfig, DistillationLossFn, prepare_loss_input
+
+    student, data, gt = _kd_inputs(4, 9, v, k, dtype, seed=v + k)
+    xo = student.to(torch.float32).clone().requires_grad_(True)
+    s_lp, t_lp, h = D.distillation_topk_logprobs(xo, data["teacher_topk_logits"], data["teacher_topk_indices"], zero_outside,
+                                                 zero_outside and kl_type != "forward")
+    want, wm = D.distillation_loss(kl_type, 0.3, zero_outside, s_lp, t_lp, h, data, gt)
+    want.backward()
+
+    fn = DistillationLossFn(DistillationLossConfig(kl_type=kl_type, mixed_kl_weight=0.3, zero_outside_topk=zero_outside))
+    xg = student.to(DEV).requires_grad_(True)
+    ddev = {k_: t.to(DEV) for k_, t in data.items()}
+    loss_input, d2 = prepare_loss_input(xg, ddev, fn)
+    assert (loss_input["student_topk_logprobs"].detach().cpu() - s_lp.detach()).abs().max().item() <= tol
+    assert (loss_input["teacher_topk_logprobs"].cpu() - t_lp).abs().max().item() <= 1e-5
+    assert (loss_input["H_all"] is None) == (h is None)
+    got, gm = fn(data=d2, global_valid_seqs=None, global_valid_toks=gt.to(DEV), **loss_input)
+    got.backward()
+    assert abs(got.item() - want.item()) <= (1e-4 if dtype == torch.float32 else 2e-3) * abs(want.item()) + 1e-6
+    assert gm["num_valid_samples"] == wm["num_valid_samples"] and abs(gm["loss"] - got.item()) < 1e-7
+    scale = xo.grad.abs().max().item() + 1e-30
+    diff = (xg.grad.float().cpu() - xo.grad).abs().max().item()
+    assert diff <= (1e-4 if dtype == torch.float32 else 2.0 ** -7) * scale
+    assert torch.all(xg.grad[:, -1] == 0)  # the last position feeds nothing
+
+
+def test_distillation_loss_without_masks_and_with_duplicate_indices():
+    from oracle import distill as D
+    from rl_amd.algorithms.loss import DistillationLossConfig, DistillationLossFn, prepare_loss_input
+
+    student, data, _gt = _kd_inputs(2, 6, 300, 8, torch.float32, seed=3)
+    data["teacher_topk_indices"][:, :, 3] = data["teacher_topk_indices"][:, :, 1]  # a repeated id: its gradients add up
+    plain = {k: v for k, v in data.items() if k not in ("token_mask", "sample_mask")}
+    xo = student.clone().requires_grad_(True)
+    s_lp, t_lp, h = D.distillation_topk_logprobs(xo, plain["teacher_topk_logits"], plain["teacher_topk_indices"], False, False)
+    want, _ = D.distillation_loss("mixed", 0.5, False, s_lp, t_lp, h, plain, None)
+    want.backward()
+    fn = DistillationLossFn(DistillationLossConfig())
+    xg = student.to(DEV).requires_grad_(True)
+    loss_input, d2 = prepare_loss_input(xg, {k: v.to(DEV) for k, v in plain.items()}, fn)
+    got, _ = fn(data=d2, global_valid_seqs=None, global_valid_toks=None, **loss_input)
+    got.backward()
+    assert abs(got.item() - want.item()) <= 1e-4 * abs(want.item()) + 1e-7
+    assert (xg.grad.cpu() - xo.grad).abs().max().item() <= 1e-4 * xo.grad.abs().max().item()
+
+
+def test_distillation_rejects_an_empty_top_k():
+    from rl_amd.algorithms.loss import DistillationLossConfig, DistillationLossFn, prepare_loss_input
+
+    fn = DistillationLossFn(DistillationLossConfig())
+    data = {"input_ids": torch.zeros(1, 3, dtype=torch.long), "teacher_topk_logits": torch.zeros(1, 3, 0),
+            "teacher_topk_indices": torch.zeros(1, 3, 0, dtype=torch.long)}
+    with pytest.raises(ValueError):
+        prepare_loss_input(torch.zeros(1, 3, 16, device=DEV), data, fn)
+    with pytest.raises(AssertionError):
+        DistillationLossFn(DistillationLossConfig(kl_type="sideways"))
