@@ -14,6 +14,7 @@ from .loss_functions import (
     DistillationLossFn,
     DPOLossConfig,
     DPOLossFn,
+    DraftCrossEntropyLossFn,
     NLLLossFn,
     PreferenceLossFn,
 )
@@ -26,7 +27,7 @@ from .wrapper import (
 
 __all__ = [
     "fused_logits_clipped_pg_loss", "fused_packed_logits_clipped_pg_loss", "why_not_fusable", "why_not_fusable_packed",
-    "ClippedPGLossConfig", "ClippedPGLossFn", "DistillationLossConfig", "DistillationLossFn", "DPOLossConfig", "DPOLossFn", "NLLLossFn", "PreferenceLossFn", "LossFunction", "LossInputType", "LossType",
+    "ClippedPGLossConfig", "ClippedPGLossFn", "DistillationLossConfig", "DistillationLossFn", "DPOLossConfig", "DPOLossFn", "DraftCrossEntropyLossFn", "NLLLossFn", "PreferenceLossFn", "LossFunction", "LossInputType", "LossType",
     "MetricNormalizer", "prepare_loss_input", "prepare_packed_loss_input", "SequencePackingFusionLossWrapper",
     "SequencePackingLossWrapper", "wrap_loss_fn_with_input_preparation",
 ]

@@ -504,3 +504,25 @@ class DistillationLossFn(LossFunction):
         if home != dev:
             loss = loss.to(home)
         return loss, {"loss": float(loss.item()), "num_valid_samples": data["input_ids"].shape[0]}
+
+
+class DraftCrossEntropyLossFn(LossFunction):
+    """Soft-target cross entropy for draft-model training (``loss_functions.py:66-108``): per token
+    ``-sum_v softmax(teacher)_v log_softmax(student)_v`` from one streaming pass over both logit
+    tensors, then the masked mean over the tokens."""
+
+    loss_type = LossType.TOKEN_LEVEL
+    input_type = LossInputType.DRAFT
+
+    def __init__(self, vocab_parallel_group: Optional[Any] = None):
+        self.vocab_parallel_group = vocab_parallel_group
+
+    def __call__(self, teacher_logits, student_logits, token_mask, data, global_valid_seqs, global_valid_toks):
+        from ...distributed.model_utils import DistributedCrossEntropy
+
+        per_token = DistributedCrossEntropy.apply(student_logits, teacher_logits, self.vocab_parallel_group, False)
+        dev = per_token.device
+        # masked_mean(x, mask, Gt) = sum(x * mask) / (Gt + 1e-8): the NLL kernel's reduction with the sign flipped
+        nll, _metrics = _FusedNll.apply(per_token, _f32(token_mask, dev), _f32(data["sample_mask"], dev),
+                                        _global_valid(1.0, global_valid_toks, dev))
+        return -nll

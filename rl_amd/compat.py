@@ -44,7 +44,8 @@ _PATCHED = {
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
     "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],
     "nemo_rl.algorithms.loss.utils": ["prepare_loss_input", "prepare_packed_loss_input"],
-    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn"],
+    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn",
+                                               "DraftCrossEntropyLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
     "nemo_rl.models.megatron.train": ["LogprobsPostProcessor"],

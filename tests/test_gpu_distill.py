@@ -181,3 +181,27 @@ def test_distillation_rejects_an_empty_top_k():
         prepare_loss_input(torch.zeros(1, 3, 16, device=DEV), data, fn)
     with pytest.raises(AssertionError):
         DistillationLossFn(DistillationLossConfig(kl_type="sideways"))
+
+
+def test_draft_cross_entropy_loss():
+    """``DraftCrossEntropyLossFn`` against the reference's own non-parallel formula
+    (``loss_functions.py:96-101``) evaluated on the CPU."""
+    from rl_amd.algorithms.loss import DraftCrossEntropyLossFn
+
+    g = torch.Generator().manual_seed(21)
+    b, s, v = 3, 7, 1000
+    teacher = torch.randn(b, s, v, generator=g) * 2
+    student = torch.randn(b, s, v, generator=g) * 2
+    tm = (torch.rand(b, s, generator=g) < 0.7).float()
+    sm = torch.tensor([1.0, 0.0, 0.5])
+    gt = (tm * sm.unsqueeze(-1)).sum()
+    xo = student.clone().requires_grad_(True)
+    per_token = OD.soft_cross_entropy(xo, teacher)
+    want = (per_token * tm * sm.unsqueeze(-1)).sum() / (gt + 1e-8)
+    want.backward()
+    xg = student.to(DEV).requires_grad_(True)
+    got = DraftCrossEntropyLossFn()(teacher.to(DEV), xg, tm.to(DEV), {"sample_mask": sm.to(DEV)}, None, gt.to(DEV))
+    got.backward()
+    assert abs(got.item() - want.item()) <= 1e-4 * abs(want.item())
+    assert (xg.grad.cpu() - xo.grad).abs().max().item() <= 1e-4 * xo.grad.abs().max().item()
+    assert torch.all(xg.grad[1] == 0)
