@@ -48,7 +48,11 @@ Pinning status (what fixes each function besides its own text):
                            the chosen rows, SFT-only == rescaled NLL) and a
                            loop-per-pair brute force
                            (``tests/test_oracle_preference.py``).
-* ``lmhead.*``             PARITY UNPINNED against the reference (its only test
-                           needs Megatron, two GPUs and a model download);
-                           pinned here to ``logprob(hidden @ W.T)`` in fp32.
+* ``lmhead.*``             pinned: forward == ``log_softmax(hidden @ W.T).gather``,
+                           backward == torch autograd of that unfused form,
+                           chunked == unchunked.  PARITY UNPINNED only for the
+                           rounding of the reference's dW (accumulated per chunk
+                           in the weights' dtype; the reference's one test of
+                           this path needs Megatron, two GPUs and a model
+                           download).
 """

@@ -1,9 +1,13 @@
 """Oracle: fused lm_head -> token log-probabilities (hidden states in, no
 materialised full-sequence logits).
 
-Test infrastructure only (see ``oracle/__init__.py``).  PARITY UNPINNED against
-the reference (no runnable reference test exists for this path); pinned to the
-unfused ``rows_logprob(hidden @ W.T)`` identity by ``tests/test_oracle_logprob.py``.
+Test infrastructure only (see ``oracle/__init__.py``).  Pinned by the identity the
+path reduces to: forward == ``log_softmax(hidden @ W.T).gather(target)`` and
+backward == torch autograd of that unfused form, chunked == unchunked
+(``tests/test_oracle_logprob.py::test_lmhead_equals_unfused_and_autograd``).  The
+reference holds no vectors for this path (its only test needs Megatron, two GPUs
+and a model download); PARITY UNPINNED only for the rounding of the reference's
+dW, which it accumulates per chunk in the weights' dtype.
 
 Restates ``nemo_rl/distributed/model_utils.py:2119-2134`` (roll, drop last
 column) and ``:2152-2215, 2240-2291`` (forward / backward per sequence chunk)
