@@ -27,7 +27,12 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (scaled by the same counters on a 4 GiB copy), valid for one microbatch of the named workload
-MEASURED_TRAFFIC_BYTES = {"c2": 16.90e9 + 19.95e9}  # fused_logits_loss_kernel
+MEASURED_TRAFFIC_BYTES = {
+    "c2": 16.90e9 + 19.95e9,  # fused_logits_loss_kernel
+    "c4": 14.72e9 + 19.92e9,  # topk_topp_stream_kernel (backward): rows of masked tokens are zero-filled unread
+    "c4_fwd": 23.54e9,        # topk_topp_fwd_kernel: the row once plus the re-read of the chunks that reach the bound
+    "c5": 33.41e9 + 34.38e9,  # fused_logits_loss_kernel, packed
+}
 THREE_PASS_BWD_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}  # logprob_bwd_kernel
 
 WORKLOADS = {
@@ -241,10 +246,12 @@ def bench_topk(args, torch, w):
         "algorithmic_bytes_per_token": 3 * row_bytes,
         "hbm_frac_end_to_end": 3 * row_bytes * tokens * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": "topk_topp_stream_kernel (backward)", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": bwd["avg_ms"],
+                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES["c4"] if not args.seqs else None, "avg_launch_ms": bwd["avg_ms"],
                      "algorithmic_bytes_per_launch": 2 * row_bytes * rows},
         "roofline_fwd": {"bound": "hbm", "kernel": "topk_topp_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
+                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"],
+                         "traffic": MEASURED_TRAFFIC_BYTES["c4_fwd"] if not args.seqs else None},
         "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
     }))
 
@@ -384,7 +391,7 @@ def bench_packed(args, torch, w):
                    "api": "SequencePackingFusionLossWrapper(ClippedPGLossFn, prepare_packed_loss_input)(logits, batch, ...) + "
                           "autograd.grad -> nrl_fused_packed_logits_grpo_loss"},
         "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel (packed)", "achieved": gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": fk,
+                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["c5"], "avg_launch_ms": fk,
                      "algorithmic_bytes_per_launch": alg},
         "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in km.items()},
     }
