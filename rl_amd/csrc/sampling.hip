@@ -68,6 +68,7 @@ template <int CAP> struct SelShared {
     int sel_cnt[2][kSelWaves * 3];
     Lse2 lse_w[kSelWaves];
     int count;
+    int n_hit;  // chunks whose maximum reaches the bound (their list lives in expv until the finish phase)
 };
 
 // k-th largest (1-based) of the workgroup's kChunks keys (kSub per thread, in registers); every thread
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         }
         if ((tid & (kWave - 1)) == 0) sh.lse_w[tid / kWave] = acc;
     }
-    if (tid == 0) sh.count = 0;
+    if (tid == 0) { sh.count = 0; sh.n_hit = 0; }
     __syncthreads();
     if (FULL_LSE) {
         Lse2 tot = sh.lse_w[0];
@@ -297,8 +298,8 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     }
 
     // ---- pass 2: collect candidates ----
-    // Only the chunks whose maximum reaches the bound can hold candidates; a thread re-reads just those
-    // of its own chunks (with top-k that is about k of the 2048 chunks, a few percent of the row).
+    // Only the chunks whose maximum reaches the bound can hold candidates (with top-k that is about k of the
+    // 2048 chunks, a few percent of the row).
     auto push = [&](uint32_t key, int64_t index) {
         if (key >= bound_key) {
             const int pos = atomicAdd(&sh.count, 1);
@@ -311,26 +312,43 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
 #pragma unroll
         for (int k = 0; k < EPV; ++k) push(order_key(scale_logit<DT, TEMP>(t[k], a.tparam)), head + vi * EPV + k);
     };
-    constexpr int kBatch = 8;  // loads of one chunk in flight together (a chunk of a 152k row is 9-10 vectors)
+    // The hit chunks go to a list and their vectors are then dealt out evenly, a few per thread with the
+    // loads in flight together: a thread that re-read only its own hit chunks left most lanes of a wave
+    // idle through several thousand instructions, which cost more than the streaming pass.
+    static_assert(kChunks <= 65536 && kChunks * 2 <= CAP * 4, "the hit list is 16-bit chunk ids inside expv");
+    uint16_t* hit = reinterpret_cast<uint16_t*>(sh.expv);
+#pragma unroll
+    for (int u = 0; u < kSub; ++u)
+        if (mx_key[u] >= bound_key) hit[atomicAdd(&sh.n_hit, 1)] = static_cast<uint16_t>(tid * kSub + u);
+    if (mx_key[0] >= bound_key) {  // chunk 0 also took the unaligned head / tail elements
+        if (tid < head) push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam)), tid);
+        if (tail0 + tid < vocab)
+            push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam)), tail0 + tid);
+    }
+    __syncthreads();
     const int64_t n_full = nvec / (kSub * kSelBlock);  // vectors every chunk got in the main loop of pass 1
+    const int per_chunk = static_cast<int>(n_full) + 1;  // ... plus its slot of the ragged end
+    const int n_items = sh.n_hit * per_chunk;
+    // vector index of item number `item`, or -1 (the ragged slot of a chunk that has none)
+    auto item_vec = [&](int item) -> int64_t {
+        if (item >= n_items) return -1;
+        const int h = item / per_chunk, j = item - h * per_chunk;
+        const int cu = hit[h], t = cu / kSub, u = cu - t * kSub;
+        const int64_t vi = j < n_full ? j * static_cast<int64_t>(kSub * kSelBlock) + u * kSelBlock + t : base + u * kSelBlock + t;
+        return vi < nvec ? vi : -1;
+    };
+    constexpr int kBatch = 4;
+    for (int i0 = tid; i0 < n_items; i0 += kBatch * kSelBlock) {
+        int64_t vi[kBatch];
+        u32x4 q[kBatch];
 #pragma unroll
-    for (int u = 0; u < kSub; ++u) {
-        if (mx_key[u] < bound_key) continue;
-        for (int64_t b0 = 0; b0 < n_full; b0 += kBatch) {
-            u32x4 q[kBatch];
-#pragma unroll
-            for (int j = 0; j < kBatch; ++j)
-                if (b0 + j < n_full) q[j] = xv[(b0 + j) * (kSub * kSelBlock) + u * kSelBlock + tid];
-#pragma unroll
-            for (int j = 0; j < kBatch; ++j)
-                if (b0 + j < n_full) push_raw(q[j], (b0 + j) * (kSub * kSelBlock) + u * kSelBlock + tid);
+        for (int j = 0; j < kBatch; ++j) {
+            vi[j] = item_vec(i0 + j * kSelBlock);
+            if (vi[j] >= 0) q[j] = xv[vi[j]];
         }
-        if (base + u * kSelBlock + tid < nvec) push_raw(xv[base + u * kSelBlock + tid], base + u * kSelBlock + tid);  // ragged end
-        if (u == 0) {  // chunk 0 also took the unaligned head / tail elements
-            if (tid < head) push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam)), tid);
-            if (tail0 + tid < vocab)
-                push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam)), tail0 + tid);
-        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (vi[j] >= 0) push_raw(q[j], vi[j]);
     }
     __syncthreads();
     const int n = sh.count;
