@@ -118,13 +118,13 @@ int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t total_toke
  * logprob_out (may be NULL, then rows->targets may be NULL): x_t - lse_kept, or -inf when the target
  * was filtered out.  logprob_unfiltered_out / lse_full_out (may be NULL): the same row's unfiltered
  * logprob (what the KL penalty needs, loss/utils.py:104-118) from the same pass.
- * overflow_flag: device int32 set to 1 if some row's kept set exceeded the on-chip candidate list
- * (4096 entries; such rows come back as NaN).  top_k above 2048 is not supported.
+ * Rows whose kept set exceeds the on-chip candidate list (4096 entries: a flat distribution under
+ * top-p alone, many exact ties, a top_k in the thousands) take a second, slower kernel in the same
+ * call that searches the threshold instead of sorting; there is no limit on top_k or on the kept set.
  * ------------------------------------------------------------------------------------------ */
 int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
                               float* thr_out, int32_t* tie_out, float* lse_kept_out,
-                              float* logprob_unfiltered_out, float* lse_full_out,
-                              int32_t* overflow_flag, void* stream);
+                              float* logprob_unfiltered_out, float* lse_full_out, void* stream);
 
 /* dlogits_v = keep_v * g * (onehot_v - exp(x_v - lse_kept)); layout arguments as nrl_logprob_bwd. */
 int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,

@@ -19,7 +19,8 @@
 // kept.  The backward streams the row once more: d_v = keep_v * g * (onehot_v - exp(x_v - lse_kept)).
 //
 // Rows whose candidate list would exceed the LDS capacity (very flat distributions under top-p
-// alone, or thousands of exact ties) raise the overflow flag instead of producing a wrong result.
+// alone, thousands of exact ties, or a top_k in the thousands) are marked and finished by
+// topk_topp_wide_kernel, which finds the same predicate by bitwise threshold search over the row.
 
 #include <float.h>
 #include <math.h>
@@ -30,6 +31,9 @@ namespace nrl {
 
 constexpr int kSelBlock = 256;
 constexpr int kSelWaves = kSelBlock / kWave;
+constexpr int kMassBins = 64;
+constexpr int kWideGrid = 2048;
+constexpr int32_t kTieUnresolved = -1;  // tie[] marker: the row's kept set did not fit the candidate list
 constexpr int kSub = 8;                      // chunk maxima per thread
 constexpr int kChunks = kSelBlock * kSub;    // 2048
 constexpr int kCap = 4096;                   // candidate capacity (LDS); rows under a small top-k use kCapSmall
@@ -68,6 +72,7 @@ template <int CAP> struct SelShared {
     int sel_cnt[2][kSelWaves * 3];
     Lse2 lse_w[kSelWaves];
     int count;
+    float mass_bin[kMassBins];  // top-p alone: probability mass per log-probability bin
     int n_hit;  // chunks whose maximum reaches the bound (their list lives in expv until the finish phase)
 };
 
@@ -173,7 +178,6 @@ struct SelArgs {
     float* lse_kept;     // [rows]
     float* logprob_full; // [rows] or NULL: unfiltered logprob of the target
     float* lse_full;     // [rows] or NULL
-    int32_t* overflow;   // device flag
 };
 
 template <int DT, int TEMP, bool FULL_LSE, int CAP>
@@ -292,9 +296,46 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     if (use_k) {
         if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, mx_key, a.top_k);
     } else {
-        // top-p alone: elements with probability <= (1-p)/V sum to at most 1-p and are the smallest
-        const float b = lse_full + logf((1.0f - a.top_p) / static_cast<float>(vocab));
-        bound_key = order_key(b) + 1u;  // strictly above the bound
+        // top-p alone: elements with probability <= (1-p)/V sum to at most 1-p and are the smallest ...
+        const float cut = 1.0f - a.top_p;
+        const float span = logf(static_cast<float>(vocab) / cut);  // from that probability up to 1, in nats
+        const float b0 = lse_full - span;
+        // ... but a long tail leaves thousands of elements above that.  One more pass over the row (it was
+        // just read) sorts the probability of everything above b0 into kMassBins equal log-probability bins;
+        // the bins below the edge where the mass from the bottom first exceeds 1-p cannot be kept either.
+        const float to_bin = static_cast<float>(kMassBins) / span;
+        for (int i = tid; i < kMassBins; i += kSelBlock) sh.mass_bin[i] = 0.f;
+        __syncthreads();
+        auto bin = [&](float x) {
+            if (x > b0) {
+                const int j = static_cast<int>((x - b0) * to_bin);
+                atomicAdd(&sh.mass_bin[j < kMassBins - 1 ? j : kMassBins - 1], expf(x - lse_full));
+            }
+        };
+        for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
+            float t[EPV];
+            Row<DT>::decode(xv[vi], t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) bin(scale_logit<DT, TEMP>(t[k], a.tparam));
+        }
+        if (tid < head) bin(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam));
+        if (tail0 + tid < vocab) bin(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam));
+        __syncthreads();
+        // every wave: lane j takes bin j and the mass of the bins from j upwards; the row's mass below the
+        // lower edge of bin j is 1 minus that.  The highest edge whose mass below stays under 1-p (less a
+        // margin for the rounding of the sums: the list may hold more than the kept set, never less) bounds
+        // the candidates; with none the bound stays at b0.
+        static_assert(kMassBins == kWave, "one bin per lane");
+        float above = sh.mass_bin[tid & (kWave - 1)];
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const float up = __shfl_down(above, off, kWave);
+            if ((tid & (kWave - 1)) + off < kWave) above += up;
+        }
+        const unsigned long long ok = __ballot(1.0f - above <= cut * 0.999f - 1e-5f);
+        const int edge = ok ? 63 - __builtin_clzll(ok) : 0;
+        // just under the edge, so that an element the rounding of its bin number put into bin `edge` counts
+        bound_key = edge > 0 ? order_key(b0 + (static_cast<float>(edge) - 0.01f) / to_bin) : order_key(b0) + 1u;
     }
 
     // ---- pass 2: collect candidates ----
@@ -355,9 +396,8 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     if (n > CAP || n == 0) {
         // the kept set does not fit the candidate list (or the row holds no finite value)
         if (tid == 0) {
-            if (n > CAP) atomicExch(a.overflow, 1);
             a.thr[r] = __builtin_nanf("");
-            a.tie[r] = 0;
+            a.tie[r] = n > CAP ? kTieUnresolved : 0;  // unresolved rows are finished by topk_topp_wide_kernel
             a.lse_kept[r] = __builtin_nanf("");
             if (a.logprob) a.logprob[r] = __builtin_nanf("");
             if (a.lse_full) a.lse_full[r] = lse_full;
@@ -435,6 +475,206 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                 if (a.logprob_full) a.logprob_full[r] = lpf;
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// rows whose kept set does not fit the on-chip candidate list (top-p alone over a flat distribution, or a
+// very large top_k): the same keep predicate found without a sort, by searching the threshold key bit by
+// bit with one streaming pass over the row per two bits.  The row (at most a few hundred KB) stays in L2
+// between passes.  Sums are carried in double, so the cumulative mass at the boundary differs from the
+// sorted fp32 running sum of the fast path only in which of two nearly equal neighbours falls first.
+// ---------------------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ void block_sum3(T (&v)[3], T* shm) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) v[c] += __shfl_down(v[c], off, kWave);
+    __syncthreads();  // the previous round's readers are done with shm
+    if (lane == 0)
+#pragma unroll
+        for (int c = 0; c < 3; ++c) shm[wave * 3 + c] = v[c];
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+        T t = shm[c];
+#pragma unroll
+        for (int w = 1; w < kSelWaves; ++w) t += shm[w * 3 + c];
+        v[c] = t;
+    }
+}
+
+template <int DT, int TEMP> struct WideRow {
+    const char* row;
+    const u32x4* xv;
+    int64_t vocab, head, nvec, tail0;
+    float tparam;
+    // f(scaled logit, vocabulary index) for every element of the row, each exactly once
+    template <typename F> __device__ __forceinline__ void for_each(F f) const {
+        constexpr int EPV = Row<DT>::EPV;
+        const int tid = threadIdx.x;
+        for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
+            float t[EPV];
+            Row<DT>::decode(xv[vi], t);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) f(scale_logit<DT, TEMP>(t[k], tparam), head + vi * EPV + k);
+        }
+        if (tid < head) f(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), tparam), static_cast<int64_t>(tid));
+        if (tail0 + tid < vocab) f(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), tparam), tail0 + tid);
+    }
+};
+
+template <int DT, int TEMP>
+__global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, int64_t n_rows) {
+    __shared__ double shm_d[kSelWaves * 3];
+    __shared__ long long shm_i[kSelWaves * 3];
+    __shared__ float shm_m[kSelWaves];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const bool use_k = a.top_k > 0, use_p = a.top_p < 1.0f;
+    for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
+        if (a.tie[r] != kTieUnresolved) continue;  // the same word for every thread of the workgroup
+        const int64_t o = r / a.n_inner, i_in = r - o * a.n_inner;
+        WideRow<DT, TEMP> w;
+        w.row = static_cast<const char*>(a.logits) + (o * a.stride_outer + i_in * a.stride_inner) * Row<DT>::BYTES;
+        w.vocab = a.vocab;
+        w.head = sel_row_head<DT>(w.row, w.vocab);
+        w.nvec = (w.vocab - w.head) / Row<DT>::EPV;
+        w.tail0 = w.head + w.nvec * Row<DT>::EPV;
+        w.xv = reinterpret_cast<const u32x4*>(w.row + w.head * Row<DT>::BYTES);
+        w.tparam = a.tparam;
+
+        // row maximum
+        float m = -FLT_MAX;
+        w.for_each([&](float x, int64_t) { m = fmaxf(m, x); });
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) m = fmaxf(m, __shfl_down(m, off, kWave));
+        __syncthreads();
+        if (lane == 0) shm_m[wave] = m;
+        __syncthreads();
+        m = shm_m[0];
+#pragma unroll
+        for (int q = 1; q < kSelWaves; ++q) m = fmaxf(m, shm_m[q]);
+        const uint32_t max_key = order_key(m);
+
+        // top-k: the largest key with at least top_k keys at or above it (ties at that key are all kept)
+        uint32_t k_key = 0u;
+        if (use_k && a.top_k < w.vocab) {
+            for (int bit = 30; bit >= 0; bit -= 2) {
+                long long cnt[3] = {0, 0, 0};
+                const uint32_t c1 = k_key | (1u << bit), c2 = k_key | (2u << bit), c3 = k_key | (3u << bit);
+                w.for_each([&](float x, int64_t) {
+                    const uint32_t key = order_key(x);
+                    cnt[0] += key >= c1;
+                    cnt[1] += key >= c2;
+                    cnt[2] += key >= c3;
+                });
+                block_sum3(cnt, shm_i);
+                const uint32_t step = cnt[2] >= a.top_k ? 3u : cnt[1] >= a.top_k ? 2u : cnt[0] >= a.top_k ? 1u : 0u;
+                k_key |= step << bit;
+            }
+        }
+
+        // mass of the top-k survivors (Z) and of the whole row
+        double mass[3] = {0.0, 0.0, 0.0};
+        w.for_each([&](float x, int64_t) {
+            const double e = static_cast<double>(expf(x - m));
+            mass[0] += order_key(x) >= k_key ? e : 0.0;
+            mass[1] += e;
+        });
+        block_sum3(mass, shm_d);
+        const double z = mass[0];
+        const float lse_full = m + logf(static_cast<float>(mass[1]));
+
+        uint32_t thr_key = k_key;
+        int32_t tie = 0;
+        double kept_mass = z;
+        if (use_p) {
+            // ascending cumulative probability; elements fall while it stays <= 1 - p.  The threshold is
+            // the largest key c whose strictly-lower survivors together weigh <= (1 - p) Z.
+            const double target = static_cast<double>(1.0f - a.top_p) * z;
+            uint32_t c = 0u;
+            for (int bit = 30; bit >= 0; bit -= 2) {
+                double lt[3] = {0.0, 0.0, 0.0};
+                const uint32_t c1 = c | (1u << bit), c2 = c | (2u << bit), c3 = c | (3u << bit);
+                w.for_each([&](float x, int64_t) {
+                    const uint32_t key = order_key(x);
+                    const double e = key >= k_key ? static_cast<double>(expf(x - m)) : 0.0;
+                    lt[0] += key < c1 ? e : 0.0;
+                    lt[1] += key < c2 ? e : 0.0;
+                    lt[2] += key < c3 ? e : 0.0;
+                });
+                block_sum3(lt, shm_d);
+                const uint32_t step = lt[2] <= target ? 3u : lt[1] <= target ? 2u : lt[0] <= target ? 1u : 0u;
+                c |= step << bit;
+            }
+            if (c > max_key) c = max_key;  // the largest element always survives
+            if (c < k_key) c = k_key;
+            thr_key = c;
+            // how many of the elements equal to the threshold fall too (the ones with the smallest indices)
+            double below[3] = {0.0, 0.0, 0.0};
+            long long n_eq[3] = {0, 0, 0};
+            w.for_each([&](float x, int64_t) {
+                const uint32_t key = order_key(x);
+                below[0] += (key >= k_key && key < c) ? static_cast<double>(expf(x - m)) : 0.0;
+                n_eq[0] += key == c;
+            });
+            block_sum3(below, shm_d);
+            block_sum3(n_eq, shm_i);
+            const double e_thr = static_cast<double>(expf(key_value(c) - m));
+            long long drop = 0;
+            if (e_thr > 0.0 && n_eq[0] > 1) {
+                const double room = (target - below[0]) / e_thr;
+                drop = room <= 0.0 ? 0 : room >= static_cast<double>(n_eq[0] - 1) ? n_eq[0] - 1 : static_cast<long long>(room);
+                while (drop + 1 <= n_eq[0] - 1 && below[0] + static_cast<double>(drop + 1) * e_thr <= target) ++drop;
+                while (drop > 0 && below[0] + static_cast<double>(drop) * e_thr > target) --drop;
+            }
+            if (drop > 0) {
+                // index of the first survivor among the equal elements: the largest index with at most
+                // `drop` equal elements before it
+                int64_t idx = 0;
+                int top_bit = 0;
+                while ((int64_t{1} << (top_bit + 1)) < w.vocab) ++top_bit;
+                top_bit |= 1;  // pairs of bits, so start from an odd position
+                for (int bit = top_bit - 1; bit >= 0; bit -= 2) {
+                    long long before[3] = {0, 0, 0};
+                    const int64_t i1 = idx | (int64_t{1} << bit), i2 = idx | (int64_t{2} << bit), i3 = idx | (int64_t{3} << bit);
+                    w.for_each([&](float x, int64_t j) {
+                        const bool eq = order_key(x) == c;
+                        before[0] += eq && j < i1;
+                        before[1] += eq && j < i2;
+                        before[2] += eq && j < i3;
+                    });
+                    block_sum3(before, shm_i);
+                    const int64_t step = before[2] <= drop ? 3 : before[1] <= drop ? 2 : before[0] <= drop ? 1 : 0;
+                    idx |= step << bit;
+                }
+                tie = static_cast<int32_t>(idx);
+            }
+            kept_mass = z - below[0] - static_cast<double>(drop) * e_thr;
+            if (!(kept_mass > 0.0)) kept_mass = e_thr;
+        }
+        const float thr = key_value(thr_key);
+        const float lse_kept = m + logf(static_cast<float>(kept_mass));
+        if (tid == 0) {
+            a.thr[r] = thr;
+            a.lse_kept[r] = lse_kept;
+            if (a.lse_full) a.lse_full[r] = lse_full;
+            if (a.targets && a.logprob) {
+                const int64_t tg = a.targets[o * a.ts_outer + i_in * a.ts_inner];
+                float lp = -INFINITY, lpf = 0.f;
+                if (tg >= 0 && tg < w.vocab) {
+                    const float xt = scale_logit<DT, TEMP>(Row<DT>::load1(w.row, tg), a.tparam);
+                    const bool kept = xt > thr || (xt == thr && tg >= tie);
+                    if (kept) lp = xt - lse_kept;
+                    lpf = xt - lse_full;
+                }
+                a.logprob[r] = lp;
+                if (a.logprob_full) a.logprob_full[r] = lpf;
+            }
+        }
+        __syncthreads();      // every thread has read tie[r] == unresolved before it is replaced
+        if (tid == 0) a.tie[r] = tie;
     }
 }
 
@@ -563,15 +803,14 @@ using namespace nrl;
 
 extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
                                          float* thr_out, int32_t* tie_out, float* lse_kept_out,
-                                         float* logprob_unfiltered_out, float* lse_full_out, int32_t* overflow_flag,
-                                         void* stream) {
+                                         float* logprob_unfiltered_out, float* lse_full_out, void* stream) {
     if (int e = check_sel_rows(rows, logprob_out != nullptr)) return e;
     const bool use_k = top_k > 0, use_p = top_p < 1.0f;
     if (!use_k && !use_p) return fail(NRL_E_INVALID, "neither top-k nor top-p is active");
     if (use_p && !(top_p > 0.f)) return fail(NRL_E_INVALID, "top_p must be in (0, 1]");
     const int64_t n = rows->n_outer * rows->n_inner;
     if (n == 0) return NRL_OK;
-    if (!thr_out || !tie_out || !lse_kept_out || !overflow_flag) return fail(NRL_E_INVALID, "null state output");
+    if (!thr_out || !tie_out || !lse_kept_out) return fail(NRL_E_INVALID, "null state output");
     SelArgs a;
     a.logits = rows->logits; a.n_inner = rows->n_inner; a.vocab = rows->vocab;
     a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
@@ -579,7 +818,7 @@ extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, fl
     a.top_k = use_k ? static_cast<int>(top_k > (1ll << 30) ? (1ll << 30) : top_k) : 0;
     a.top_p = use_p ? top_p : 1.0f;
     a.logprob = logprob_out; a.thr = thr_out; a.tie = tie_out; a.lse_kept = lse_kept_out;
-    a.logprob_full = logprob_unfiltered_out; a.lse_full = lse_full_out; a.overflow = overflow_flag;
+    a.logprob_full = logprob_unfiltered_out; a.lse_full = lse_full_out;
     const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
     const bool full = !use_k || logprob_unfiltered_out != nullptr || lse_full_out != nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -593,7 +832,12 @@ extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, fl
     } else {
         NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, false, kCap><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
     }
-    return check_launch("topk_topp_logprob_fwd");
+    if (int e = check_launch("topk_topp_logprob_fwd")) return e;
+    // rows the candidate list could not hold are finished here; with none, every workgroup leaves after
+    // reading its rows' markers
+    const unsigned grid = static_cast<unsigned>(n < kWideGrid ? n : kWideGrid);
+    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_wide_kernel<DT, TEMP><<<dim3(grid), dim3(kSelBlock), 0, s>>>(a, n));
+    return check_launch("topk_topp_logprob_fwd (wide rows)");
 }
 
 extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,

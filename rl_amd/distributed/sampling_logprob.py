@@ -12,17 +12,6 @@ from .._lib import NRL_TEMP_RCP
 
 _OPS = torch.ops.rl_amd
 
-_OVERFLOW = (
-    "top-k/top-p: a row's kept set exceeds the 4096-entry on-chip candidate list (a very flat distribution under "
-    "top-p alone, thousands of exact ties, or top_k > 2048); combine top_p with a top_k <= 2048"
-)
-
-
-def _check_overflow(flag: torch.Tensor) -> None:
-    if int(flag.item()) != 0:
-        raise RuntimeError(_OVERFLOW)
-
-
 def _norm_k(top_k) -> int:
     return int(top_k) if top_k is not None and top_k > 0 else 0
 
@@ -42,10 +31,9 @@ def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, wa
     targets = targets.to(logits.device)
     if targets.dtype != torch.int64:
         targets = targets.long()
-    lp, thr, tie, lse, lpu, flag = _OPS.topk_topp_logprob_fwd(
+    lp, thr, tie, lse, lpu = _OPS.topk_topp_logprob_fwd(
         logits, targets, n_inner, _norm_k(top_k), _norm_p(top_p), 1.0, NRL_TEMP_RCP, want_unfiltered
     )
-    _check_overflow(flag)
     ctx.saved = (not inference_only) and ctx.needs_input_grad[0]
     if ctx.saved:
         ctx.save_for_backward(logits, targets, thr, tie, lse)
@@ -111,8 +99,7 @@ class _FilterLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits3d, top_k, top_p):
         x = logits3d.detach()
-        _, thr, tie, _, _, flag = _OPS.topk_topp_logprob_fwd(x, None, x.shape[1], top_k, top_p, 1.0, NRL_TEMP_RCP, False)
-        _check_overflow(flag)
+        _, thr, tie, _, _ = _OPS.topk_topp_logprob_fwd(x, None, x.shape[1], top_k, top_p, 1.0, NRL_TEMP_RCP, False)
         filtered, keep = _OPS.topk_topp_filter(x, thr, tie, 1.0, NRL_TEMP_RCP)
         keep = keep.bool()
         ctx.save_for_backward(keep)

@@ -243,7 +243,7 @@ for _name, _fn in (("logprob_packed_fwd", _logprob_packed_fwd), ("logprob_packed
 # ------------------------------------------------------------------------------------------------
 _LIB.define(
     "topk_topp_logprob_fwd(Tensor logits, Tensor? targets, int n_inner, int top_k, float top_p, float temperature, "
-    "int temp_mode, bool want_unfiltered) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)"
+    "int temp_mode, bool want_unfiltered) -> (Tensor, Tensor, Tensor, Tensor, Tensor)"
 )
 _LIB.define(
     "topk_topp_logprob_bwd(Tensor logits, Tensor targets, Tensor thr, Tensor tie, Tensor lse_kept, Tensor grad, "
@@ -255,7 +255,7 @@ _LIB.define(
 
 
 def _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, temp_mode, want_unfiltered):
-    """-> (logprob [B,n] (empty without targets), thr, tie, lse_kept, unfiltered logprob (or empty), overflow flag)."""
+    """-> (logprob [B,n] (empty without targets), thr, tie, lse_kept, unfiltered logprob (or empty))."""
     _need_gpu(logits, targets)
     b, s, v = logits.shape
     dummy = targets if targets is not None else torch.zeros((b, max(n_inner, 1)), dtype=torch.int64, device=logits.device)
@@ -270,14 +270,13 @@ def _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, 
         tie = torch.empty((b, n_inner), dtype=torch.int32, device=dev)
         lse = torch.empty((b, n_inner), **f32)
         lpu = torch.empty((b, n_inner) if want_unfiltered else (0,), **f32)
-        flag = torch.zeros((1,), dtype=torch.int32, device=dev)
         with _timed("topk_topp_fwd"):
             code = _lib.load().nrl_topk_topp_logprob_fwd(
                 C.byref(rows), int(top_k), float(top_p), _ptr(lp if targets is not None else None), _ptr(thr), _ptr(tie),
-                _ptr(lse), _ptr(lpu if want_unfiltered else None), None, _ptr(flag), _stream(),
+                _ptr(lse), _ptr(lpu if want_unfiltered else None), None, _stream(),
             )
     _lib.check(code, "nrl_topk_topp_logprob_fwd")
-    return lp, thr, tie, lse, lpu, flag
+    return lp, thr, tie, lse, lpu
 
 
 def _topk_topp_logprob_bwd(logits, targets, thr, tie, lse_kept, grad, n_inner, temperature, temp_mode):

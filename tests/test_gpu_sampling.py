@@ -120,11 +120,89 @@ def test_c4_slice_bf16_temperature_topk_topp():
     assert torch.equal(lp.cpu(), got)
 
 
-def test_flat_distribution_under_top_p_alone_fails_loudly():
-    x = torch.zeros(1, 2, 151936, device=DEV)   # every token tied: the nucleus is ~144k tokens wide
-    ids = torch.zeros(1, 2, dtype=torch.long, device=DEV)
-    with pytest.raises(RuntimeError, match="candidate list"):
-        MU.from_parallel_logits_to_logprobs(x, ids, 0, 151936, None, sampling_params=TrainingSamplingParams(top_p=0.95))
+def _boundary_only(got_keep, want_keep, x, slack):
+    """The two masks may differ only in a handful of elements whose values sit at the threshold: the
+    oracle's running sum is sequential fp32 over tens of thousands of terms, the kernel's is double."""
+    diff = got_keep ^ want_keep
+    per_row = diff.reshape(-1, x.shape[-1]).sum(-1)
+    assert int(per_row.max()) <= slack, per_row.tolist()
+    for r in torch.nonzero(per_row).flatten().tolist():
+        xr, dr, wr = x.reshape(-1, x.shape[-1])[r], diff.reshape(-1, x.shape[-1])[r], want_keep.reshape(-1, x.shape[-1])[r]
+        thr = xr[wr].min()
+        below = xr[~wr].max() if bool((~wr).any()) else thr
+        # every disputed element is one of the smallest kept or largest dropped values
+        assert float(xr[dr].max()) <= float(thr) + 1e-6 + abs(float(thr)) * 1e-2 and float(xr[dr].min()) >= float(below) - 1e-6 - abs(float(below)) * 1e-2
+
+
+WIDE = [
+    (None, 0.9, 50257, 2.5, torch.float32),      # nucleus of tens of thousands of tokens
+    (None, 0.5, 65544, 2.5, torch.bfloat16),     # a small nucleus, but more candidates above the chunk bound than fit
+    (None, 0.97, 151936, 1.0, torch.bfloat16),
+    (3000, 1.0, 20000, 2.5, torch.float32),      # top_k beyond the candidate list's reach
+    (3000, 0.8, 20000, 1.0, torch.float32),
+    (5000, 0.9, 8199, 1.0, torch.bfloat16),      # bf16: many exact ties at both boundaries
+]
+
+
+@pytest.mark.parametrize("k,p,vocab,sigma,dtype", WIDE)
+def test_kept_sets_beyond_the_candidate_list(k, p, vocab, sigma, dtype):
+    """Rows whose kept set exceeds the 4096-entry on-chip list take the threshold-search kernel.  Same
+    oracle; the top-p boundary may move by a few near-equal elements (see _boundary_only), which moves
+    the kept mass by parts in 1e5, hence the 1e-4 bound on the logprobs."""
+    g = torch.Generator().manual_seed(vocab + (k or 7))
+    b, s = 2, 4
+    logits = (torch.randn(b, s, vocab, generator=g) * sigma).to(dtype)
+    ids = torch.randint(0, vocab, (b, s), generator=g)
+    top = logits.float().argmax(-1)
+    ids[:, 1:] = torch.where(torch.rand(b, s - 1, generator=g) < 0.5, top[:, :-1], ids[:, 1:])
+    x32 = logits.float()
+    want_keep = OS.keep_mask_rows(x32.reshape(-1, vocab), k, p).reshape(b, s, vocab)
+    _, got_keep = apply_top_k_top_p(logits.to(DEV), k, p)
+    got_keep = got_keep.cpu()
+    if p >= 1.0:
+        assert torch.equal(got_keep, want_keep)                  # top-k alone: no running sum, exact
+    else:
+        _boundary_only(got_keep, want_keep, x32, slack=8)
+    # logprobs and gradient, judged on the targets both sides keep
+    xo = x32.clone().requires_grad_(True)
+    want = OL.from_logits_to_logprobs(xo, ids, top_k=k, top_p=p)
+    xg = logits.to(DEV).requires_grad_(True)
+    got = MU.from_parallel_logits_to_logprobs(xg, ids.to(DEV), 0, vocab, None,
+                                              sampling_params=TrainingSamplingParams(top_k=k, top_p=p))
+    gc = got.detach().cpu()
+    tgt_keep_w = torch.isfinite(want.detach())
+    tgt_keep_g = torch.isfinite(gc)
+    both = tgt_keep_w & tgt_keep_g
+    assert both.any() and int((tgt_keep_w ^ tgt_keep_g).sum()) <= 1
+    assert (gc[both] - want.detach()[both]).abs().max().item() <= (1e-4 if dtype == torch.float32 else 2e-3)
+    up = torch.randn(b, s - 1, generator=g)
+    (torch.where(both, want, torch.zeros_like(want)) * up).sum().backward()
+    (torch.where(both.to(DEV), got, torch.zeros_like(got)) * up.to(DEV)).sum().backward()
+    gg, wg = xg.grad.float().cpu()[:, :-1], xo.grad[:, :-1]
+    agree = ~(got_keep ^ want_keep)[:, :-1]
+    scale = wg.abs().max().item() + 1e-30
+    tol = 1e-4 if dtype == torch.float32 else 2.0 ** -7
+    assert bool((((gg - wg).abs() <= wg.abs() * tol + 1e-4 * scale) | ~agree).all())
+    assert torch.all(gg[~got_keep[:, :-1]] == 0)
+
+
+def test_every_token_tied_under_top_p_alone():
+    """151936 equal logits: the nucleus is ~144k tokens wide and the cut runs through one giant tie, where
+    the smallest indices fall.  The oracle's sequential fp32 sum of 151936 equal terms drifts, so the
+    count is compared with the exact one (drop floor((1 - p) V) tokens) and with the oracle loosely."""
+    vocab, p = 151936, 0.95
+    x = torch.zeros(1, 2, vocab, device=DEV)
+    _, keep = apply_top_k_top_p(x, None, p)
+    keep = keep[0, 0].cpu()
+    n_drop = int((~keep).sum())
+    cut = float(torch.tensor(1.0) - torch.tensor(p))           # 1 - p in fp32, as the kernel forms it
+    assert abs(n_drop - math.floor(cut * vocab)) <= 1
+    assert not keep[:n_drop].any() and keep[n_drop:].all()      # the dropped ones are the smallest indices
+    want_keep = OS.keep_mask_rows(torch.zeros(1, vocab), None, p)[0]
+    assert int((want_keep ^ keep).sum()) <= 64
+    ids = torch.tensor([[5, vocab - 1]], device=DEV)
+    lp = MU.from_parallel_logits_to_logprobs(x, ids, 0, vocab, None, sampling_params=TrainingSamplingParams(top_p=p)).cpu()
+    assert abs(lp[0, 0].item() + math.log(vocab - n_drop)) <= 1e-5
 
 
 def test_prepare_loss_input_with_sampling_and_kl():
