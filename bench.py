@@ -32,6 +32,9 @@ MEASURED_TRAFFIC_BYTES = {
     "c4": 14.72e9 + 19.92e9,  # topk_topp_stream_kernel (backward): rows of masked tokens are zero-filled unread
     "c4_fwd": 23.54e9,        # topk_topp_fwd_kernel: the row once plus the re-read of the chunks that reach the bound
     "c5": 33.41e9 + 34.38e9,  # fused_logits_loss_kernel, packed
+    # lmhead_fwd_kernel: L2 fills (W and hidden-state tiles re-fetched by every 4 x 8 patch of tiles that uses
+    # them; 114 GB if the workgroups of a patch stayed in step) + the partial log-sum-exp records written
+    "c3_fwd": 207.8e9 + 1.28e9,
 }
 THREE_PASS_BWD_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}  # logprob_bwd_kernel
 
@@ -460,7 +463,8 @@ def bench_lmhead(args, torch, w):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "tokens": n, "hidden": h, "vocab": v},
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tf, "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "avg_launch_ms": fwd_ms},
+                     "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["c3_fwd"] if not args.seqs else None,
+                     "avg_launch_ms": fwd_ms},
         "roofline_bwd": {"bound": "mfma", "kernel": "lmhead backward (grad + dH + dW GEMMs)", "achieved": bwd_alg_tf,
                          "achieved_incl_recompute": bwd_exec_tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": bwd_alg_tf / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": bwd_ms},
