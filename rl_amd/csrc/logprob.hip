@@ -14,6 +14,11 @@
 #include <float.h>
 
 #include "common.hpp"
+#ifdef NRL_NT_ZERO
+#define NRL_ZERO_STORE(v, p) __builtin_nontemporal_store(v, p)
+#else
+#define NRL_ZERO_STORE(v, p) (*(p) = (v))
+#endif
 
 namespace nrl {
 
@@ -105,7 +110,7 @@ template <int DT> __device__ __forceinline__ void row_zero(void* row, int64_t vo
     const int64_t nvec = (vocab - head) / EPV;
     u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(row) + head * Row<DT>::BYTES);
     const u32x4 z = {0u, 0u, 0u, 0u};
-    for (int64_t i = tid; i < nvec; i += kBlock) __builtin_nontemporal_store(z, ov + i);
+    for (int64_t i = tid; i < nvec; i += kBlock) NRL_ZERO_STORE(z, ov + i);
     if (tid < head) Row<DT>::store1(row, tid, 0.f);
     const int64_t tail0 = head + nvec * EPV;
     if (tail0 + tid < vocab) Row<DT>::store1(row, tail0 + tid, 0.f);

@@ -708,8 +708,14 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_stream_kernel(SelBwdArgs 
     const int64_t vocab = a.vocab;
     float g = 0.f;
     if (MODE == 0 && i_in < a.n_inner) g = a.grad[o * a.gs_outer + i_in * a.gs_inner];
-    if (MODE == 0 && g == 0.f) {
-        for (int64_t e = tid; e < vocab; e += kSelBlock) Row<DT>::store1(out, e, 0.f);
+    if (MODE == 0 && g == 0.f) {  // dropped position or masked token: the gradient row is exactly zero
+        const int64_t zh = sel_row_head<DT>(out, vocab);
+        const int64_t zn = (vocab - zh) / EPV;
+        u32x4* zv = reinterpret_cast<u32x4*>(out + zh * Row<DT>::BYTES);
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int64_t v = tid; v < zn; v += kSelBlock) zv[v] = z;
+        if (tid < zh) Row<DT>::store1(out, tid, 0.f);
+        if (zh + zn * EPV + tid < vocab) Row<DT>::store1(out, zh + zn * EPV + tid, 0.f);
         return;
     }
     const int64_t rr = o * a.n_inner + i_in;
