@@ -532,6 +532,13 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
     __shared__ float shm_m[kSelWaves];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const bool use_k = a.top_k > 0, use_p = a.top_p < 1.0f;
+    {
+        // the usual case is that no row of this workgroup is marked: look at all of them at once and leave
+        bool mine = false;
+        for (int64_t r = blockIdx.x + static_cast<int64_t>(tid) * gridDim.x; r < n_rows; r += static_cast<int64_t>(kSelBlock) * gridDim.x)
+            mine |= a.tie[r] == kTieUnresolved;
+        if (!__syncthreads_or(mine)) return;
+    }
     for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
         if (a.tie[r] != kTieUnresolved) continue;  // the same word for every thread of the workgroup
         const int64_t o = r / a.n_inner, i_in = r - o * a.n_inner;
