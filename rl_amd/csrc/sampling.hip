@@ -32,6 +32,11 @@ namespace nrl {
 constexpr int kSelBlock = 256;
 constexpr int kSelWaves = kSelBlock / kWave;
 constexpr int kMassBins = 64;
+#ifndef NRL_LOOSE_HITS
+#define NRL_LOOSE_HITS 768
+#endif
+constexpr int kLooseHits = NRL_LOOSE_HITS;  // top-p alone: more hit chunks than this under the chunk maxima's bound -> bound from the row
+constexpr int kMassCopies = 8;  // copies of the histogram, by lane: most elements fall into the few lowest bins
 constexpr int kWideGrid = 2048;
 constexpr int32_t kTieUnresolved = -1;  // tie[] marker: the row's kept set did not fit the candidate list
 constexpr int kSub = 8;                      // chunk maxima per thread
@@ -72,7 +77,7 @@ template <int CAP> struct SelShared {
     int sel_cnt[2][kSelWaves * 3];
     Lse2 lse_w[kSelWaves];
     int count;
-    float mass_bin[kMassBins];  // top-p alone: probability mass per log-probability bin
+    float mass_bin[kMassCopies * kMassBins];  // top-p alone: probability mass per log-probability bin
     int n_hit;  // chunks whose maximum reaches the bound (their list lives in expv until the finish phase)
 };
 
@@ -180,8 +185,11 @@ struct SelArgs {
     float* lse_full;     // [rows] or NULL
 };
 
-template <int DT, int TEMP, bool FULL_LSE, int CAP>
+// PONLY: top-p without top-k (its own instantiation, so that the mass histogram costs the top-k variants
+// neither registers nor LDS); otherwise top-k is on, with or without top-p.
+template <int DT, int TEMP, bool FULL_LSE, int CAP, bool PONLY = false>
 __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
+    static_assert(!PONLY || FULL_LSE, "top-p alone normalises over the whole row");
     __shared__ SelShared<CAP> sh;
     constexpr int EPV = Row<DT>::EPV;
     const int tid = threadIdx.x;
@@ -290,28 +298,51 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     }
 
     // ---- lower bound of everything that can be kept ----
-    const bool use_k = a.top_k > 0;
+    constexpr bool use_k = !PONLY;
     const bool use_p = a.top_p < 1.0f;
     uint32_t bound_key = 0u;
-    if (use_k) {
-        if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, mx_key, a.top_k);
-    } else {
-        // top-p alone: elements with probability <= (1-p)/V sum to at most 1-p and are the smallest ...
-        const float cut = 1.0f - a.top_p;
-        const float span = logf(static_cast<float>(vocab) / cut);  // from that probability up to 1, in nats
-        const float b0 = lse_full - span;
-        // ... but a long tail leaves thousands of elements above that.  One more pass over the row (it was
-        // just read) sorts the probability of everything above b0 into kMassBins equal log-probability bins;
-        // the bins below the edge where the mass from the bottom first exceeds 1-p cannot be kept either.
-        const float to_bin = static_cast<float>(kMassBins) / span;
-        for (int i = tid; i < kMassBins; i += kSelBlock) sh.mass_bin[i] = 0.f;
+    // top-p alone: elements with probability <= (1-p)/V sum to at most 1-p and are the smallest, which puts
+    // a first bound b0 under the kept set; but a long tail leaves thousands of elements above b0.  The
+    // probability of a set of elements above b0, sorted into kMassBins equal log-probability bins, gives a
+    // better one: if the bins from j upwards already hold more than p of the row's mass, everything below
+    // bin j weighs less than 1-p and cannot be kept.  First the set is the 2048 chunk maxima (already in
+    // registers; enough whenever the kept set is a few hundred tokens), and only if that proves nothing or
+    // leaves too many candidates the whole row, read once more.
+    const float cut = 1.0f - a.top_p;
+    const float span = logf(static_cast<float>(vocab) / cut);  // from probability (1-p)/V up to 1, in nats
+    const float b0 = lse_full - span;
+    const float to_bin = static_cast<float>(kMassBins) / span;
+    auto bin = [&](float x) {
+        if (x > b0) {
+            const int j = static_cast<int>((x - b0) * to_bin);
+            atomicAdd(&sh.mass_bin[(tid & (kMassCopies - 1)) * kMassBins + (j < kMassBins - 1 ? j : kMassBins - 1)], expf(x - lse_full));
+        }
+    };
+    // called by every thread between two barriers around the binning; returns the bound (the same in all)
+    auto bound_from_bins = [&]() -> uint32_t {
+        // every wave: lane j takes bin j and the mass of the bins from j upwards.  The highest edge whose
+        // mass below stays under 1-p (less a margin for the rounding of the sums: the list may hold more
+        // than the kept set, never less) bounds the candidates; with none the bound stays at b0.
+        static_assert(kMassBins == kWave, "one bin per lane");
+        float above = 0.f;
+#pragma unroll
+        for (int q = 0; q < kMassCopies; ++q) above += sh.mass_bin[q * kMassBins + (tid & (kWave - 1))];
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const float up = __shfl_down(above, off, kWave);
+            if ((tid & (kWave - 1)) + off < kWave) above += up;
+        }
+        const unsigned long long ok = __ballot(1.0f - above <= cut * 0.999f - 1e-5f);
+        const int edge = ok ? 63 - __builtin_clzll(ok) : 0;
+        // just under the edge, so that an element the rounding of its bin number put into bin `edge` counts
+        return edge > 0 ? order_key(b0 + (static_cast<float>(edge) - 0.01f) / to_bin) : order_key(b0) + 1u;
+    };
+    auto clear_bins = [&]() {
+        for (int i = tid; i < kMassCopies * kMassBins; i += kSelBlock) sh.mass_bin[i] = 0.f;
+    };
+    auto bound_from_row = [&]() -> uint32_t {
+        clear_bins();
         __syncthreads();
-        auto bin = [&](float x) {
-            if (x > b0) {
-                const int j = static_cast<int>((x - b0) * to_bin);
-                atomicAdd(&sh.mass_bin[j < kMassBins - 1 ? j : kMassBins - 1], expf(x - lse_full));
-            }
-        };
         for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
             float t[EPV];
             Row<DT>::decode(xv[vi], t);
@@ -321,24 +352,29 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         if (tid < head) bin(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam));
         if (tail0 + tid < vocab) bin(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam));
         __syncthreads();
-        // every wave: lane j takes bin j and the mass of the bins from j upwards; the row's mass below the
-        // lower edge of bin j is 1 minus that.  The highest edge whose mass below stays under 1-p (less a
-        // margin for the rounding of the sums: the list may hold more than the kept set, never less) bounds
-        // the candidates; with none the bound stays at b0.
-        static_assert(kMassBins == kWave, "one bin per lane");
-        float above = sh.mass_bin[tid & (kWave - 1)];
+        return bound_from_bins();
+    };
+    bool whole_row = true;  // top-p alone: the bound already rests on the whole row
+    if (use_k) {
+        if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, mx_key, a.top_k);
+    } else {
+        clear_bins();
+        __syncthreads();
 #pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            const float up = __shfl_down(above, off, kWave);
-            if ((tid & (kWave - 1)) + off < kWave) above += up;
+        for (int u = 0; u < kSub; ++u) bin(mx[u]);
+        __syncthreads();
+        bound_key = bound_from_bins();
+        whole_row = bound_key == order_key(b0) + 1u;  // the maxima alone prove nothing: go to the row at once
+        if (whole_row) {
+            __syncthreads();  // every wave is done with the bins
+            bound_key = bound_from_row();
         }
-        const unsigned long long ok = __ballot(1.0f - above <= cut * 0.999f - 1e-5f);
-        const int edge = ok ? 63 - __builtin_clzll(ok) : 0;
-        // just under the edge, so that an element the rounding of its bin number put into bin `edge` counts
-        bound_key = edge > 0 ? order_key(b0 + (static_cast<float>(edge) - 0.01f) / to_bin) : order_key(b0) + 1u;
     }
 
-    // ---- pass 2: collect candidates ----
+    // ---- pass 2: collect candidates (top-p alone: once more with the bound from the whole row if the list
+    // did not hold what the chunk maxima's bound lets through) ----
+    int n = 0;
+    for (;;) {
     // Only the chunks whose maximum reaches the bound can hold candidates (with top-k that is about k of the
     // 2048 chunks, a few percent of the row).
     auto push = [&](uint32_t key, int64_t index) {
@@ -367,6 +403,14 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             push(order_key(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam)), tail0 + tid);
     }
     __syncthreads();
+    if (!use_k && !whole_row && sh.n_hit > kLooseHits) {
+        // the bound from the chunk maxima lets too many chunks through: the row's own is worth its pass
+        __syncthreads();  // every thread has read the hit count
+        if (tid == 0) { sh.count = 0; sh.n_hit = 0; }
+        whole_row = true;
+        bound_key = bound_from_row();
+        continue;
+    }
     const int64_t n_full = nvec / (kSub * kSelBlock);  // vectors every chunk got in the main loop of pass 1
     const int per_chunk = static_cast<int>(n_full) + 1;  // ... plus its slot of the ragged end
     const int n_items = sh.n_hit * per_chunk;
@@ -392,7 +436,13 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             if (vi[j] >= 0) push_raw(q[j], vi[j]);
     }
     __syncthreads();
-    const int n = sh.count;
+    n = sh.count;
+    if (use_k || whole_row || n <= CAP) break;
+    __syncthreads();  // every thread has read the count
+    if (tid == 0) { sh.count = 0; sh.n_hit = 0; }
+    whole_row = true;
+    bound_key = bound_from_row();
+    }
     if (n > CAP || n == 0) {
         // the kept set does not fit the candidate list (or the row holds no finite value)
         if (tid == 0) {
@@ -836,7 +886,9 @@ extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, fl
     const bool full = !use_k || logprob_unfiltered_out != nullptr || lse_full_out != nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool small = use_k && a.top_k <= kSmallTopK;
-    if (full && small) {
+    if (!use_k) {
+        NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true, kCap, true><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    } else if (full && small) {
         NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true, kCapSmall><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
     } else if (full) {
         NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_fwd_kernel<DT, TEMP, true, kCap><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
