@@ -6,8 +6,10 @@
 //                  wants the unfiltered logprob too, the online log-sum-exp of the full row);
 //   select         the k-th largest chunk maximum is a lower bound of the k-th largest element
 //                  (found two bits per round with wave ballots, the maxima staying in registers);
-//                  for top-p alone the bound is lse + log((1-p)/V): everything below it is dropped
-//                  whatever the order;
+//                  for top-p alone the bound starts at lse + log((1-p)/V) (everything below it is
+//                  dropped whatever the order) and is raised with a 64-bin histogram of probability
+//                  over log-probability, filled from the chunk maxima and, only if that is not
+//                  enough, from the row read once more;
 //   pass 2         re-reads only the chunks whose maximum reaches the bound (about k of 2048) and
 //                  appends the elements above the bound to an LDS list;
 //   finish         bitonic sort of the list by (value, index), top-k threshold with ties kept,
