@@ -39,7 +39,10 @@ constexpr int kMassBins = 64;
 #endif
 constexpr int kLooseHits = NRL_LOOSE_HITS;  // top-p alone: more hit chunks than this under the chunk maxima's bound -> bound from the row
 constexpr int kMassCopies = 8;  // copies of the histogram, by lane: most elements fall into the few lowest bins
-constexpr int kWideGrid = 2048;
+#ifndef NRL_WIDE_GRID
+#define NRL_WIDE_GRID 2048
+#endif
+constexpr int kWideGrid = NRL_WIDE_GRID;
 constexpr int32_t kTieUnresolved = -1;  // tie[] marker: the row's kept set did not fit the candidate list
 constexpr int kSub = 8;                      // chunk maxima per thread
 constexpr int kChunks = kSelBlock * kSub;    // 2048
@@ -635,9 +638,10 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
         }
 
         // mass of the top-k survivors (Z) and of the whole row
+        auto wexp = [&](float x) { return static_cast<double>(fast_exp2((x - m) * kLog2e)); };
         double mass[3] = {0.0, 0.0, 0.0};
         w.for_each([&](float x, int64_t) {
-            const double e = static_cast<double>(expf(x - m));
+            const double e = wexp(x);
             mass[0] += order_key(x) >= k_key ? e : 0.0;
             mass[1] += e;
         });
@@ -650,37 +654,51 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
         double kept_mass = z;
         if (use_p) {
             // ascending cumulative probability; elements fall while it stays <= 1 - p.  The threshold is
-            // the largest key c whose strictly-lower survivors together weigh <= (1 - p) Z.
+            // the largest key c whose strictly-lower survivors together weigh <= (1 - p) Z.  `base` carries
+            // the mass of the survivors below c from round to round, so a round only looks at the keys in
+            // the still undecided range [c, c + 3 * 2^bit): after the first few rounds nearly every element
+            // is skipped before its exponential.
             const double target = static_cast<double>(1.0f - a.top_p) * z;
             uint32_t c = 0u;
+            double base = 0.0;
             for (int bit = 30; bit >= 0; bit -= 2) {
-                double lt[3] = {0.0, 0.0, 0.0};
                 const uint32_t c1 = c | (1u << bit), c2 = c | (2u << bit), c3 = c | (3u << bit);
+                const uint32_t lo = c > k_key ? c : k_key;
+                double seg[3] = {0.0, 0.0, 0.0};  // survivors in [c, c1), [c1, c2), [c2, c3)
                 w.for_each([&](float x, int64_t) {
                     const uint32_t key = order_key(x);
-                    const double e = key >= k_key ? static_cast<double>(expf(x - m)) : 0.0;
-                    lt[0] += key < c1 ? e : 0.0;
-                    lt[1] += key < c2 ? e : 0.0;
-                    lt[2] += key < c3 ? e : 0.0;
+                    if (key >= lo && key < c3) {
+                        const double e = wexp(x);
+                        seg[0] += key < c1 ? e : 0.0;
+                        seg[1] += (key >= c1 && key < c2) ? e : 0.0;
+                        seg[2] += key >= c2 ? e : 0.0;
+                    }
                 });
-                block_sum3(lt, shm_d);
-                const uint32_t step = lt[2] <= target ? 3u : lt[1] <= target ? 2u : lt[0] <= target ? 1u : 0u;
-                c |= step << bit;
+                block_sum3(seg, shm_d);
+                const double l1 = base + seg[0], l2 = l1 + seg[1], l3 = l2 + seg[2];
+                if (l3 <= target) { c = c3; base = l3; }
+                else if (l2 <= target) { c = c2; base = l2; }
+                else if (l1 <= target) { c = c1; base = l1; }
             }
-            if (c > max_key) c = max_key;  // the largest element always survives
-            if (c < k_key) c = k_key;
+            bool clamped = false;
+            if (c > max_key) { c = max_key; clamped = true; }  // the largest element always survives
+            if (c < k_key) { c = k_key; clamped = true; }
             thr_key = c;
             // how many of the elements equal to the threshold fall too (the ones with the smallest indices)
-            double below[3] = {0.0, 0.0, 0.0};
+            double below[3] = {clamped ? 0.0 : base, 0.0, 0.0};
             long long n_eq[3] = {0, 0, 0};
-            w.for_each([&](float x, int64_t) {
-                const uint32_t key = order_key(x);
-                below[0] += (key >= k_key && key < c) ? static_cast<double>(expf(x - m)) : 0.0;
-                n_eq[0] += key == c;
-            });
-            block_sum3(below, shm_d);
+            if (clamped) {
+                w.for_each([&](float x, int64_t) {
+                    const uint32_t key = order_key(x);
+                    below[0] += (key >= k_key && key < c) ? wexp(x) : 0.0;
+                    n_eq[0] += key == c;
+                });
+                block_sum3(below, shm_d);
+            } else {
+                w.for_each([&](float x, int64_t) { n_eq[0] += order_key(x) == c; });
+            }
             block_sum3(n_eq, shm_i);
-            const double e_thr = static_cast<double>(expf(key_value(c) - m));
+            const double e_thr = wexp(key_value(c));
             long long drop = 0;
             if (e_thr > 0.0 && n_eq[0] > 1) {
                 const double room = (target - below[0]) / e_thr;
