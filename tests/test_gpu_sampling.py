@@ -138,6 +138,9 @@ WIDE = [
     (None, 0.9, 50257, 2.5, torch.float32),      # nucleus of tens of thousands of tokens
     (None, 0.5, 65544, 2.5, torch.bfloat16),     # a small nucleus, but more candidates above the chunk bound than fit
     (None, 0.97, 151936, 1.0, torch.bfloat16),
+    (None, 0.9, 151936, 4.0, torch.bfloat16),    # ~700 tokens: too many chunks pass the chunk maxima's bound, the row's own is used
+    (None, 0.9, 151936, 5.0, torch.float32),     # ~100 tokens: the bound from the chunk maxima suffices
+    (None, 0.9, 151936, 8.0, torch.bfloat16),    # a handful of tokens
     (3000, 1.0, 20000, 2.5, torch.float32),      # top_k beyond the candidate list's reach
     (3000, 0.8, 20000, 1.0, torch.float32),
     (5000, 0.9, 8199, 1.0, torch.bfloat16),      # bf16: many exact ties at both boundaries
