@@ -214,3 +214,47 @@ def test_config5_packed_row_full_shape():
     want_lp = OL.rows_logprob(rows, tgt)
     got_lp = torch.stack([lp[si, p - int(cu[si])] for p, si in zip(picks, seq_of)]).detach().cpu()
     assert (got_lp - want_lp).abs().max().item() <= 2e-3
+
+
+def test_config3_fused_lm_head_full_width_three_chunks():
+    """Benchmark config 3 at its full width (H = 4096, V = 151936) over 33068 tokens: the backward runs in
+    three token chunks, the last one ragged, so dW is accumulated across launches.  Sixteen sampled tokens
+    (some in every chunk) are checked against the oracle: their logprobs, their rows of dH, and -- with the
+    upstream gradient zero everywhere else -- the whole of dW, which then is exactly what those sixteen
+    contribute.  Every other row of dH must be exactly zero."""
+    from oracle import lmhead as OH
+
+    n, h, v = 2 * 16384 + 300, 4096, V_QWEN
+    g = torch.Generator(device=DEV).manual_seed(3003)
+    hid = torch.randn((n, 1, h), generator=g, device=DEV).to(torch.bfloat16)
+    w = torch.empty((v, h), dtype=torch.bfloat16, device=DEV)
+    for lo in range(0, v, 16384):  # in slices: the fp32 temporary of the whole matrix is 2.5 GB
+        w[lo:lo + 16384] = (torch.randn((min(16384, v - lo), h), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    ids = torch.randint(0, v, (1, n), generator=g, device=DEV)
+    cg = torch.Generator().manual_seed(33)
+    pick = torch.cat([torch.randint(0, 16384, (5,), generator=cg), torch.randint(16384, 32768, (5,), generator=cg),
+                      torch.randint(32768, n - 1, (6,), generator=cg)]).unique()
+    up = torch.zeros((1, n - 1), device=DEV)
+    up[0, pick.to(DEV)] = (torch.randn(pick.numel(), generator=cg) * 1e-2 + 0.05).to(DEV)
+
+    hg, wg = hid.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    lp = MU.from_parallel_hidden_states_to_logprobs(hg, wg, False, ids, 0, v, None)
+    assert lp.shape == (1, n - 1) and bool(torch.isfinite(lp).all()) and bool((lp <= 0).all())
+    (lp * up).sum().backward()
+
+    # oracle on the sampled tokens only (position t predicts ids[t + 1])
+    hs, ws = hid[pick.to(DEV)].cpu(), w.cpu()
+    tgt = ids[0, (pick + 1).to(DEV)].cpu().unsqueeze(0)                  # [1, n_pick]
+    want_lp = OH.hidden_to_logprobs_rows(hs, ws, tgt)[0]
+    got_lp = lp[0, pick.to(DEV)].detach().cpu()
+    logit_scale = 8.0   # |logit| stays under 8 for hidden ~ N(0,1), W ~ N(0,0.02), H = 4096 (std 1.28)
+    assert (got_lp - want_lp).abs().max().item() <= 2.0 ** -7 * logit_scale + 2e-3
+    want_dh, want_dw = OH.hidden_to_logprobs_backward(hs, ws, tgt, up[0, pick.to(DEV)].cpu().unsqueeze(0))
+    got_dh = hg.grad[:, 0].float().cpu()
+    rest = torch.ones(n, dtype=torch.bool)
+    rest[pick] = False
+    assert bool((got_dh[rest] == 0).all())
+    for got, want in ((got_dh[pick], want_dh[:, 0].float()), (wg.grad.float().cpu(), want_dw.float())):
+        scale = want.abs().max().item()
+        assert (got - want).abs().max().item() <= 1e-2 * scale
+        assert ((got - want).norm() / want.norm()).item() <= 4e-3
