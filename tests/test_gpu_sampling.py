@@ -189,6 +189,32 @@ def test_kept_sets_beyond_the_candidate_list(k, p, vocab, sigma, dtype):
     assert torch.all(gg[~got_keep[:, :-1]] == 0)
 
 
+def test_wide_rows_with_masked_vocabulary_entries():
+    """-inf logits (a masked part of the vocabulary) carry no mass and are never kept, also on the
+    threshold-search path; a top_k that reaches into them keeps only finite entries plus nothing else."""
+    g = torch.Generator().manual_seed(77)
+    vocab = 30011
+    x = torch.randn(1, 3, vocab, generator=g) * 0.5
+    x[..., torch.randperm(vocab, generator=g)[: vocab // 10]] = -math.inf
+    ids = torch.randint(0, vocab, (1, 3), generator=g)
+    for k, p in ((None, 0.9), (6000, 0.95), (6000, 1.0)):
+        want_keep = OS.keep_mask_rows(x.reshape(-1, vocab), k, p).reshape(x.shape)
+        _, keep = apply_top_k_top_p(x.to(DEV), k, p)
+        keep = keep.cpu()
+        assert not bool(keep[torch.isinf(x)].any())
+        if p >= 1.0:
+            assert torch.equal(keep, want_keep)
+        else:
+            _boundary_only(keep, want_keep, x, slack=8)
+        want = OL.from_logits_to_logprobs(x, ids, top_k=k, top_p=p)
+        got = MU.from_parallel_logits_to_logprobs(x.to(DEV), ids.to(DEV), 0, vocab, None,
+                                                  sampling_params=TrainingSamplingParams(top_k=k, top_p=p)).cpu()
+        both = torch.isfinite(want) & torch.isfinite(got)
+        assert int((torch.isfinite(want) ^ torch.isfinite(got)).sum()) <= 1
+        if both.any():
+            assert (got[both] - want[both]).abs().max().item() <= 1e-4
+
+
 def test_every_token_tied_under_top_p_alone():
     """151936 equal logits: the nucleus is ~144k tokens wide and the cut runs through one giant tie, where
     the smallest indices fall.  The oracle's sequential fp32 sum of 151936 equal terms drifts, so the
