@@ -72,6 +72,19 @@ int nrl_logprob_fwd(const nrl_rows* rows, float* logprob_out, float* lse_out, vo
  * lengths: int64 [n_outer] device; out: fp32 [n_outer, n_inner + 1].  Padding rows are never read. */
 int nrl_logprob_post_fwd(const nrl_rows* rows, const int64_t* lengths, float* out, void* stream);
 
+/* The stable log-softmax itself, materialised: y_v = (x_v - max) - log(sum_u exp(x_u - max)), fp32
+ * arithmetic, written in the logits' dtype.  Replaces _compute_distributed_log_softmax[_with_grad]
+ * (nemo_rl/distributed/model_utils.py:33-79) at TP = 1; the logprob entry points above never
+ * materialise it.  Row r at logits + r*row_stride / out + r*out_row_stride (elements, unit column stride). */
+int nrl_log_softmax_fwd(const void* logits, int32_t dtype, int64_t n_rows, int64_t vocab,
+                        int64_t row_stride, void* out, int64_t out_row_stride, void* stream);
+
+/* Its backward (what autograd derives from :49-67): dx_v = g_v - exp(y_v) * sum_u g_u, from the saved
+ * forward output; logprobs, grad and dx share the dtype. */
+int nrl_log_softmax_bwd(const void* logprobs, int32_t dtype, int64_t n_rows, int64_t vocab,
+                        int64_t lp_row_stride, const void* grad, int64_t grad_row_stride, void* dx,
+                        int64_t dx_row_stride, void* stream);
+
 /* K2  dlogits = g * (onehot(target) - exp(x - lse)), written once in the logits' dtype.
  * Replaces DistributedLogprob.backward / ChunkedDistributedLogprob.backward (:167-207, 333-380).
  * grad: fp32 upstream gradient of the logprobs, element (o, i) at

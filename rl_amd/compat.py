@@ -40,6 +40,7 @@ _PATCHED = {
         "dtensor_from_parallel_logits_to_logprobs", "get_logprobs_from_vocab_parallel_logits",
         "get_distillation_topk_logprobs_from_logits",
         "ChunkedDistributedEntropy", "ChunkedDistributedGatherLogprob", "DistributedCrossEntropy",
+        "_compute_distributed_log_softmax", "_compute_distributed_log_softmax_with_grad",
     ],
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
     "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],

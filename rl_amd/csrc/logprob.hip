@@ -373,6 +373,66 @@ static RowArgs make_row_args(const nrl_rows* r, float tparam) {
     return a;
 }
 
+// ---------------------------------------------------------------------------------------------
+// log-softmax of whole rows, materialised (the stand-alone form of the stable log-softmax every logprob
+// path starts from) and its backward dx_v = g_v - exp(y_v) * sum_u g_u
+// ---------------------------------------------------------------------------------------------
+// out_v = f(in_v [, in2_v]) over one row, by 16-byte vectors when the rows are congruent modulo 16 bytes
+template <int DT, bool TWO, typename F>
+__device__ __forceinline__ void row_apply(const void* in, const void* in2, void* out, int64_t vocab, F f) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const int64_t head = row_head<DT>(in, vocab);
+    if (row_head<DT>(out, vocab) != head || (TWO && row_head<DT>(in2, vocab) != head)) {
+        for (int64_t i = tid; i < vocab; i += kBlock)
+            Row<DT>::store1(out, i, f(Row<DT>::load1(in, i), TWO ? Row<DT>::load1(in2, i) : 0.f));
+        return;
+    }
+    const int64_t nvec = (vocab - head) / EPV;
+    const u32x4* av = reinterpret_cast<const u32x4*>(static_cast<const char*>(in) + head * Row<DT>::BYTES);
+    const u32x4* bv = TWO ? reinterpret_cast<const u32x4*>(static_cast<const char*>(in2) + head * Row<DT>::BYTES) : nullptr;
+    u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(out) + head * Row<DT>::BYTES);
+    for (int64_t i = tid; i < nvec; i += kBlock) {
+        float x[EPV], y[EPV], o[EPV];
+        Row<DT>::decode(av[i], x);
+        if (TWO) Row<DT>::decode(bv[i], y);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) o[k] = f(x[k], TWO ? y[k] : 0.f);
+        ov[i] = Row<DT>::encode(o);
+    }
+    if (tid < head) Row<DT>::store1(out, tid, f(Row<DT>::load1(in, tid), TWO ? Row<DT>::load1(in2, tid) : 0.f));
+    const int64_t tail0 = head + nvec * EPV;
+    if (tail0 + tid < vocab)
+        Row<DT>::store1(out, tail0 + tid, f(Row<DT>::load1(in, tail0 + tid), TWO ? Row<DT>::load1(in2, tail0 + tid) : 0.f));
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void log_softmax_fwd_kernel(const void* __restrict__ logits, int64_t vocab, int64_t row_stride,
+                                                                 void* __restrict__ out, int64_t out_stride) {
+    __shared__ Lse smem[kWaves];
+    const int64_t r = blockIdx.x;
+    const char* row = static_cast<const char*>(logits) + r * row_stride * Row<DT>::BYTES;
+    char* o = static_cast<char*>(out) + r * out_stride * Row<DT>::BYTES;
+    const Lse t = row_online_lse<DT, 0>(row, vocab, 1.0f, smem);
+    const float m = t.m, log_s = logf(t.s);
+    row_apply<DT, false>(row, nullptr, o, vocab, [&](float x, float) { return (x - m) - log_s; });
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void log_softmax_bwd_kernel(const void* __restrict__ logprobs, int64_t vocab, int64_t lp_stride,
+                                                                 const void* __restrict__ grad, int64_t g_stride,
+                                                                 void* __restrict__ dx, int64_t dx_stride) {
+    __shared__ float smem[kWaves];
+    const int64_t r = blockIdx.x;
+    const char* y = static_cast<const char*>(logprobs) + r * lp_stride * Row<DT>::BYTES;
+    const char* g = static_cast<const char*>(grad) + r * g_stride * Row<DT>::BYTES;
+    char* d = static_cast<char*>(dx) + r * dx_stride * Row<DT>::BYTES;
+    float part = 0.f;
+    for (int64_t i = threadIdx.x; i < vocab; i += kBlock) part += Row<DT>::load1(g, i);
+    const float sum_g = block_sum<float, kWaves>(part, smem);
+    row_apply<DT, true>(g, y, d, vocab, [&](float gv, float yv) { return gv - fast_exp2(yv * kLog2e) * sum_g; });
+}
+
 #define NRL_DISPATCH(DT_, TC_, ...)                                                         \
     switch ((DT_) * 3 + (TC_)) {                                                            \
         case NRL_F32 * 3 + 0: { constexpr int DT = NRL_F32, TEMP = 0; __VA_ARGS__; break; }        \
@@ -504,4 +564,30 @@ extern "C" int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t
                  logprob_packed_bwd_kernel<DT, TEMP><<<dim3((unsigned)total_tokens), dim3(kBlock), 0, s>>>(
                      a, lse, grad, dlogits, d_row_stride));
     return check_launch("logprob_packed_bwd");
+}
+
+extern "C" int nrl_log_softmax_fwd(const void* logits, int32_t dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                   void* out, int64_t out_row_stride, void* stream) {
+    if (dtype != NRL_F32 && dtype != NRL_BF16 && dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown logits dtype %d", dtype);
+    if (n_rows < 0 || vocab <= 0 || row_stride < vocab || out_row_stride < vocab) return fail(NRL_E_INVALID, "bad shape or stride");
+    if (n_rows == 0) return NRL_OK;
+    if (!logits || !out) return fail(NRL_E_INVALID, "null logits or out");
+    if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(dtype, 0, log_softmax_fwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logits, vocab, row_stride, out, out_row_stride));
+    return check_launch("log_softmax_fwd");
+}
+
+extern "C" int nrl_log_softmax_bwd(const void* logprobs, int32_t dtype, int64_t n_rows, int64_t vocab, int64_t lp_row_stride,
+                                   const void* grad, int64_t grad_row_stride, void* dx, int64_t dx_row_stride, void* stream) {
+    if (dtype != NRL_F32 && dtype != NRL_BF16 && dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown dtype %d", dtype);
+    if (n_rows < 0 || vocab <= 0 || lp_row_stride < vocab || grad_row_stride < vocab || dx_row_stride < vocab)
+        return fail(NRL_E_INVALID, "bad shape or stride");
+    if (n_rows == 0) return NRL_OK;
+    if (!logprobs || !grad || !dx) return fail(NRL_E_INVALID, "null logprobs, grad or dx");
+    if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(dtype, 0, log_softmax_bwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logprobs, vocab, lp_row_stride, grad,
+                                                                                                   grad_row_stride, dx, dx_row_stride));
+    return check_launch("log_softmax_bwd");
 }

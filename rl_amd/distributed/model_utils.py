@@ -93,6 +93,40 @@ def _rows_logprob(logits, targets, n_inner, vocab_start, vocab_end, inference_on
     return _RowsLogprob.apply(logits, targets, n_inner, vocab_start, vocab_end, inference_only, float(temperature))
 
 
+class _LogSoftmaxRows(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits):
+        x = logits.detach()
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+        out = _OPS.log_softmax_fwd(x2)
+        ctx.save_for_backward(out)
+        return out.view(logits.shape)
+
+    @staticmethod
+    def backward(ctx, grad):
+        (out,) = ctx.saved_tensors
+        g2 = grad.reshape(out.shape)
+        if g2.stride(-1) != 1:
+            g2 = g2.contiguous()
+        return _OPS.log_softmax_bwd(out, g2.to(out.dtype)).view(grad.shape)
+
+
+def _compute_distributed_log_softmax_with_grad(vocab_parallel_logits: torch.Tensor, group: Any) -> torch.Tensor:
+    """``model_utils.py:33-67`` on one rank: the stable log-softmax of every row, same shape and dtype as the
+    input, differentiable.  The arithmetic is fp32 whatever the input dtype (the reference subtracts the
+    maximum and exponentiates in the input dtype; its callers on this path cast to fp32 first)."""
+    _require_single_rank(group, "_compute_distributed_log_softmax_with_grad")
+    return _LogSoftmaxRows.apply(vocab_parallel_logits)
+
+
+@torch.no_grad()
+def _compute_distributed_log_softmax(vocab_parallel_logits: torch.Tensor, group: Any) -> torch.Tensor:
+    """``model_utils.py:70-79``: the same without a graph."""
+    return _compute_distributed_log_softmax_with_grad(vocab_parallel_logits, group)
+
+
 class DistributedLogprob(torch.autograd.Function):
     """``model_utils.py:120-207``.  ``apply(logits, target, vocab_start_index, vocab_end_index, group,
     inference_only=False)`` with ``target`` already shifted; every position is computed."""

@@ -241,6 +241,50 @@ for _name, _fn in (("logprob_packed_fwd", _logprob_packed_fwd), ("logprob_packed
 # ------------------------------------------------------------------------------------------------
 # K3: top-k / top-p
 # ------------------------------------------------------------------------------------------------
+_LIB.define("log_softmax_fwd(Tensor logits) -> Tensor")
+_LIB.define("log_softmax_bwd(Tensor logprobs, Tensor grad) -> Tensor")
+
+
+def _rows2d(t, name):
+    if t.dim() != 2 or (t.stride(1) != 1 and t.shape[1] > 1):
+        raise ValueError(f"{name} must be [rows, V] with a contiguous vocabulary axis")
+    return t
+
+
+def _log_softmax_fwd(logits):
+    """[rows, V] -> log-softmax in the same dtype (fp32 arithmetic)."""
+    _need_gpu(logits)
+    _rows2d(logits, "logits")
+    n, v = logits.shape
+    with torch.cuda.device(logits.device):
+        out = torch.empty((n, v), dtype=logits.dtype, device=logits.device)
+        with _timed("log_softmax_fwd"):
+            code = _lib.load().nrl_log_softmax_fwd(_ptr(logits), _dtype_code(logits), n, v, logits.stride(0) if n > 1 else v,
+                                                   _ptr(out), v, _stream())
+    _lib.check(code, "nrl_log_softmax_fwd")
+    return out
+
+
+def _log_softmax_bwd(logprobs, grad):
+    _need_gpu(logprobs, grad)
+    _rows2d(logprobs, "logprobs")
+    _rows2d(grad, "grad")
+    if grad.shape != logprobs.shape or grad.dtype != logprobs.dtype:
+        raise ValueError("grad must have the shape and dtype of the log-probabilities")
+    n, v = logprobs.shape
+    with torch.cuda.device(logprobs.device):
+        dx = torch.empty((n, v), dtype=logprobs.dtype, device=logprobs.device)
+        with _timed("log_softmax_bwd"):
+            code = _lib.load().nrl_log_softmax_bwd(_ptr(logprobs), _dtype_code(logprobs), n, v, logprobs.stride(0) if n > 1 else v,
+                                                   _ptr(grad), grad.stride(0) if n > 1 else v, _ptr(dx), v, _stream())
+    _lib.check(code, "nrl_log_softmax_bwd")
+    return dx
+
+
+for _name, _fn in (("log_softmax_fwd", _log_softmax_fwd), ("log_softmax_bwd", _log_softmax_bwd)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
 _LIB.define(
     "topk_topp_logprob_fwd(Tensor logits, Tensor? targets, int n_inner, int top_k, float top_p, float temperature, "
     "int temp_mode, bool want_unfiltered) -> (Tensor, Tensor, Tensor, Tensor, Tensor)"

@@ -223,3 +223,39 @@ def test_fused_temperature_matches_in_place_divide(dtype):
         want = OL.rows_logprob(scaled, ids)
         got, lse = torch.ops.rl_amd.logprob_fwd(xg, idg, 5, 0, vocab, t, mode, True)
         assert (got.cpu() - want).abs().max().item() <= 1e-5  # same rounded inputs -> fp32-level agreement
+
+
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 2003), (torch.float32, 4096), (torch.bfloat16, 4099), (torch.float16, 777)])
+def test_materialised_log_softmax_and_its_gradient(dtype, vocab):
+    """``_compute_distributed_log_softmax[_with_grad]`` (``model_utils.py:33-79``) at TP = 1 against the
+    oracle's restatement: values within 1e-5 (fp32) or one unit in the last place of the narrow dtype,
+    gradient ``g - softmax * sum(g)`` against torch autograd of the oracle."""
+    g = torch.Generator().manual_seed(vocab)
+    x = (torch.randn(3, 5, vocab, generator=g) * 2.5).to(dtype)
+    up = torch.randn(3, 5, vocab, generator=g).to(dtype)
+    xo = x.float().clone().requires_grad_(True)
+    want = OL.stable_log_softmax(xo)
+    (want * up.float()).sum().backward()
+    xg = x.to(DEV).requires_grad_(True)
+    got = MU._compute_distributed_log_softmax_with_grad(xg, None)
+    assert got.dtype == dtype and got.shape == x.shape
+    (got.float() * up.to(DEV).float()).sum().backward()
+    gv, wv = got.detach().float().cpu(), want.detach()
+    if dtype == torch.float32:
+        assert (gv - wv).abs().max().item() <= 1e-5
+        scale = xo.grad.abs().max().item()
+        assert (xg.grad.cpu() - xo.grad).abs().max().item() <= 1e-4 * scale
+    else:
+        ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        assert bool(((gv - wv).abs() <= wv.abs() * ulp + 1e-6).all())
+        # the saved output is in the narrow dtype, so softmax = exp(y) carries its rounding (|y| * ulp relative)
+        scale = xo.grad.abs().max().item()
+        assert (xg.grad.float().cpu() - xo.grad).abs().max().item() <= 20 * ulp * scale
+    with torch.no_grad():
+        same = MU._compute_distributed_log_softmax(x.to(DEV), None)
+    assert torch.equal(same, got.detach()) and not same.requires_grad
+    # a view with a padded row stride goes through without a copy of the values changing
+    wide = torch.zeros(4, vocab + 8, dtype=dtype)
+    wide[:, :vocab] = x[0, :4]
+    sl = MU._compute_distributed_log_softmax(wide.to(DEV)[:, :vocab], None)
+    assert torch.equal(sl.cpu(), got.detach().cpu()[0, :4])

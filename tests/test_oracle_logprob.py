@@ -228,3 +228,19 @@ def test_logprobs_post_process_brute_force():
     unpacked = L.logprobs_post_process(packed_logits, packed_ids, torch.tensor(lengths), cu_seqlens=cu,
                                         original_batch_size=b, original_seq_len=s)
     assert torch.allclose(unpacked, got, atol=1e-6)
+
+
+def test_stable_log_softmax_is_the_textbook_one():
+    """``model_utils.py:49-67``: against the library routine in float64 and a brute-force loop on a tiny row
+    (a dropped maximum, a wrong sign of the log term or a sum over the wrong axis fails one of them)."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(4, 6, 300, generator=g) * 3 + 40.0      # large offset: an unshifted exp would overflow fp32 sums' precision
+    got = L.stable_log_softmax(x)
+    want = torch.log_softmax(x.double(), dim=-1)
+    assert (got.double() - want).abs().max().item() <= 2e-5
+    row = [0.5, -1.25, 3.0, 3.0, -7.0]
+    z = sum(math.exp(v) for v in row)
+    brute = [v - math.log(z) for v in row]
+    small = L.stable_log_softmax(torch.tensor([row]))
+    assert all(abs(float(small[0, i]) - brute[i]) <= 1e-6 for i in range(len(row)))
+    assert abs(float(small.exp().sum()) - 1.0) <= 1e-6
