@@ -284,7 +284,7 @@ def _log_softmax_fwd(logits):
     _rows2d(logits, "logits")
     n, v = logits.shape
     with torch.cuda.device(logits.device):
-        out = torch.empty((n, v), dtype=logits.dtype, device=logits.device)
+        out = _grad_buffer((n, v), logits)
         with _timed("log_softmax_fwd"):
             code = _lib.load().nrl_log_softmax_fwd(_ptr(logits), _dtype_code(logits), n, v, logits.stride(0) if n > 1 else v,
                                                    _ptr(out), v, _stream())
@@ -300,7 +300,7 @@ def _log_softmax_bwd(logprobs, grad):
         raise ValueError("grad must have the shape and dtype of the log-probabilities")
     n, v = logprobs.shape
     with torch.cuda.device(logprobs.device):
-        dx = torch.empty((n, v), dtype=logprobs.dtype, device=logprobs.device)
+        dx = _grad_buffer((n, v), logprobs)
         with _timed("log_softmax_bwd"):
             code = _lib.load().nrl_log_softmax_bwd(_ptr(logprobs), _dtype_code(logprobs), n, v, logprobs.stride(0) if n > 1 else v,
                                                    _ptr(grad), grad.stride(0) if n > 1 else v, _ptr(dx), v, _stream())
@@ -653,7 +653,7 @@ def _topk_logsoftmax_bwd(logits, indices, logprobs, grad):
             raise ValueError(f"{name} must be fp32 [{b}, {s}, {k}], got {t.dtype} {tuple(t.shape)}")
     logprobs, grad = logprobs.contiguous(), grad.contiguous()
     with torch.cuda.device(logits.device):
-        d = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+        d = _grad_buffer(logits.shape, logits)
         code = _lib.load().nrl_topk_logsoftmax_bwd(C.byref(rows), _ptr(indices), k, _ptr(logprobs), _ptr(grad), _ptr(d),
                                                    d.stride(0), d.stride(1), _stream())
     _lib.check(code, "nrl_topk_logsoftmax_bwd")
@@ -969,7 +969,7 @@ def _neg_entropy_bwd(logits, lse, h, grad):
     b, s, _ = logits.shape
     lse, h, grad = _row_scalar(lse, b, s, "lse"), _row_scalar(h, b, s, "h"), _row_scalar(grad, b, s, "grad")
     with torch.cuda.device(logits.device):
-        d = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+        d = _grad_buffer(logits.shape, logits)
         with _timed("neg_entropy_bwd"):
             code = _lib.load().nrl_neg_entropy_bwd(C.byref(rows), _ptr(lse), _ptr(h), _ptr(grad), _ptr(d), d.stride(0), d.stride(1), _stream())
     _lib.check(code, "nrl_neg_entropy_bwd")
@@ -1007,7 +1007,7 @@ def _gather_logprob_bwd(logits, indices, vocab_start, vocab_end, lse, grad):
         raise ValueError(f"grad must be fp32 [{b}, {s}, {k}], got {grad.dtype} {tuple(grad.shape)}")
     grad = grad.contiguous()
     with torch.cuda.device(logits.device):
-        d = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+        d = _grad_buffer(logits.shape, logits)
         with _timed("gather_logprob_bwd"):
             code = _lib.load().nrl_gather_logprob_bwd(C.byref(rows), _ptr(indices), k, _ptr(lse), _ptr(grad), _ptr(d),
                                                       d.stride(0), d.stride(1), _stream())
@@ -1046,7 +1046,7 @@ def _soft_cross_entropy_bwd(student, teacher, lse_student, lse_teacher, grad):
     b, s, _ = student.shape
     lx, ly, grad = _row_scalar(lse_student, b, s, "lse_student"), _row_scalar(lse_teacher, b, s, "lse_teacher"), _row_scalar(grad, b, s, "grad")
     with torch.cuda.device(student.device):
-        d = torch.empty(student.shape, dtype=student.dtype, device=student.device)
+        d = _grad_buffer(student.shape, student)
         with _timed("soft_cross_entropy_bwd"):
             code = _lib.load().nrl_soft_cross_entropy_bwd(C.byref(rows), _ptr(teacher), teacher.stride(0), teacher.stride(1),
                                                           _ptr(lx), _ptr(ly), _ptr(grad), _ptr(d), d.stride(0), d.stride(1), _stream())
