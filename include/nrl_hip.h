@@ -92,7 +92,12 @@ int nrl_log_softmax_bwd(const void* logprobs, int32_t dtype, int64_t n_rows, int
  * dlogits: same dtype as the logits; row (o, i) at dlogits + o*d_stride_outer + i*d_stride_inner
  * for 0 <= i < d_n_inner; rows with i >= rows->n_inner (positions the forward dropped) are
  * zero-filled.  dlogits may alias the logits (in-place gradient).  Rows whose g is exactly 0 are
- * zero-filled without reading the logits. */
+ * zero-filled without reading the logits.
+ * Placement: every kernel here that reads logits and writes a tensor of the same shape streams one row in
+ * and another out at a fixed distance, and HBM serves the pair up to 17 % slower when (dlogits - logits) is
+ * a multiple of 512 KiB (rows of a power-of-two size) or 64 - 256 KiB past a multiple of 2 MiB (V = 151936
+ * bf16).  A separate output buffer is best started about 1.69 MiB (0x1B0000) past a multiple of 2 MiB
+ * relative to the logits. */
 int nrl_logprob_bwd(const nrl_rows* rows, const float* lse, const float* grad,
                     int64_t grad_stride_outer, int64_t grad_stride_inner, void* dlogits,
                     int64_t d_n_inner, int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
