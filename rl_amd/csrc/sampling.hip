@@ -125,9 +125,11 @@ __device__ __forceinline__ float wave_seq_sum_desc(const float* e, int n) {
     float s = 0.f;
     for (int blk = (n - 1) / kWave; blk >= 0; --blk) {
         const int idx = blk * kWave + lane;
+        // lanes past the end hold 0 and come first in this order, where adding them changes nothing; with a
+        // fixed trip count the loop unrolls into 64 lane reads with constant indices
         const float v = idx < n ? e[idx] : 0.f;
-        const int top = n - 1 - blk * kWave < kWave - 1 ? n - 1 - blk * kWave : kWave - 1;
-        for (int i = top; i >= 0; --i) s += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), i));
+#pragma unroll
+        for (int i = kWave - 1; i >= 0; --i) s += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), i));
     }
     return s;
 }
@@ -316,10 +318,13 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     const float cut = 1.0f - a.top_p;
     const float span = logf(static_cast<float>(vocab) / cut);  // from probability (1-p)/V up to 1, in nats
     const float b0 = lse_full - span;
-    const float to_bin = static_cast<float>(kMassBins) / span;
+    // The bins start a quarter of the span above b0: an edge lower than that would keep thousands of tokens,
+    // more than the list holds anyway, and the many elements just above b0 would each cost an LDS atomic.
+    const float hb = b0 + 0.25f * span;
+    const float to_bin = static_cast<float>(kMassBins) / (0.75f * span);
     auto bin = [&](float x) {
-        if (x > b0) {
-            const int j = static_cast<int>((x - b0) * to_bin);
+        if (x > hb) {
+            const int j = static_cast<int>((x - hb) * to_bin);
             atomicAdd(&sh.mass_bin[(tid & (kMassCopies - 1)) * kMassBins + (j < kMassBins - 1 ? j : kMassBins - 1)], expf(x - lse_full));
         }
     };
@@ -340,7 +345,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         const unsigned long long ok = __ballot(1.0f - above <= cut * 0.999f - 1e-5f);
         const int edge = ok ? 63 - __builtin_clzll(ok) : 0;
         // just under the edge, so that an element the rounding of its bin number put into bin `edge` counts
-        return edge > 0 ? order_key(b0 + (static_cast<float>(edge) - 0.01f) / to_bin) : order_key(b0) + 1u;
+        return ok ? order_key(hb + (static_cast<float>(edge) - 0.01f) / to_bin) : order_key(b0) + 1u;
     };
     auto clear_bins = [&]() {
         for (int i = tid; i < kMassCopies * kMassBins; i += kSelBlock) sh.mass_bin[i] = 0.f;
@@ -348,11 +353,21 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     auto bound_from_row = [&]() -> uint32_t {
         clear_bins();
         __syncthreads();
-        for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
-            float t[EPV];
-            Row<DT>::decode(xv[vi], t);
+        for (int64_t vb = 0; vb < nvec; vb += kSub * kSelBlock) {  // kSub loads in flight per thread
+            u32x4 q[kSub];
 #pragma unroll
-            for (int k = 0; k < EPV; ++k) bin(scale_logit<DT, TEMP>(t[k], a.tparam));
+            for (int u = 0; u < kSub; ++u) {
+                const int64_t vi = vb + u * kSelBlock + tid;
+                if (vi < nvec) q[u] = xv[vi];
+            }
+#pragma unroll
+            for (int u = 0; u < kSub; ++u) {
+                if (vb + u * kSelBlock + tid >= nvec) continue;
+                float t[EPV];
+                Row<DT>::decode(q[u], t);
+#pragma unroll
+                for (int k = 0; k < EPV; ++k) bin(scale_logit<DT, TEMP>(t[k], a.tparam));
+            }
         }
         if (tid < head) bin(scale_logit<DT, TEMP>(Row<DT>::load1(row, tid), a.tparam));
         if (tail0 + tid < vocab) bin(scale_logit<DT, TEMP>(Row<DT>::load1(row, tail0 + tid), a.tparam));
@@ -493,18 +508,26 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                 cum = fmaxf(0.f, (s_full - s_k) / s_full);
                 s_k = s_full;
             }
-            n_keep = 1;
-            bool done = false;
-            for (int blk = (n_k - 1) / kWave; blk >= 0 && !done; --blk) {
+            // Elements fall, smallest first, while the running sum stays <= 1 - p; the sum only grows, so
+            // counting the steps that end at or under the cut counts the fallen.  Whole blocks of 64 with
+            // constant lane indices: lanes past the end come first and add nothing (each counts as a step
+            // under the cut and is taken off again), index 0 is always kept and never enters the sum.
+            const int top_blk = (n_k - 1) / kWave;
+            int steps_under = 0;
+            for (int blk = top_blk; blk >= 0; --blk) {
                 const int idx = blk * kWave + tid;
-                const float v = idx < n_k ? sh.expv[idx] : 0.f;
-                const int top = n_k - 1 - blk * kWave < kWave - 1 ? n_k - 1 - blk * kWave : kWave - 1;
-                for (int i = top; i >= 0; --i) {
-                    if (blk * kWave + i < 1) break;  // index 0 is always kept
-                    cum += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), i)) / s_k;
-                    if (cum > cut) { n_keep = blk * kWave + i + 1; done = true; break; }
+                const float v = (idx >= 1 && idx < n_k) ? sh.expv[idx] / s_k : 0.f;
+#pragma unroll
+                for (int i = kWave - 1; i >= 0; --i) {
+                    cum += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), i));
+                    steps_under += cum <= cut ? 1 : 0;
                 }
+                if (!(cum <= cut)) break;  // nothing further down can fall (also leaves on a NaN)
             }
+            const int fallen = steps_under - ((top_blk + 1) * kWave - n_k);
+            n_keep = n_k - fallen;
+            if (n_keep < 1) n_keep = 1;
+            if (n_keep > n_k) n_keep = n_k;
         }
         const float s = wave_seq_sum_desc(sh.expv, n_keep);
         const unsigned long long last = sh.cand[n_keep - 1];

@@ -189,6 +189,37 @@ def test_kept_sets_beyond_the_candidate_list(k, p, vocab, sigma, dtype):
     assert torch.all(gg[~got_keep[:, :-1]] == 0)
 
 
+def test_top_p_cut_at_multiples_of_the_wave_width():
+    """The finish phase walks the sorted candidates 64 at a time; kept sets of exactly 64, 128, 192 ... entries
+    put the cut on the first element of such a block.  Crafted rows (distinct descending values above a
+    negligible floor) and seeded Gaussian rows whose nuclei happen to be 1024 and 576 tokens wide."""
+    vocab = 5000
+    for n_keep, n_top in ((64, 100), (128, 200), (192, 300), (256, 257), (63, 100), (65, 100)):
+        # n_top tokens with probabilities ~ 1/n_top each (slightly decreasing), the rest negligible; the cut
+        # 1 - p falls between the cumulative mass of n_top - n_keep and n_top - n_keep + 1 of the smallest
+        logit = torch.full((vocab,), -60.0)
+        vals = 2.0 + torch.linspace(0.0, 0.01, n_top)            # ascending, almost equal
+        idx = torch.randperm(vocab, generator=torch.Generator().manual_seed(n_keep))[:n_top]
+        logit[idx] = vals
+        prob = torch.softmax(logit.double(), -1)[idx]             # ascending like vals
+        cum = prob.cumsum(0)
+        n_drop = n_top - n_keep
+        cut = float((cum[n_drop - 1] + cum[n_drop]) / 2)
+        p = 1.0 - cut
+        x = logit.view(1, 1, vocab).repeat(1, 2, 1)
+        want = OS.keep_mask_rows(x.reshape(-1, vocab), None, p).reshape(x.shape)
+        assert int(want[0, 0].sum()) == n_keep
+        _, keep = apply_top_k_top_p(x.to(DEV), None, p)
+        assert torch.equal(keep.cpu(), want), n_keep
+        _, keep_k = apply_top_k_top_p(x.to(DEV), n_top + 50, p)   # the same cut reached through the top-k path
+        assert torch.equal(keep_k.cpu(), OS.keep_mask_rows(x.reshape(-1, vocab), n_top + 50, p).reshape(x.shape)), n_keep
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(1, 32, 151936, generator=g) * 4.0).to(torch.bfloat16)
+    want = OS.keep_mask_rows(x.float().reshape(-1, 151936), None, 0.9).reshape(x.shape)
+    _, keep = apply_top_k_top_p(x.to(DEV), None, 0.9)
+    assert torch.equal(keep.cpu(), want)
+
+
 def test_wide_rows_with_masked_vocabulary_entries():
     """-inf logits (a masked part of the vocabulary) carry no mass and are never kept, also on the
     threshold-search path; a top_k that reaches into them keeps only finite entries plus nothing else."""
