@@ -37,8 +37,8 @@ __global__ __launch_bounds__(kAdvBlock) void prompt_hash_kernel(const int64_t* p
     if (threadIdx.x == 0) hashes[b] = h;
 }
 
-__global__ __launch_bounds__(kAdvBlock) void prompt_group_kernel(const int64_t* prompts, int64_t batch, int64_t len,
-                                                                 int64_t stride, const uint64_t* hashes, int32_t* group) {
+__global__ __launch_bounds__(kAdvBlock) void prompt_group_kernel(const int64_t* prompts, int64_t len, int64_t stride,
+                                                                 const uint64_t* hashes, int32_t* group) {
     __shared__ int sm_flag[kAdvWaves];
     const int64_t b = blockIdx.x;
     const uint64_t hb = hashes[b];
@@ -231,7 +231,7 @@ extern "C" int nrl_group_baseline_std(const int64_t* prompts, int64_t batch, int
     int32_t* group = group_out ? group_out : reinterpret_cast<int32_t*>(hashes + batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     prompt_hash_kernel<<<dim3((unsigned)batch), dim3(kAdvBlock), 0, s>>>(prompts, prompt_len, prompt_stride, hashes);
-    prompt_group_kernel<<<dim3((unsigned)batch), dim3(kAdvBlock), 0, s>>>(prompts, batch, prompt_len, prompt_stride, hashes, group);
+    prompt_group_kernel<<<dim3((unsigned)batch), dim3(kAdvBlock), 0, s>>>(prompts, prompt_len, prompt_stride, hashes, group);
     group_stats_kernel<<<dim3((unsigned)((batch + 127) / 128)), dim3(128), 0, s>>>(
         group, batch, rewards, valid, std_rewards, leave_one_out, normalize, baseline_out, std_out, adv_out);
     return check_launch("group_baseline_std");

@@ -574,7 +574,7 @@ extern "C" int nrl_log_softmax_fwd(const void* logits, int32_t dtype, int64_t n_
     if (!logits || !out) return fail(NRL_E_INVALID, "null logits or out");
     if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    NRL_DISPATCH(dtype, 0, log_softmax_fwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logits, vocab, row_stride, out, out_row_stride));
+    NRL_DISPATCH(dtype, 0, (void)TEMP; log_softmax_fwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logits, vocab, row_stride, out, out_row_stride));
     return check_launch("log_softmax_fwd");
 }
 
@@ -587,7 +587,7 @@ extern "C" int nrl_log_softmax_bwd(const void* logprobs, int32_t dtype, int64_t 
     if (!logprobs || !grad || !dx) return fail(NRL_E_INVALID, "null logprobs, grad or dx");
     if (n_rows >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    NRL_DISPATCH(dtype, 0, log_softmax_bwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logprobs, vocab, lp_row_stride, grad,
+    NRL_DISPATCH(dtype, 0, (void)TEMP; log_softmax_bwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logprobs, vocab, lp_row_stride, grad,
                                                                                                    grad_row_stride, dx, dx_row_stride));
     return check_launch("log_softmax_bwd");
 }
