@@ -52,6 +52,9 @@ WORKLOADS = {
     "c5": dict(seqs=0, seq_len=131072, vocab=131072, dtype="bf16", mb_seqs=0, std=3.0, spike_p=0.0,
                desc="benchmark config 5: sequences of U[2048,32768] tokens packed into one 131072-token row, V=131072 bf16, "
                     "sequence-level-normalised loss, k3 KL beta=0.001, fwd+bwd to dlogits"),
+    "post": dict(seqs=16, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=3.0, spike_p=0.0,
+                 desc="forward-only LogprobsPostProcessor (prev / reference logprobs): 16 seq x 4096 tok right-padded to "
+                      "lengths U[2048,4096], V=151936 bf16"),
     "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
                desc="benchmark config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
 }
@@ -314,6 +317,54 @@ def bench_distill(args, torch, w):
     }))
 
 
+def bench_post(args, torch, w):
+    """The forward-only post-processor the policy worker runs for prev_logprobs and reference_policy_logprobs."""
+    from types import SimpleNamespace
+
+    from rl_amd import ops
+    from rl_amd.models.automodel.train import LogprobsPostProcessor
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    b, s, v = w["seqs"], w["seq_len"], w["vocab"]
+    g = torch.Generator(device=dev).manual_seed(7007)
+    logits = torch.empty((b, s, v), dtype=torch.bfloat16, device=dev).normal_(0.0, w["std"], generator=g)
+    ids = torch.randint(0, v, (b, s), generator=g, device=dev)
+    lengths = torch.randint(s // 2, s + 1, (b,), generator=g, device=dev)
+    pp = LogprobsPostProcessor({"logprob_chunk_size": None}, None, None, None, 1)
+    inputs = SimpleNamespace(seq_len=s, input_ids=ids)
+
+    def step():
+        return pp(logits, {"input_lengths": lengths}, inputs, b, s)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = EventTimer(torch)
+    ops.KERNEL_TIMER = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    km = timer.summary()
+    live_rows = int((lengths - 1).clamp(min=0).sum().item())   # rows 0 .. length-2 of a sequence are read
+    alg = live_rows * v * 2
+    k_ms = km["logprob_post_fwd"]["avg_ms"]
+    gbs = alg / (k_ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "forward-only token logprobs (post-processor) tokens/s at V=151936; % of HBM peak",
+        "value": b * s * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["desc"], "sequences": b, "seq_len": s, "vocab": v, "rows_read": live_rows},
+        "roofline": {"bound": "hbm", "kernel": "logprob_post_fwd_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": k_ms, "algorithmic_bytes_per_launch": alg},
+        "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in km.items()},
+    }))
+
+
 def bench_packed(args, torch, w):
     """One packed row through SequencePackingFusionLossWrapper (single pass), then the three-pass packed path."""
     from rl_amd import ops
@@ -494,6 +545,8 @@ def main():
         return bench_distill(args, torch, w)
     if args.workload == "c5":
         return bench_packed(args, torch, w)
+    if args.workload == "post":
+        return bench_post(args, torch, w)
     if args.seqs:
         w["seqs"] = args.seqs
         w["mb_seqs"] = min(w["mb_seqs"], args.seqs)
