@@ -1,0 +1,204 @@
+"""Seeded random sweeps against the CPU oracle: shapes, dtypes, strided views and loss configurations that
+no hand-written case lists.  Every draw is reproducible from the seed in the test id."""
+
+import math
+import random
+
+import pytest
+import torch
+
+from oracle import logprob as OL
+from oracle import loss as O
+from rl_amd.algorithms.logits_sampling_utils import TrainingSamplingParams
+from rl_amd.algorithms.loss import (ClippedPGLossConfig, ClippedPGLossFn, prepare_loss_input,
+                                    wrap_loss_fn_with_input_preparation)
+from rl_amd.distributed import model_utils as MU
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _close(a, b, rel, abs_):
+    if math.isinf(a) or math.isinf(b) or math.isnan(a) or math.isnan(b):
+        return a == b or (math.isnan(a) and math.isnan(b))
+    return abs(a - b) <= rel * abs(b) + abs_
+
+
+def _views(rng, b, s, v, dtype, seed):
+    """Logits as a plain tensor, as a column slice of a wider buffer, or as a slice along the sequence."""
+    g = torch.Generator().manual_seed(seed)
+    kind = rng.choice(["plain", "pad", "seqslice"])
+    if kind == "pad":
+        return (torch.randn(b, s, v + 24, generator=g) * 2.5).to(dtype), (lambda t: t[..., 8:8 + v]), kind
+    if kind == "seqslice":
+        return (torch.randn(b, s + 3, v, generator=g) * 2.5).to(dtype), (lambda t: t[:, 2:2 + s]), kind
+    return (torch.randn(b, s, v, generator=g) * 2.5).to(dtype), (lambda t: t), kind
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_views_and_dtypes(seed):
+    rng = random.Random(1000 + seed)
+    b, s = rng.randint(1, 5), rng.randint(2, 40)
+    v = rng.choice([rng.randint(3, 70), rng.randint(100, 3000), rng.choice([4096, 8192, 32000, 50257, 65536 + 8, 131072])])
+    dtype = rng.choice([torch.float32, torch.bfloat16, torch.float16])
+    buf, sl, kind = _views(rng, b, s, v, dtype, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    ids = torch.randint(0, v, (b, s), generator=g)
+    logits_cpu = sl(buf)
+    xo = logits_cpu.float().clone().requires_grad_(True)
+    lp_want = OL.next_token_logprobs(ids, xo)
+    dbuf = buf.to(DEV).requires_grad_(True)
+    x = sl(dbuf)
+    lp = MU.get_next_token_logprobs_from_logits(ids.to(DEV), x)
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert (lp.detach().cpu() - lp_want.detach()).abs().max().item() <= tol * max(1.0, lp_want.detach().abs().max().item() / 10)
+
+    tm = (torch.rand(b, s, generator=g) < 0.7).float()
+    tm[:, 0] = 0
+    sm = (torch.rand(b, generator=g) < 0.8).float()
+    cur = torch.cat([torch.zeros(b, 1), lp_want.detach()], 1)
+    noisy = lambda: cur + 0.05 * torch.randn(b, s, generator=g)  # noqa: E731
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm,
+            "advantages": torch.randn(b, 1, generator=g).expand(b, s).contiguous(),
+            "prev_logprobs": noisy(), "generation_logprobs": noisy(), "reference_policy_logprobs": noisy()}
+    gs, gt = sm.sum() + 1, (tm[:, 1:] * sm.unsqueeze(-1)).sum() + 1
+    cfg = rng.choice([dict(), dict(token_level_loss=False), dict(reference_policy_kl_penalty=0.0, ratio_clip_max=0.28),
+                      dict(use_importance_sampling_correction=True, truncated_importance_sampling_type="tis",
+                           truncated_importance_sampling_ratio=1.02)])
+    want, _ = O.clipped_pg_loss(O.LossConfig(**cfg), lp_want, data, gs, gt)
+    want.backward()
+    fn = ClippedPGLossFn(ClippedPGLossConfig(**cfg))
+    got, _ = wrap_loss_fn_with_input_preparation(x, {k: t.to(DEV) for k, t in data.items()}, gs.to(DEV), gt.to(DEV), fn,
+                                                 prepare_loss_input)
+    got.backward()
+    if dtype == torch.float32:
+        assert abs(got.item() - want.item()) <= 1e-4 * abs(want.item()) + 1e-6
+    else:
+        assert abs(got.item() - want.item()) <= 2e-3 * abs(want.item()) + 1e-5
+    scale = xo.grad.abs().max().item() + 1e-30
+    assert (sl(dbuf.grad).float().cpu() - xo.grad).abs().max().item() <= (1e-4 if dtype == torch.float32 else 2.0 ** -7) * scale + 1e-12
+    if kind != "plain":  # nothing outside the view is written
+        outside = torch.ones_like(buf, dtype=torch.bool)
+        sl(outside)[...] = False
+        assert bool((dbuf.grad.cpu()[outside] == 0).all())
+
+    if v >= 16:
+        k = rng.choice([None, rng.randint(1, min(v, 64))])
+        p = rng.choice([1.0, 0.9, 0.5])
+        if k is None and p == 1.0:
+            k = 5
+        want_s = OL.next_token_logprobs(ids, logits_cpu.float(), top_k=k, top_p=p)
+        got_s = MU.get_next_token_logprobs_from_logits(ids.to(DEV), sl(buf.to(DEV)),
+                                                       sampling_params=TrainingSamplingParams(top_k=k, top_p=p, temperature=1.0)).cpu()
+        fin = torch.isfinite(want_s)
+        assert bool((torch.isfinite(got_s) == fin).all())
+        if fin.any():
+            assert (got_s[fin] - want_s[fin]).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2)
+
+
+def _random_config(rng):
+    c = {}
+    if rng.random() < 0.3:
+        c["token_level_loss"] = False
+    if rng.random() < 0.5:
+        c["reference_policy_kl_penalty"] = rng.choice([0.0, 0.001, 0.05])
+    if rng.random() < 0.5:
+        c["reference_policy_kl_type"] = rng.choice(["k1", "k2", "k3"])
+    if rng.random() < 0.3:
+        c["use_on_policy_kl_approximation"] = True
+    if rng.random() < 0.2:
+        c["kl_input_clamp_value"] = rng.choice([None, 0.05, 5.0])
+    if rng.random() < 0.2:
+        c["kl_output_clamp_value"] = rng.choice([None, 0.001, 3.0])
+    if rng.random() < 0.4:
+        c["ratio_clip_max"] = rng.choice([0.28, 0.02, 0.5])
+        c["ratio_clip_min"] = rng.choice([0.2, 0.01])
+    if rng.random() < 0.1:
+        c["use_kl_in_reward"] = True
+    mode = rng.choice(["plain", "plain", "cispo", "noratio", "onpolicy", "gspo", "dual"])
+    if mode == "cispo":
+        c["use_cispo"], c["token_level_loss"] = True, True
+    if mode == "noratio":
+        c["disable_ppo_ratio"] = True
+    if mode == "onpolicy":
+        c["force_on_policy_ratio"] = True
+    if mode == "gspo":
+        c["sequence_level_importance_ratios"], c["token_level_loss"] = True, False
+    if mode == "dual":
+        c["ratio_clip_c"] = rng.choice([1.5, 3.0])
+    if rng.random() < 0.5:
+        c["use_importance_sampling_correction"] = True
+        kind = rng.choice([None, "tis", "icepop", "seq-mask-tis"])
+        if kind == "seq-mask-tis" and c.get("sequence_level_importance_ratios"):
+            kind = "tis"
+        if kind:
+            c["truncated_importance_sampling_type"] = kind
+            c["truncated_importance_sampling_ratio"] = rng.choice([1.01, 1.05, 2.0])
+            if kind != "tis" or rng.random() < 0.5:
+                c["truncated_importance_sampling_ratio_min"] = rng.choice([0.5, 0.97, 0.99])
+    if rng.random() < 0.15 and mode != "cispo":
+        c["positive_example_nll_weight"] = 0.3
+    return c
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_loss_configurations(seed):
+    """Loss, every metric and the gradient through the wrapper (single pass when it applies) and through the
+    three-pass path, for configurations drawn over all switches of ``ClippedPGLossConfig``."""
+    rng = random.Random(2000 + seed)
+    cfg = _random_config(rng)
+    try:
+        O.check_config(O.LossConfig(**cfg))
+    except AssertionError:
+        with pytest.raises(AssertionError):   # the product rejects what the reference rejects
+            ClippedPGLossFn(ClippedPGLossConfig(**cfg))
+        return
+    b, s, v = rng.randint(1, 6), rng.randint(2, 33), rng.choice([17, 130, 1000, 2003, 4096])
+    dtype = rng.choice([torch.float32, torch.bfloat16])
+    g = torch.Generator().manual_seed(seed)
+    logits = (torch.randn(b, s, v, generator=g) * 2).to(dtype)
+    ids = torch.randint(0, v, (b, s), generator=g)
+    kind = rng.choice(["rand", "prefix", "none", "onesample"])
+    tm = (torch.rand(b, s, generator=g) < 0.7).float()
+    if kind == "prefix":
+        tm = (torch.arange(s).unsqueeze(0) >= torch.randint(0, s, (b, 1), generator=g)).float()
+    if kind == "none":
+        tm = torch.zeros(b, s)
+    tm[:, 0] = 0
+    sm = (torch.rand(b, generator=g) < 0.8).float()
+    if kind == "onesample":
+        sm = torch.zeros(b)
+        sm[rng.randrange(b)] = 1
+    xo = logits.float().clone().requires_grad_(True)
+    lp_want = OL.next_token_logprobs(ids, xo)
+    cur = torch.cat([torch.zeros(b, 1), lp_want.detach()], 1)
+    noise = rng.choice([0.02, 0.3])
+    noisy = lambda: cur + noise * torch.randn(b, s, generator=g)  # noqa: E731
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm,
+            "advantages": torch.randn(b, 1, generator=g).expand(b, s).contiguous(),
+            "prev_logprobs": noisy(), "generation_logprobs": noisy(), "reference_policy_logprobs": noisy(),
+            "rewards": torch.randn(b, generator=g)}
+    gs, gt = sm.sum() + rng.choice([0, 1]), (tm[:, 1:] * sm.unsqueeze(-1)).sum() + rng.choice([0, 1])
+    want, wm = O.clipped_pg_loss(O.LossConfig(**cfg), lp_want, data, gs, gt)
+    if want.requires_grad and math.isfinite(want.item()):
+        want.backward()
+    gref = xo.grad if xo.grad is not None else torch.zeros_like(xo)
+    fn = ClippedPGLossFn(ClippedPGLossConfig(**cfg))
+    ddev = {k: t.to(DEV) for k, t in data.items()}
+    lt = 2e-4 if dtype == torch.float32 else 4e-3
+    for path in ("wrapper", "three-pass"):
+        x = logits.to(DEV).requires_grad_(True)
+        if path == "wrapper":
+            got, gm = wrap_loss_fn_with_input_preparation(x, dict(ddev), gs.to(DEV), gt.to(DEV), fn, prepare_loss_input)
+        else:
+            loss_input, prepared = prepare_loss_input(x, dict(ddev), fn)
+            got, gm = fn(data=prepared, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+        if got.requires_grad and math.isfinite(got.item()):
+            got.backward()
+        assert _close(got.item(), want.item(), lt, 1e-5 if dtype != torch.float32 else 2e-6), (path, cfg)
+        assert set(gm) == set(wm)
+        for key in wm:
+            assert _close(float(gm[key]), float(wm[key]), lt * 2, 1e-4 if dtype != torch.float32 else 1e-5), (path, key, cfg)
+        ggot = (x.grad if x.grad is not None else torch.zeros_like(x)).float().cpu()
+        scale = gref.abs().max().item() + 1e-30
+        assert (ggot - gref).abs().max().item() <= (2e-4 if dtype == torch.float32 else 2.0 ** -6) * scale + 1e-12, (path, cfg)
