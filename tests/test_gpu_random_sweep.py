@@ -202,3 +202,105 @@ def test_random_loss_configurations(seed):
         ggot = (x.grad if x.grad is not None else torch.zeros_like(x)).float().cpu()
         scale = gref.abs().max().item() + 1e-30
         assert (ggot - gref).abs().max().item() <= (2e-4 if dtype == torch.float32 else 2.0 ** -6) * scale + 1e-12, (path, cfg)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_packed_batches(seed):
+    """Random sequence lengths (including empty and one-token sequences), random padding inside the spans and
+    an unused tail, through the packed logprob op, the packed single pass and the three-pass packed path."""
+    from rl_amd.algorithms.loss import SequencePackingFusionLossWrapper, prepare_packed_loss_input
+
+    rng = random.Random(3000 + seed)
+    b = rng.randint(1, 6)
+    lens = [rng.choice([0, 1, 2, rng.randint(3, 30)]) if rng.random() < 0.3 else rng.randint(3, 30) for _ in range(b)]
+    if max(lens) < 3:
+        lens[0] = 7
+    pads = [rng.choice([0, 0, rng.randint(1, 6)]) for _ in range(b)]
+    width = max(lens) + rng.choice([0, 0, 3])
+    tail = rng.choice([0, 0, 5])
+    vocab = rng.choice([130, 1000, 2003, 4096])
+    dtype = rng.choice([torch.float32, torch.bfloat16])
+    g = torch.Generator().manual_seed(seed)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    cup = torch.tensor([0] + list((torch.tensor(lens) + torch.tensor(pads)).cumsum(0)), dtype=torch.int32)
+    total = int(cup[-1]) + tail
+    logits = (torch.randn(1, total, vocab, generator=g) * 2.5).to(dtype)
+    ids = torch.zeros(b, width, dtype=torch.int64)
+    tm = torch.zeros(b, width, dtype=torch.int64)
+    for i, n in enumerate(lens):
+        ids[i, :n] = torch.randint(0, vocab, (n,), generator=g)
+        if n > 2:
+            tm[i, int(torch.randint(1, n - 1, (1,), generator=g)):n] = 1
+    sm = (torch.rand(b, generator=g) < 0.8).long()
+    targets = OL.pack_input_ids(ids, cu, cup, roll_shift=-1)
+    xo = logits.float().clone().requires_grad_(True)
+    lp_want = OL.packed_logits_to_logprobs(xo[:, : int(cup[-1])], targets, cup, width, target_is_pre_rolled=True)
+    cur = torch.cat([torch.zeros(b, 1), lp_want.detach()], 1)
+    noisy = lambda: cur + 0.05 * torch.randn(b, width, generator=g)  # noqa: E731
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm,
+            "advantages": torch.randn(b, 1, generator=g).expand(b, width).contiguous(),
+            "prev_logprobs": noisy(), "generation_logprobs": noisy(), "reference_policy_logprobs": noisy()}
+    gs, gt = sm.sum() + 1, (tm[:, 1:] * sm.unsqueeze(-1)).sum() + 1
+    cfg = rng.choice([dict(), dict(token_level_loss=False, reference_policy_kl_penalty=0.001), dict(use_cispo=True),
+                      dict(force_on_policy_ratio=True)])
+    want, wm = O.clipped_pg_loss(O.LossConfig(**cfg), lp_want, data, gs, gt)
+    want.backward()
+
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    padded_targets = torch.cat([targets, torch.zeros(1, total - targets.shape[1], dtype=targets.dtype)], 1)  # one per packed position
+    got_lp = MU.from_parallel_logits_to_logprobs_packed_sequences(logits.to(DEV), padded_targets.to(DEV), cup.to(DEV), width, 0, vocab, None,
+                                                                  target_is_pre_rolled=True)
+    assert (got_lp.cpu() - lp_want.detach()).abs().max().item() <= tol * max(1.0, lp_want.detach().abs().max().item() / 10)
+
+    fn = ClippedPGLossFn(ClippedPGLossConfig(**cfg))
+    ddev = {k: t.to(DEV) for k, t in data.items()}
+    lt = 2e-4 if dtype == torch.float32 else 4e-3
+    grads = []
+    for path in ("wrapper", "three-pass"):
+        x = logits.to(DEV).requires_grad_(True)
+        if path == "wrapper":
+            wrapped = SequencePackingFusionLossWrapper(fn, prepare_packed_loss_input, cu.to(DEV), cup.to(DEV))
+            got, gm = wrapped(x, dict(ddev), gs.to(DEV), gt.to(DEV))
+        else:
+            loss_input, prepared = prepare_packed_loss_input(x, dict(ddev), fn, cu.to(DEV), cup.to(DEV))
+            got, gm = fn(data=prepared, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+        if got.requires_grad:
+            got.backward()
+        assert _close(got.item(), want.item(), lt, 1e-5 if dtype != torch.float32 else 2e-6), (path, cfg, lens, pads)
+        assert set(gm) == set(wm)
+        for key in wm:
+            assert _close(float(gm[key]), float(wm[key]), lt * 2, 1e-4 if dtype != torch.float32 else 1e-5), (path, key)
+        grads.append((x.grad if x.grad is not None else torch.zeros_like(x)).float().cpu())
+    scale = xo.grad.abs().max().item() + 1e-30
+    for gq in grads:
+        assert (gq - xo.grad).abs().max().item() <= (2e-4 if dtype == torch.float32 else 2.0 ** -6) * scale + 1e-12
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_lm_head_shapes(seed):
+    """Fused lm_head over random token counts, hidden widths (multiples of 64 take the 256 x 256 core, others
+    the 128-wide one) and vocabulary sizes that are not multiples of any tile."""
+    from oracle import lmhead as OH
+
+    rng = random.Random(4000 + seed)
+    s, b = rng.randint(2, 150), rng.randint(1, 3)
+    h = rng.choice([64, 128, 192, 72, 200, 256])
+    v = rng.choice([rng.randint(40, 700), 1000, 2500, 4099])
+    g = torch.Generator().manual_seed(seed)
+    hid = torch.randn(s, b, h, generator=g).to(torch.bfloat16)
+    w = (torch.randn(v, h, generator=g) * 0.05).to(torch.bfloat16)
+    ids = torch.randint(0, v, (b, s), generator=g)
+    up = torch.randn(b, s, generator=g) * 1e-3
+    up[:, -1] = 0
+    want = OH.hidden_to_logprobs(hid, w, ids)
+    want_dh, want_dw = OH.hidden_to_logprobs_backward(hid, w, ids.roll(-1, -1), up)
+    hg, wg = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp = MU.from_parallel_hidden_states_to_logprobs(hg, wg, False, ids.to(DEV), 0, v, None)
+    logit_scale = (hid.float() @ w.float().T).abs().max().item()
+    err = (lp.detach().cpu() - want).abs()
+    assert err.max().item() <= 2.0 ** -7 * logit_scale + 2e-3
+    (lp * up[:, :-1].to(DEV)).sum().backward()
+    for got, ref in ((hg.grad.float().cpu(), want_dh), (wg.grad.float().cpu(), want_dw.float())):
+        scale = ref.abs().max().item() + 1e-30
+        assert (got - ref).abs().max().item() <= 1e-2 * scale
+        assert ((got - ref).norm() / (ref.norm() + 1e-30)).item() <= 5e-3
