@@ -304,3 +304,36 @@ def test_random_lm_head_shapes(seed):
         scale = ref.abs().max().item() + 1e-30
         assert (got - ref).abs().max().item() <= 1e-2 * scale
         assert ((got - ref).norm() / (ref.norm() + 1e-30)).item() <= 5e-3
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_prompt_groups_and_advantages(seed):
+    """Random numbers of prompts and group sizes (singletons included), tiny alphabets (near-duplicate prompts),
+    random validity masks and reward distributions, with and without leave-one-out and separate std rewards."""
+    from oracle import advantage as OA
+
+    rng = random.Random(5000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    n_prompts, plen = rng.randint(1, 40), rng.randint(1, 50)
+    base = torch.randint(0, rng.choice([2, 5, 50000]), (n_prompts, plen), generator=g)
+    sizes = [rng.choice([1, 1, 2, 3, 8, 16]) for _ in range(n_prompts)]
+    prompts = torch.cat([base[i:i + 1].repeat(k, 1) for i, k in enumerate(sizes)], 0)
+    prompts = prompts[torch.randperm(prompts.shape[0], generator=g)]
+    n = prompts.shape[0]
+    kind = rng.choice(["bernoulli", "normal", "constant"])
+    rewards = {"bernoulli": (torch.rand(n, generator=g) < 0.5).float(), "normal": torch.randn(n, generator=g) * 3,
+               "constant": torch.full((n,), 0.75)}[kind]
+    valid = (torch.rand(n, generator=g) < rng.choice([1.0, 0.9, 0.3])).float()
+    loo = rng.random() < 0.5
+    std_rewards = torch.randn(n, generator=g) if rng.random() < 0.3 else None
+    wb, ws = OA.baseline_and_std_per_prompt(prompts, rewards, valid, loo, std_rewards)
+    gb, gs_, _, gid = torch.ops.rl_amd.group_baseline_std(prompts.to(DEV), rewards.to(DEV), valid.to(DEV),
+                                                          None if std_rewards is None else std_rewards.to(DEV), loo, False)
+    want_gid = OA.group_ids_by_prompt(prompts).tolist()
+    first = {}
+    for i, v in enumerate(want_gid):
+        first.setdefault(v, i)
+    assert gid.cpu().tolist() == [first[v] for v in want_gid]            # bit-exact grouping
+    torch.testing.assert_close(gb.cpu(), wb, rtol=1e-5, atol=1e-6)
+    # E[r^2] - E[r]^2 cancels: compare the variance, not its root, near zero
+    torch.testing.assert_close(gs_.cpu().square(), ws.square(), rtol=1e-4, atol=2e-5 * (1.0 + float(rewards.abs().max()) ** 2))
