@@ -335,5 +335,9 @@ def test_random_prompt_groups_and_advantages(seed):
         first.setdefault(v, i)
     assert gid.cpu().tolist() == [first[v] for v in want_gid]            # bit-exact grouping
     torch.testing.assert_close(gb.cpu(), wb, rtol=1e-5, atol=1e-6)
+    # the decisions the driver takes on the std (dynamic sampling keeps std != 0, normalisation divides where
+    # std > 0) must not flip; with exactly representable rewards the reference's own formula is exact
+    if kind != "normal" and std_rewards is None:
+        assert torch.equal(gs_.cpu() > 0, ws > 0) and torch.equal(gs_.cpu() != 0, ws != 0)
     # E[r^2] - E[r]^2 cancels: compare the variance, not its root, near zero
     torch.testing.assert_close(gs_.cpu().square(), ws.square(), rtol=1e-4, atol=2e-5 * (1.0 + float(rewards.abs().max()) ** 2))
