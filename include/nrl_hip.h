@@ -10,7 +10,8 @@
  *   - return value: 0 = ok, negative = NRL_E_* below; nrl_last_error() gives the text for the
  *     calling thread;
  *   - the library keeps no state between calls: entry points may be called from any host
- *     thread (forward pass and autograd thread alike).
+ *     thread (forward pass and autograd thread alike).  The one exception is
+ *     nrl_grpo_loss_fwd_bwd_static, which owns a fixed device array (see there).
  *
  * The reference (NVIDIA NeMo-RL) has no FFI; each entry point names the Python code whose
  * arithmetic it replaces (paths relative to the reference tree).
@@ -217,6 +218,19 @@ int64_t nrl_grpo_loss_workspace_bytes(int64_t batch);
 int nrl_grpo_loss_fwd_bwd(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out,
                           float* dlp_out, float* dlpu_out, float* metrics_out, void* workspace,
                           int64_t workspace_bytes, void* stream);
+
+/* nrl_grpo_loss_fwd_bwd without a workspace argument and without any allocation.  It has no counterpart in
+ * the reference; it is for callers that cannot allocate device memory around the call: code under HIP graph
+ * capture, tight loops, harnesses that forbid hipMalloc.  The per-sequence partial sums live in a fixed
+ * array in the library's device image (NRL_GRPO_STATIC_MAX_BATCH * 160 bytes = 1.25 MiB on every GPU the
+ * library runs on, held until the process ends); in->batch above NRL_GRPO_STATIC_MAX_BATCH returns
+ * NRL_E_WORKSPACE.  Inputs, outputs and results are those of nrl_grpo_loss_fwd_bwd, bit for bit.
+ * The first call on a device resolves that device's copy of the array (hipGetSymbolAddress; make it outside a
+ * graph capture).  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
+ * host threads) race; calls in stream order do not, and nothing needs clearing between them. */
+#define NRL_GRPO_STATIC_MAX_BATCH 8192
+int nrl_grpo_loss_fwd_bwd_static(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out,
+                                 float* dlp_out, float* dlpu_out, float* metrics_out, void* stream);
 
 /* Fused variant: one pass over the logits computes the token logprob (as K1), the loss terms and
  * d loss / d logprob of that token (as K4) and writes dlogits (as K2) from the row held on chip:

@@ -16,6 +16,7 @@ NRL_F32, NRL_BF16, NRL_F16 = 0, 1, 2
 NRL_TEMP_DIV, NRL_TEMP_RCP = 0, 1
 NRL_TIS = {None: 0, "tis": 1, "icepop": 2, "seq-mask-tis": 3}
 NRL_GRPO_N_METRICS = 24
+NRL_GRPO_STATIC_MAX_BATCH = 8192
 
 METRIC_SLOTS = {
     "loss": 0, "probs_ratio": 1, "probs_ratio_clamped": 2, "probs_ratio_min": 3, "probs_ratio_max": 4,
@@ -79,6 +80,7 @@ SIGNATURES = {
     "nrl_topk_topp_filter": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P, _I64, _I64, _P, _P]),
     "nrl_grpo_loss_workspace_bytes": (_I64, [_I64]),
     "nrl_grpo_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _P, _I64, _P]),
+    "nrl_grpo_loss_fwd_bwd_static": (C.c_int, [C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _P]),
     "nrl_fused_workspace_bytes": (_I64, [_I64, _I64]),
     "nrl_fused_packed_workspace_bytes": (_I64, [_I64, _I64, _I64]),
     "nrl_fused_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _F, _P, _I64,

@@ -15,6 +15,8 @@
 #include <float.h>
 #include <math.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #ifdef NRL_NT_ZERO
 #define NRL_ZERO_STORE(v, p) __builtin_nontemporal_store(v, p)
@@ -601,28 +603,16 @@ extern "C" int64_t nrl_grpo_loss_workspace_bytes(int64_t batch) {
     return (batch < 1 ? 1 : batch) * P_COUNT * static_cast<int64_t>(sizeof(double));
 }
 
-extern "C" int nrl_grpo_loss_fwd_bwd(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,
-                                     float* dlpu_out, float* metrics_out, void* workspace, int64_t workspace_bytes,
-                                     void* stream) {
-    if (!cfg) return fail(NRL_E_INVALID, "cfg is NULL");
-    if (int e = check_inputs(in, !cfg->force_on_policy_ratio, cfg->has_kl != 0, true)) return e;
-    if (cfg->kl_type < 1 || cfg->kl_type > 3) return fail(NRL_E_INVALID, "kl_type must be 1, 2 or 3");
-    if (cfg->tis_type < 0 || cfg->tis_type > 3) return fail(NRL_E_INVALID, "bad tis_type");
-    if (cfg->sequence_level_importance_ratios && cfg->token_level_loss)
-        return fail(NRL_E_INVALID, "sequence-level importance ratios need a sequence-level loss");
-    if (cfg->has_nll && !in->correct_mask) return fail(NRL_E_INVALID, "correct_mask is NULL");
-    if (!loss_out || !metrics_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
-    if (workspace_bytes < nrl_grpo_loss_workspace_bytes(in->batch)) return fail(NRL_E_WORKSPACE, "workspace too small");
-    if (reinterpret_cast<uintptr_t>(workspace) & 7) return fail(NRL_E_INVALID, "workspace must be 8-byte aligned");
+static int grpo_loss_impl(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out, float* dlp_out, float* dlpu_out,
+                          float* metrics_out, double* parts, void* stream, const char* what) {
     const bool split = in->lpu != nullptr && cfg->has_kl;
-    if (in->batch * in->sm1 > 0 && (!dlp_out || (split && !dlpu_out))) return fail(NRL_E_INVALID, "null gradient output");
     GrpoArgs a;
     a.cfg = *cfg;
     a.in = *in;
     if (!cfg->has_kl) a.in.lpu = nullptr;
     a.dlp = dlp_out;
     a.dlpu = split ? dlpu_out : nullptr;
-    a.parts = static_cast<double*>(workspace);
+    a.parts = parts;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (in->batch > 0) {
         const bool gspo = cfg->sequence_level_importance_ratios && !cfg->disable_ppo_ratio && !cfg->force_on_policy_ratio;
@@ -635,7 +625,78 @@ extern "C" int nrl_grpo_loss_fwd_bwd(const nrl_grpo_cfg* cfg, const nrl_grpo_inp
         const unsigned blocks = (unsigned)((total + 255) / 256 > 1024 ? 1024 : (total + 255) / 256);
         grpo_nll_grad_kernel<<<dim3(blocks), dim3(256), 0, s>>>(a);
     }
-    return check_launch("grpo_loss_fwd_bwd");
+    return check_launch(what);
+}
+
+// argument checks shared by the two loss entry points (everything except the workspace)
+static int grpo_loss_check(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, const float* loss_out, const float* dlp_out,
+                           const float* dlpu_out, const float* metrics_out) {
+    if (!cfg) return fail(NRL_E_INVALID, "cfg is NULL");
+    if (int e = check_inputs(in, !cfg->force_on_policy_ratio, cfg->has_kl != 0, true)) return e;
+    if (cfg->kl_type < 1 || cfg->kl_type > 3) return fail(NRL_E_INVALID, "kl_type must be 1, 2 or 3");
+    if (cfg->tis_type < 0 || cfg->tis_type > 3) return fail(NRL_E_INVALID, "bad tis_type");
+    if (cfg->sequence_level_importance_ratios && cfg->token_level_loss)
+        return fail(NRL_E_INVALID, "sequence-level importance ratios need a sequence-level loss");
+    if (cfg->has_nll && !in->correct_mask) return fail(NRL_E_INVALID, "correct_mask is NULL");
+    if (!loss_out || !metrics_out) return fail(NRL_E_INVALID, "null output");
+    const bool split = in->lpu != nullptr && cfg->has_kl;
+    if (in->batch * in->sm1 > 0 && (!dlp_out || (split && !dlpu_out))) return fail(NRL_E_INVALID, "null gradient output");
+    return NRL_OK;
+}
+
+extern "C" int nrl_grpo_loss_fwd_bwd(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,
+                                     float* dlpu_out, float* metrics_out, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
+    if (int e = grpo_loss_check(cfg, in, loss_out, dlp_out, dlpu_out, metrics_out)) return e;
+    if (!workspace) return fail(NRL_E_INVALID, "null workspace");
+    if (workspace_bytes < nrl_grpo_loss_workspace_bytes(in->batch)) return fail(NRL_E_WORKSPACE, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7) return fail(NRL_E_INVALID, "workspace must be 8-byte aligned");
+    return grpo_loss_impl(cfg, in, loss_out, dlp_out, dlpu_out, metrics_out, static_cast<double*>(workspace), stream,
+                          "grpo_loss_fwd_bwd");
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same loss for callers that cannot allocate: the per-sequence partial sums live in a fixed
+// device array instead of a caller workspace.  Every GPU holds its own copy of the array at its own
+// address; the name `scratch` is only a host-side handle, the address comes from hipGetSymbolAddress
+// once per device and is what the kernels receive.
+// ---------------------------------------------------------------------------------------------
+namespace nrl {
+constexpr int64_t kStaticMaxBatch = NRL_GRPO_STATIC_MAX_BATCH;
+constexpr int kStaticMaxDevices = 64;
+static __device__ __align__(256) double scratch[kStaticMaxBatch * P_COUNT];  // 1.25 MiB per GPU
+static std::mutex scratch_mutex;
+static double* scratch_ptr[kStaticMaxDevices] = {nullptr};
+
+// device address of this GPU's `scratch`, resolved on the first call with that GPU current
+static int scratch_for_current_device(double** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(NRL_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kStaticMaxDevices) return fail(NRL_E_UNSUPPORTED, "device index %d beyond %d", dev, kStaticMaxDevices);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(NRL_E_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        scratch_ptr[dev] = static_cast<double*>(p);
+    }
+    *out = scratch_ptr[dev];
+    return NRL_OK;
+}
+}  // namespace nrl
+
+extern "C" int nrl_grpo_loss_fwd_bwd_static(const nrl_grpo_cfg* cfg, const nrl_grpo_inputs* in, float* loss_out,
+                                            float* dlp_out, float* dlpu_out, float* metrics_out, void* stream) {
+    if (int e = grpo_loss_check(cfg, in, loss_out, dlp_out, dlpu_out, metrics_out)) return e;
+    if (in->batch > kStaticMaxBatch)
+        return fail(NRL_E_WORKSPACE, "batch %lld exceeds the %lld sequences the static scratch holds; use nrl_grpo_loss_fwd_bwd",
+                    (long long)in->batch, (long long)kStaticMaxBatch);
+    double* parts = nullptr;
+    if (int e = scratch_for_current_device(&parts)) return e;
+    // rows 0 .. batch-1 of the scratch are rewritten in full by the first launch before the second reads
+    // them, and nothing beyond `batch` rows is read, so a previous call's contents need no clearing
+    return grpo_loss_impl(cfg, in, loss_out, dlp_out, dlpu_out, metrics_out, parts, stream, "grpo_loss_fwd_bwd_static");
 }
 
 extern "C" int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out, float* metrics_out,
