@@ -52,7 +52,7 @@ def prepare_loss_input(
     if loss_fn.input_type != LossInputType.LOGPROB:
         raise ValueError(f"Unknown loss function input type: {loss_fn.input_type}")
 
-    def logprobs_with(params):
+    def logprobs_with(params, chunk):
         return get_next_token_logprobs_from_logits(
             input_ids=data["input_ids"],
             next_token_logits=logits,
@@ -61,20 +61,20 @@ def prepare_loss_input(
             vocab_parallel_group=vocab_parallel_group,
             context_parallel_group=context_parallel_group,
             sampling_params=params,
-            chunk_size=chunk_size if params is not None else None,
+            chunk_size=chunk,
         )
 
     if getattr(loss_fn, "use_fused_linear_logprobs", False):
         # the model forward already produced next-token logprobs (loss/utils.py:77-83)
         logprobs = logits.to(torch.float32)[:, : data["input_ids"].shape[1] - 1]
     else:
-        logprobs = logprobs_with(sampling_params)
+        logprobs = logprobs_with(sampling_params, chunk_size)  # loss/utils.py:85-94: the main call chunks
 
     if need_top_k_or_top_p_filtering(sampling_params):
         mask = data["token_mask"] * data["sample_mask"].unsqueeze(-1)
         logprobs = mask_out_neg_inf_logprobs(logprobs, mask[:, 1:].to(logprobs.device), "curr_logprobs")
         if _wants_unfiltered_kl(loss_fn):
-            data["curr_logprobs_unfiltered"] = logprobs_with(None)
+            data["curr_logprobs_unfiltered"] = logprobs_with(None, None)  # :108-118: the unfiltered pass does not
     return {"next_token_logprobs": logprobs}, data
 
 
