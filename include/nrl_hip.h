@@ -103,6 +103,21 @@ int nrl_logprob_bwd(const nrl_rows* rows, const float* lse, const float* grad,
                     int64_t grad_stride_outer, int64_t grad_stride_inner, void* dlogits,
                     int64_t d_n_inner, int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
 
+/* dst[o, i, :] = src[o, i, :] * (factor[0] / divisor), fp32 product narrowed once to `dtype`; row (o, i) at
+ * base + o*stride_outer + i*stride_inner; dst may be src (in place).  `factor` is a DEVICE scalar, so the
+ * caller never waits for its value; in place with factor[0] / divisor exactly 1 no row is read or written.
+ * Replaces two elementwise passes of the reference:
+ *   - the in-place temperature divide apply_temperature_scaling = logits.div_(T)
+ *     (nemo_rl/models/automodel/train.py:180-194, nemo_rl/models/megatron/train.py:203-217) and its backward,
+ *     with factor = 1 and divisor = T: x * (1 / T) with the quotient in fp32, which is how the GPU divide by a
+ *     scalar rounds;
+ *   - the multiplication autograd applies to a gradient when the loss was scaled after the loss function
+ *     returned (automodel/train.py:547 multiplies by dp_size * cp_size, megatron/train.py:590-592 by
+ *     num_microbatches / cp_size), applied to a gradient the single-pass entry points have already written. */
+int nrl_scale_rows(const void* src, void* dst, int32_t dtype, int64_t n_outer, int64_t n_inner, int64_t vocab,
+                   int64_t src_stride_outer, int64_t src_stride_inner, int64_t dst_stride_outer,
+                   int64_t dst_stride_inner, const float* factor, float divisor, void* stream);
+
 /* Packed sequences (one [1, T, V] row of logits, sequences delimited by cu_seqlens_padded).
  * Replaces from_parallel_logits_to_logprobs_packed_sequences (model_utils.py:1085-1196) at
  * CP = 1: position p of sequence s (start = cu[s], len = cu[s+1]-cu[s]) uses target

@@ -33,6 +33,12 @@ Pinning status (what fixes each function besides its own text):
                            sampling_importance_ratio, probs_ratio*): restated
                            from the source text and checked against
                            independent float64 formulas only.
+* ``loss.sequence_packing_loss``  pinned: the identity the reference's own test
+                           states (per-sequence wrapper == one loss call on the
+                           unpacked batch, loss and gradient to 1e-5,
+                           ``tests/unit/algorithms/test_sequence_packing_fusion.py:190-265``)
+                           for additive metrics, and brute force for the
+                           min / max merging (``tests/test_oracle_loss.py``).
 * ``advantage.*``          pinned: golden vectors of the reference's unit tests.
 * ``advantage.seq_logprob_error_masking``  pinned by brute-force loops on tiny
                            inputs (the reference's tests only mock it).

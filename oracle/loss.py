@@ -277,6 +277,43 @@ def clipped_pg_loss(
     return loss, metrics
 
 
+_MIN_METRICS = ("probs_ratio_min", "probs_ratio_clamped_min")
+_MAX_METRICS = ("probs_ratio_max", "probs_ratio_clamped_max")
+
+
+def sequence_packing_loss(cfg: LossConfig, packed_logits, data, cu_seqlens, cu_seqlens_padded, global_valid_seqs,
+                          global_valid_toks, logprob_fn):
+    """``SequencePackingLossWrapper.__call__`` (``loss/wrapper.py:65-166``) around ``prepare_loss_input`` +
+    ``ClippedPGLossFn`` at CP = 1: sequence ``i`` owns the packed positions
+    ``[cu_padded[i], cu_padded[i+1])``, its data rows are cut to the unpadded length (:87-93), the loss is
+    called once per sequence and summed (:136), metrics are summed except the ratio extrema, which are
+    combined with min / max while infinite sentinels of empty sequences are skipped (:137-164).
+    ``logprob_fn(input_ids, logits)`` is the oracle's next-token logprob."""
+    cup = cu_seqlens if cu_seqlens_padded is None else cu_seqlens_padded
+    total, merged = 0, {}
+    for i in range(len(cu_seqlens) - 1):
+        n_real = int(cu_seqlens[i + 1] - cu_seqlens[i])
+        start, n_pad = int(cup[i]), int(cup[i + 1] - cup[i])
+        row = {k: (v[i : i + 1, :n_real] if isinstance(v, torch.Tensor) and v.ndim > 1 and v.shape[1] > 1 else
+                   (v[i : i + 1] if isinstance(v, torch.Tensor) else v)) for k, v in data.items()}
+        piece = packed_logits.narrow(1, start, n_pad)
+        lp = logprob_fn(row["input_ids"], piece)
+        loss, metrics = clipped_pg_loss(cfg, lp, row, global_valid_seqs, global_valid_toks)
+        total = total + loss
+        for k, v in metrics.items():
+            if k in _MIN_METRICS:
+                merged.setdefault(k, float("inf"))
+                if v not in (float("inf"), float("-inf")):
+                    merged[k] = min(merged[k], v)
+            elif k in _MAX_METRICS:
+                merged.setdefault(k, float("-inf"))
+                if v not in (float("inf"), float("-inf")):
+                    merged[k] = max(merged[k], v)
+            else:
+                merged[k] = merged.get(k, 0) + v
+    return total, merged
+
+
 def nll_loss(next_token_logprobs, data, global_valid_toks):
     """``NLLLossFn`` scalar branch (``loss_functions.py:818-842``)."""
     mask = data["token_mask"][:, 1:] * data["sample_mask"].unsqueeze(-1)

@@ -4,8 +4,8 @@
 backward of the logprob op do (``nemo_rl/algorithms/loss/wrapper.py:292-322``), but the logits are
 read once and the gradient written once: the kernel keeps each row on chip between the
 log-sum-exp and the gradient and evaluates the token's loss terms in between.  The gradient exists
-as soon as the forward returns; ``backward`` hands it to autograd (scaled if the upstream gradient
-is not the ``loss_scale`` it was computed with).
+as soon as the forward returns; ``backward`` hands it to autograd, rescaled in place on the device when
+the upstream gradient is not the ``loss_scale`` it was computed with.
 """
 
 from __future__ import annotations
@@ -15,8 +15,9 @@ from typing import Any, Optional
 import torch
 
 from ... import ops as _ops  # noqa: F401
-from ..._lib import METRIC_SLOTS
-from .loss_functions import ClippedPGLossFn, _f32, _global_valid
+from ..._deferred import pending_temperature
+from ..._lib import NRL_TEMP_RCP
+from .loss_functions import ClippedPGLossFn, _f32, _global_valid, metrics_record_to_dict
 
 _OPS = torch.ops.rl_amd
 
@@ -54,59 +55,48 @@ def why_not_fusable(loss_fn, logits, data, sampling_params=None) -> Optional[str
     return None
 
 
-def _metrics_dict(metrics, loss_fn, sample_mask_in):
-    beta = loss_fn.reference_policy_kl_penalty
-    m = metrics.cpu().tolist()
-    get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
-    n_valid = get("num_valid_samples")
-    out = {
-        "loss": get("loss"),
-        "probs_ratio": get("probs_ratio"),
-        "probs_ratio_clamped": get("probs_ratio_clamped"),
-        "probs_ratio_min": get("probs_ratio_min"),
-        "probs_ratio_max": get("probs_ratio_max"),
-        "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
-        "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
-        "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
-        "token_mult_prob_error": get("token_mult_prob_error"),
-        "gen_kl_error": get("gen_kl_error"),
-        "policy_kl_error": get("policy_kl_error"),
-        "js_divergence_error": get("js_divergence_error"),
-        "sampling_importance_ratio": get("sampling_importance_ratio"),
-        "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
-        "approx_entropy": get("approx_entropy"),
-    }
-    if loss_fn.truncated_importance_sampling_ratio is not None:
-        out["is_oob_ratio"] = get("is_oob_ratio")
-    out["positive_nll_loss"] = get("positive_nll_loss")
-    return out
+def _rescale(dlogits, grad_loss, loss_scale):
+    """The stored gradient was computed for an upstream factor of ``loss_scale``.  Whatever factor autograd
+    actually delivers is applied in place by one kernel that reads it from the device: the host never waits
+    for its value, no second ``[B, S, V]`` tensor exists, and when the two agree (the normal case) the kernel
+    touches no memory."""
+    if not isinstance(grad_loss, torch.Tensor) or not grad_loss.is_cuda:
+        grad_loss = torch.as_tensor(grad_loss, dtype=torch.float32, device=dlogits.device)
+    view = dlogits if dlogits.dim() == 3 else dlogits.unsqueeze(0)
+    _OPS.scale_rows_(view, grad_loss, float(loss_scale))
+    return dlogits
+
+
+def _hand_over(ctx, grad_loss):
+    dlogits, ctx.dlogits = ctx.dlogits, None
+    if dlogits is None:
+        raise RuntimeError("the single-pass loss hands its gradient buffer to autograd once; a second backward "
+                           "through the same loss needs a new forward")
+    return _rescale(dlogits, grad_loss, ctx.loss_scale)
+
 
 class _FusedLogitsLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams,
-                loss_scale, in_place):
+                loss_scale, in_place, temperature):
         x = logits.detach()
         if in_place:
             loss, lp, metrics = _OPS.fused_logits_grpo_loss_(
-                x, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams, loss_scale)
+                x, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams, loss_scale,
+                temperature, NRL_TEMP_RCP)
             dlogits = x  # the caller declared the logits dead; their storage now holds the gradient
         else:
             loss, dlogits, lp, metrics = _OPS.fused_logits_grpo_loss(
-                x, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams, loss_scale)
-        ctx.save_for_backward(dlogits)
+                x, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags, fparams, loss_scale,
+                temperature, NRL_TEMP_RCP)
+        ctx.dlogits = dlogits  # an intermediate, neither input nor output: held directly so it can be rescaled in place
         ctx.loss_scale = loss_scale
         ctx.mark_non_differentiable(lp, metrics)
         return loss, lp, metrics
 
     @staticmethod
     def backward(ctx, grad_loss, _g_lp, _g_metrics):
-        (dlogits,) = ctx.saved_tensors
-        factor = float(grad_loss) / ctx.loss_scale
-        if factor != 1.0:
-            # the stored gradient was final for the announced loss_scale; any other upstream factor costs one
-            # more pass (computed in fp32 per element, no fp32 copy of the tensor)
-            dlogits = dlogits * factor
-        return (dlogits,) + (None,) * 13
+        return (_hand_over(ctx, grad_loss),) + (None,) * 14
 
 
 def fused_logits_clipped_pg_loss(
@@ -144,29 +134,26 @@ def fused_logits_clipped_pg_loss(
         logits, ids[:, 1:], n_inner, prev, _f32(data["generation_logprobs"][:, 1:], dev), ref,
         _f32(data["advantages"][:, 1:], dev), _f32(data["token_mask"][:, 1:], dev), _f32(sample_mask_in, dev),
         _global_valid(global_valid_seqs, global_valid_toks, dev), iflags, fparams, float(loss_scale), bool(in_place),
+        pending_temperature(logits),  # a divide apply_temperature_scaling left to this kernel
     )
-    return loss, _metrics_dict(metrics, loss_fn, sample_mask_in)
+    return loss, metrics_record_to_dict(metrics, loss_fn, sample_mask_in)
 
 
 class _FusedPackedLogitsLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits2d, targets, cu, unpacked_seqlen, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags,
-                fparams, loss_scale):
+                fparams, loss_scale, temperature):
         loss, dlogits, lp, metrics = _OPS.fused_packed_logits_grpo_loss(
             logits2d.detach(), targets, True, cu, unpacked_seqlen, prev, gen, ref, adv, token_mask, sample_mask, global_valid,
-            iflags, fparams, loss_scale)
-        ctx.save_for_backward(dlogits)
+            iflags, fparams, loss_scale, temperature, NRL_TEMP_RCP)
+        ctx.dlogits = dlogits  # an intermediate, neither input nor output: held directly so it can be rescaled in place
         ctx.loss_scale = loss_scale
         ctx.mark_non_differentiable(lp, metrics)
         return loss, lp, metrics
 
     @staticmethod
     def backward(ctx, grad_loss, _g_lp, _g_metrics):
-        (dlogits,) = ctx.saved_tensors
-        factor = float(grad_loss) / ctx.loss_scale
-        if factor != 1.0:
-            dlogits = dlogits * factor
-        return (dlogits,) + (None,) * 13
+        return (_hand_over(ctx, grad_loss),) + (None,) * 14
 
 
 def why_not_fusable_packed(loss_fn, logits, data, sampling_params=None) -> Optional[str]:
@@ -205,5 +192,6 @@ def fused_packed_logits_clipped_pg_loss(logits, data, loss_fn, cu_seqlens_q, cu_
         _f32(data["generation_logprobs"][:, 1:], dev), ref, _f32(data["advantages"][:, 1:], dev),
         _f32(data["token_mask"][:, 1:], dev), _f32(sample_mask_in, dev),
         _global_valid(global_valid_seqs, global_valid_toks, dev), iflags, fparams, float(loss_scale),
+        pending_temperature(logits),
     )
-    return loss, _metrics_dict(metrics, loss_fn, sample_mask_in)
+    return loss, metrics_record_to_dict(metrics, loss_fn, sample_mask_in)

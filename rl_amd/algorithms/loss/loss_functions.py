@@ -68,6 +68,36 @@ def _global_valid(seqs, toks, dev) -> torch.Tensor:
     return torch.stack(parts)
 
 
+def metrics_record_to_dict(metrics: torch.Tensor, loss_fn, sample_mask_in: torch.Tensor) -> dict:
+    """The kernels' metrics record -> the dictionary ``ClippedPGLossFn`` returns (``loss_functions.py:767-788``);
+    fetching the record is the one device -> host synchronisation of a loss call."""
+    beta = loss_fn.reference_policy_kl_penalty
+    m = metrics.cpu().tolist()
+    get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
+    n_valid = get("num_valid_samples")
+    out = {
+        "loss": get("loss"),
+        "probs_ratio": get("probs_ratio"),
+        "probs_ratio_clamped": get("probs_ratio_clamped"),
+        "probs_ratio_min": get("probs_ratio_min"),
+        "probs_ratio_max": get("probs_ratio_max"),
+        "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
+        "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
+        "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
+        "token_mult_prob_error": get("token_mult_prob_error"),
+        "gen_kl_error": get("gen_kl_error"),
+        "policy_kl_error": get("policy_kl_error"),
+        "js_divergence_error": get("js_divergence_error"),
+        "sampling_importance_ratio": get("sampling_importance_ratio"),
+        "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
+        "approx_entropy": get("approx_entropy"),
+    }
+    if loss_fn.truncated_importance_sampling_ratio is not None:
+        out["is_oob_ratio"] = get("is_oob_ratio")
+    out["positive_nll_loss"] = get("positive_nll_loss")
+    return out
+
+
 class _FusedLoss(torch.autograd.Function):
     """loss, metrics = kernel(lp, lpu, ...); the kernel also returns d loss / d lp (and / d lpu), so the
     backward is a scalar multiply."""
@@ -244,30 +274,7 @@ class ClippedPGLossFn(LossFunction):
         )
         if home != dev:
             loss = loss.to(home)
-        m = metrics.cpu().tolist()  # the one synchronisation of the call
-        get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
-        n_valid = get("num_valid_samples")
-        out = {
-            "loss": get("loss"),
-            "probs_ratio": get("probs_ratio"),
-            "probs_ratio_clamped": get("probs_ratio_clamped"),
-            "probs_ratio_min": get("probs_ratio_min"),
-            "probs_ratio_max": get("probs_ratio_max"),
-            "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
-            "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
-            "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
-            "token_mult_prob_error": get("token_mult_prob_error"),
-            "gen_kl_error": get("gen_kl_error"),
-            "policy_kl_error": get("policy_kl_error"),
-            "js_divergence_error": get("js_divergence_error"),
-            "sampling_importance_ratio": get("sampling_importance_ratio"),
-            "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
-            "approx_entropy": get("approx_entropy"),
-        }
-        if self.truncated_importance_sampling_ratio is not None:
-            out["is_oob_ratio"] = get("is_oob_ratio")
-        out["positive_nll_loss"] = get("positive_nll_loss")
-        return loss, out
+        return loss, metrics_record_to_dict(metrics, self, sample_mask_in)
 
 
 class _FusedNll(torch.autograd.Function):

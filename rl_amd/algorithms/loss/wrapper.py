@@ -3,6 +3,7 @@
 
 from __future__ import annotations
 
+import functools
 import math
 from typing import Any, Callable, Optional
 
@@ -12,6 +13,20 @@ from .interfaces import LossFunction
 
 _MIN_KEYS = {"probs_ratio_min", "probs_ratio_clamped_min"}
 _MAX_KEYS = {"probs_ratio_max", "probs_ratio_clamped_max"}
+
+
+def _bound_keywords(prepare_fn, base, allowed) -> Optional[dict]:
+    """The workers never pass ``prepare_loss_input`` bare: they bind ``sampling_params`` / ``d2t`` /
+    ``chunk_size`` with ``functools.partial`` first (``models/megatron/train.py:506-533``,
+    ``models/automodel/train.py:624-627``).  Returns the bound keywords when ``prepare_fn`` is ``base`` itself
+    or such a partial of it (keywords from ``allowed`` only, no positional arguments), else ``None``."""
+    if prepare_fn is base:
+        return {}
+    if isinstance(prepare_fn, functools.partial) and prepare_fn.func is base and not prepare_fn.args:
+        kw = dict(prepare_fn.keywords)
+        if set(kw) <= set(allowed):
+            return kw
+    return None
 
 
 def _slice_row(data, idx: int):
@@ -95,9 +110,10 @@ class SequencePackingFusionLossWrapper:
 
         # a ClippedPGLossFn whose token gradient needs no other token's logprob: logits -> loss -> gradient
         # in one pass over the packed row, as in wrap_loss_fn_with_input_preparation
-        if (self.prepare_fn is prepare_packed_loss_input and torch.is_grad_enabled()
+        bound = _bound_keywords(self.prepare_fn, prepare_packed_loss_input, ("sampling_params", "chunk_size"))
+        if (bound is not None and torch.is_grad_enabled()
                 and isinstance(next_token_logits, torch.Tensor) and next_token_logits.requires_grad
-                and why_not_fusable_packed(self.loss_fn, next_token_logits, data) is None):
+                and why_not_fusable_packed(self.loss_fn, next_token_logits, data, bound.get("sampling_params")) is None):
             from ...distributed.model_utils import _group_size
 
             if _group_size(self.vocab_parallel_group) == 1 and _group_size(self.context_parallel_group) == 1:
@@ -125,8 +141,12 @@ def wrap_loss_fn_with_input_preparation(next_token_logits, data, global_valid_se
     from .fused import fused_logits_clipped_pg_loss, why_not_fusable
     from .utils import prepare_loss_input
 
-    if (prepare_fn is prepare_loss_input and torch.is_grad_enabled() and isinstance(next_token_logits, torch.Tensor)
-            and next_token_logits.requires_grad and why_not_fusable(loss_fn, next_token_logits, data) is None):
+    # chunk_size only bounds the reference's working set and d2t belongs to the draft-model loss: neither changes
+    # what the single pass computes, top-k / top-p filtering (checked by why_not_fusable) does
+    bound = _bound_keywords(prepare_fn, prepare_loss_input, ("sampling_params", "d2t", "chunk_size"))
+    if (bound is not None and bound.get("d2t") is None and torch.is_grad_enabled()
+            and isinstance(next_token_logits, torch.Tensor) and next_token_logits.requires_grad
+            and why_not_fusable(loss_fn, next_token_logits, data, bound.get("sampling_params")) is None):
         from ...distributed.model_utils import _group_size
 
         if _group_size(vocab_parallel_group) == 1 and _group_size(context_parallel_group) == 1:

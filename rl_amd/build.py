@@ -40,7 +40,7 @@ def build(verbose: bool = True) -> str:
     for src in sources():
         obj = os.path.join(LIB_DIR, os.path.basename(src)[:-4] + ".o")
         objs.append(obj)
-        cmd = [hipcc, *HIPCC_FLAGS, *os.environ.get("NRL_EXTRA_HIPCC_FLAGS", "").split(), "-c", src, "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

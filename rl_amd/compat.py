@@ -3,7 +3,8 @@
 ``install()`` either registers ``nemo_rl.distributed.model_utils``, ``nemo_rl.algorithms.loss`` (and
 its sub-modules), ``nemo_rl.algorithms.loss_functions``, ``nemo_rl.algorithms.utils``,
 ``nemo_rl.algorithms.logits_sampling_utils``, ``nemo_rl.algorithms.advantage_estimator`` and
-``nemo_rl.models.automodel.train`` / ``nemo_rl.models.megatron.train`` (their ``LogprobsPostProcessor``) as
+``nemo_rl.models.automodel.train`` / ``nemo_rl.models.megatron.train`` (their post-processors and
+``apply_temperature_scaling``) as
 aliases of the ``rl_amd`` modules (when NeMo-RL is not importable), or replaces the hot-path
 attributes of an existing NeMo-RL install in place.
 """
@@ -43,13 +44,14 @@ _PATCHED = {
         "_compute_distributed_log_softmax", "_compute_distributed_log_softmax_with_grad",
     ],
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
-    "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation"],
+    "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation", "SequencePackingLossWrapper",
+                                        "SequencePackingFusionLossWrapper"],
     "nemo_rl.algorithms.loss.utils": ["prepare_loss_input", "prepare_packed_loss_input"],
     "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn",
                                                "DraftCrossEntropyLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
-    "nemo_rl.models.automodel.train": ["LogprobsPostProcessor"],
-    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor"],
+    "nemo_rl.models.automodel.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling"],
+    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor", "apply_temperature_scaling"],
     "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking", "dynamic_sampling"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }

@@ -18,11 +18,6 @@
 #include <mutex>
 
 #include "common.hpp"
-#ifdef NRL_NT_ZERO
-#define NRL_ZERO_STORE(v, p) __builtin_nontemporal_store(v, p)
-#else
-#define NRL_ZERO_STORE(v, p) (*(p) = (v))
-#endif
 #include "grpo_token.hpp"
 
 namespace nrl {
@@ -433,7 +428,7 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
             if (i < a.n_inner) w = in.token_mask[o * in.token_mask_stride + i] * in.sample_mask[o];
             if (w != 0.f) break;
             u32x4* ov = reinterpret_cast<u32x4*>(out_row(r));
-            for (int v = tid; v < nvec; v += kFusedBlock) NRL_ZERO_STORE(zero, ov + v);
+            for (int v = tid; v < nvec; v += kFusedBlock) ov[v] = zero;
             if (i < a.n_inner) {
                 const int64_t tok = o * a.n_inner + i;
                 if (tid < T_COUNT) a.terms[tok * T_COUNT + tid] = 0.f;

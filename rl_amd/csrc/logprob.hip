@@ -14,44 +14,17 @@
 #include <float.h>
 
 #include "common.hpp"
-#ifdef NRL_NT_ZERO
-#define NRL_ZERO_STORE(v, p) __builtin_nontemporal_store(v, p)
-#else
-#define NRL_ZERO_STORE(v, p) (*(p) = (v))
-#endif
 
 namespace nrl {
 
-#ifndef NRL_ROW_BLOCK
-#define NRL_ROW_BLOCK 256
-#endif
-#ifndef NRL_ROW_UNROLL
-#define NRL_ROW_UNROLL 4
-#endif
-#ifndef NRL_K2_NT_STORE
-#define NRL_K2_NT_STORE 1
-#endif
-#ifndef NRL_K2_NT_LOAD
-#define NRL_K2_NT_LOAD 1
-#endif
-constexpr int kBlock = NRL_ROW_BLOCK;
+constexpr int kBlock = 256;  // one workgroup of 4 wave64 per row
 constexpr int kWaves = kBlock / kWave;
-constexpr int kUnroll = NRL_ROW_UNROLL;
+constexpr int kUnroll = 4;   // 16-byte loads in flight per lane
 
-template <typename P> __device__ __forceinline__ u32x4 k2_load(const P* p) {
-#if NRL_K2_NT_LOAD
-    return __builtin_nontemporal_load(p);
-#else
-    return *p;
-#endif
-}
-template <typename P> __device__ __forceinline__ void k2_store(u32x4 v, P* p) {
-#if NRL_K2_NT_STORE
-    __builtin_nontemporal_store(v, p);
-#else
-    *p = v;
-#endif
-}
+// rows that are read and written in the same pass stream through non-temporal loads and stores; rows
+// that are only written (zero gradients) use plain stores, which a pure write stream sustains faster
+template <typename P> __device__ __forceinline__ u32x4 k2_load(const P* p) { return __builtin_nontemporal_load(p); }
+template <typename P> __device__ __forceinline__ void k2_store(u32x4 v, P* p) { __builtin_nontemporal_store(v, p); }
 
 // number of leading elements before the first 16-byte boundary of a row
 template <int DT> __device__ __forceinline__ int64_t row_head(const void* row, int64_t vocab) {
@@ -110,7 +83,7 @@ template <int DT> __device__ __forceinline__ void row_zero(void* row, int64_t vo
     const int64_t nvec = (vocab - head) / EPV;
     u32x4* ov = reinterpret_cast<u32x4*>(static_cast<char*>(row) + head * Row<DT>::BYTES);
     const u32x4 z = {0u, 0u, 0u, 0u};
-    for (int64_t i = tid; i < nvec; i += kBlock) NRL_ZERO_STORE(z, ov + i);
+    for (int64_t i = tid; i < nvec; i += kBlock) ov[i] = z;
     if (tid < head) Row<DT>::store1(row, tid, 0.f);
     const int64_t tail0 = head + nvec * EPV;
     if (tail0 + tid < vocab) Row<DT>::store1(row, tail0 + tid, 0.f);
@@ -406,6 +379,26 @@ __device__ __forceinline__ void row_apply(const void* in, const void* in2, void*
         Row<DT>::store1(out, tail0 + tid, f(Row<DT>::load1(in, tail0 + tid), TWO ? Row<DT>::load1(in2, tail0 + tid) : 0.f));
 }
 
+// sum of one row's elements (fp32 partials per lane, fixed-order workgroup reduction), 16-byte vectors
+template <int DT> __device__ __forceinline__ float row_sum(const void* row, int64_t vocab, float* smem) {
+    constexpr int EPV = Row<DT>::EPV;
+    const int tid = threadIdx.x;
+    const int64_t head = row_head<DT>(row, vocab);
+    const int64_t nvec = (vocab - head) / EPV;
+    const u32x4* xv = reinterpret_cast<const u32x4*>(static_cast<const char*>(row) + head * Row<DT>::BYTES);
+    float part = 0.f;
+    for (int64_t i = tid; i < nvec; i += kBlock) {
+        float t[EPV];
+        Row<DT>::decode(xv[i], t);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) part += t[k];
+    }
+    if (tid < head) part += Row<DT>::load1(row, tid);
+    const int64_t tail0 = head + nvec * EPV;
+    if (tail0 + tid < vocab) part += Row<DT>::load1(row, tail0 + tid);
+    return block_sum<float, kWaves>(part, smem);
+}
+
 template <int DT>
 __global__ __launch_bounds__(kBlock) void log_softmax_fwd_kernel(const void* __restrict__ logits, int64_t vocab, int64_t row_stride,
                                                                  void* __restrict__ out, int64_t out_stride) {
@@ -427,10 +420,24 @@ __global__ __launch_bounds__(kBlock) void log_softmax_bwd_kernel(const void* __r
     const char* y = static_cast<const char*>(logprobs) + r * lp_stride * Row<DT>::BYTES;
     const char* g = static_cast<const char*>(grad) + r * g_stride * Row<DT>::BYTES;
     char* d = static_cast<char*>(dx) + r * dx_stride * Row<DT>::BYTES;
-    float part = 0.f;
-    for (int64_t i = threadIdx.x; i < vocab; i += kBlock) part += Row<DT>::load1(g, i);
-    const float sum_g = block_sum<float, kWaves>(part, smem);
+    const float sum_g = row_sum<DT>(g, vocab, smem);
     row_apply<DT, true>(g, y, d, vocab, [&](float gv, float yv) { return gv - fast_exp2(yv * kLog2e) * sum_g; });
+}
+
+// dst = src * (factor[0] / divisor) over strided rows (dst may be src): fp32 product, one narrowing to the
+// rows' dtype.  The factor lives on the device so that the host never waits for it; when dst is src and the
+// quotient is exactly 1 every workgroup leaves after reading it and no row is touched.
+template <int DT>
+__global__ __launch_bounds__(kBlock) void scale_rows_kernel(const void* src, void* dst, int64_t n_inner, int64_t vocab,
+                                                            int64_t src_outer, int64_t src_inner, int64_t dst_outer,
+                                                            int64_t dst_inner, const float* __restrict__ factor, float divisor) {
+    const float f = factor[0] / divisor;
+    if (f == 1.f && src == dst) return;
+    const int64_t r = blockIdx.x;
+    const int64_t o = r / n_inner, i = r - o * n_inner;
+    const char* in = static_cast<const char*>(src) + (o * src_outer + i * src_inner) * Row<DT>::BYTES;
+    char* out = static_cast<char*>(dst) + (o * dst_outer + i * dst_inner) * Row<DT>::BYTES;
+    row_apply<DT, false>(in, nullptr, out, vocab, [&](float x, float) { return x * f; });
 }
 
 #define NRL_DISPATCH(DT_, TC_, ...)                                                         \
@@ -590,4 +597,21 @@ extern "C" int nrl_log_softmax_bwd(const void* logprobs, int32_t dtype, int64_t 
     NRL_DISPATCH(dtype, 0, (void)TEMP; log_softmax_bwd_kernel<DT><<<dim3((unsigned)n_rows), dim3(kBlock), 0, s>>>(logprobs, vocab, lp_row_stride, grad,
                                                                                                    grad_row_stride, dx, dx_row_stride));
     return check_launch("log_softmax_bwd");
+}
+
+extern "C" int nrl_scale_rows(const void* src, void* dst, int32_t dtype, int64_t n_outer, int64_t n_inner, int64_t vocab,
+                              int64_t src_stride_outer, int64_t src_stride_inner, int64_t dst_stride_outer,
+                              int64_t dst_stride_inner, const float* factor, float divisor, void* stream) {
+    if (dtype != NRL_F32 && dtype != NRL_BF16 && dtype != NRL_F16) return fail(NRL_E_INVALID, "unknown dtype %d", dtype);
+    if (n_outer < 0 || n_inner < 0 || vocab <= 0) return fail(NRL_E_INVALID, "bad shape");
+    if (!(divisor != 0.f)) return fail(NRL_E_INVALID, "divisor must not be zero");
+    const int64_t n = n_outer * n_inner;
+    if (n == 0) return NRL_OK;
+    if (!src || !dst || !factor) return fail(NRL_E_INVALID, "null src, dst or factor");
+    if (n >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    NRL_DISPATCH(dtype, 0, (void)TEMP; scale_rows_kernel<DT><<<dim3((unsigned)n), dim3(kBlock), 0, s>>>(
+                                 src, dst, n_inner, vocab, src_stride_outer, src_stride_inner, dst_stride_outer,
+                                 dst_stride_inner, factor, divisor));
+    return check_launch("scale_rows");
 }

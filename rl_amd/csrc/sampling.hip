@@ -34,15 +34,9 @@ namespace nrl {
 constexpr int kSelBlock = 256;
 constexpr int kSelWaves = kSelBlock / kWave;
 constexpr int kMassBins = 64;
-#ifndef NRL_LOOSE_HITS
-#define NRL_LOOSE_HITS 768
-#endif
-constexpr int kLooseHits = NRL_LOOSE_HITS;  // top-p alone: more hit chunks than this under the chunk maxima's bound -> bound from the row
+constexpr int kLooseHits = 768;  // top-p alone: more hit chunks than this under the chunk maxima's bound -> bound from the row
 constexpr int kMassCopies = 8;  // copies of the histogram, by lane: most elements fall into the few lowest bins
-#ifndef NRL_WIDE_GRID
-#define NRL_WIDE_GRID 2048
-#endif
-constexpr int kWideGrid = NRL_WIDE_GRID;
+constexpr int kWideGrid = 2048;  // workgroups of the threshold-search kernel (more in flight measured faster than fewer)
 constexpr int32_t kTieUnresolved = -1;  // tie[] marker: the row's kept set did not fit the candidate list
 constexpr int kSub = 8;                      // chunk maxima per thread
 constexpr int kChunks = kSelBlock * kSub;    // 2048

@@ -16,6 +16,7 @@ from typing import Any, Optional
 import torch
 
 from .. import ops as _ops  # noqa: F401  (registers torch.ops.rl_amd.*)
+from .._deferred import pending_temperature, refuse_pending
 from .._lib import NRL_TEMP_RCP
 from ..algorithms.logits_sampling_utils import (
     TrainingSamplingParams,
@@ -57,6 +58,8 @@ def _prep_rows(logits, targets):
 def _fwd_rows(ctx, logits, targets, n_inner, vocab_start, vocab_end, inference_only, temperature):
     """Shared forward: saves the logits (no copy), the targets and one fp32 log-sum-exp per row;
     the softmax is never materialised."""
+    if temperature == 1.0:
+        temperature = pending_temperature(logits)  # a divide apply_temperature_scaling left to this kernel
     logits, targets = _prep_rows(logits.detach(), targets)
     save = (not inference_only) and ctx.needs_input_grad[0]
     out, lse = _OPS.logprob_fwd(logits, targets, n_inner, vocab_start, vocab_end, temperature, NRL_TEMP_RCP, save)
@@ -96,6 +99,7 @@ def _rows_logprob(logits, targets, n_inner, vocab_start, vocab_end, inference_on
 class _LogSoftmaxRows(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits):
+        refuse_pending(logits, "_compute_distributed_log_softmax")
         x = logits.detach()
         x2 = x.reshape(-1, x.shape[-1])
         if x2.stride(-1) != 1:
@@ -227,14 +231,14 @@ def from_parallel_logits_to_logprobs(
     b, s = target.shape
     if vocab_parallel_logits.shape[1] < s:
         raise ValueError(f"logits cover {vocab_parallel_logits.shape[1]} positions, targets {s}")
+    if s - 1 <= 0:  # nothing to predict (a one-token or empty sequence): torch's gather returns an empty result
+        return torch.zeros((b, 0), dtype=torch.float32, device=vocab_parallel_logits.device)
     if need_top_k_or_top_p_filtering(sampling_params):
         from .sampling_logprob import rows_logprob_sampled
 
         return rows_logprob_sampled(
             vocab_parallel_logits, target[:, 1:], s - 1, sampling_params.top_k, sampling_params.top_p, inference_only
         )
-    if s - 1 == 0:
-        return torch.zeros((b, 0), dtype=torch.float32, device=vocab_parallel_logits.device)
     return _rows_logprob(
         vocab_parallel_logits, target[:, 1:], s - 1, vocab_start_index, vocab_end_index, inference_only
     )
@@ -341,15 +345,16 @@ def get_logprobs_from_vocab_parallel_logits(
 # ------------------------------------------------------------------------------------------------
 class _PackedLogprob(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, inference_only):
+    def forward(ctx, logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, inference_only,
+                temperature):
         save = (not inference_only) and ctx.needs_input_grad[0]
         out, lse = _OPS.logprob_packed_fwd(
-            logits2d.detach(), targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, 1.0,
+            logits2d.detach(), targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, temperature,
             NRL_TEMP_RCP, save,
         )
         if save:
             ctx.save_for_backward(logits2d.detach(), targets1d, cu_dev, lse)
-            ctx.meta = (pre_rolled, unpacked_seqlen, vocab_start, vocab_end)
+            ctx.meta = (pre_rolled, unpacked_seqlen, vocab_start, vocab_end, temperature)
         ctx.saved = save
         return out
 
@@ -358,12 +363,12 @@ class _PackedLogprob(torch.autograd.Function):
         if not ctx.saved:
             raise RuntimeError("backward through a logprob computed with inference_only=True")
         logits2d, targets1d, cu_dev, lse = ctx.saved_tensors
-        pre_rolled, unpacked_seqlen, vocab_start, vocab_end = ctx.meta
+        pre_rolled, unpacked_seqlen, vocab_start, vocab_end, temperature = ctx.meta
         d = _OPS.logprob_packed_bwd(
-            logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, 1.0, NRL_TEMP_RCP,
+            logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, vocab_start, vocab_end, temperature, NRL_TEMP_RCP,
             lse, grad_out.float(),
         )
-        return d, None, None, None, None, None, None, None
+        return d, None, None, None, None, None, None, None, None
 
 
 def _checked_cu_seqlens(cu_seqlens_padded: torch.Tensor, total: int, n_targets: int, device) -> torch.Tensor:
@@ -405,6 +410,7 @@ def from_parallel_logits_to_logprobs_packed_sequences(
     _require_single_rank(cp_group, "from_parallel_logits_to_logprobs_packed_sequences")
     if vocab_parallel_logits.dim() != 3 or vocab_parallel_logits.shape[0] != 1:
         raise ValueError(f"expected packed logits [1, T, V], got {tuple(vocab_parallel_logits.shape)}")
+    temperature = pending_temperature(vocab_parallel_logits)  # a divide apply_temperature_scaling left to the kernel
     logits2d = vocab_parallel_logits.squeeze(0)
     if logits2d.stride(-1) != 1:
         logits2d = logits2d.contiguous()
@@ -416,11 +422,11 @@ def from_parallel_logits_to_logprobs_packed_sequences(
 
         return packed_logprob_sampled(
             logits2d, targets1d, target_is_pre_rolled, cu_dev, int(unpacked_seqlen), sampling_params.top_k,
-            sampling_params.top_p, inference_only,
+            sampling_params.top_p, inference_only, temperature,
         )
     return _PackedLogprob.apply(
         logits2d, targets1d, bool(target_is_pre_rolled), cu_dev, int(unpacked_seqlen), vocab_start_index,
-        vocab_end_index, inference_only,
+        vocab_end_index, inference_only, temperature,
     )
 
 

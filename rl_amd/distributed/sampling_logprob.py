@@ -8,6 +8,7 @@ from __future__ import annotations
 import torch
 
 from .. import ops as _ops  # noqa: F401
+from .._deferred import pending_temperature, refuse_pending
 from .._lib import NRL_TEMP_RCP
 
 _OPS = torch.ops.rl_amd
@@ -20,9 +21,11 @@ def _norm_p(top_p) -> float:
     return float(top_p) if top_p is not None else 1.0
 
 
-def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, want_unfiltered=False):
+def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, want_unfiltered=False, temperature=1.0):
     """Shared forward of the filtered-logprob autograd functions: saves the logits (no copy), the targets
     and three numbers per row (threshold, tie index, kept log-sum-exp)."""
+    if temperature == 1.0:
+        temperature = pending_temperature(logits)  # a divide apply_temperature_scaling left to this kernel
     logits = logits.detach()
     if logits.dim() != 3:
         raise ValueError(f"expected logits [B, S, V], got {tuple(logits.shape)}")
@@ -32,12 +35,13 @@ def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, wa
     if targets.dtype != torch.int64:
         targets = targets.long()
     lp, thr, tie, lse, lpu = _OPS.topk_topp_logprob_fwd(
-        logits, targets, n_inner, _norm_k(top_k), _norm_p(top_p), 1.0, NRL_TEMP_RCP, want_unfiltered
+        logits, targets, n_inner, _norm_k(top_k), _norm_p(top_p), temperature, NRL_TEMP_RCP, want_unfiltered
     )
     ctx.saved = (not inference_only) and ctx.needs_input_grad[0]
     if ctx.saved:
         ctx.save_for_backward(logits, targets, thr, tie, lse)
         ctx.n_inner = n_inner
+        ctx.temperature = temperature
     return (lp, lpu) if want_unfiltered else lp
 
 
@@ -46,27 +50,28 @@ def _sampled_bwd(ctx, grad_lp):
         raise RuntimeError("backward through a logprob computed with inference_only=True")
     logits, targets, thr, tie, lse = ctx.saved_tensors
     return _OPS.topk_topp_logprob_bwd(
-        logits, targets, thr, tie, lse, grad_lp.float().contiguous(), ctx.n_inner, 1.0, NRL_TEMP_RCP
+        logits, targets, thr, tie, lse, grad_lp.float().contiguous(), ctx.n_inner, ctx.temperature, NRL_TEMP_RCP
     )
 
 
 class _RowsLogprobSampled(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, logits, targets, n_inner, top_k, top_p, inference_only):
-        return _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only)
+    def forward(ctx, logits, targets, n_inner, top_k, top_p, inference_only, temperature):
+        return _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, temperature=temperature)
 
     @staticmethod
     def backward(ctx, grad_lp):
-        return _sampled_bwd(ctx, grad_lp), None, None, None, None, None
+        return _sampled_bwd(ctx, grad_lp), None, None, None, None, None, None
 
 
-def rows_logprob_sampled(logits, targets, n_inner, top_k, top_p, inference_only=False):
+def rows_logprob_sampled(logits, targets, n_inner, top_k, top_p, inference_only=False, temperature=1.0):
     """logits [B,S,V], targets [B,>=n_inner] aligned with the rows -> fp32 [B,n_inner]; a target outside
     the kept set gives ``-inf`` (``model_utils.py:445-452``)."""
-    return _RowsLogprobSampled.apply(logits, targets, n_inner, top_k, top_p, inference_only)
+    return _RowsLogprobSampled.apply(logits, targets, n_inner, top_k, top_p, inference_only, float(temperature))
 
 
-def packed_logprob_sampled(logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, top_k, top_p, inference_only):
+def packed_logprob_sampled(logits2d, targets1d, pre_rolled, cu_dev, unpacked_seqlen, top_k, top_p, inference_only,
+                           temperature=1.0):
     """Packed ``[T, V]`` logits under filtering -> unpacked ``[n_seq, unpacked_seqlen-1]``.  Every packed
     position is one row of the selection kernel; the per-sequence roll and the unpacking are index
     tensors built from ``cu_seqlens`` (sizes ``[T]`` and ``[n_seq, L]``)."""
@@ -85,7 +90,8 @@ def packed_logprob_sampled(logits2d, targets1d, pre_rolled, cu_dev, unpacked_seq
     else:
         tgt_idx = torch.where(pos + 1 < stop, pos + 1, start)
     tgt = torch.where(inside, targets1d[tgt_idx.clamp(max=targets1d.shape[0] - 1)], torch.zeros_like(pos))
-    lp_flat = rows_logprob_sampled(logits2d.unsqueeze(0), tgt.unsqueeze(0), total, top_k, top_p, inference_only)[0]
+    lp_flat = rows_logprob_sampled(logits2d.unsqueeze(0), tgt.unsqueeze(0), total, top_k, top_p, inference_only,
+                                   temperature)[0]
     # out[s, p] = lp_flat[cu[s] + p] for p < min(len_s - 1, width)
     p = torch.arange(width, device=dev).unsqueeze(0)
     lens = (cu[1:] - cu[:-1]).unsqueeze(-1)
@@ -115,6 +121,7 @@ class _FilterLogits(torch.autograd.Function):
 def filter_logits(logits, top_k, top_p):
     """``apply_top_k_top_p``: filtered logits (``-inf`` outside the kept set) and the boolean keep mask, same
     shape as ``logits``; gradients pass through where kept."""
+    refuse_pending(logits, "apply_top_k_top_p")
     shape = logits.shape
     x = logits.reshape(1, -1, shape[-1]) if logits.dim() != 3 else logits
     if x.stride(-1) != 1:

@@ -16,10 +16,57 @@ import torch
 
 from .. import _need_single_gpu
 from ... import ops  # noqa: F401  (registers torch.ops.rl_amd)
+from ..._deferred import pending_temperature
 from ..._lib import NRL_TEMP_RCP
 from ...algorithms.logits_sampling_utils import TrainingSamplingParams, need_top_k_or_top_p_filtering
 from ...algorithms.loss.utils import mask_out_neg_inf_logprobs
 from ...distributed import model_utils as MU
+from ...temperature import apply_temperature_scaling, deferred_temperature  # noqa: F401
+
+
+class LossPostProcessor:
+    """``LossPostProcessor`` of the DTensor worker (``nemo_rl/models/automodel/train.py:540-653``): logits of one
+    microbatch -> ``(loss, metrics)``.  Same constructor and call signature as the reference class.
+
+    The reference prepares the loss input and calls the loss as two steps; here the unpacked case goes through
+    ``wrap_loss_fn_with_input_preparation``, which does the same two steps unless the loss is a
+    ``ClippedPGLossFn`` the single pass covers - then logits -> loss -> gradient is one kernel.  Packed
+    microbatches take ``SequencePackingLossWrapper`` with the unpadded boundaries for both arguments, as the
+    reference does."""
+
+    def __init__(self, loss_fn: Any, cfg: Any, device_mesh: Any, cp_mesh: Any, tp_mesh: Any, cp_size: int, dp_size: int,
+                 enable_seq_packing: bool = False, sampling_params: Optional[TrainingSamplingParams] = None):
+        self.loss_fn = loss_fn
+        self.cfg = cfg
+        self.device_mesh = device_mesh
+        self.cp_mesh = cp_mesh
+        self.tp_mesh = tp_mesh
+        self.cp_size = cp_size
+        self.dp_size = dp_size
+        self.enable_seq_packing = enable_seq_packing
+        self.sampling_params = sampling_params
+        _need_single_gpu(cp_size, "LossPostProcessor")
+
+    def __call__(self, logits: torch.Tensor, data_dict: Any, processed_inputs: Any, global_valid_seqs: torch.Tensor,
+                 global_valid_toks: torch.Tensor, sequence_dim: int = 1):
+        from functools import partial
+
+        from ...algorithms.loss import (
+            SequencePackingLossWrapper,
+            prepare_loss_input,
+            wrap_loss_fn_with_input_preparation,
+        )
+
+        if type(logits).__name__ == "DTensor":
+            raise NotImplementedError("LossPostProcessor: vocabulary-parallel (DTensor) logits need more than one GPU")
+        prepare = partial(prepare_loss_input, sampling_params=self.sampling_params)
+        if self.enable_seq_packing:
+            cu = processed_inputs.flash_attn_kwargs.cu_seqlens_q
+            wrapped = SequencePackingLossWrapper(loss_fn=self.loss_fn, prepare_fn=prepare, cu_seqlens_q=cu,
+                                                 cu_seqlens_q_padded=cu)
+            return wrapped(logits, data_dict, global_valid_seqs, global_valid_toks)
+        return wrap_loss_fn_with_input_preparation(logits, data_dict, global_valid_seqs, global_valid_toks, self.loss_fn,
+                                                   prepare)
 
 
 class LogprobsPostProcessor:
@@ -72,9 +119,10 @@ class LogprobsPostProcessor:
                 token_logprobs = token_logprobs * (torch.arange(seq_len, device=lp.device)[None, :] < lengths)
             else:
                 lengths = torch.as_tensor(data_dict["input_lengths"]).to(device=logits.device, dtype=torch.int64).contiguous()
+                temperature = pending_temperature(logits)  # a divide apply_temperature_scaling left to this kernel
                 x = logits if logits.stride(-1) == 1 else logits.contiguous()
                 token_logprobs = torch.ops.rl_amd.logprob_post_fwd(
-                    x, input_ids[:, 1:], lengths, input_ids.shape[1] - 1, 0, x.shape[-1], 1.0, NRL_TEMP_RCP)
+                    x, input_ids[:, 1:], lengths, input_ids.shape[1] - 1, 0, x.shape[-1], temperature, NRL_TEMP_RCP)
         if filtering:  # ``train.py:799-804``
             mask = data_dict["token_mask"] * data_dict["sample_mask"].unsqueeze(-1)
             token_logprobs = mask_out_neg_inf_logprobs(token_logprobs, mask.to(token_logprobs.device), "prev_logprobs")

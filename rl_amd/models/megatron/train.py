@@ -16,10 +16,82 @@ from typing import Any, Callable, Dict, Optional, Tuple
 import torch
 
 from ... import ops  # noqa: F401  (registers torch.ops.rl_amd)
+from ..._deferred import pending_temperature
 from ..._lib import NRL_TEMP_RCP
 from ...algorithms.logits_sampling_utils import TrainingSamplingParams, need_top_k_or_top_p_filtering
 from ...algorithms.loss.utils import mask_out_neg_inf_logprobs
 from ...distributed import model_utils as MU
+from ...temperature import apply_temperature_scaling, deferred_temperature  # noqa: F401
+
+
+class LossPostProcessor:
+    """``LossPostProcessor`` of the Megatron worker (``nemo_rl/models/megatron/train.py:442-597``) for one GPU
+    (tensor- and context-parallel size 1, so no ``megatron.core`` state is consulted): ``__call__`` returns the
+    function the forward step applies to the model's output tensor, ``output -> (loss, metrics)``.
+
+    ``prepare_loss_input`` is bound to ``sampling_params`` / ``d2t`` / ``chunk_size`` with ``functools.partial``
+    exactly as the reference binds it, so the wrappers below see what a real worker hands them; a
+    ``ClippedPGLossFn`` the single pass covers then runs logits -> loss -> gradient as one kernel.  The loss is
+    multiplied by ``num_microbatches`` (``:583-594``, undoing the schedule's averaging); the gradient the single
+    pass has already written is rescaled on the device by whatever factor autograd delivers.  The draft-model
+    wrapper (``student_logits`` in the data) is not part of this path."""
+
+    def __init__(self, loss_fn: Any, cfg: Any, num_microbatches: int = 1, cp_normalize: bool = True,
+                 sampling_params: Optional[TrainingSamplingParams] = None, draft_model: Any = None,
+                 prepare_fn: Optional[Callable[..., Any]] = None):
+        if draft_model is not None:
+            raise NotImplementedError("LossPostProcessor: the draft-model loss is outside this build")
+        self.loss_fn = loss_fn
+        self.cfg = cfg
+        self.num_microbatches = num_microbatches
+        self.cp_normalize = cp_normalize
+        self.sampling_params = sampling_params
+        self.prepare_fn = prepare_fn
+        self.d2t = None
+
+    def __call__(self, data_dict: Any, packed_seq_params: Any = None, global_valid_seqs: Optional[torch.Tensor] = None,
+                 global_valid_toks: Optional[torch.Tensor] = None) -> Callable[[torch.Tensor], Tuple[torch.Tensor, Dict[str, Any]]]:
+        from functools import partial
+
+        from ...algorithms.loss import (
+            SequencePackingFusionLossWrapper,
+            SequencePackingLossWrapper,
+            prepare_loss_input,
+            prepare_packed_loss_input,
+            wrap_loss_fn_with_input_preparation,
+        )
+
+        chunk = self.cfg.get("logprob_chunk_size", None)
+        if self.prepare_fn is not None:
+            prepare = self.prepare_fn
+        else:
+            prepare = partial(prepare_loss_input, sampling_params=self.sampling_params, d2t=self.d2t, chunk_size=chunk)
+        if "student_logits" in data_dict:
+            raise NotImplementedError("LossPostProcessor: the draft-model loss is outside this build")
+        if self.cfg["sequence_packing"]["enabled"] and packed_seq_params is not None:
+            if self.cfg.get("sequence_packing", {}).get("fuse_loss", False):
+                assert self.prepare_fn is None, (
+                    "sequence_packing.fuse_loss=true does not support a custom prepare_fn (e.g. the value model's "
+                    "value-specific prep). Disable fuse_loss for the value model."
+                )
+                wrapper_cls = SequencePackingFusionLossWrapper
+                prepare = partial(prepare_packed_loss_input, sampling_params=self.sampling_params, chunk_size=chunk)
+            else:
+                wrapper_cls = SequencePackingLossWrapper
+            wrapped = wrapper_cls(loss_fn=self.loss_fn, prepare_fn=prepare, cu_seqlens_q=packed_seq_params.cu_seqlens_q,
+                                  cu_seqlens_q_padded=packed_seq_params.cu_seqlens_q_padded, vocab_parallel_rank=0,
+                                  vocab_parallel_group=None, context_parallel_group=None)
+        else:
+            wrapped = partial(wrap_loss_fn_with_input_preparation, loss_fn=self.loss_fn, prepare_fn=prepare,
+                              vocab_parallel_rank=0, vocab_parallel_group=None, context_parallel_group=None)
+        wrapped = partial(wrapped, data=data_dict, global_valid_seqs=global_valid_seqs, global_valid_toks=global_valid_toks)
+        num_microbatches = self.num_microbatches
+
+        def counteract_schedule_averaging(*args, **kwargs):
+            loss, metrics = wrapped(*args, **kwargs)
+            return loss * num_microbatches, metrics  # context-parallel size 1: no division
+
+        return counteract_schedule_averaging
 
 
 class LogprobsPostProcessor:
@@ -60,11 +132,12 @@ class LogprobsPostProcessor:
                     token_logprobs = torch.cat([torch.zeros_like(lp[:, :1]), lp], dim=1)
                 else:
                     # logprob of every next token and the zero column in front in one launch; no position is padding
+                    temperature = pending_temperature(output_tensor)  # a divide left to this kernel
                     x = output_tensor if output_tensor.stride(-1) == 1 else output_tensor.contiguous()
                     ids = unpacked_input_ids.to(x.device)
                     full = torch.full((ids.shape[0],), ids.shape[1], dtype=torch.int64, device=x.device)
                     token_logprobs = torch.ops.rl_amd.logprob_post_fwd(
-                        x, ids[:, 1:], full, ids.shape[1] - 1, 0, x.shape[-1], 1.0, NRL_TEMP_RCP)
+                        x, ids[:, 1:], full, ids.shape[1] - 1, 0, x.shape[-1], temperature, NRL_TEMP_RCP)
                 if filtering:  # ``train.py:672-677``
                     mask = data_dict["token_mask"] * data_dict["sample_mask"].unsqueeze(-1)
                     token_logprobs = mask_out_neg_inf_logprobs(token_logprobs, mask.to(token_logprobs.device), "prev_logprobs")

@@ -13,6 +13,7 @@ import os
 import torch
 
 from . import _lib
+from ._deferred import refuse_pending
 
 _DTYPES = {torch.float32: _lib.NRL_F32, torch.bfloat16: _lib.NRL_BF16, torch.float16: _lib.NRL_F16}
 
@@ -184,8 +185,35 @@ def _logprob_post_fwd(logits, targets, lengths, n_inner, vocab_start, vocab_end,
     return out
 
 
+_LIB.define("scale_rows_(Tensor(a!) x, Tensor factor, float divisor) -> ()")
+_LIB.define("scale_rows(Tensor x, Tensor factor, float divisor) -> Tensor")
+
+
+def _scale_rows(x, factor, divisor, in_place=False):
+    """``x * (factor / divisor)`` for a ``[B, S, V]`` tensor and a device scalar ``factor``, in ``x``'s dtype.  The
+    host does not wait for the factor's value; in place, a factor equal to the divisor touches no memory."""
+    _need_gpu(x, factor)
+    if x.dim() != 3 or (x.stride(2) != 1 and x.shape[2] > 1):
+        raise ValueError(f"expected [B, S, V] with a contiguous last axis, got {tuple(x.shape)} strides {x.stride()}")
+    if factor.numel() != 1:
+        raise ValueError("factor must hold one element")
+    f = factor.detach().reshape(1).to(torch.float32)
+    b, s, v = x.shape
+    with torch.cuda.device(x.device):
+        out = x if in_place else torch.empty((b, s, v), dtype=x.dtype, device=x.device)
+        with _timed("scale_rows"):
+            code = _lib.load().nrl_scale_rows(_ptr(x), _ptr(out), _dtype_code(x), b, s, v, x.stride(0), x.stride(1),
+                                              out.stride(0), out.stride(1), _ptr(f), float(divisor), _stream())
+    _lib.check(code, "nrl_scale_rows")
+    return out
+
+
+def _scale_rows_inplace(x, factor, divisor):
+    _scale_rows(x, factor, divisor, in_place=True)
+
+
 for _name, _fn in (("logprob_fwd", _logprob_fwd), ("logprob_bwd", _logprob_bwd), ("logprob_bwd_", _logprob_bwd_inplace),
-                   ("logprob_post_fwd", _logprob_post_fwd)):
+                   ("logprob_post_fwd", _logprob_post_fwd), ("scale_rows_", _scale_rows_inplace), ("scale_rows", _scale_rows)):
     _LIB.impl(_name, _fn, "CUDA")
     _LIB.impl(_name, _fn, "CPU")  # raises: there is no CPU path
 
@@ -487,24 +515,25 @@ def _grpo_loss(lp, lpu, prev, gen, ref, adv, token_mask, sample_mask, correct_ma
 
 _LIB.define(
     "fused_logits_grpo_loss(Tensor logits, Tensor targets, int n_inner, Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, "
-    "Tensor token_mask, Tensor sample_mask, Tensor global_valid, int[] iflags, float[] fparams, float loss_scale) "
-    "-> (Tensor, Tensor, Tensor, Tensor)"
+    "Tensor token_mask, Tensor sample_mask, Tensor global_valid, int[] iflags, float[] fparams, float loss_scale, "
+    "float temperature, int temp_mode) -> (Tensor, Tensor, Tensor, Tensor)"
 )
 _LIB.define(
     "fused_logits_grpo_loss_(Tensor(a!) logits, Tensor targets, int n_inner, Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, "
-    "Tensor token_mask, Tensor sample_mask, Tensor global_valid, int[] iflags, float[] fparams, float loss_scale) "
-    "-> (Tensor, Tensor, Tensor)"
+    "Tensor token_mask, Tensor sample_mask, Tensor global_valid, int[] iflags, float[] fparams, float loss_scale, "
+    "float temperature, int temp_mode) -> (Tensor, Tensor, Tensor)"
 )
 
 
 def _fused_logits_grpo_loss(logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid, iflags,
-                            fparams, loss_scale, in_place=False):
-    """-> (loss, dlogits, logprobs [B, n_inner], metrics)."""
+                            fparams, loss_scale, temperature, temp_mode, in_place=False):
+    """-> (loss, dlogits, logprobs [B, n_inner], metrics).  ``temperature`` != 1 divides the logits inside the
+    pass the way an in-place ``div_`` of the tensor would have rounded them (``temp_mode``: on the GPU or the CPU)."""
     if len(iflags) != len(_CFG_INT) or len(fparams) != len(_CFG_FLT):
         raise ValueError("malformed loss configuration")
     _need_gpu(logits, targets)
     b, s, v = logits.shape
-    rows = _rows(logits, targets, n_inner, 0, v, 1.0, _lib.NRL_TEMP_RCP)
+    rows = _rows(logits, targets, n_inner, 0, v, float(temperature), int(temp_mode))
     dev = logits.device
     lp_shape = torch.empty((b, n_inner), dtype=torch.float32, device=dev)
     inp, keep, _, _ = _grpo_inputs(lp_shape, None, prev, gen, ref, adv, token_mask, sample_mask, None, global_valid)
@@ -533,9 +562,10 @@ def _fused_logits_grpo_loss(logits, targets, n_inner, prev, gen, ref, adv, token
 
 
 def _fused_logits_grpo_loss_inplace(logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask, global_valid,
-                                    iflags, fparams, loss_scale):
+                                    iflags, fparams, loss_scale, temperature, temp_mode):
     loss, _, lp, metrics = _fused_logits_grpo_loss(logits, targets, n_inner, prev, gen, ref, adv, token_mask, sample_mask,
-                                                   global_valid, iflags, fparams, loss_scale, in_place=True)
+                                                   global_valid, iflags, fparams, loss_scale, temperature, temp_mode,
+                                                   in_place=True)
     return loss, lp, metrics
 
 
@@ -546,12 +576,13 @@ for _name, _fn in (("fused_logits_grpo_loss", _fused_logits_grpo_loss), ("fused_
 _LIB.define(
     "fused_packed_logits_grpo_loss(Tensor logits, Tensor targets, bool pre_rolled, Tensor cu_seqlens, int unpacked_seqlen, "
     "Tensor? prev, Tensor gen, Tensor? ref, Tensor adv, Tensor token_mask, Tensor sample_mask, Tensor global_valid, "
-    "int[] iflags, float[] fparams, float loss_scale) -> (Tensor, Tensor, Tensor, Tensor)"
+    "int[] iflags, float[] fparams, float loss_scale, float temperature, int temp_mode) "
+    "-> (Tensor, Tensor, Tensor, Tensor)"
 )
 
 
 def _fused_packed_logits_grpo_loss(logits, targets, pre_rolled, cu_seqlens, unpacked_seqlen, prev, gen, ref, adv, token_mask,
-                                   sample_mask, global_valid, iflags, fparams, loss_scale):
+                                   sample_mask, global_valid, iflags, fparams, loss_scale, temperature, temp_mode):
     """Packed [T, V] logits -> (loss, dlogits [T, V], logprobs [n_seq, unpacked_seqlen - 1], metrics)."""
     if len(iflags) != len(_CFG_INT) or len(fparams) != len(_CFG_FLT):
         raise ValueError("malformed loss configuration")
@@ -566,7 +597,7 @@ def _fused_packed_logits_grpo_loss(logits, targets, pre_rolled, cu_seqlens, unpa
     rows.targets = targets.data_ptr()
     rows.tgt_stride_outer, rows.tgt_stride_inner = 0, 1
     rows.vocab_start, rows.vocab_end = 0, v
-    rows.temperature, rows.temp_mode = 1.0, _lib.NRL_TEMP_RCP
+    rows.temperature, rows.temp_mode = float(temperature), int(temp_mode)
     dev = logits.device
     lp = torch.empty((n_seq, n_inner), dtype=torch.float32, device=dev)
     inp, keep, _, _ = _grpo_inputs(lp, None, prev, gen, ref, adv, token_mask, sample_mask, None, global_valid)
@@ -931,6 +962,7 @@ def _plain_rows(logits, vocab_start=0, vocab_end=None):
         raise ValueError(f"expected logits [B, S, V], got {tuple(logits.shape)}")
     if logits.stride(2) != 1 and logits.shape[2] > 1:
         raise ValueError("the vocabulary axis of the logits must be contiguous")
+    refuse_pending(logits, "this op")
     b, s, v = logits.shape
     r = _lib.NrlRows()
     r.logits = logits.data_ptr()

@@ -1,0 +1,74 @@
+"""Temperature scaling of the model's logits (``apply_temperature_scaling``,
+``nemo_rl/models/automodel/train.py:180-194`` and ``nemo_rl/models/megatron/train.py:203-217``).
+
+The reference divides the logits tensor in place, in its own dtype, right after the model forward; the
+Megatron worker even drops the return value, so "the tensor the model returned now holds scaled values"
+is the contract.  ``apply_temperature_scaling`` here keeps it: one HIP pass ``x * (1 / T)`` over the
+tensor (how a GPU ``div_`` by a scalar rounds), differentiable like ``div_``.
+
+That pass costs a full read + write of ``[B, S, V]``.  The logprob kernels can apply the same divide,
+with the same rounding of value and gradient, while they stream the row anyway.  Because nothing in
+the tensor itself can say "not divided yet" without risking a silently unscaled read elsewhere, that is
+an explicit opt-in: inside ``with deferred_temperature():`` ``apply_temperature_scaling`` leaves the
+memory alone and records (storage, T) for the calling thread; the logprob / loss entry points of this
+package look the logits they are handed up in that record (views of the recorded tensor share its
+storage) and divide inside their kernels.  Whoever opens the context promises that, until it closes,
+only those entry points read the logits.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+
+from . import ops  # noqa: F401  (registers torch.ops.rl_amd)
+from ._deferred import _state, deferred_temperature, pending_temperature  # noqa: F401
+
+_OPS = torch.ops.rl_amd
+
+
+def _one(device) -> torch.Tensor:
+    return torch.ones((), dtype=torch.float32, device=device)
+
+
+class _DivideInPlace(torch.autograd.Function):
+    """``logits.div_(T)`` with GPU rounding: value ``round(x * (1/T))``, gradient ``round(g * (1/T))``."""
+
+    @staticmethod
+    def forward(ctx, logits, temperature):
+        ctx.mark_dirty(logits)
+        ctx.temperature = temperature
+        view = logits if logits.dim() == 3 else logits.view(-1, 1, logits.shape[-1])
+        _OPS.scale_rows_(view, _one(logits.device), temperature)
+        return logits
+
+    @staticmethod
+    def backward(ctx, grad):
+        g3 = grad if grad.dim() == 3 else grad.reshape(-1, 1, grad.shape[-1])
+        if g3.stride(-1) != 1:
+            g3 = g3.contiguous()
+        return _OPS.scale_rows(g3, _one(grad.device), ctx.temperature).view(grad.shape), None
+
+
+def apply_temperature_scaling(logits: torch.Tensor, sampling_params: Optional[Any]) -> torch.Tensor:
+    """Same contract as the reference function: returns ``logits``, divided in place by the temperature
+    when there is one and it is not 1.  Inside ``deferred_temperature()`` the divide is left to the
+    logprob kernels instead (see the module text)."""
+    if sampling_params is None or sampling_params.temperature == 1.0:
+        return logits
+    t = float(sampling_params.temperature)
+    if getattr(_state, "depth", 0) > 0:
+        if not logits.is_cuda:
+            raise RuntimeError("deferred_temperature() needs GPU logits")
+        _state.pending.append((logits.untyped_storage().data_ptr(), t))
+        return logits
+    if not logits.is_cuda:
+        raise RuntimeError("rl_amd runs on the GPU only (got CPU logits); there is no CPU fallback")
+    if logits.dim() < 1 or logits.stride(-1) != 1 or not logits.is_contiguous():
+        raise ValueError("apply_temperature_scaling expects a contiguous logits tensor")
+    if torch.is_grad_enabled() and logits.requires_grad:
+        return _DivideInPlace.apply(logits, t)
+    view = logits if logits.dim() == 3 else logits.view(-1, 1, logits.shape[-1])
+    _OPS.scale_rows_(view, _one(logits.device), t)
+    return logits

@@ -99,3 +99,38 @@ def synthetic_grpo_batch(n_prompts, group, seq, vocab, seed, logits_dtype=torch.
         "logits": logits, "input_ids": ids, "token_mask": token_mask, "sample_mask": sample_mask,
         "rewards": rewards, "prompt_ids": prompt_ids, "generator": g,
     }
+
+
+def packed_grpo_case(lens, pads, width, vocab, dtype, seed, tail=0, empty_mask_rows=(), dead_rows=(), float_masks=False):
+    """Unpacked ``[B, width]`` loss data plus the packed ``[1, T, V]`` logits of the same sequences (CPU):
+    sequence i holds ``lens[i]`` tokens inside a span of ``lens[i] + pads[i]`` packed positions, ``tail``
+    unused positions follow.  ``empty_mask_rows`` get an all-zero token mask, ``dead_rows`` a zero sample mask.
+    Returns (logits, data, cu_seqlens, cu_seqlens_padded, global_valid_seqs, global_valid_toks)."""
+    b = len(lens)
+    g = torch.Generator().manual_seed(seed)
+    lens_t, pads_t = torch.tensor(lens), torch.tensor(pads)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lens_t.cumsum(0)]).to(torch.int32)
+    cup = torch.cat([torch.zeros(1, dtype=torch.int64), (lens_t + pads_t).cumsum(0)]).to(torch.int32)
+    total = int(cup[-1]) + tail
+    logits = (torch.randn(1, total, vocab, generator=g) * 2.5).to(dtype)
+    ids = torch.zeros(b, width, dtype=torch.int64)
+    mdt = torch.float32 if float_masks else torch.int64
+    tm = torch.zeros(b, width, dtype=mdt)
+    for i, n in enumerate(lens):
+        ids[i, :n] = torch.randint(0, vocab, (n,), generator=g)
+        if n > 2 and i not in empty_mask_rows:
+            tm[i, int(torch.randint(1, n - 1, (1,), generator=g)):n] = 1
+    sm = torch.ones(b, dtype=mdt)
+    for i in dead_rows:
+        sm[i] = 0
+    from oracle import logprob as OL
+
+    targets = OL.pack_input_ids(ids, cu, cup, roll_shift=-1)
+    cur = OL.packed_logits_to_logprobs(logits.float()[:, : int(cup[-1])], targets, cup, width, target_is_pre_rolled=True)
+    near = lambda: torch.cat([torch.zeros(b, 1), cur + 0.05 * torch.randn(b, width - 1, generator=g)], 1)  # noqa: E731
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm,
+            "advantages": torch.randn(b, 1, generator=g).expand(b, width).contiguous(),
+            "prev_logprobs": near(), "generation_logprobs": near(), "reference_policy_logprobs": near()}
+    gs = sm.sum().float()
+    gt = (tm[:, 1:] * sm.unsqueeze(-1)).sum().float()
+    return logits, data, cu, cup, gs, gt

@@ -168,3 +168,56 @@ def test_diagnostics_against_float64_formulas():
     assert m["probs_ratio_max"] == pytest.approx(float(r[mask.bool()].max()), rel=1e-5)
     assert m["approx_entropy"] == pytest.approx(-mean(torch.exp(c - g) * c), rel=1e-5)
     assert m["num_valid_samples"] == 2.0
+
+
+def _packed_oracle_case(**kw):
+    from helpers import packed_grpo_case
+
+    return packed_grpo_case(dtype=torch.float32, seed=13, **kw)
+
+
+def test_sequence_packing_loss_equals_one_call_on_the_unpacked_batch():
+    """The identity the reference's own test states for its two wrappers
+    (``tests/unit/algorithms/test_sequence_packing_fusion.py:190-265``): with global normalisers the per-sequence
+    losses add up to the loss of the whole unpacked batch, and so do the gradients."""
+    from oracle import logprob as OL
+
+    logits, data, cu, cup, gs, gt = _packed_oracle_case(lens=[9, 5, 12, 7], pads=[3, 1, 0, 5], width=14, vocab=64)
+    for cfg in (O.LossConfig(), O.LossConfig(token_level_loss=False, reference_policy_kl_penalty=0.01)):
+        x1 = logits.clone().requires_grad_(True)
+        l1, m1 = O.sequence_packing_loss(cfg, x1, data, cu, cup, gs, gt, OL.next_token_logprobs)
+        l1.backward()
+        x2 = logits.clone().requires_grad_(True)
+        targets = OL.pack_input_ids(data["input_ids"], cu, cup, roll_shift=-1)
+        lp = OL.packed_logits_to_logprobs(x2[:, : int(cup[-1])], targets, cup, 14, target_is_pre_rolled=True)
+        l2, m2 = O.clipped_pg_loss(cfg, lp, data, gs, gt)
+        l2.backward()
+        torch.testing.assert_close(l1, l2, atol=1e-6, rtol=1e-5)
+        torch.testing.assert_close(x1.grad, x2.grad, atol=1e-7, rtol=1e-5)
+        for k in ("probs_ratio_min", "probs_ratio_max", "probs_ratio_clamped_min", "probs_ratio_clamped_max",
+                  "probs_ratio", "token_mult_prob_error", "num_valid_samples"):
+            assert m1[k] == pytest.approx(m2[k], rel=1e-5), k
+
+
+def test_sequence_packing_loss_extrema_skip_empty_sequences():
+    """Brute force for the min / max merge (``loss/wrapper.py:145-164``): the merged extrema are the extrema over
+    all valid tokens; a sequence without valid tokens contributes its +-inf sentinels, which are skipped; with no
+    valid token anywhere the sentinels stay."""
+    from oracle import logprob as OL
+
+    logits, data, cu, cup, gs, gt = _packed_oracle_case(lens=[6, 4, 8], pads=[2, 0, 1], width=8, vocab=32, empty_mask_rows=(1,))
+    _, m = O.sequence_packing_loss(O.LossConfig(), logits, data, cu, cup, gs, gt, OL.next_token_logprobs)
+    ratios = []
+    for i in (0, 2):
+        n = int(cu[i + 1] - cu[i])
+        piece = logits[:, int(cup[i]) : int(cup[i + 1])]
+        lp = OL.next_token_logprobs(data["input_ids"][i : i + 1, :n], piece)[0]
+        r = torch.exp(lp - data["prev_logprobs"][i, 1:n])
+        ratios.append(r[data["token_mask"][i, 1:n] > 0])
+    allr = torch.cat(ratios)
+    assert m["probs_ratio_min"] == pytest.approx(allr.min().item(), rel=1e-6)
+    assert m["probs_ratio_max"] == pytest.approx(allr.max().item(), rel=1e-6)
+    assert m["probs_ratio_clamped_min"] == pytest.approx(allr.clamp(0.8, 1.2).min().item(), rel=1e-6)
+    data["token_mask"] = torch.zeros_like(data["token_mask"])
+    _, m = O.sequence_packing_loss(O.LossConfig(), logits, data, cu, cup, gs, gt, OL.next_token_logprobs)
+    assert m["probs_ratio_min"] == float("inf") and m["probs_ratio_max"] == float("-inf")
