@@ -14,8 +14,11 @@
 //          bf16) and folded into a running (max, sum-exp) per token column without any cross-lane
 //          traffic while the workgroup walks its vocabulary tiles; the target's logit is captured on the
 //          way.  Only [tokens] sized partials leave the chip.
-//   GRAD   backward: recomputed tile -> g * (onehot - exp(x - lse)) written as bf16 both row-major
-//          (for dH = G W) and transposed (for dW = G^T hidden) for one token chunk at a time.
+//   GRAD   backward: recomputed tile -> the softmax part -g * exp(x - lse) of the logits' gradient, written as
+//          bf16 row-major (for dH = G W) and, with the one-hot term g at the target added, transposed (for
+//          dW = G^T hidden), for one token chunk at a time.  The one-hot term of dH, g * W[target], is added
+//          in fp32 by its own kernel: it is the one large element of a row of G, and narrowing it to bf16
+//          would put its rounding error (up to 2^-8, coherent over the row) straight into dH.
 //   STORE / ACCUM  plain fp32 C = or C += for dH and dW.
 // The vocabulary is walked in tiles while the token chunk bounds what is materialised:
 // chunk x V bf16 for G and G^T (5 GB each at chunk 16384, V 151936) instead of N x V.
@@ -134,7 +137,7 @@ struct CoreA {
 
 // ---------------------------------------------------------------------------------------------
 // Core B: 256 x 256 tile (wave tile 128 x 128: 16 MFMA tiles, 256 accumulator registers, one wave per
-// SIMD), K a multiple of 64.  Two LDS buffers per operand (4 x 32 KiB); slab k+1 is fetched by direct
+// SIMD), K a multiple of 64.  Two LDS buffers per operand (4 x 32 KiB); slabs k+1 and k+2 are fetched by direct
 // global-to-LDS loads while slab k is consumed, one barrier per slab.  A 64-element row is 8 chunks
 // of 16 bytes; chunk c of row r sits at chunk position c ^ ((r >> 1) & 7), which keeps the rows unpadded
 // (a wave's direct load fills 1 KiB contiguously) and the wave's 16-byte fragment reads (32 rows x 2
@@ -183,41 +186,57 @@ struct CoreB {
                      : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
     }
 
-    static constexpr int DMA_EVERY = 2;  // one direct load behind every second MFMA of the first 32
+    static constexpr int KS = BK / 16;
+    static constexpr int LATE = ROUNDS;  // of a slab's 16 direct loads, those issued during the following slab's first k step
 
-    // Consume slab buffer BUF while the direct loads of slab k_next go into the other buffer.  One wave per
-    // SIMD: nothing else hides latencies, so the order is fixed by hand -- the 16 direct loads go out one
-    // behind every second MFMA of the first half of the slab (their address arithmetic runs in the shadow of
-    // the matrix pipe, and the four waves do not queue up at the load unit), and the 8 fragment reads of k
-    // step ks + 1 follow the first 8 MFMAs of step ks.
+    // One slab out of buffer BUF with one wave per SIMD: nothing else hides latencies, so the order is fixed by
+    // hand.  On entry the fragments of the slab's k step 0 are in flight into set 0; on exit those of the next
+    // slab (buffer BUF ^ 1) are.  The fragments of the last k step are in registers once that step starts, so
+    // from there on this wave no longer reads BUF: the wait for the other buffer's direct loads and the workgroup
+    // barrier sit at the start of the last step, no LDS latency is exposed between two slabs, and the freed
+    // buffer starts filling at once with the slab after the next (k_load): half of its 16 direct loads go out
+    // behind every second MFMA of this last step, the other half (k_late, into BUF ^ 1 as seen from the next
+    // slab) behind every second MFMA of the next slab's first step.  Measured against all 16 in one step, or 4 /
+    // 2 early: this split was fastest on every shape.  The 8 fragment reads of k step ks + 1 follow the first 8
+    // MFMAs of step ks.
     template <int BUF>
-    __device__ static __forceinline__ void compute(const Ctx& c, unsigned char* lds, f32x16 (&acc)[NI][NJ], int64_t k_next) {
-        static_assert(NI == 4 && NJ == 4, "wait_frags names four fragments per operand");
-        bf16x8 af[2][NI], bfr[2][NJ];
-        // fragment read number f of k step ks: 0..NI-1 operand A, NI..NI+NJ-1 operand B
-        auto frag_one = [&](int ks, int set, int f) {
-            if (f < NI) af[set][f] = lds_read16(c.aoff[ks], BUF * TILE_BYTES + f * 32 * BK * 2);
-            else bfr[set][f - NI] = lds_read16(c.boff[ks], BUF * TILE_BYTES + (f - NI) * 32 * BK * 2);
+    __device__ static __forceinline__ void compute(const Ctx& c, unsigned char* lds, f32x16 (&acc)[NI][NJ],
+                                                   bf16x8 (&af)[2][NI], bf16x8 (&bfr)[2][NJ], int64_t k_load, int64_t k_late) {
+        auto frag_one = [&](int buf, int ks, int set, int f) {
+            if (f < NI) af[set][f] = lds_read16(c.aoff[ks], buf * TILE_BYTES + f * 32 * BK * 2);
+            else bfr[set][f - NI] = lds_read16(c.boff[ks], buf * TILE_BYTES + (f - NI) * 32 * BK * 2);
         };
 #pragma unroll
-        for (int f = 0; f < NI + NJ; ++f) frag_one(0, 0, f);
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             wait_frags(af[ks & 1], bfr[ks & 1]);
+            if (ks == KS - 1) {
+                // this wave is done reading BUF; the other buffer's loads (issued during the previous slab's
+                // last step and this slab's first steps) must have landed before anyone reads it
+                asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+            }
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
-                    const int idx = i * NJ + j, n = ks * NI * NJ + idx;  // MFMA number within the step / the slab
+                    const int idx = i * NJ + j;
                     __builtin_amdgcn_sched_barrier(0);
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
-                    if (n % DMA_EVERY == 0 && n / DMA_EVERY < 2 * ROUNDS) {
+                    constexpr int EARLY = 2 * ROUNDS - LATE, GAP = NI * NJ / EARLY;
+                    if (ks == KS - 1 && idx % GAP == 0) {
+                        // the freed buffer takes the slab after the next: direct loads behind this step's MFMAs
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_one(c, lds, BUF ^ 1, k_next, n / DMA_EVERY);
+                        issue_one(c, lds, BUF, k_load, idx / GAP);
                     }
-                    if (ks + 1 < BK / 16 && idx < NI + NJ) {
+                    const int n = ks * NI * NJ + idx;
+                    if (n % 2 == 0 && n / 2 < LATE) {
+                        // ... and the rest of the slab that the previous slab started loading into the other buffer
                         __builtin_amdgcn_sched_barrier(0);
-                        frag_one(ks + 1, (ks + 1) & 1, idx);
+                        issue_one(c, lds, BUF ^ 1, k_late, EARLY + n / 2);
+                    }
+                    if (idx < NI + NJ) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (ks + 1 < KS) frag_one(BUF, ks + 1, (ks + 1) & 1, idx);
+                        else frag_one(BUF ^ 1, 0, 0, idx);
                     }
                 }
             }
@@ -225,16 +244,16 @@ struct CoreB {
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    // End of a slab: the direct loads must have landed in LDS and every wave must be done reading the
-    // buffer they will overwrite next.  The compiler does not track direct loads against LDS reads, so the
-    // wait is written by hand.
-    __device__ static __forceinline__ void slab_barrier() {
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    }
-
     __device__ static __forceinline__ void tile(const GemmOperands& op, int64_t row0, int64_t col0, f32x16 (&acc)[NI][NJ],
                                                 unsigned char* lds) {
-        const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        static_assert(NI + NJ <= NI * NJ && 2 * ROUNDS == NI * NJ, "one direct load behind each MFMA of a k step");
+        static_assert(LATE >= 0 && LATE < 2 * ROUNDS && (NI * NJ) % (2 * ROUNDS - LATE) == 0 && LATE <= 3 * NI * NJ / 2, "load schedule");
+        // (an opaque copy of the thread index: everything derived from it below is recomputed per tile, about a
+        // hundred instructions, instead of being hoisted out of the caller's tile loop and kept in registers, or
+        // spilled, across its epilogue)
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int wm = wave >> 1, wn = wave & 1;
         Ctx c;
         c.wave = wave;
@@ -250,30 +269,41 @@ struct CoreB {
             c.vob[j] = static_cast<uint32_t>((r < last_b ? r : last_b) * op.ldb + cg * 8) * 2u;
         }
         const int fr = lane & 31, fh = lane >> 5;
-        // the buffer's address inside LDS (the low half of its generic address)
         const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             const uint32_t sw = static_cast<uint32_t>(((ks * 2 + fh) ^ ((fr >> 1) & 7)) * 16);
             c.aoff[ks] = lds_base + static_cast<uint32_t>((wm * 128 + fr) * BK * 2) + sw;
             c.boff[ks] = lds_base + static_cast<uint32_t>(2 * TILE_BYTES + (wn * 128 + fr) * BK * 2) + sw;
         }
         const int64_t nk = op.k / BK;
         const int64_t k_last = (nk - 1) * BK;
-        // every wave has passed the barrier that ended the previous tile's last slab, so buffer 0 is free
+        auto slab_k = [&](int64_t kt) { return kt < nk ? kt * BK : k_last; };  // past the end: the last slab again, unused
+        // every wave has passed the barrier inside the previous tile's last slab and has since only read
+        // registers, so both buffers are free: slab 0 and slab 1 start now
         issue(c, lds, 0, 0);
-        slab_barrier();
-        // after the last slab the loads re-fetch it into the idle buffer (no branch in the slab body)
-        for (int64_t kt = 0; kt + 1 < nk; kt += 2) {
-            compute<0>(c, lds, acc, (kt + 1) * BK);
-            slab_barrier();
-            compute<1>(c, lds, acc, kt + 2 < nk ? (kt + 2) * BK : k_last);
-            slab_barrier();
+#pragma unroll
+        for (int d = 0; d < 2 * ROUNDS - LATE; ++d) issue_one(c, lds, 1, slab_k(1), d);
+        // slab 0 has landed everywhere
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * ROUNDS - LATE) : "memory");
+        bf16x8 af[2][NI], bfr[2][NJ];
+#pragma unroll
+        for (int f = 0; f < NI + NJ; ++f) {
+            if (f < NI) af[0][f] = lds_read16(c.aoff[0], f * 32 * BK * 2);
+            else bfr[0][f - NI] = lds_read16(c.boff[0], (f - NI) * 32 * BK * 2);
         }
-        if (nk & 1) {
-            compute<0>(c, lds, acc, k_last);
-            slab_barrier();
+        int64_t kt = 0;
+        for (; kt + 1 < nk; kt += 2) {
+            compute<0>(c, lds, acc, af, bfr, slab_k(kt + 2), slab_k(kt + 1));
+            compute<1>(c, lds, acc, af, bfr, slab_k(kt + 3), slab_k(kt + 2));
         }
+        if (kt < nk) compute<0>(c, lds, acc, af, bfr, k_last, k_last);
+        // The last slab read ahead into fragments nobody uses.  Their registers must stay allocated until the
+        // reads have returned: the compiler takes an asm output for complete at once, and a register it hands
+        // out again (a load address, say) would be overwritten when the LDS data arrives.
+        wait_frags(af[0], bfr[0]);
+        // likewise the direct loads the last slab issued (copies of itself, never read) must not outlive the tile
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     }
 };
 
@@ -336,16 +366,17 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     const int64_t tok0 = bx * BT;
     const int split = static_cast<int>(by);
     const int64_t n_tiles = (a.op.m + BV - 1) / BV;
-    // this lane's token columns and their (local) target rows
-    int64_t tok[NJ];
-    int tgt[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        tok[j] = tok0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+    // (local) target row of each of the tile's token columns, -1 where there is none; kept in LDS so that the
+    // registers it would occupy through the K loop stay free
+    __shared__ int tgt_s[BT];
+    static_assert(BT <= GB_THREADS, "one thread per token column fills the target table");
+    if (tid < BT) {
         int64_t t = -1;
-        if (tok[j] < a.op.n) t = a.targets[tok[j]] - a.vocab_start;
-        tgt[j] = (t >= 0 && t < a.op.m) ? static_cast<int>(t) : -1;
+        if (tok0 + tid < a.op.n) t = a.targets[tok0 + tid] - a.vocab_start;
+        tgt_s[tid] = (t >= 0 && t < a.op.m) ? static_cast<int>(t) : -1;
     }
+    __syncthreads();
+    const int col = wn * (NJ * 32) + (lane & 31);  // this lane's token column of tile j is col + j * 32
     float run_m[NJ], run_s[NJ];
 #pragma unroll
     for (int j = 0; j < NJ; ++j) { run_m[j] = -1e30f; run_s[j] = 0.f; }
@@ -359,44 +390,42 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
         // below this lane's first row vb.  Only the last vocabulary tile needs the rows-past-the-end mask.
         const int vb = static_cast<int>(v0) + wm * 128 + 4 * (lane >> 5);
         const int limit = static_cast<int>(a.op.m) - vb;  // rows with off < limit exist
+        // One 32 x 32 block (16 accumulator registers) at a time, so that only those 16 values are live next to
+        // the accumulators: running maximum and sum are rescaled per block (one extra exponential per 16).
         auto fold_tile = [&](auto masked_tag) {
             constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                __builtin_amdgcn_sched_barrier(0);
-                const int toff = tgt[j] - vb;  // the target's row as an offset, if it is in this lane at all
-                // The logits count as rounded to bf16 (the matmul output dtype).  Rounding is monotone, so the
-                // maximum is taken over the raw accumulators and rounded once.
-                float raw = -INFINITY;
+                const int tg = tgt_s[col + j * 32];
+                const int toff = tg - vb;  // the target's row as an offset, if it is in this lane at all
 #pragma unroll
-                for (int i = 0; i < NI; ++i)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const int off = i * 32 + 8 * (e >> 2) + (e & 3);
-                        raw = fmaxf(raw, (!MASKED || off < limit) ? acc[i][j][e] : -INFINITY);
-                    }
-                const float mx = fmaxf(run_m[j], round_bf16(raw));
-                const float mx2 = mx * kLog2e;
-                // (the subtraction is exact where an FMA against the rounded mx2 would leave a huge residual
-                // while both maxima are still the -1e30 start value)
-                float sx = run_s[j] * fast_exp2((run_m[j] - mx) * kLog2e);
-#pragma unroll
-                for (int i = 0; i < NI; ++i)
+                for (int i = 0; i < NI; ++i) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    // The logits count as rounded to bf16 (the matmul output dtype).  Rounding is monotone, so the
+                    // maximum is taken over the raw accumulators and rounded once.
+                    float x[16];
+                    float raw = -INFINITY;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int off = i * 32 + 8 * (e >> 2) + (e & 3);
-                        const float p = fast_exp2(__builtin_fmaf(round_bf16(acc[i][j][e]), kLog2e, -mx2));
-                        sx += (!MASKED || off < limit) ? p : 0.f;
+                        x[e] = (!MASKED || off < limit) ? acc[i][j][e] : -INFINITY;
+                        raw = fmaxf(raw, x[e]);
                     }
-                run_m[j] = mx;
-                run_s[j] = sx;
-                if (toff >= 0 && toff < 128 && (toff & 4) == 0) {  // rare: the target's row is one of this lane's
-                    float xt = 0.f;
+                    const float mx = fmaxf(run_m[j], round_bf16(raw));
+                    const float mx2 = mx * kLog2e;
+                    // (the subtraction is exact where an FMA against the rounded mx2 would leave a huge residual
+                    // while both maxima are still the -1e30 start value)
+                    float sx = run_s[j] * fast_exp2((run_m[j] - mx) * kLog2e);
 #pragma unroll
-                    for (int i = 0; i < NI; ++i)
+                    for (int e = 0; e < 16; ++e) sx += fast_exp2(__builtin_fmaf(round_bf16(x[e]), kLog2e, -mx2));
+                    run_m[j] = mx;
+                    run_s[j] = sx;
+                    if (tg >= 0 && toff >= i * 32 && toff < i * 32 + 32 && (toff & 4) == 0) {  // rare: the target's row is here
+                        float xt = 0.f;
 #pragma unroll
-                        for (int e = 0; e < 16; ++e) xt = toff == i * 32 + 8 * (e >> 2) + (e & 3) ? acc[i][j][e] : xt;
-                    a.xt[tok[j]] = round_bf16(xt);
+                        for (int e = 0; e < 16; ++e) xt = toff == i * 32 + 8 * (e >> 2) + (e & 3) ? x[e] : xt;
+                        a.xt[tok0 + col + j * 32] = round_bf16(xt);
+                    }
                 }
             }
         };
@@ -475,9 +504,11 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     {
         const int64_t grow = row0 + tid;
         int64_t t = -1;
-        float l = 0.f, g = 0.f;
+        // rows past the chunk repeat its last row's operand: give them a log-sum-exp that keeps exp(x - lse)
+        // finite, and a zero gradient
+        float l = 128.f, g = 0.f;
         if (grow < a.op.m) { t = a.targets[grow] - a.vocab_start; l = a.lse[grow]; g = a.grad[grow]; }
-        tgt_local[tid] = (t >= 0 && t < a.op.n) ? static_cast<int>(t) : -1;
+        tgt_local[tid] = (t >= 0 && t < a.op.n && g != 0.f) ? static_cast<int>(t) : -1;
         lse_l[tid] = l * kLog2e;
         g_l[tid] = g;
     }
@@ -486,41 +517,43 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     zero_acc<Core>(acc);
     Core::tile(a.op, row0, col0, acc, lds);
     const int64_t m_pad = ((a.op.m + 63) / 64) * 64;
-    // gradient of the lane's 4 consecutive tokens (accumulator rows) of tile (i, j), group q, as two bf16 pairs
-    auto grad4 = [&](int i, int j, int q, uint32_t& p01, uint32_t& p23) {
+    // gradient of the lane's 4 consecutive tokens (accumulator rows) of tile (i, j), group q, as two bf16 pairs:
+    // s01 / s23 the softmax part alone (for G), p01 / p23 with the one-hot term (for G^T)
+    auto grad4 = [&](int i, int j, int q, uint32_t& p01, uint32_t& p23, uint32_t& s01, uint32_t& s23) {
         const int64_t c = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
         const bool col_ok = c < a.op.n;
-        float gv[4];
+        float gv[4], sv[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int e = q * 4 + u;
             const int rl = wm * 128 + i * 32 + acc_row(e, lane);
             const bool row_ok = row0 + rl < a.op.m;
-            gv[u] = 0.f;
-            if (row_ok && col_ok) {
+            gv[u] = sv[u] = 0.f;
+            if (row_ok && col_ok && g_l[rl] != 0.f) {
                 const float x = round_bf16(acc[i][j][e]);
                 const float p = fast_exp2(__builtin_fmaf(x, kLog2e, -lse_l[rl]));
-                gv[u] = ((tgt_local[rl] == c ? 1.f : 0.f) - p) * g_l[rl];
+                sv[u] = -p * g_l[rl];
+                gv[u] = tgt_local[rl] == c ? g_l[rl] + round_bf16(sv[u]) : sv[u];
             }
         }
         p01 = pack_bf16x2(gv[0], gv[1]);
         p23 = pack_bf16x2(gv[2], gv[3]);
+        s01 = pack_bf16x2(sv[0], sv[1]);
+        s23 = pack_bf16x2(sv[2], sv[3]);
     };
-    // The whole tile's gradients as bf16 pairs.  A group of 4 accumulator rows is the same for every j, so
-    // its per-token values are read from LDS once; out-of-range elements become zero by a select, not a branch.
+    // The softmax part of the whole tile's gradients as bf16 pairs.  A group of 4 accumulator rows is the same for
+    // every j, so its per-token values are read from LDS once; columns past the vocabulary become zero by a select.
     auto grad_all = [&](uint32_t (&p01)[NI][NJ][4], uint32_t (&p23)[NI][NJ][4]) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int rl = wm * 128 + i * 32 + acc_row(q * 4, lane);  // first of the 4 consecutive rows
-                float lse_r[4], g_r[4];
-                int tgt_r[4];
+                float lse_r[4], ng_r[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     lse_r[u] = lse_l[rl + u];
-                    g_r[u] = row0 + rl + u < a.op.m ? g_l[rl + u] : 0.f;
-                    tgt_r[u] = tgt_local[rl + u];
+                    ng_r[u] = -g_l[rl + u];  // zero for rows past the chunk and for tokens without a gradient
                 }
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
@@ -530,8 +563,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
                     for (int u = 0; u < 4; ++u) {
                         const float x = round_bf16(acc[i][j][q * 4 + u]);
                         const float p = fast_exp2(__builtin_fmaf(x, kLog2e, -lse_r[u]));
-                        const float v = ((tgt_r[u] == c ? 1.f : 0.f) - p) * g_r[u];
-                        gv[u] = (c < a.op.n && g_r[u] != 0.f) ? v : 0.f;  // (also keeps 0 * inf out of the padding)
+                        gv[u] = c < a.op.n ? p * ng_r[u] : 0.f;
                     }
                     p01[i][j][q] = pack_bf16x2(gv[0], gv[1]);
                     p23[i][j][q] = pack_bf16x2(gv[2], gv[3]);
@@ -541,6 +573,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     };
     if constexpr (Core::LDS_BYTES >= BM * BN * 2) {
         // Both layouts leave through LDS so that every global store is a 16-byte piece of a 512-byte run.
+        static_assert(BM == GB_THREADS, "one thread per token row patches the one-hot term");
         // Pass 1, [vocab][token]: a lane's 4 tokens are one 8-byte unit; unit U of row v sits at U ^ (v & 63).
         // Pass 2, [token][vocab]: 2-byte writes; the 16-byte chunk C of row t sits at C ^ ((t >> 2) & 7).
         constexpr int RV = BN / 8;  // 16-byte pieces per token row of the tile
@@ -557,6 +590,14 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
                     const int unit = (t0 >> 2) ^ (v & 63);
                     *reinterpret_cast<uint2*>(lds + v * (BM * 2) + unit * 8) = uint2{p01[i][j][q], p23[i][j][q]};
                 }
+        }
+        __syncthreads();
+        {   // the one-hot term of G^T: token `tid` adds its g at its target's row, if that row is in this tile
+            const int v = tgt_local[tid] - static_cast<int>(col0);
+            if (tgt_local[tid] >= 0 && v >= 0 && v < BN) {
+                uint16_t* cell = reinterpret_cast<uint16_t*>(lds + v * (BM * 2) + (((tid >> 2) ^ (v & 63)) * 8) + (tid & 3) * 2);
+                *cell = static_cast<uint16_t>(f32_to_bf16_bits(g_l[tid] + bf16_bits_to_f32(*cell)));
+            }
         }
         __syncthreads();
 #pragma unroll 4
@@ -603,15 +644,15 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
             for (int i = 0; i < NI; ++i) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {  // four groups of four consecutive rows
-                    uint32_t p01, p23;
-                    grad4(i, j, q, p01, p23);
+                    uint32_t p01, p23, s01, s23;
+                    grad4(i, j, q, p01, p23, s01, s23);
                     const int64_t r_first = row0 + wm * 128 + i * 32 + acc_row(q * 4, lane);
                     if (c < a.ldg) {
                         uint16_t* gp = a.g + r_first * a.ldg + c;
-                        if (r_first + 0 < m_pad) gp[0] = static_cast<uint16_t>(p01);
-                        if (r_first + 1 < m_pad) gp[a.ldg] = static_cast<uint16_t>(p01 >> 16);
-                        if (r_first + 2 < m_pad) gp[2 * a.ldg] = static_cast<uint16_t>(p23);
-                        if (r_first + 3 < m_pad) gp[3 * a.ldg] = static_cast<uint16_t>(p23 >> 16);
+                        if (r_first + 0 < m_pad) gp[0] = static_cast<uint16_t>(s01);
+                        if (r_first + 1 < m_pad) gp[a.ldg] = static_cast<uint16_t>(s01 >> 16);
+                        if (r_first + 2 < m_pad) gp[2 * a.ldg] = static_cast<uint16_t>(s23);
+                        if (r_first + 3 < m_pad) gp[3 * a.ldg] = static_cast<uint16_t>(s23 >> 16);
                     }
                     if (col_ok && r_first < a.ldgt) {
                         uint2 v;
@@ -670,6 +711,20 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
     };
     if (interior) write_back(std::true_type{});
     else write_back(std::false_type{});
+}
+
+// dH[n, :] += g_n * W[target_n, :] in fp32: the one-hot term of dH = G W, kept out of the bf16 product.
+// One workgroup per token; tokens without a gradient or with a target outside the shard add nothing.
+__global__ __launch_bounds__(256) void lmhead_onehot_dh_kernel(float* dh, int64_t ld_dh, const float* grad, const int64_t* targets,
+                                                              int64_t vocab_start, int64_t vocab, const uint16_t* w, int64_t ldw,
+                                                              int64_t h) {
+    const int64_t n = blockIdx.x;
+    const float g = grad[n];
+    const int64_t t = targets[n] - vocab_start;
+    if (g == 0.f || t < 0 || t >= vocab) return;
+    const uint16_t* wr = w + t * ldw;
+    float* out = dh + n * ld_dh;
+    for (int64_t c = threadIdx.x; c < h; c += 256) out[c] += g * bf16_bits_to_f32(wr[c]);
 }
 
 // dst[c, r] = src[r, c] for r < rows, c < cols; dst row stride ldd, columns [rows, pad_cols) zero-filled
@@ -837,6 +892,8 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         GemmOperands dh;
         dh.a = g; dh.lda = vp; dh.b = wt; dh.ldb = vp; dh.m = rows; dh.n = h; dh.k = vp;
         launch_gemm<false>(dh, dhidden_out + t0 * ld_dh, ld_dh, s);
+        lmhead_onehot_dh_kernel<<<dim3((unsigned)rows), dim3(256), 0, s>>>(dhidden_out + t0 * ld_dh, ld_dh, grad + t0, targets + t0,
+                                                                          vocab_start, vocab, w, ldw, h);
         // dW += G^T [V, rows] * (hidden^T [H, rows])^T
         transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((rows_pad + 63) / 64)), dim3(256), 0, s>>>(
             hid + t0 * ldh, rows, h, ldh, ht, chunk, rows_pad);

@@ -254,7 +254,13 @@ def test_config3_fused_lm_head_full_width_three_chunks():
     rest = torch.ones(n, dtype=torch.bool)
     rest[pick] = False
     assert bool((got_dh[rest] == 0).all())
-    for got, want in ((got_dh[pick], want_dh[:, 0].float()), (wg.grad.float().cpu(), want_dw.float())):
-        scale = want.abs().max().item()
-        assert (got - want).abs().max().item() <= 1e-2 * scale
-        assert ((got - want).norm() / want.norm()).item() <= 4e-3
+    # element-wise bound from the one narrowing of G to bf16 (see tests/test_gpu_lmhead.py); dH here has been cast
+    # to bf16 by autograd, which adds one more 2^-8
+    from test_gpu_lmhead import narrowing_bounds
+
+    o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hs[:, 0], ws, tgt[0], up[0, pick.to(DEV)].cpu())
+    torch.testing.assert_close(o_dh, want_dh[:, 0].float(), rtol=1e-4, atol=1e-9)
+    assert bool(((got_dh[pick] - o_dh).abs() <= b_dh + 2.0 ** -8 * o_dh.abs()).all())
+    assert bool(((wg.grad.float().cpu() - o_dw).abs() <= b_dw).all())
+    assert ((got_dh[pick] - o_dh).norm() / o_dh.norm()).item() <= 2.5e-3   # the bf16 cast autograd applies to dH
+    assert ((wg.grad.float().cpu() - o_dw).norm() / o_dw.norm()).item() <= 3e-3
