@@ -25,18 +25,46 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (scaled by the same counters on a 4 GiB copy), valid for one microbatch of the named workload
-MEASURED_TRAFFIC_BYTES = {
-    "c2": 16.90e9 + 19.95e9,  # fused_logits_loss_kernel
-    "c4": 14.72e9 + 19.92e9,  # topk_topp_stream_kernel (backward): rows of masked tokens are zero-filled unread
-    "c4_fwd": 23.54e9,        # topk_topp_fwd_kernel: the row once plus the re-read of the chunks that reach the bound
-    "c5": 33.41e9 + 34.38e9,  # fused_logits_loss_kernel, packed
-    # lmhead_fwd_kernel: L2 fills (W and hidden-state tiles re-fetched by every 4 x 8 patch of tiles that uses
-    # them; 114 GB if the workgroups of a patch stayed in step) + the partial log-sum-exp records written
-    "c3_fwd": 207.8e9 + 1.28e9,
-}
-THREE_PASS_BWD_TRAFFIC_BYTES = {"c2": 16.83e9 + 19.92e9}  # logprob_bwd_kernel
+def load_measured_traffic():
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, from the committed table
+    ``profiles/measured_traffic.md`` (key -> dict(kernel, read, write, profile)); each row names the profile
+    summary it was taken from, so a figure that no longer matches its kernel can be traced and re-measured."""
+    table = {}
+    path = os.path.join(ROOT, "profiles", "measured_traffic.md")
+    try:
+        with open(path) as fh:
+            for line in fh:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) == 6 and cells[0] not in ("key", "---") and not set(cells[0]) <= set("-"):
+                    try:
+                        table[cells[0]] = dict(kernel=cells[1], shape=cells[2], read=float(cells[3]), write=float(cells[4]),
+                                               profile=cells[5])
+                    except ValueError:
+                        pass
+    except OSError:
+        pass
+    return table
+
+
+MEASURED_TRAFFIC = load_measured_traffic()
+
+
+def hbm_roofline(kernel, alg_bytes, avg_ms, traffic_key=None, **extra):
+    """The roofline record of an HBM-bound kernel: ``achieved`` = algorithmic bytes / average launch time;
+    ``traffic`` = measured bytes per launch (or None when no profile covers this launch shape) and
+    ``frac_measured`` = those bytes / the same time / peak."""
+    gbs = alg_bytes / (avg_ms * 1e-3) / 1e9
+    rec = {"bound": "hbm", "kernel": kernel, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+           "traffic": None, "avg_launch_ms": avg_ms, "algorithmic_bytes_per_launch": alg_bytes}
+    row = MEASURED_TRAFFIC.get(traffic_key) if traffic_key else None
+    if row is not None:
+        moved = row["read"] + row["write"]
+        rec["traffic"] = moved
+        rec["frac_measured"] = moved / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        rec["traffic_profile"] = row["profile"]
+    rec.update(extra)
+    return rec
+
 
 WORKLOADS = {
     # name: (sequences, seq_len, vocab, dtype, sequences per microbatch, logit std, spike p)
@@ -55,8 +83,9 @@ WORKLOADS = {
     "post": dict(seqs=16, seq_len=4096, vocab=151936, dtype="bf16", mb_seqs=16, std=3.0, spike_p=0.0,
                  desc="forward-only LogprobsPostProcessor (prev / reference logprobs): 16 seq x 4096 tok right-padded to "
                       "lengths U[2048,4096], V=151936 bf16"),
-    "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0,
-               desc="benchmark config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32"),
+    "c1": dict(seqs=32, seq_len=512, vocab=32000, dtype="f32", mb_seqs=32, std=2.0, spike_p=0.0, group=4, response_suffix=64,
+               desc="benchmark config 1: 8 prompts x 4 = 32 seq x 512 tok, V=32000 fp32, response suffix U[64,512], Bernoulli "
+                    "rewards -> group-normalised advantages"),
 }
 
 
@@ -67,7 +96,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--seqs", type=int, default=None, help="override the number of sequences (smaller test runs)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true",
+                    help="skip the baseline legs (oracle on the host cores, oracle's op sequence on the GPU, copy bandwidth)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 4 GiB device-to-device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
@@ -114,8 +144,11 @@ def make_microbatch(torch, w, n_seq, seed, dev):
         view = logits[:, :-1]
         idx = ids[:, 1:].unsqueeze(-1)
         view.scatter_add_(-1, idx, hit.unsqueeze(-1))
-    lo, hi = (256, 1024) if s >= 2048 else (max(1, s // 8), max(2, s // 4))
-    prefix = torch.randint(lo, hi + 1, (n_seq,), generator=g, device=dev)
+    if w.get("response_suffix"):   # config 1: the response is a suffix of random length U[64, S]
+        prefix = s - torch.randint(w["response_suffix"], s + 1, (n_seq,), generator=g, device=dev)
+    else:
+        lo, hi = (256, 1024) if s >= 2048 else (max(1, s // 8), max(2, s // 4))
+        prefix = torch.randint(lo, hi + 1, (n_seq,), generator=g, device=dev)
     token_mask = (torch.arange(s, device=dev).unsqueeze(0) >= prefix.unsqueeze(-1)).to(torch.int64)
     token_mask[:, 0] = 0
     sample_mask = torch.ones(n_seq, dtype=torch.float32, device=dev)
@@ -135,54 +168,227 @@ def make_microbatch(torch, w, n_seq, seed, dev):
     })
 
 
-def cpu_baseline(torch, w, seconds):
-    """The oracle (pure PyTorch restatement of the reference op sequence) on the host cores, on a
-    bounded sample of the same workload: real vocabulary and dtype, fewer rows."""
+def timed(torch, ops, args, step):
+    """W untimed steps, then K timed ones bracketed by synchronisation; HIP events around every kernel launch of
+    the timed region (on the stream the ops launch on).  -> (seconds, per-kernel summary)."""
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = EventTimer(torch)
+    ops.KERNEL_TIMER = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ops.KERNEL_TIMER = None
+    return dt, timer.summary()
+
+
+# ------------------------------------------------------------------------------------------------
+# Baseline legs: the oracle (the CPU restatement of the reference's op sequence) on the host cores, the same
+# op sequence with stock torch ops on the GPU, and the device's copy bandwidth.  Reported next to the
+# measurement; none of it is on the product path.
+# ------------------------------------------------------------------------------------------------
+def oracle_sample(torch, w, kind, device, rows):
+    """One bounded sample of workload ``w`` for the oracle on ``device``: -> (run, rows, unit text).  ``run()`` does one
+    forward (+ loss + backward where the workload has one) of the reference's op sequence on about ``rows``
+    rows of the real vocabulary and dtype; inputs are built once, outside the timed call."""
+    from oracle import distill as OD
+    from oracle import lmhead as OH
     from oracle import logprob as OL
     from oracle import loss as O
 
-    cores = os.cpu_count() or 1
-    threads = min(cores, 16)
-    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(1002)
     dtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
     v = w["vocab"]
+    s = 64 if rows >= 64 else rows
+    n_seq = max(1, rows // s)
+    rows = n_seq * s
 
-    def run(n_seq, s):
-        g = torch.Generator().manual_seed(1002)
-        logits = (torch.randn(n_seq, s, v, generator=g) * w["std"]).to(dtype).requires_grad_(True)
-        ids = torch.randint(0, v, (n_seq, s), generator=g)
-        base = -torch.rand(n_seq, s, generator=g) * 3
-        tm = torch.ones(n_seq, s, dtype=torch.int64)
-        tm[:, : s // 8] = 0
-        data = {"token_mask": tm, "sample_mask": torch.ones(n_seq), "advantages": torch.randn(n_seq, 1, generator=g).expand(n_seq, s),
-                "prev_logprobs": base, "generation_logprobs": base, "reference_policy_logprobs": base + 0.05}
-        t0 = time.perf_counter()
-        lp = OL.next_token_logprobs(ids, logits)
-        loss, _ = O.clipped_pg_loss(O.LossConfig(), lp, data, torch.tensor(float(n_seq)), tm[:, 1:].sum().float())
+    def loss_data(n, width, beta_ref=True):
+        base = -torch.rand(n, width, generator=g) * 3
+        tm = torch.ones(n, width, dtype=torch.int64)
+        tm[:, : max(1, width // 8)] = 0
+        d = {"token_mask": tm, "sample_mask": torch.ones(n), "advantages": torch.randn(n, 1, generator=g).expand(n, width).contiguous(),
+             "prev_logprobs": base, "generation_logprobs": base.clone()}
+        if beta_ref:
+            d["reference_policy_logprobs"] = base + 0.05
+        return {k: t.to(device) for k, t in d.items()}, torch.tensor(float(n), device=device), tm[:, 1:].sum().float().to(device)
+
+    if kind == "lmhead":
+        h = w["hidden"]
+        hidden = torch.randn(s, n_seq, h, generator=g).to(torch.bfloat16).to(device).requires_grad_(True)
+        weight = (torch.randn(v, h, generator=g) * 0.02).to(torch.bfloat16).to(device).requires_grad_(True)
+        ids = torch.randint(0, v, (n_seq, s), generator=g).to(device)
+        data, gs, gt = loss_data(n_seq, s)
+
+        def run():
+            hidden.grad = weight.grad = None
+            lp = OH.hidden_to_logprobs(hidden, weight, ids)
+            loss, _ = O.clipped_pg_loss(O.LossConfig(), lp, data, gs, gt)
+            loss.backward()
+
+        return run, rows, f"{rows} tokens, H={h}, V={v} bf16: hidden -> logprobs -> loss -> (dH, dW) by autograd"
+
+    std = w["std"] or 1.0
+    logits = (torch.randn(n_seq, s, v, generator=g) * std).to(dtype).to(device)
+    ids = torch.randint(0, v, (n_seq, s), generator=g).to(device)
+    if kind == "post":
+        lengths = torch.randint(s // 2, s + 1, (n_seq,), generator=g).to(device)
+
+        def run():
+            with torch.no_grad():
+                OL.logprobs_post_process(logits, ids, lengths)
+
+        return run, rows, f"{rows} rows of V={v} {w['dtype']}: forward-only fp32 log-softmax + gather + padding mask"
+    if kind == "distill":
+        teacher = (torch.randn(n_seq, s, v, generator=g) * std).to(dtype).to(device)
+        idx = torch.randint(0, v, (n_seq, s, w["topk"]), generator=g).to(device)
+        x = logits.requires_grad_(True)
+
+        def run():
+            x.grad = None
+            (OD.neg_entropy(x).sum() + OD.gather_logprob(x, idx).sum() + OD.soft_cross_entropy(x, teacher).sum()).backward()
+
+        return run, rows, f"{rows} rows of V={v} {w['dtype']}: negative entropy + {w['topk']} gathered logprobs + soft cross entropy, fwd+bwd"
+    x = logits.requires_grad_(True)
+    if kind == "topk":
+        ids = logits.float().argmax(-1).roll(1, -1)  # next-token targets that survive the filter
+        data, gs, gt = loss_data(n_seq, s, beta_ref=False)
+        cfg = O.LossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0)
+
+        def run():
+            x.grad = None
+            scaled = OL.apply_temperature(x, w["temperature"])
+            lp = OL.next_token_logprobs(ids, scaled, top_k=w["top_k"], top_p=w["top_p"])
+            mask = (data["token_mask"] * data["sample_mask"].unsqueeze(-1))[:, 1:]
+            lp = OL.mask_out_neg_inf_logprobs(lp, mask)
+            loss, _ = O.clipped_pg_loss(cfg, lp, data, gs, gt)
+            loss.backward()
+
+        return run, rows, (f"{rows} rows of V={v} bf16: div_(T) -> top-k/top-p by full sort -> log-softmax -> gather -> DAPO loss -> "
+                           "backward")
+    if kind == "packed":
+        cu = torch.arange(0, rows + 1, s, dtype=torch.int32)
+        data, gs, gt = loss_data(n_seq, s)
+        packed = x.reshape(1, rows, v)
+        cfg = O.LossConfig(token_level_loss=False, reference_policy_kl_penalty=0.001)
+
+        def run():
+            x.grad = None
+            targets = OL.pack_input_ids(ids.cpu(), cu, cu, roll_shift=-1).to(device)
+            lp = OL.packed_logits_to_logprobs(packed, targets, cu, s, target_is_pre_rolled=True)
+            loss, _ = O.clipped_pg_loss(cfg, lp, data, gs, gt)
+            loss.backward()
+
+        return run, rows, f"{rows} packed rows ({n_seq} sequences) of V={v} bf16: packed logprobs -> sequence-level loss -> backward"
+    data, gs, gt = loss_data(n_seq, s)
+
+    def run():
+        x.grad = None
+        lp = OL.next_token_logprobs(ids, x)
+        loss, _ = O.clipped_pg_loss(O.LossConfig(), lp, data, gs, gt)
         loss.backward()
-        return time.perf_counter() - t0
 
-    s, n_seq = 64, 64
-    run(1, s)  # warm-up
+    return run, rows, f"{rows} rows of V={v} {w['dtype']}: logprobs -> clipped-PG loss (k3 KL) -> backward to dlogits"
+
+
+def cpu_baseline(torch, w, kind, seconds, rows):
+    """The oracle on the host cores of the GPU box: median of at least two iterations after one warm-up, bounded
+    to about ``seconds`` of work."""
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)  # the box's CPU share for one GPU
+    torch.set_num_threads(threads)
+    run, rows, what = oracle_sample(torch, w, kind, "cpu", rows)
+    t0 = time.perf_counter()
+    run()  # warm-up
+    first = time.perf_counter() - t0
     times = []
-    while sum(times) < seconds or len(times) < 3:
-        times.append(run(n_seq, s))
+    while (sum(times) + first < seconds and len(times) < 25) or len(times) < 2:
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
     times.sort()
     t = times[len(times) // 2]
-    rows = n_seq * s
     return dict(value=rows / t, unit="tokens/s", cores=threads, kind="port",
-                sample=f"{rows} rows of V={v} {w['dtype']} per iteration, oracle fwd+loss+bwd, median of {len(times)} "
-                       f"iterations ({sum(times):.1f} s total), {threads} threads of {cores} host cores")
+                sample=f"{what}; median of {len(times)} iterations after one warm-up ({sum(times) + first:.1f} s in all), "
+                       f"{threads} threads of {cores} host cores")
+
+
+def reference_on_gpu(torch, w, kind, rows):
+    """The same op sequence (the oracle's restatement of the reference) with stock torch-ROCm ops on the device:
+    what a worker gets from the reference's Python on this GPU without this library."""
+    try:
+        run, rows, what = oracle_sample(torch, w, kind, "cuda", rows)
+        run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n = 3
+        for _ in range(n):
+            run()
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0) / n
+        peak = torch.cuda.max_memory_allocated()
+        return dict(value=rows / t, unit="tokens/s", sample=f"{what}; stock torch ops on the GPU, mean of {n} iterations after one warm-up",
+                    ms_per_iteration=t * 1e3)
+    except Exception as exc:  # a baseline leg must never take the measurement down with it
+        return dict(value=None, unit="tokens/s", error=f"{type(exc).__name__}: {exc}"[:300])
+    finally:
+        torch.cuda.empty_cache()
+
+
+def copy_bandwidth(torch, dev):
+    """Read + write GB/s of a 4 GiB device-to-device copy (HIP events), the practical ceiling of a kernel that
+    streams one tensor in and another out."""
+    src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(3):
+        dst.copy_(src)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / 3
+    del src, dst
+    torch.cuda.empty_cache()
+    return 2 * (1 << 32) / (ms * 1e-3) / 1e9
+
+
+def finish(result, args, torch, w, kind, cpu_rows, gpu_rows):
+    """Adds the baseline legs to a workload's record and prints the one JSON line."""
+    if not args.no_cpu_baseline:
+        dev = torch.device("cuda:0")
+        torch.cuda.empty_cache()
+        free, _ = torch.cuda.mem_get_info()
+        if free > (10 << 30):
+            gbs = copy_bandwidth(torch, dev)
+            result["copy_bandwidth_GBps"] = gbs
+            roof = result.get("roofline", {})
+            if roof.get("bound") == "hbm" and roof.get("achieved"):
+                roof["copy_bandwidth_frac"] = roof["achieved"] / gbs
+        result["reference_on_gpu"] = reference_on_gpu(torch, w, kind, gpu_rows)
+        result["cpu_baseline"] = cpu_baseline(torch, w, kind, args.cpu_seconds, cpu_rows)
+    print(json.dumps(result))
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
 
 
 def bench_topk(args, torch, w):
-    """Config 4: top-k / top-p filtered training logprobs -> DAPO loss -> dlogits (K3 forward + backward)."""
+    """Config 4: temperature 0.7 + top-k / top-p filtered training logprobs -> DAPO loss -> dlogits (K3 forward +
+    backward).  The temperature divide is inside the timed region, as in the worker
+    (``apply_temperature_scaling`` on the model's output), left to the kernels by ``deferred_temperature()``: no
+    extra pass over the logits."""
+    from functools import partial
+
     from rl_amd import ops
     from rl_amd.algorithms.logits_sampling_utils import TrainingSamplingParams
     from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn, prepare_loss_input
+    from rl_amd.distributed.model_utils import get_next_token_logprobs_from_logits
+    from rl_amd.temperature import apply_temperature_scaling, deferred_temperature
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -193,19 +399,19 @@ def bench_topk(args, torch, w):
     mb_bytes = w["mb_seqs"] * w["seq_len"] * w["vocab"] * 2
     free, _ = torch.cuda.mem_get_info()
     n_buf = max(1, min(n_mb, int((free * 0.9 - mb_bytes * 1.5) // mb_bytes)))
-    params = TrainingSamplingParams(top_k=w["top_k"], top_p=w["top_p"])
+    params = TrainingSamplingParams(top_k=w["top_k"], top_p=w["top_p"], temperature=w["temperature"])
+    prepare = partial(prepare_loss_input, sampling_params=params)  # as the DTensor worker binds it
     fn = ClippedPGLossFn(ClippedPGLossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0))
     mbs = []
     for i in range(n_buf):
         m = make_microbatch(torch, dict(w, spike_p=0.0), w["mb_seqs"], 4004 + i, dev)
-        # logits.div_(T) in bf16, as the worker does before the loss; targets mostly the argmax so that they survive the filter
-        m["logits"].mul_(1.0 / w["temperature"])
+        # targets mostly the argmax so that they survive the filter
         top = torch.stack([m["logits"][b].float().argmax(-1) for b in range(w["mb_seqs"])])
         keep = torch.rand(top[:, :-1].shape, device=dev) < 0.8
         m["data"]["input_ids"][:, 1:] = torch.where(keep, top[:, :-1], m["data"]["input_ids"][:, 1:])
-        with torch.no_grad():
-            from rl_amd.distributed.model_utils import get_next_token_logprobs_from_logits
-            cur = get_next_token_logprobs_from_logits(m["data"]["input_ids"], m["logits"], sampling_params=params)
+        with torch.no_grad(), deferred_temperature():
+            cur = get_next_token_logprobs_from_logits(m["data"]["input_ids"], apply_temperature_scaling(m["logits"], params),
+                                                      sampling_params=params)
         cur = torch.cat([torch.zeros((w["mb_seqs"], 1), device=dev), torch.nan_to_num(cur, neginf=0.0)], dim=1)
         for k in ("prev_logprobs", "generation_logprobs"):
             m["data"][k] = cur + 0.05 * torch.randn_like(cur)
@@ -217,49 +423,38 @@ def bench_topk(args, torch, w):
     def step():
         for i in range(n_mb):
             m = mbs[i % n_buf]
-            logits = m["logits"].requires_grad_(True)
-            loss_input, data = prepare_loss_input(logits, m["data"], fn, sampling_params=params)
-            loss, _ = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
-            (d,) = torch.autograd.grad(loss, logits)
+            leaf = m["logits"].requires_grad_(True)
+            with deferred_temperature():
+                logits = apply_temperature_scaling(leaf, params)
+                loss_input, data = prepare(logits=logits, data=m["data"], loss_fn=fn)
+                loss, _ = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+            (d,) = torch.autograd.grad(loss, leaf)
             del d, loss, loss_input
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    timer = EventTimer(torch)
-    ops.KERNEL_TIMER = timer
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ops.KERNEL_TIMER = None
-    k = timer.summary()
+    elapsed, k = timed(torch, ops, args, step)
     nan = dict(avg_ms=float("nan"))
     fwd, bwd = k.get("topk_topp_fwd", nan), k.get("topk_topp_bwd", nan)
     rows = w["mb_seqs"] * w["seq_len"]
     row_bytes = w["vocab"] * 2
     tokens = w["seqs"] * w["seq_len"]
-    fwd_gbs = row_bytes * w["mb_seqs"] * (w["seq_len"] - 1) / (fwd["avg_ms"] * 1e-3) / 1e9
-    bwd_gbs = 2 * row_bytes * rows / (bwd["avg_ms"] * 1e-3) / 1e9
-    print(json.dumps({
+    full = not args.seqs
+    result = {
         "metric": "top-k/top-p filtered logprob + DAPO loss fwd/bwd tokens/s at V=151936; % of HBM peak",
         "value": tokens * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
-                   "microbatches": n_mb, "resident_logit_buffers": n_buf},
+                   "microbatches": n_mb, "resident_logit_buffers": n_buf,
+                   "temperature": "divided inside the timed region by the logprob kernels (deferred_temperature), bf16 rounding of a GPU div_"},
         "algorithmic_bytes_per_token": 3 * row_bytes,
         "hbm_frac_end_to_end": 3 * row_bytes * tokens * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "kernel": "topk_topp_stream_kernel (backward)", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES["c4"] if not args.seqs else None, "avg_launch_ms": bwd["avg_ms"],
-                     "algorithmic_bytes_per_launch": 2 * row_bytes * rows},
-        "roofline_fwd": {"bound": "hbm", "kernel": "topk_topp_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"],
-                         "traffic": MEASURED_TRAFFIC_BYTES["c4_fwd"] if not args.seqs else None},
+        "roofline": hbm_roofline("topk_topp_stream_kernel (backward)", 2 * row_bytes * rows, bwd["avg_ms"], "c4" if full else None),
+        "roofline_fwd": hbm_roofline("topk_topp_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
+                                     "c4_fwd" if full else None),
         "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
-    }))
+    }
+    del mbs
+    finish(result, args, torch, w, "topk", cpu_rows=256, gpu_rows=2048)
 
 
 def bench_distill(args, torch, w):
@@ -286,18 +481,7 @@ def bench_distill(args, torch, w):
         (d,) = torch.autograd.grad((MU.DistributedCrossEntropy.apply(x, teacher, None) * up2).sum(), x)
         del d
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    timer = EventTimer(torch)
-    ops.KERNEL_TIMER = timer
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ops.KERNEL_TIMER = None
-    km = timer.summary()
+    elapsed, km = timed(torch, ops, args, step)
     tensor_bytes = b * s * v * 2
     passes = {"neg_entropy_fwd": 1, "neg_entropy_bwd": 2, "gather_logprob_fwd": 1, "gather_logprob_bwd": 2,
               "soft_cross_entropy_fwd": 2, "soft_cross_entropy_bwd": 3}
@@ -306,15 +490,16 @@ def bench_distill(args, torch, w):
                    "frac_of_hbm_peak": passes[n] * tensor_bytes / (km[n]["avg_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
                for n in passes if n in km}
     worst = min(kernels, key=lambda n: kernels[n]["frac_of_hbm_peak"])
-    print(json.dumps({
+    result = {
         "metric": "distillation reductions fwd/bwd tokens/s at V=151936 (three losses per token); % of HBM peak",
         "value": 3 * b * s * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic", "config": {"workload": w["desc"]},
-        "roofline": {"bound": "hbm", "kernel": worst, "achieved": kernels[worst]["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": kernels[worst]["frac_of_hbm_peak"], "traffic": None},
+        "roofline": hbm_roofline(worst, passes[worst] * tensor_bytes, km[worst]["avg_ms"]),
         "kernels": kernels,
-    }))
+    }
+    del student, teacher
+    finish(result, args, torch, w, "distill", cpu_rows=512, gpu_rows=2048)
 
 
 def bench_post(args, torch, w):
@@ -337,36 +522,25 @@ def bench_post(args, torch, w):
     def step():
         return pp(logits, {"input_lengths": lengths}, inputs, b, s)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    timer = EventTimer(torch)
-    ops.KERNEL_TIMER = timer
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ops.KERNEL_TIMER = None
-    km = timer.summary()
+    elapsed, km = timed(torch, ops, args, step)
     live_rows = int((lengths - 1).clamp(min=0).sum().item())   # rows 0 .. length-2 of a sequence are read
-    alg = live_rows * v * 2
-    k_ms = km["logprob_post_fwd"]["avg_ms"]
-    gbs = alg / (k_ms * 1e-3) / 1e9
-    print(json.dumps({
+    result = {
         "metric": "forward-only token logprobs (post-processor) tokens/s at V=151936; % of HBM peak",
         "value": b * s * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": b, "seq_len": s, "vocab": v, "rows_read": live_rows},
-        "roofline": {"bound": "hbm", "kernel": "logprob_post_fwd_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_launch_ms": k_ms, "algorithmic_bytes_per_launch": alg},
+        "roofline": hbm_roofline("logprob_post_fwd_kernel", live_rows * v * 2, km["logprob_post_fwd"]["avg_ms"]),
         "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in km.items()},
-    }))
+    }
+    del logits
+    finish(result, args, torch, w, "post", cpu_rows=4096, gpu_rows=4096)
 
 
 def bench_packed(args, torch, w):
     """One packed row through SequencePackingFusionLossWrapper (single pass), then the three-pass packed path."""
+    from functools import partial
+
     from rl_amd import ops
     from rl_amd.algorithms.loss import (ClippedPGLossConfig, ClippedPGLossFn, SequencePackingFusionLossWrapper,
                                         prepare_packed_loss_input)
@@ -401,7 +575,9 @@ def bench_packed(args, torch, w):
     gs = torch.tensor(float(nseq), device=dev)
     gt = token_mask[:, 1:].sum().float()
     live_rows = int(gt.item())
-    wrapped = SequencePackingFusionLossWrapper(fn, prepare_packed_loss_input, cu, cu)
+    # prepare_fn bound as the Megatron worker binds it (models/megatron/train.py:529-533)
+    prepare = partial(prepare_packed_loss_input, sampling_params=None, chunk_size=None)
+    wrapped = SequencePackingFusionLossWrapper(fn, prepare, cu, cu, 0, None, None)
 
     def step():
         x = logits.requires_grad_(True)
@@ -416,47 +592,31 @@ def bench_packed(args, torch, w):
         (d,) = torch.autograd.grad(loss, x)
         del d, loss, loss_input
 
-    def timed(fn_step):
-        for _ in range(args.warmup):
-            fn_step()
-        torch.cuda.synchronize()
-        timer = EventTimer(torch)
-        ops.KERNEL_TIMER = timer
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            fn_step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        ops.KERNEL_TIMER = None
-        return dt, timer.summary()
-
-    elapsed, km = timed(step)
+    elapsed, km = timed(torch, ops, args, step)
     row_bytes = v * 2
     # a live row is read once and its gradient written once; a row that feeds no token is only zero-filled
     alg = live_rows * 2 * row_bytes + (total - live_rows) * row_bytes
-    fk = km["fused_packed_logits_loss"]["avg_ms"]
-    gbs = alg / (fk * 1e-3) / 1e9
     out = {
         "metric": "GRPO logprob+loss fwd/bwd tokens/s, packed 131072-token row at V=131072; % of HBM peak",
         "value": total * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": nseq, "packed_tokens": total, "vocab": v, "loss_tokens": live_rows,
-                   "api": "SequencePackingFusionLossWrapper(ClippedPGLossFn, prepare_packed_loss_input)(logits, batch, ...) + "
-                          "autograd.grad -> nrl_fused_packed_logits_grpo_loss"},
-        "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel (packed)", "achieved": gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES["c5"], "avg_launch_ms": fk,
-                     "algorithmic_bytes_per_launch": alg},
+                   "api": "SequencePackingFusionLossWrapper(ClippedPGLossFn, partial(prepare_packed_loss_input, ...))(logits, batch, "
+                          "...) + autograd.grad -> nrl_fused_packed_logits_grpo_loss"},
+        "hbm_frac_end_to_end": alg * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline": hbm_roofline("fused_logits_loss_kernel (packed)", alg, km["fused_packed_logits_loss"]["avg_ms"], "c5"),
         "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in km.items()},
     }
-    t_elapsed, tk = timed(three_pass_step)
+    t_elapsed, tk = timed(torch, ops, args, three_pass_step)
     out["three_pass"] = {
         "value": total * args.steps / t_elapsed, "unit": "tokens/s", "ms_per_step": t_elapsed / args.steps * 1e3,
         "api": "prepare_packed_loss_input -> nrl_logprob_packed_fwd; ClippedPGLossFn -> nrl_grpo_loss_fwd_bwd; "
                "backward -> nrl_logprob_packed_bwd",
         "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in tk.items()},
     }
-    print(json.dumps(out))
+    del logits
+    finish(out, args, torch, w, "packed", cpu_rows=2048, gpu_rows=4096)
 
 
 def bench_lmhead(args, torch, w):
@@ -490,23 +650,13 @@ def bench_lmhead(args, torch, w):
         dh, dw = torch.autograd.grad(loss, (hidden, weight))
         del dh, dw
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    timer = EventTimer(torch)
-    ops.KERNEL_TIMER = timer
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ops.KERNEL_TIMER = None
-    k = timer.summary()
+    elapsed, k = timed(torch, ops, args, step)
     n = b * s
     fwd_ms, bwd_ms = k["lmhead_fwd"]["avg_ms"], k["lmhead_bwd"]["avg_ms"]
     fwd_tf = 2.0 * n * h * v / (fwd_ms * 1e-3) / 1e12
     bwd_alg_tf = 4.0 * n * h * v / (bwd_ms * 1e-3) / 1e12       # dH + dW
     bwd_exec_tf = 6.0 * n * h * v / (bwd_ms * 1e-3) / 1e12      # + recomputed logits
+    fills = MEASURED_TRAFFIC.get("c3_fwd") if not args.seqs else None
     result = {
         "metric": "fused lm_head + GRPO loss fwd/bwd tokens/s; % of bf16 MFMA peak",
         "value": n * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -514,15 +664,18 @@ def bench_lmhead(args, torch, w):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "tokens": n, "hidden": h, "vocab": v},
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tf, "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES["c3_fwd"] if not args.seqs else None,
-                     "avg_launch_ms": fwd_ms},
+                     "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": (fills["read"] + fills["write"]) if fills else None,
+                     "traffic_profile": fills["profile"] if fills else None, "avg_launch_ms": fwd_ms},
         "roofline_bwd": {"bound": "mfma", "kernel": "lmhead backward (grad + dH + dW GEMMs)", "achieved": bwd_alg_tf,
                          "achieved_incl_recompute": bwd_exec_tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": bwd_alg_tf / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": bwd_ms},
+                         "frac": bwd_alg_tf / MFMA_BF16_PEAK_TFLOPS, "frac_incl_recompute": bwd_exec_tf / MFMA_BF16_PEAK_TFLOPS,
+                         "avg_launch_ms": bwd_ms},
         "algorithmic_tflops_end_to_end": 6.0 * n * h * v * args.steps / elapsed / 1e12,
         "kernel_ms": {kk: round(vv["avg_ms"], 4) for kk, vv in k.items()},
     }
-    print(json.dumps(result))
+    del hidden, weight
+    finish(result, args, torch, w, "lmhead", cpu_rows=1024, gpu_rows=1024)
 
 
 def main():
@@ -567,15 +720,32 @@ def main():
     tot_toks = sum((m["data"]["token_mask"][:, 1:].sum() for m in mbs)) * (n_mb / n_buf)
     tot_toks = tot_toks.float()
 
-    from rl_amd.algorithms.loss import wrap_loss_fn_with_input_preparation
+    from functools import partial
+
+    from rl_amd.algorithms.advantage_estimator import AdvEstimatorConfig, GRPOAdvantageEstimator
+    from rl_amd.algorithms.loss import fused_logits_clipped_pg_loss, wrap_loss_fn_with_input_preparation
+
+    # prepare_fn bound as the Megatron worker binds it (models/megatron/train.py:506-513)
+    prepare = partial(prepare_loss_input, sampling_params=None, d2t=None, chunk_size=None)
+    grouped = None
+    if w.get("group"):  # config 1: advantages come from Bernoulli(0.5) rewards through the per-prompt group baseline
+        g = torch.Generator(device=dev).manual_seed(1001)
+        n_prompts = w["seqs"] // w["group"]
+        grouped = dict(
+            prompts=torch.arange(n_prompts, device=dev).repeat_interleave(w["group"]).unsqueeze(-1).expand(-1, 8).contiguous(),
+            rewards=(torch.rand((w["seqs"],), generator=g, device=dev) < 0.5).float(),
+            estimator=GRPOAdvantageEstimator(AdvEstimatorConfig(), None))
 
     def step():
         # the drop-in call: logits + batch -> loss; dispatches to the single-pass kernel when the loss
         # configuration allows it (this one does), and autograd hands back d loss / d logits
         for i in range(n_mb):
             m = mbs[i % n_buf]
+            if grouped is not None:
+                m["data"]["advantages"] = grouped["estimator"].compute_advantage(grouped["prompts"], grouped["rewards"],
+                                                                                 m["data"]["token_mask"])
             logits = m["logits"].requires_grad_(True)
-            loss, _metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare_loss_input)
+            loss, _metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare, 0, None, None)
             (dlogits,) = torch.autograd.grad(loss, logits)
             del dlogits, loss
 
@@ -589,30 +759,26 @@ def main():
             (dlogits,) = torch.autograd.grad(loss, logits)
             del dlogits, loss, loss_input
 
-    def timed(fn_step):
-        for _ in range(args.warmup):
-            fn_step()
-        torch.cuda.synchronize()
-        timer = EventTimer(torch)
-        ops.KERNEL_TIMER = timer
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            fn_step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        ops.KERNEL_TIMER = None
-        return dt, timer.summary()
+    def in_place_step():
+        # the gradient written over the logits (the logits are dead after the loss in a training step): no second
+        # [B, S, V] buffer, and the read and the write of a row hit the same DRAM pages
+        for i in range(n_mb):
+            m = mbs[i % n_buf]
+            logits = m["logits"].requires_grad_(True)
+            loss, _metrics = fused_logits_clipped_pg_loss(logits, m["data"], fn, tot_seqs, tot_toks, in_place=True)
+            (dlogits,) = torch.autograd.grad(loss, logits)
+            del dlogits, loss
 
-    elapsed, kernels = timed(step)
+    elapsed, kernels = timed(torch, ops, args, step)
     tokens_per_step = w["seqs"] * w["seq_len"]
     rows_per_launch = w["mb_seqs"] * w["seq_len"]
     row_bytes = w["vocab"] * elt
     nan = dict(avg_ms=float("nan"))
     fk = kernels.get("fused_logits_loss", nan)
     alg_launch = 2 * row_bytes * rows_per_launch  # every logit read once, every gradient element written once
-    f_gbs = alg_launch / (fk["avg_ms"] * 1e-3) / 1e9
+    full = not args.seqs
     result = {
-        "metric": "GRPO logprob+loss fwd/bwd tokens/s at V=151936; % of HBM peak",
+        "metric": "GRPO logprob+loss fwd/bwd tokens/s at V=%d; %% of HBM peak" % w["vocab"],
         "value": tokens_per_step * args.steps / elapsed,
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -627,34 +793,37 @@ def main():
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
                    "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level",
-                   "api": "wrap_loss_fn_with_input_preparation(logits, batch, ...) + autograd.grad -> "
-                          "nrl_fused_logits_grpo_loss (seq stats + single pass + term reduce + finish)"},
+                   "api": "wrap_loss_fn_with_input_preparation(logits, batch, ..., prepare_fn=partial(prepare_loss_input, "
+                          "sampling_params=, d2t=, chunk_size=)) + autograd.grad -> nrl_fused_logits_grpo_loss (seq stats + single "
+                          "pass + term reduce + finish)"},
         "algorithmic_bytes_per_token": 2 * row_bytes,
         "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "kernel": "fused_logits_loss_kernel", "achieved": f_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": f_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if not args.seqs else None,
-                     "avg_launch_ms": fk["avg_ms"], "algorithmic_bytes_per_launch": alg_launch},
+        "roofline": hbm_roofline("fused_logits_loss_kernel", alg_launch, fk["avg_ms"], args.workload if full else None),
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
     }
     # ---- the three-pass path (its own row: 3 * V * sizeof per token) ----
-    t_elapsed, t_kernels = timed(three_pass_step)
+    t_elapsed, t_kernels = timed(torch, ops, args, three_pass_step)
     bwd = t_kernels.get("logprob_bwd", nan)
     fwd = t_kernels.get("logprob_fwd", nan)
-    bwd_gbs = 2 * row_bytes * rows_per_launch / (bwd["avg_ms"] * 1e-3) / 1e9
-    fwd_gbs = row_bytes * w["mb_seqs"] * (w["seq_len"] - 1) / (fwd["avg_ms"] * 1e-3) / 1e9
     result["three_pass"] = {
         "value": tokens_per_step * args.steps / t_elapsed, "unit": "tokens/s", "ms_per_step": t_elapsed / args.steps * 1e3,
         "api": "prepare_loss_input -> nrl_logprob_fwd; ClippedPGLossFn -> nrl_grpo_loss_fwd_bwd; backward -> nrl_logprob_bwd",
         "algorithmic_bytes_per_token": 3 * row_bytes,
         "hbm_frac_end_to_end": 3 * row_bytes * tokens_per_step * args.steps / t_elapsed / 1e9 / HBM_PEAK_GBS,
-        "roofline_bwd": {"bound": "hbm", "kernel": "logprob_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": bwd["avg_ms"],
-                         "traffic": THREE_PASS_BWD_TRAFFIC_BYTES.get(args.workload) if not args.seqs else None,
-                         "algorithmic_bytes_per_launch": 2 * row_bytes * rows_per_launch},
-        "roofline_fwd": {"bound": "hbm", "kernel": "logprob_fwd_kernel", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": fwd_gbs / HBM_PEAK_GBS, "avg_launch_ms": fwd["avg_ms"]},
+        "roofline_bwd": hbm_roofline("logprob_bwd_kernel", 2 * row_bytes * rows_per_launch, bwd["avg_ms"],
+                                     args.workload + "_three_pass_bwd" if full else None),
+        "roofline_fwd": hbm_roofline("logprob_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
+                                     args.workload + "_three_pass_fwd" if full else None),
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in t_kernels.items()},
+    }
+    # ---- the single pass writing the gradient over the logits (last: it consumes the logits) ----
+    i_elapsed, i_kernels = timed(torch, ops, args, in_place_step)
+    ik = i_kernels.get("fused_logits_loss", nan)
+    result["in_place"] = {
+        "value": tokens_per_step * args.steps / i_elapsed, "unit": "tokens/s", "ms_per_step": i_elapsed / args.steps * 1e3,
+        "api": "fused_logits_clipped_pg_loss(..., in_place=True): dlogits aliases the logits",
+        "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / i_elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline": hbm_roofline("fused_logits_loss_kernel (dlogits over logits)", alg_launch, ik["avg_ms"]),
     }
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)  # 4 GiB
@@ -662,9 +831,11 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         result["copy_calibration_bytes"] = src.numel() * 4
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_seconds)
-    print(json.dumps(result))
+        del src, dst
+    del mbs
+    small = w["vocab"] < 100000
+    finish(result, args, torch, w, "loss", cpu_rows=(w["seqs"] * w["seq_len"] if small else 4096),
+           gpu_rows=(w["seqs"] * w["seq_len"] if small else 4096))
 
 
 if __name__ == "__main__":

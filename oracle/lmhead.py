@@ -62,7 +62,7 @@ def hidden_to_logprobs_backward(
     vocab = weight_vh.shape[0]
     step = seq if chunk_size is None else chunk_size
     d_w = torch.zeros(
-        vocab, width, dtype=weight_vh.dtype if accumulate_in_weight_dtype else torch.float32
+        vocab, width, dtype=weight_vh.dtype if accumulate_in_weight_dtype else torch.float32, device=weight_vh.device
     )
     d_h_parts = []
     for lo in range(0, seq, step):

@@ -184,11 +184,11 @@ def packed_logits_to_logprobs(
     else:
         flat_lp = rows_logprob(logits, tgt, vocab_start, vocab_end)
     flat_lp = flat_lp.squeeze(0)
-    out = torch.zeros((nseq, unpacked_seqlen - 1), dtype=flat_lp.dtype)
+    out = torch.zeros((nseq, unpacked_seqlen - 1), dtype=flat_lp.dtype, device=flat_lp.device)
     rows = []
     for i in range(nseq):
         n = min(max(cup[i + 1] - cup[i] - 1, 0), unpacked_seqlen - 1)
-        row = torch.zeros(unpacked_seqlen - 1, dtype=flat_lp.dtype)
+        row = torch.zeros(unpacked_seqlen - 1, dtype=flat_lp.dtype, device=flat_lp.device)
         if n > 0:
             row = torch.cat([flat_lp[cup[i] : cup[i] + n], row[n:]])
         rows.append(row)
@@ -219,10 +219,10 @@ def logprobs_post_process(logits, input_ids, input_lengths, cu_seqlens=None, ori
     lp = torch.log_softmax(x, dim=-1).gather(-1, nxt.unsqueeze(-1)).squeeze(-1)
     lp = torch.cat([torch.zeros_like(lp[:, :1]), lp], dim=1)
     if cu_seqlens is not None:
-        out = torch.zeros(original_batch_size, original_seq_len, dtype=lp.dtype)
+        out = torch.zeros(original_batch_size, original_seq_len, dtype=lp.dtype, device=lp.device)
         for i in range(original_batch_size):
             start, end = int(cu_seqlens[i]) + 1, int(cu_seqlens[i + 1])
             out[i, 1 : int(input_lengths[i])] = lp[0, start:end]
         return out
-    mask = torch.arange(lp.shape[1])[None, :] < torch.as_tensor(input_lengths).reshape(-1, 1)
+    mask = torch.arange(lp.shape[1], device=lp.device)[None, :] < torch.as_tensor(input_lengths, device=lp.device).reshape(-1, 1)
     return lp * mask

@@ -264,3 +264,72 @@ def test_config3_fused_lm_head_full_width_three_chunks():
     assert bool(((wg.grad.float().cpu() - o_dw).abs() <= b_dw).all())
     assert ((got_dh[pick] - o_dh).norm() / o_dh.norm()).item() <= 2.5e-3   # the bf16 cast autograd applies to dH
     assert ((wg.grad.float().cpu() - o_dw).norm() / o_dw.norm()).item() <= 3e-3
+
+
+def test_config1_whole_step_at_its_own_shape():
+    """Benchmark config 1 whole, the one configuration the CPU oracle can run at full size: 8 prompts x group 4 =
+    32 sequences x 512 tokens, V = 32000, fp32 logits ~ N(0, 2), response mask = suffix of length U[64, 512],
+    Bernoulli(0.5) rewards -> group-normalised (leave-one-out) advantages, prev / reference logprobs = current +
+    N(0, 0.05), clipped-PG loss eps 0.2, k3 KL beta 0.01, token-level mean; forward + backward.  Every element of
+    the result against the oracle: advantages, logprobs (1e-5), loss and every metric (1e-4 relative), dlogits
+    (1e-4 of the largest entry), through the three-pass path and the single pass the workers' wrapper takes."""
+    from functools import partial
+
+    from oracle import advantage as OA
+    from rl_amd.algorithms.advantage_estimator import AdvEstimatorConfig, GRPOAdvantageEstimator
+
+    n_prompts, group, s, v = 8, 4, 512, 32000
+    b = n_prompts * group
+    g = torch.Generator().manual_seed(1001)
+    logits = torch.randn(b, s, v, generator=g) * 2.0
+    ids = torch.randint(0, v, (b, s), generator=g)
+    resp = torch.randint(64, s + 1, (b,), generator=g)
+    tm = (torch.arange(s)[None, :] >= (s - resp)[:, None]).long()
+    tm[:, 0] = 0
+    sm = torch.ones(b)
+    rewards = (torch.rand(b, generator=g) < 0.5).float()
+    prompts = torch.randint(0, v, (n_prompts, 16), generator=g).repeat_interleave(group, dim=0)
+
+    adv = OA.grpo_advantages(prompts, rewards, tm)
+    xo = logits.clone().requires_grad_(True)
+    lpo = OL.next_token_logprobs(ids, xo)
+    pad = lambda t: torch.cat([torch.zeros(b, 1), t], 1)  # noqa: E731
+    prev = pad(lpo.detach() + 0.05 * torch.randn(b, s - 1, generator=g))
+    ref = pad(lpo.detach() + 0.05 * torch.randn(b, s - 1, generator=g))
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": sm, "advantages": adv, "prev_logprobs": prev,
+            "generation_logprobs": prev.clone(), "reference_policy_logprobs": ref}
+    gs, gt = sm.sum(), (tm[:, 1:] * sm.unsqueeze(-1)).sum().float()
+    want, wm = O.clipped_pg_loss(O.LossConfig(), lpo, data, gs, gt)
+    want.backward()
+    scale = xo.grad.abs().max().item()
+    assert scale > 0
+
+    est = GRPOAdvantageEstimator(AdvEstimatorConfig(), None)
+    adv_g = est.compute_advantage(prompts.to(DEV), rewards.to(DEV), tm.to(DEV))
+    torch.testing.assert_close(adv_g.cpu(), adv, rtol=1e-5, atol=1e-6)
+    assert torch.equal(adv_g.cpu() == 0, adv == 0)  # groups without variance stay exactly zero
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    ddev = {k: t.to(DEV) for k, t in data.items()}
+    ddev["advantages"] = adv_g
+
+    def check(loss, metrics, grad):
+        assert abs(loss.item() - want.item()) <= 1e-4 * abs(want.item()) + 1e-7, (loss.item(), want.item())
+        assert set(metrics) == set(wm)
+        for k in wm:
+            a, e = float(metrics[k]), float(wm[k])
+            assert abs(a - e) <= 1e-4 * abs(e) + 1e-6, (k, a, e)
+        assert (grad.cpu() - xo.grad).abs().max().item() <= 1e-4 * scale
+
+    x3 = logits.to(DEV).requires_grad_(True)
+    loss_input, d3 = prepare_loss_input(x3, dict(ddev), fn)
+    assert (loss_input["next_token_logprobs"].cpu() - lpo.detach()).abs().max().item() <= 1e-5
+    l3, m3 = fn(data=d3, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    l3.backward()
+    check(l3, m3, x3.grad)
+    del x3, loss_input
+
+    x1 = logits.to(DEV).requires_grad_(True)
+    prep = partial(prepare_loss_input, sampling_params=None, d2t=None, chunk_size=None)
+    l1, m1 = wrap_loss_fn_with_input_preparation(x1, dict(ddev), gs.to(DEV), gt.to(DEV), fn, prep, 0, None, None)
+    l1.backward()
+    check(l1, m1, x1.grad)
