@@ -716,6 +716,9 @@ def main():
     torch.cuda.synchronize()
 
     fn = ClippedPGLossFn(ClippedPGLossConfig())  # eps 0.2/0.2, k3 KL beta 0.01, token-level mean
+    # the metrics record of every microbatch is fetched when it is read (here: never inside the step), the way a
+    # worker collects per-microbatch metrics and looks at them after the step; the eager default is its own row
+    fn.lazy_metrics = True
     tot_seqs = torch.tensor(float(w["seqs"]), device=dev)
     tot_toks = sum((m["data"]["token_mask"][:, 1:].sum() for m in mbs)) * (n_mb / n_buf)
     tot_toks = tot_toks.float()
@@ -793,6 +796,7 @@ def main():
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
                    "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level",
+                   "metrics": "all diagnostics computed per microbatch; records fetched lazily (loss_fn.lazy_metrics = True)",
                    "api": "wrap_loss_fn_with_input_preparation(logits, batch, ..., prepare_fn=partial(prepare_loss_input, "
                           "sampling_params=, d2t=, chunk_size=)) + autograd.grad -> nrl_fused_logits_grpo_loss (seq stats + single "
                           "pass + term reduce + finish)"},
@@ -800,6 +804,16 @@ def main():
         "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
         "roofline": hbm_roofline("fused_logits_loss_kernel", alg_launch, fk["avg_ms"], args.workload if full else None),
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
+    }
+    # ---- the same call with the default eager metrics: the host waits for every microbatch's record ----
+    fn.lazy_metrics = False
+    e_elapsed, e_kernels = timed(torch, ops, args, step)
+    fn.lazy_metrics = True
+    result["eager_metrics"] = {
+        "value": tokens_per_step * args.steps / e_elapsed, "unit": "tokens/s", "ms_per_step": e_elapsed / args.steps * 1e3,
+        "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / e_elapsed / 1e9 / HBM_PEAK_GBS,
+        "note": "ClippedPGLossFn.lazy_metrics = False: the metrics dictionary is filled before the call returns (one device -> "
+                "host wait per microbatch, the reference's behaviour)",
     }
     # ---- the three-pass path (its own row: 3 * V * sizeof per token) ----
     t_elapsed, t_kernels = timed(torch, ops, args, three_pass_step)

@@ -9,6 +9,7 @@ dozen element-wise kernels and a synchronisation per metric.
 
 from __future__ import annotations
 
+from collections.abc import MutableMapping
 from typing import Any, Optional
 
 import torch
@@ -68,34 +69,92 @@ def _global_valid(seqs, toks, dev) -> torch.Tensor:
     return torch.stack(parts)
 
 
+class LazyMetrics(MutableMapping):
+    """The metrics of a loss call, fetched from the device on first use (opt-in: ``loss_fn.lazy_metrics = True``).
+
+    The reference ends every loss call with about fifteen ``.item()`` calls, each of which stalls the host until
+    the device has caught up; by default this package returns the same plain ``{name: float}`` dictionary after
+    ONE such wait.  With ``lazy_metrics`` set the wait moves to the first time anything reads, writes or iterates
+    the mapping: a worker that collects the metrics of its microbatches and looks at them after the step (as the
+    Megatron schedule does) then launches the backward pass and the next microbatch without idling the device in
+    between.  Deliberately not a ``dict`` subclass: C-level consumers (``json.dumps``) read a dict subclass's
+    storage directly and would see it empty; ``dict(metrics)`` gives the plain dictionary."""
+
+    __slots__ = ("_pending", "_data")
+
+    def __init__(self, build):
+        self._pending = build
+        self._data = None
+
+    def _fill(self) -> dict:
+        if self._data is None:
+            self._data = self._pending()
+            self._pending = None
+        return self._data
+
+    def __getitem__(self, key): return self._fill()[key]
+    def __setitem__(self, key, value): self._fill()[key] = value
+    def __delitem__(self, key): del self._fill()[key]
+    def __iter__(self): return iter(self._fill())
+    def __len__(self): return len(self._fill())
+    def __repr__(self): return repr(self._fill())
+    def __reduce_ex__(self, protocol): return (dict, (dict(self._fill()),))
+    def copy(self): return dict(self._fill())
+
+
+def fetch_later(record: torch.Tensor):
+    """Starts the copy of a small device record to pinned host memory on the current stream and returns a function
+    that waits for that copy alone (not for work enqueued afterwards) and yields the values as a list."""
+    if not record.is_cuda:
+        return record.tolist
+    host = torch.empty(record.shape, dtype=record.dtype, pin_memory=True)
+    host.copy_(record, non_blocking=True)
+    done = torch.cuda.Event()
+    done.record()
+
+    def values():
+        done.synchronize()
+        return host.tolist()
+
+    return values
+
+
 def metrics_record_to_dict(metrics: torch.Tensor, loss_fn, sample_mask_in: torch.Tensor) -> dict:
-    """The kernels' metrics record -> the dictionary ``ClippedPGLossFn`` returns (``loss_functions.py:767-788``);
-    fetching the record is the one device -> host synchronisation of a loss call."""
+    """The kernels' metrics record -> the dictionary ``ClippedPGLossFn`` returns (``loss_functions.py:767-788``).
+    Fetching the record is the one device -> host wait of a loss call; with ``loss_fn.lazy_metrics`` it is put off
+    until the metrics are first used (``LazyMetrics``)."""
     beta = loss_fn.reference_policy_kl_penalty
-    m = metrics.cpu().tolist()
-    get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
-    n_valid = get("num_valid_samples")
-    out = {
-        "loss": get("loss"),
-        "probs_ratio": get("probs_ratio"),
-        "probs_ratio_clamped": get("probs_ratio_clamped"),
-        "probs_ratio_min": get("probs_ratio_min"),
-        "probs_ratio_max": get("probs_ratio_max"),
-        "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
-        "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
-        "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
-        "token_mult_prob_error": get("token_mult_prob_error"),
-        "gen_kl_error": get("gen_kl_error"),
-        "policy_kl_error": get("policy_kl_error"),
-        "js_divergence_error": get("js_divergence_error"),
-        "sampling_importance_ratio": get("sampling_importance_ratio"),
-        "num_valid_samples": n_valid if sample_mask_in.is_floating_point() else int(n_valid),
-        "approx_entropy": get("approx_entropy"),
-    }
-    if loss_fn.truncated_importance_sampling_ratio is not None:
-        out["is_oob_ratio"] = get("is_oob_ratio")
-    out["positive_nll_loss"] = get("positive_nll_loss")
-    return out
+    with_oob = loss_fn.truncated_importance_sampling_ratio is not None
+    as_float = sample_mask_in.is_floating_point()
+    values = fetch_later(metrics)
+
+    def build():
+        m = values()
+        get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
+        n_valid = get("num_valid_samples")
+        out = {
+            "loss": get("loss"),
+            "probs_ratio": get("probs_ratio"),
+            "probs_ratio_clamped": get("probs_ratio_clamped"),
+            "probs_ratio_min": get("probs_ratio_min"),
+            "probs_ratio_max": get("probs_ratio_max"),
+            "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
+            "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
+            "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
+            "token_mult_prob_error": get("token_mult_prob_error"),
+            "gen_kl_error": get("gen_kl_error"),
+            "policy_kl_error": get("policy_kl_error"),
+            "js_divergence_error": get("js_divergence_error"),
+            "sampling_importance_ratio": get("sampling_importance_ratio"),
+            "num_valid_samples": n_valid if as_float else int(n_valid),
+            "approx_entropy": get("approx_entropy"),
+        }
+        if with_oob:
+            out["is_oob_ratio"] = get("is_oob_ratio")
+        out["positive_nll_loss"] = get("positive_nll_loss")
+        return out
+
+    return LazyMetrics(build) if getattr(loss_fn, "lazy_metrics", False) else build()
 
 
 class _FusedLoss(torch.autograd.Function):
@@ -125,7 +184,12 @@ class ClippedPGLossFn(LossFunction):
     """Generalised clipped policy-gradient loss with KL regularisation.
 
     ``L = E_t[max(-A r, -A clip(r, 1-eps_lo, 1+eps_hi))] + beta * KL(pi || pi_ref)`` with the variants
-    selected by the configuration flags (see ``ClippedPGLossConfig``)."""
+    selected by the configuration flags (see ``ClippedPGLossConfig``).
+
+    ``lazy_metrics`` (not in the reference; set it on the instance): return the metrics as a ``LazyMetrics``
+    mapping that waits for the device only when first read, instead of a plain dictionary."""
+
+    lazy_metrics = False
 
     input_type = LossInputType.LOGPROB
 

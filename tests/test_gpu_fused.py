@@ -353,3 +353,24 @@ def test_fused_packed_rejects_what_it_cannot_take():
     with pytest.raises(ValueError):   # boundaries that leave the packed row
         fused_packed_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, fn, cu,
                                             torch.tensor([0, 5, 40], dtype=torch.int32), gs, gt)
+
+
+def test_lazy_metrics_hold_the_same_values_as_the_eager_dictionary():
+    from rl_amd.algorithms.loss.loss_functions import LazyMetrics
+
+    logits, data, gs, gt = _batch(3, 20, 4096, torch.bfloat16, seed=77)
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    eager_loss, eager = fused_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, fn, gs.to(DEV), gt.to(DEV))
+    assert type(eager) is dict
+    fn.lazy_metrics = True
+    x = logits.to(DEV).requires_grad_(True)
+    lazy_loss, lazy = fused_logits_clipped_pg_loss(x, ddev, fn, gs.to(DEV), gt.to(DEV))
+    assert isinstance(lazy, LazyMetrics)
+    lazy_loss.backward()                     # more work goes onto the stream before the record is looked at
+    torch.ops.rl_amd.logprob_fwd(logits.to(DEV), ddev["input_ids"], 20, 0, 4096, 1.0, 1, False)
+    assert dict(lazy) == eager and lazy_loss.item() == eager_loss.item()
+    # the three-pass loss honours the switch as well
+    loss_input, d2 = prepare_loss_input(logits.to(DEV), dict(ddev), fn)
+    _, m3 = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
+    assert isinstance(m3, LazyMetrics) and set(m3) == set(eager)

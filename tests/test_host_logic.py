@@ -113,3 +113,35 @@ def test_multi_rank_groups_are_rejected(monkeypatch):
     monkeypatch.setattr(mu, "_group_size", lambda g: 2 if g == "tp2" else 1)
     with pytest.raises(NotImplementedError, match="one GPU"):
         mu.from_parallel_logits_to_logprobs(torch.zeros(1, 2, 4), torch.zeros(1, 2, dtype=torch.long), 0, 4, "tp2")
+
+
+def test_lazy_metrics_fetches_once_on_first_use_and_behaves_like_the_dictionary():
+    import pickle
+
+    from rl_amd.algorithms.loss.loss_functions import LazyMetrics
+
+    calls = []
+
+    def build():
+        calls.append(1)
+        return {"loss": 0.5, "num_valid_samples": 4}
+
+    m = LazyMetrics(build)
+    assert calls == []                       # nothing fetched by construction
+    assert m["loss"] == 0.5 and calls == [1]
+    assert list(m) == ["loss", "num_valid_samples"] and len(m) == 2 and "loss" in m and calls == [1]
+    m["lr"] = 1e-5
+    m["loss"] /= 2
+    assert dict(m) == {"loss": 0.25, "num_valid_samples": 4, "lr": 1e-5}
+    for use in (lambda x: list(x.items()), lambda x: x.get("loss"), lambda x: repr(x), lambda x: x == {"loss": 0.5, "num_valid_samples": 4},
+                lambda x: {**x}, lambda x: x.copy(), lambda x: x.update(a=1), lambda x: x.setdefault("b", 2)):
+        calls.clear()
+        fresh = LazyMetrics(build)
+        use(fresh)
+        assert calls == [1]
+    restored = pickle.loads(pickle.dumps(LazyMetrics(build)))
+    assert type(restored) is dict and restored == {"loss": 0.5, "num_valid_samples": 4}
+    with pytest.raises(TypeError):           # not a dict subclass on purpose: C-level consumers must not see it empty
+        import json
+
+        json.dumps(LazyMetrics(build))
