@@ -40,7 +40,24 @@ struct GemmOperands {
     const uint16_t* a;  // [M, K] row stride lda
     const uint16_t* b;  // [N, K] row stride ldb
     int64_t lda, ldb, m, n, k;  // k multiple of 8; slabs beyond k read as zero
+    // An extent that only the device knows (the number of tokens that carry a gradient): when `live` is set, the
+    // kernel replaces m (live_dim 1) or k (live_dim 2, rounded up to 64) by clamp(live[0] - live_from, 0, that
+    // extent) before it starts, and leaves at once when nothing is left.
+    const int32_t* live = nullptr;
+    int64_t live_from = 0;
+    int live_dim = 0;
 };
+
+// applies the device-side extent; false when the product is empty
+__device__ __forceinline__ bool resolve_live(GemmOperands& op) {
+    if (op.live) {
+        int64_t r = static_cast<int64_t>(op.live[0]) - op.live_from;
+        r = r < 0 ? 0 : r;
+        if (op.live_dim == 1) op.m = r < op.m ? r : op.m;
+        else { r = (r + 63) / 64 * 64; op.k = r < op.k ? r : op.k; }
+    }
+    return op.m > 0 && op.k > 0 && op.n > 0;
+}
 
 // accumulator element e (0..15) of lane l in a 32x32 tile: column l % 32, row 8*(e/4) + 4*(l/32) + e%4
 __device__ __forceinline__ int acc_row(int e, int lane) { return 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3); }
@@ -498,6 +515,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     __shared__ float lse_l[BM], g_l[BM];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    if (!resolve_live(a.op)) return;
     int64_t bx, by;
     if (!patch_tile(blockIdx.x, (a.op.m + BM - 1) / BM, (a.op.n + BN - 1) / BN, bx, by)) return;
     const int64_t row0 = bx * BM, col0 = by * BN;
@@ -670,17 +688,35 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
 // plain GEMM with fp32 output: C = A B^T or C += A B^T
 // ---------------------------------------------------------------------------------------------
 template <class Core, bool ACCUM>
-__global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, float* c, int64_t ldc) {
+__global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, float* c, int64_t ldc, const int32_t* row_map) {
     constexpr int NI = Core::NI, NJ = Core::NJ, BM = Core::BM, BN = Core::BN;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    if (!resolve_live(op)) return;
     int64_t bx, by;
     if (!patch_tile(blockIdx.x, (op.m + BM - 1) / BM, (op.n + BN - 1) / BN, bx, by)) return;
     const int64_t row0 = bx * BM, col0 = by * BN;
     f32x16 acc[NI][NJ];
     zero_acc<Core>(acc);
     Core::tile(op, row0, col0, acc, lds);
+    if (row_map) {
+        // rows of the product are scattered: row r of C goes to row row_map[r] of the output (plain store only)
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int64_t r = row0 + wm * 128 + i * 32 + acc_row(e, lane);
+                if (r >= op.m) continue;
+                float* out = c + static_cast<int64_t>(row_map[r]) * ldc;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+                    if (col < op.n) out[col] = acc[i][j][e];
+                }
+            }
+        return;
+    }
     // an interior tile takes the path without per-element bounds (no divergent branch between the loads)
     const bool interior = row0 + BM <= op.m && col0 + BN <= op.n;
     auto write_back = [&](auto interior_tag) {
@@ -727,6 +763,52 @@ __global__ __launch_bounds__(256) void lmhead_onehot_dh_kernel(float* dh, int64_
     for (int64_t c = threadIdx.x; c < h; c += 256) out[c] += g * bf16_bits_to_f32(wr[c]);
 }
 
+// Order-preserving list of the tokens whose upstream gradient is not zero (one workgroup walks the vector 1024
+// entries at a time: a wave's ballot and the waves' running counts give every kept token its slot).  Tokens with a
+// zero gradient contribute nothing to dH or dW, so the backward products run on the listed tokens only.
+__global__ __launch_bounds__(1024) void live_tokens_kernel(const float* grad, int64_t n, int32_t* idx, int32_t* count) {
+    __shared__ int wave_cnt[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int base = 0;
+    for (int64_t i0 = 0; i0 < n; i0 += 1024) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool keep = i < n && grad[i] != 0.0f;
+        const unsigned long long ballot = __ballot(keep);
+        if (lane == 0) wave_cnt[wave] = __popcll(ballot);
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            before += w < wave ? wave_cnt[w] : 0;
+            total += wave_cnt[w];
+        }
+        if (keep) idx[base + before + __popcll(ballot & ((1ull << lane) - 1ull))] = static_cast<int32_t>(i);
+        base += total;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *count = base;
+}
+
+// Row i of the compact operands is token idx[i] for i < count[0]; rows from count[0] on are zero (they pad the
+// last K slab of the dW product, where anything but zero would be multiplied into the result).
+__global__ __launch_bounds__(256) void gather_live_kernel(const uint16_t* hidden, int64_t ldh, int64_t h, const int64_t* targets,
+                                                         const float* lse, const float* grad, const int32_t* idx,
+                                                         const int32_t* count, int64_t n, uint16_t* hidden_c, int64_t* targets_c,
+                                                         float* lse_c, float* grad_c) {
+    const int64_t i = blockIdx.x;
+    const bool live = i < count[0];
+    const int64_t src = live ? idx[i] : 0;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const u32x4* in = reinterpret_cast<const u32x4*>(hidden + src * ldh);
+    u32x4* out = reinterpret_cast<u32x4*>(hidden_c + i * h);
+    for (int64_t v = threadIdx.x; v < h / 8; v += 256) out[v] = live ? in[v] : zero;
+    if (threadIdx.x == 0) {
+        targets_c[i] = live ? targets[src] : 0;
+        lse_c[i] = live ? lse[src] : 0.f;
+        grad_c[i] = live ? grad[src] : 0.f;
+    }
+}
+
 // dst[c, r] = src[r, c] for r < rows, c < cols; dst row stride ldd, columns [rows, pad_cols) zero-filled
 __global__ void transpose_bf16_kernel(const uint16_t* src, int64_t rows, int64_t cols, int64_t lds_, uint16_t* dst,
                                       int64_t ldd, int64_t pad_cols) {
@@ -748,6 +830,12 @@ __global__ void f32_to_bf16_kernel(const float* src, uint16_t* dst, int64_t n) {
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
          i += static_cast<int64_t>(gridDim.x) * blockDim.x)
         dst[i] = static_cast<uint16_t>(f32_to_bf16_bits(src[i]));
+}
+
+// one workgroup per row of a [rows, width] fp32 matrix with row stride ld
+__global__ __launch_bounds__(256) void fill_zero_rows_kernel(float* p, int64_t ld, int64_t width) {
+    float* row = p + static_cast<int64_t>(blockIdx.x) * ld;
+    for (int64_t c = threadIdx.x; c < width; c += 256) row[c] = 0.f;
 }
 
 __global__ void fill_zero_u32(uint32_t* p, int64_t n) {
@@ -803,13 +891,13 @@ template <class Core> static void launch_grad(const LmGradArgs& a, hipStream_t s
                                dim3(GB_THREADS), 0, s>>>(a);
 }
 
-template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, int64_t ldc, hipStream_t s) {
+template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, int64_t ldc, hipStream_t s, const int32_t* row_map = nullptr) {
     if (op.k % CoreB::BK == 0 && op.k > 0)
         gemm_f32_kernel<CoreB, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreB::BM - 1) / CoreB::BM, (op.n + CoreB::BN - 1) / CoreB::BN)),
-                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc);
+                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
     else
         gemm_f32_kernel<CoreA, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreA::BM - 1) / CoreA::BM, (op.n + CoreA::BN - 1) / CoreA::BN)),
-                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc);
+                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
 }
 
 extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
@@ -841,14 +929,17 @@ static constexpr int64_t kBwdChunk = 16384;
 static int64_t bwd_chunk(int64_t n) { return n < kBwdChunk ? round_up(n < 1 ? 1 : n, 64) : kBwdChunk; }
 
 extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab) {
-    const int64_t chunk = bwd_chunk(n_tokens), vp = round_up(vocab, 64);
+    const int64_t n = n_tokens < 1 ? 1 : n_tokens;
+    const int64_t chunk = bwd_chunk(n_tokens), vp = round_up(vocab, 64), n_pad = round_up(n, chunk);
     int64_t b = 0;
     b += hidden_size * vp * 2;        // W^T
     b += chunk * vp * 2;              // G
     b += vocab * chunk * 2;           // G^T
     b += hidden_size * chunk * 2;     // hidden chunk^T
     b += vocab * hidden_size * 4;     // dW accumulator (fp32)
-    return b + 1024;
+    b += n_pad * hidden_size * 2;     // hidden rows of the tokens that carry a gradient
+    b += n_pad * (8 + 4 + 4 + 4);     // their targets, log-sum-exps, gradients and token indices
+    return b + 2048;
 }
 
 extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
@@ -860,47 +951,74 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
     if (vocab_end - vocab_start != vocab) return fail(NRL_E_INVALID, "vocab range does not span the rows of W");
     if (!dweight_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
     if (n_tokens > 0 && (!lse || !grad || !dhidden_out)) return fail(NRL_E_INVALID, "null argument");
+    if (n_tokens >= (1ll << 31)) return fail(NRL_E_INVALID, "too many tokens");
+    if (ld_dh < hidden_size) return fail(NRL_E_INVALID, "ld_dh shorter than the hidden size");
     if (workspace_bytes < nrl_lmhead_bwd_workspace_bytes(n_tokens, hidden_size, vocab)) return fail(NRL_E_WORKSPACE, "workspace too small");
     if (reinterpret_cast<uintptr_t>(workspace) & 255) return fail(NRL_E_INVALID, "workspace must be 256-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t chunk = bwd_chunk(n_tokens), vp = round_up(vocab, 64), h = hidden_size;
+    const int64_t n_pad = round_up(n_tokens < 1 ? 1 : n_tokens, chunk);
     char* ws = static_cast<char*>(workspace);
-    uint16_t* wt = reinterpret_cast<uint16_t*>(ws); ws += h * vp * 2;
-    uint16_t* g = reinterpret_cast<uint16_t*>(ws); ws += chunk * vp * 2;
-    uint16_t* gt = reinterpret_cast<uint16_t*>(ws); ws += vocab * chunk * 2;
-    uint16_t* ht = reinterpret_cast<uint16_t*>(ws); ws += h * chunk * 2;
-    float* dw = reinterpret_cast<float*>(ws);
+    auto take = [&](int64_t bytes) { char* p = ws; ws += (bytes + 255) / 256 * 256; return p; };
+    uint16_t* wt = reinterpret_cast<uint16_t*>(take(h * vp * 2));
+    uint16_t* g = reinterpret_cast<uint16_t*>(take(chunk * vp * 2));
+    uint16_t* gt = reinterpret_cast<uint16_t*>(take(vocab * chunk * 2));
+    uint16_t* ht = reinterpret_cast<uint16_t*>(take(h * chunk * 2));
+    float* dw = reinterpret_cast<float*>(take(vocab * h * 4));
+    uint16_t* hid_c = reinterpret_cast<uint16_t*>(take(n_pad * h * 2));
+    int64_t* tgt_c = reinterpret_cast<int64_t*>(take(n_pad * 8));
+    float* lse_c = reinterpret_cast<float*>(take(n_pad * 4));
+    float* grad_c = reinterpret_cast<float*>(take(n_pad * 4));
+    int32_t* idx = reinterpret_cast<int32_t*>(take(n_pad * 4 + 256));
+    int32_t* count = idx + n_pad;
     const uint16_t* hid = static_cast<const uint16_t*>(hidden);
     const uint16_t* w = static_cast<const uint16_t*>(weight);
 
     // W^T [H, vp] (zero-padded columns) and a zeroed fp32 dW accumulator
     transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((vp + 63) / 64)), dim3(256), 0, s>>>(w, vocab, h, ldw, wt, vp, vp);
     fill_zero_u32<<<dim3(2048), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(dw), vocab * h);
+    if (n_tokens == 0) {
+        // (nothing to add to dW)
+    } else {
+        // Tokens with a zero upstream gradient (prompt tokens, masked samples, each sequence's dropped last position)
+        // have a zero row in G: the three products run on the other tokens only.  How many those are stays on the
+        // device; the launches are sized for all tokens and the workgroups beyond the live ones leave at once.
+        live_tokens_kernel<<<dim3(1), dim3(1024), 0, s>>>(grad, n_tokens, idx, count);
+        gather_live_kernel<<<dim3((unsigned)n_pad), dim3(256), 0, s>>>(hid, ldh, h, targets, lse, grad, idx, count, n_tokens, hid_c, tgt_c,
+                                                                        lse_c, grad_c);
+        for (int64_t r = 0; r < n_tokens; r += 65535)  // dH rows of the other tokens are zero
+            fill_zero_rows_kernel<<<dim3((unsigned)(n_tokens - r < 65535 ? n_tokens - r : 65535)), dim3(256), 0, s>>>(
+                dhidden_out + r * ld_dh, ld_dh, h);
+    }
 
     for (int64_t t0 = 0; t0 < n_tokens; t0 += chunk) {
-        const int64_t rows = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;
+        const int64_t rows = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;   // upper bound: the live rows of this chunk
         const int64_t rows_pad = round_up(rows, 64);
-        // G / G^T for this chunk
+        // G / G^T for this chunk of live tokens
         LmGradArgs ga;
-        ga.op.a = hid + t0 * ldh; ga.op.b = w; ga.op.lda = ldh; ga.op.ldb = ldw; ga.op.m = rows; ga.op.n = vocab; ga.op.k = h;
-        ga.targets = targets + t0; ga.vocab_start = vocab_start; ga.lse = lse + t0; ga.grad = grad + t0;
+        ga.op.a = hid_c + t0 * h; ga.op.b = w; ga.op.lda = h; ga.op.ldb = ldw; ga.op.m = rows; ga.op.n = vocab; ga.op.k = h;
+        ga.op.live = count; ga.op.live_from = t0; ga.op.live_dim = 1;
+        ga.targets = tgt_c + t0; ga.vocab_start = vocab_start; ga.lse = lse_c + t0; ga.grad = grad_c + t0;
         ga.g = g; ga.ldg = vp; ga.gt = gt; ga.ldgt = chunk;
-        if (rows_pad < chunk) fill_zero_u32<<<dim3(2048), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(gt), vocab * chunk / 2);
         if (h % CoreB::BK == 0) launch_grad<CoreB>(ga, s);
         else launch_grad<CoreA>(ga, s);
-        // dH[chunk] = G [rows, V] * (W^T [H, V])^T
+        // dH[token of row r] = G [rows, V] * (W^T [H, V])^T, written to the tokens' own rows
         GemmOperands dh;
         dh.a = g; dh.lda = vp; dh.b = wt; dh.ldb = vp; dh.m = rows; dh.n = h; dh.k = vp;
-        launch_gemm<false>(dh, dhidden_out + t0 * ld_dh, ld_dh, s);
-        lmhead_onehot_dh_kernel<<<dim3((unsigned)rows), dim3(256), 0, s>>>(dhidden_out + t0 * ld_dh, ld_dh, grad + t0, targets + t0,
-                                                                          vocab_start, vocab, w, ldw, h);
+        dh.live = count; dh.live_from = t0; dh.live_dim = 1;
+        launch_gemm<false>(dh, dhidden_out, ld_dh, s, idx + t0);
         // dW += G^T [V, rows] * (hidden^T [H, rows])^T
         transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((rows_pad + 63) / 64)), dim3(256), 0, s>>>(
-            hid + t0 * ldh, rows, h, ldh, ht, chunk, rows_pad);
+            hid_c + t0 * h, rows, h, h, ht, chunk, rows_pad);
         GemmOperands dwo;
         dwo.a = gt; dwo.lda = chunk; dwo.b = ht; dwo.ldb = chunk; dwo.m = vocab; dwo.n = h; dwo.k = rows_pad;
+        dwo.live = count; dwo.live_from = t0; dwo.live_dim = 2;
         launch_gemm<true>(dwo, dw, h, s);
     }
+    if (n_tokens > 0)  // the one-hot term of dH in fp32, on the tokens' own rows
+        for (int64_t r = 0; r < n_tokens; r += 65535)
+            lmhead_onehot_dh_kernel<<<dim3((unsigned)(n_tokens - r < 65535 ? n_tokens - r : 65535)), dim3(256), 0, s>>>(
+                dhidden_out + r * ld_dh, ld_dh, grad + r, targets + r, vocab_start, vocab, w, ldw, h);
     // narrow dW once
     {
         uint16_t* out = static_cast<uint16_t*>(dweight_out);
