@@ -116,3 +116,51 @@ def test_lmhead_equals_unfused_path_on_gpu():
     err = (fused - unfused).abs()
     assert (err <= 2e-3).float().mean().item() >= 0.99
     assert err.max().item() <= 1e-2
+
+
+def _bwd_through_the_op(hid2d, w, tgt, up_rows):
+    v = w.shape[0]
+    _, lse = torch.ops.rl_amd.lmhead_logprob_fwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), 0, v)
+    return torch.ops.rl_amd.lmhead_logprob_bwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), lse, up_rows.to(DEV), 0, v)
+
+
+@pytest.mark.parametrize("live", ["none", "one", "last_only"])
+def test_lmhead_backward_runs_on_live_tokens_only(live):
+    """The backward products run on the tokens with a non-zero upstream gradient (the others have a zero row in the
+    logits' gradient): no such token, a single one, and one at the very end."""
+    g = torch.Generator().manual_seed(5)
+    n, h, v = 300, 64, 1000
+    hid = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    w = (torch.randn(v, h, generator=g) * 0.05).to(torch.bfloat16)
+    tgt = torch.randint(0, v, (n,), generator=g)
+    up = torch.zeros(n)
+    if live == "one":
+        up[137] = 0.5
+    elif live == "last_only":
+        up[n - 1] = -0.25
+    dh, dw = _bwd_through_the_op(hid, w, tgt, up)
+    o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
+    if live == "none":
+        assert bool((dh == 0).all()) and bool((dw.float() == 0).all())
+        return
+    assert bool((dh.cpu()[up == 0] == 0).all())
+    assert bool(((dh.cpu() - o_dh).abs() <= b_dh).all()) and bool(((dw.float().cpu() - o_dw).abs() <= b_dw).all())
+
+
+def test_lmhead_backward_live_tokens_across_the_chunk_boundary():
+    """More live tokens than one backward chunk holds (16384), ending in a partial chunk whose length is not a
+    multiple of the 64-wide K slab; masked tokens scattered in between."""
+    g = torch.Generator().manual_seed(6)
+    n, h, v = 20011, 64, 520
+    hid = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    w = (torch.randn(v, h, generator=g) * 0.05).to(torch.bfloat16)
+    tgt = torch.randint(0, v, (n,), generator=g)
+    up = torch.randn(n, generator=g) * 1e-3
+    up[torch.rand(n, generator=g) < 0.1] = 0.0
+    assert 16384 < int((up != 0).sum()) < n and int((up != 0).sum()) % 64 != 0
+    dh, dw = _bwd_through_the_op(hid, w, tgt, up)
+    o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
+    assert bool((dh.cpu()[up == 0] == 0).all())
+    assert bool(((dh.cpu() - o_dh).abs() <= b_dh).all())
+    assert bool(((dw.float().cpu() - o_dw).abs() <= b_dw).all())
+    assert ((dh.cpu() - o_dh).norm() / o_dh.norm()).item() <= 1e-4
