@@ -402,6 +402,7 @@ def bench_topk(args, torch, w):
     params = TrainingSamplingParams(top_k=w["top_k"], top_p=w["top_p"], temperature=w["temperature"])
     prepare = partial(prepare_loss_input, sampling_params=params)  # as the DTensor worker binds it
     fn = ClippedPGLossFn(ClippedPGLossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0))
+    fn.lazy_metrics = True  # metric records are fetched when read, not once per microbatch
     mbs = []
     for i in range(n_buf):
         m = make_microbatch(torch, dict(w, spike_p=0.0), w["mb_seqs"], 4004 + i, dev)
@@ -562,6 +563,7 @@ def bench_packed(args, torch, w):
     prefix = torch.randint(256, 1025, (nseq, 1), generator=g, device=dev)
     token_mask = ((torch.arange(smax, device=dev).unsqueeze(0) >= prefix) & in_seq).to(torch.int64)
     fn = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, reference_policy_kl_penalty=0.001))
+    fn.lazy_metrics = True  # metric records are fetched when read, not once per microbatch
     with torch.no_grad():
         targets = torch.cat([ids[i, : lens[i]].roll(-1) for i in range(nseq)]).unsqueeze(0)
         cur = from_parallel_logits_to_logprobs_packed_sequences(logits, targets, cu, smax, 0, v, None,
@@ -642,6 +644,7 @@ def bench_lmhead(args, torch, w):
             "prev_logprobs": prev, "generation_logprobs": prev,
             "reference_policy_logprobs": cur + 0.05 * torch.randn((b, s), generator=g, device=dev)}
     fn = ClippedPGLossFn(ClippedPGLossConfig(), use_fused_linear_logprobs=True)
+    fn.lazy_metrics = True  # metric records are fetched when read, not once per microbatch
     gs, gt = torch.tensor(float(b), device=dev), tm[:, 1:].sum().float()
 
     def step():

@@ -69,10 +69,11 @@ def mask_out_neg_inf_logprobs(logprobs: torch.Tensor, mask: torch.Tensor, logpro
     """``utils.py:227-257``: positions that are masked out or infinite become 0 (with the reference's
     warning when valid tokens are affected)."""
     is_inf = torch.isinf(logprobs)
-    hit = int((is_inf & mask.bool()).sum().item())
+    # both counts in one transfer: the warning is the only reason this function waits for the device at all
+    hit, valid = torch.stack([(is_inf & mask.bool()).sum(), mask.sum().to(torch.int64)]).tolist()
     if hit > 0:
         print(
-            f"[WARNING]: {hit}/{int(mask.sum().item())} valid tokens have -inf in {logprobs_name} "
+            f"[WARNING]: {hit}/{valid} valid tokens have -inf in {logprobs_name} "
             "(policy top-k/top-p mismatch). Masking out these positions."
         )
     keep = mask * (~is_inf).float()

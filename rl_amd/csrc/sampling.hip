@@ -3,7 +3,8 @@
 // The reference sorts every 151 936-wide row (values + int64 indices).  Here one workgroup of 256
 // threads owns a row and never sorts it:
 //   pass 1 (HBM)   streams the row keeping 2048 chunk maxima in registers (and, when the caller
-//                  wants the unfiltered logprob too, the online log-sum-exp of the full row);
+//                  wants the unfiltered logprob too, the online log-sum-exp of the full row); a chunk
+//                  is a set of whole 128-byte lines, so that what pass 2 re-reads is all used;
 //   select         the k-th largest chunk maximum is a lower bound of the k-th largest element
 //                  (found two bits per round with wave ballots, the maxima staying in registers);
 //                  for top-p alone the bound starts at lse + log((1-p)/V) (everything below it is
@@ -62,6 +63,16 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 }
 __device__ __forceinline__ float key_value(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// maximum over the 8 consecutive lanes (aligned to 8) that read one 128-byte line; every lane returns it
+__device__ __forceinline__ float line_max(float v) {
+    int x = __float_as_int(v);
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false)));   // quad_perm [1,0,3,2]
+    x = __float_as_int(v);
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false)));   // quad_perm [2,3,0,1]
+    x = __float_as_int(v);
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false)));  // row_half_mirror
 }
 
 template <int DT> __device__ __forceinline__ int64_t sel_row_head(const void* row, int64_t vocab) {
@@ -210,12 +221,20 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     Lse2 acc;
     acc.m = -FLT_MAX;
     acc.s = 0.f;
+    // A chunk is a set of whole 128-byte lines: the 8 lanes that read one line together reduce their maxima over
+    // the line, and lane j of the 8 keeps the lines of the iterations i with i % 8 == j.  The second pass then
+    // re-reads full lines; with a chunk per thread it re-read 16 bytes of a line at a time, and every such piece
+    // cost the whole line in HBM traffic.
+    const int lane8 = tid & 7;
     int64_t base = 0;
-    for (; base + kSub * kSelBlock <= nvec; base += kSub * kSelBlock) {
+    int iter = 0;
+    for (; base + kSub * kSelBlock <= nvec; base += kSub * kSelBlock, ++iter) {
         u32x4 q[kSub];
 #pragma unroll
         for (int u = 0; u < kSub; ++u) q[u] = __builtin_nontemporal_load(xv + base + u * kSelBlock + tid);
+        const bool mine = (iter & 7) == lane8;
         float v[kSub * EPV];
+        float vm_all = -FLT_MAX;
 #pragma unroll
         for (int u = 0; u < kSub; ++u) {
             float t[EPV];
@@ -227,13 +246,12 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                 v[u * EPV + k] = t[k];
                 vm = fmaxf(vm, t[k]);
             }
-            mx[u] = fmaxf(mx[u], vm);
+            vm_all = fmaxf(vm_all, vm);
+            const float lm = line_max(vm);
+            mx[u] = fmaxf(mx[u], mine ? lm : -FLT_MAX);
         }
         if (FULL_LSE) {
-            float vm = mx[0];
-#pragma unroll
-            for (int u = 1; u < kSub; ++u) vm = fmaxf(vm, mx[u]);
-            const float mn = fmaxf(acc.m, vm);
+            const float mn = fmaxf(acc.m, vm_all);
             float part = 0.f;
 #pragma unroll
             for (int k = 0; k < kSub * EPV; ++k) part += fast_exp2((v[k] - mn) * kLog2e);
@@ -241,23 +259,29 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             acc.m = mn;
         }
     }
-    // the ragged end of the row: fewer than kSub vectors per thread, vector u of a thread goes to its chunk u
-    // (so a short row still spreads over many chunks and the k-th largest chunk maximum stays a useful bound)
+    // the ragged end of the row, one more iteration with fewer than kSub vectors per thread: the same chunks
+    {
+        const bool mine = (iter & 7) == lane8;
 #pragma unroll
-    for (int u = 0; u < kSub; ++u) {
-        const int64_t vi = base + u * kSelBlock + tid;
-        if (vi >= nvec) continue;
-        float t[EPV];
-        Row<DT>::decode(xv[vi], t);
+        for (int u = 0; u < kSub; ++u) {
+            const int64_t vi = base + u * kSelBlock + tid;
+            float vm = -FLT_MAX;
+            if (vi < nvec) {
+                float t[EPV];
+                Row<DT>::decode(xv[vi], t);
 #pragma unroll
-        for (int k = 0; k < EPV; ++k) {
-            t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
-            mx[u] = fmaxf(mx[u], t[k]);
-            if (FULL_LSE) {
-                const float mn = fmaxf(acc.m, t[k]);
-                acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((t[k] - mn) * kLog2e);
-                acc.m = mn;
+                for (int k = 0; k < EPV; ++k) {
+                    t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+                    vm = fmaxf(vm, t[k]);
+                    if (FULL_LSE) {
+                        const float mn = fmaxf(acc.m, t[k]);
+                        acc.s = acc.s * fast_exp2((acc.m - mn) * kLog2e) + fast_exp2((t[k] - mn) * kLog2e);
+                        acc.m = mn;
+                    }
+                }
             }
+            const float lm = line_max(vm);  // by every lane: lanes past the end bring the identity
+            mx[u] = fmaxf(mx[u], mine ? lm : -FLT_MAX);
         }
     }
     {
@@ -425,15 +449,17 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         bound_key = bound_from_row();
         continue;
     }
-    const int64_t n_full = nvec / (kSub * kSelBlock);  // vectors every chunk got in the main loop of pass 1
-    const int per_chunk = static_cast<int>(n_full) + 1;  // ... plus its slot of the ragged end
+    const int n_full = static_cast<int>(nvec / (kSub * kSelBlock));  // whole iterations of pass 1; number n_full is the ragged end
+    const int per_chunk = ((n_full + 8) / 8) * 8;  // a line (8 vectors) per iteration the chunk's lane took
     const int n_items = sh.n_hit * per_chunk;
-    // vector index of item number `item`, or -1 (the ragged slot of a chunk that has none)
+    // vector index of item number `item`, or -1 (an iteration past the end, or a vector past the row's)
     auto item_vec = [&](int item) -> int64_t {
         if (item >= n_items) return -1;
-        const int h = item / per_chunk, j = item - h * per_chunk;
+        const int h = item / per_chunk, rem = item - h * per_chunk;
         const int cu = hit[h], t = cu / kSub, u = cu - t * kSub;
-        const int64_t vi = j < n_full ? j * static_cast<int64_t>(kSub * kSelBlock) + u * kSelBlock + t : base + u * kSelBlock + t;
+        const int i = (t & 7) + (rem & ~7);  // iteration (rem / 8) of those with i % 8 == t % 8
+        if (i > n_full) return -1;
+        const int64_t vi = i * static_cast<int64_t>(kSub * kSelBlock) + u * kSelBlock + (t & ~7) + (rem & 7);
         return vi < nvec ? vi : -1;
     };
     constexpr int kBatch = 4;
