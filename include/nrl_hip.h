@@ -287,6 +287,29 @@ int nrl_fused_packed_logits_grpo_loss(const nrl_rows* rows, int32_t target_is_pr
 int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, float* dlp_out,
                          float* metrics_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* calculate_kl (nemo_rl/algorithms/utils.py:42-101) element by element over n fp32 values: logr = reference -
+ * logprobs, clamped to +-input_clamp when has_input_clamp; kl_type 1: -logr, 2: logr^2 / 2, 3: exp(logr) - 1 - logr;
+ * multiplied by weights[i] when weights is not NULL; clamped to +-output_clamp when has_output_clamp.
+ * _bwd writes grad_kl[i] * d kl[i] / d (input) into whichever of the three outputs is not NULL: a token whose logr
+ * was clamped passes nothing (neither through the KL nor, as the reference detaches it, through its weight), a
+ * value outside the output clamp passes nothing either. */
+int nrl_calculate_kl(const float* logprobs, const float* logprobs_reference, const float* weights, int64_t n,
+                     int32_t kl_type, int32_t has_input_clamp, float input_clamp, int32_t has_output_clamp,
+                     float output_clamp, float* kl_out, void* stream);
+int nrl_calculate_kl_bwd(const float* grad_kl, const float* logprobs, const float* logprobs_reference,
+                         const float* weights, int64_t n, int32_t kl_type, int32_t has_input_clamp, float input_clamp,
+                         int32_t has_output_clamp, float output_clamp, float* dlogprobs_out, float* dreference_out,
+                         float* dweights_out, void* stream);
+
+/* masked_mean (nemo_rl/algorithms/utils.py:207-224) over the last axis of fp32 [n_rows, n_cols]:
+ * out[r] = sum_c(values * mask) / (norm + 1e-8), norm = sum_c(mask) of the row unless has_norm, then the one value
+ * at norm_device (device pointer) or, if that is NULL, norm_host.  The sums are carried in double.  denom_out
+ * (or NULL) receives norm + 1e-8 per row for _bwd: dvalues[r, c] = grad_out[r] * mask[r, c] / denom[r]. */
+int nrl_masked_mean(const float* values, const float* mask, int64_t n_rows, int64_t n_cols, const float* norm_device,
+                    float norm_host, int32_t has_norm, float* out, float* denom_out, void* stream);
+int nrl_masked_mean_bwd(const float* grad_out, const float* mask, const float* denom, int64_t n_rows, int64_t n_cols,
+                        float* dvalues_out, void* stream);
+
 /* log_softmax over the K logits of a row at the given vocabulary indices (the teacher's top-k), the
  * zero_outside_topk = False branch of get_distillation_topk_logprobs_from_logits
  * (nemo_rl/distributed/model_utils.py:1981-2005): out[r, j] = x[r, idx[r, j]] - logsumexp_j x[r, idx[r, j]].

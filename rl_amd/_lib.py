@@ -89,6 +89,10 @@ SIGNATURES = {
     "nrl_fused_packed_logits_grpo_loss": (C.c_int, [C.POINTER(NrlRows), C.c_int32, _P, _I64, C.POINTER(NrlGrpoCfg),
                                                     C.POINTER(NrlGrpoInputs), _F, _P, _I64, _P, _P, _P, _P, _I64, _P]),
     "nrl_nll_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _I64, _P]),
+    "nrl_calculate_kl": (C.c_int, [_P, _P, _P, _I64, _I32, _I32, _F, _I32, _F, _P, _P]),
+    "nrl_calculate_kl_bwd": (C.c_int, [_P, _P, _P, _P, _I64, _I32, _I32, _F, _I32, _F, _P, _P, _P, _P]),
+    "nrl_masked_mean": (C.c_int, [_P, _P, _I64, _I64, _P, _F, _I32, _P, _P, _P]),
+    "nrl_masked_mean_bwd": (C.c_int, [_P, _P, _P, _I64, _I64, _P, _P]),
     "nrl_topk_logsoftmax_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P]),
     "nrl_topk_logsoftmax_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _I64, _P, _P, _P, _I64, _I64, _P]),
     "nrl_distill_topk_loss_workspace_bytes": (_I64, [_I64, _I64]),

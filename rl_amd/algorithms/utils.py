@@ -1,8 +1,8 @@
 """Helpers around the loss (counterparts of ``nemo_rl/algorithms/utils.py:42-274``).
 
-``calculate_baseline_and_std_per_prompt`` runs the HIP grouping / statistics kernels.  The other
-helpers are thin [B, S]-sized tensor expressions kept for API compatibility; inside
-``ClippedPGLossFn`` their arithmetic is part of the fused loss kernel instead.
+``calculate_baseline_and_std_per_prompt`` runs the HIP grouping / statistics kernels, ``calculate_kl`` and
+``masked_mean`` their own small kernels (inside ``ClippedPGLossFn`` the same arithmetic is part of the fused loss
+kernel instead).  ``mask_out_neg_inf_logprobs`` is [B, S]-sized tensor plumbing around the reference's warning.
 """
 
 from __future__ import annotations
@@ -22,6 +22,44 @@ def _gpu_device() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device())
 
 
+_KL_TYPES = {"k1": 1, "k2": 2, "k3": 3}
+
+
+def _staged(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
+    """fp32, contiguous, on the GPU (host tensors, the driver's default, are copied over)."""
+    return t.detach().to(device=dev, dtype=torch.float32).contiguous()
+
+
+class _CalculateKl(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, lp, ref, weights, kl_type, input_clamp, output_clamp, out_dtype, out_device):
+        dev = lp.device if lp.is_cuda else _gpu_device()
+        parts = torch.broadcast_tensors(*[t for t in (lp, ref, weights) if t is not None])
+        staged = [_staged(t, dev) for t in parts]
+        lp32, ref32 = staged[0], staged[1]
+        w32 = staged[2] if weights is not None else None
+        ctx.save_for_backward(lp32, ref32, w32)
+        ctx.cfg = (kl_type, input_clamp, output_clamp)
+        ctx.inputs = [(t.shape, t.dtype, t.device) if t is not None else None for t in (lp, ref, weights)]
+        out = _OPS.calculate_kl(lp32, ref32, w32, kl_type, input_clamp, output_clamp)
+        return out.to(device=out_device, dtype=out_dtype)
+
+    @staticmethod
+    def backward(ctx, grad):
+        lp32, ref32, w32 = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        g = _staged(grad.expand(lp32.shape), lp32.device)
+        grads = _OPS.calculate_kl_bwd(g, lp32, ref32, w32, *ctx.cfg, need[0], need[1], bool(need[2] and w32 is not None))
+        out = []
+        for wanted, d, meta in zip(need, grads, ctx.inputs):
+            if not wanted or meta is None:
+                out.append(None)
+                continue
+            shape, dtype, device = meta
+            out.append(d.sum_to_size(shape).to(device=device, dtype=dtype) if tuple(d.shape) != tuple(shape) else d.to(device=device, dtype=dtype))
+        return (*out, None, None, None, None, None)
+
+
 def calculate_kl(
     logprobs: torch.Tensor,
     logprobs_reference: torch.Tensor,
@@ -30,28 +68,33 @@ def calculate_kl(
     output_clamp_value: float | None = 10.0,
     importance_sampling_weights: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Per-token k1 / k2 / k3 estimate of KL(policy || reference), ``utils.py:42-101``."""
-    logr = logprobs_reference - logprobs
-    if input_clamp_value is not None:
-        bounded = logr.clamp(min=-input_clamp_value, max=input_clamp_value)
-        if importance_sampling_weights is not None:
-            importance_sampling_weights = torch.where(
-                logr == bounded, importance_sampling_weights, importance_sampling_weights.detach()
-            )
-        logr = bounded
-    if kl_type == "k1":
-        kl = -logr
-    elif kl_type == "k2":
-        kl = torch.square(logr) / 2
-    elif kl_type == "k3":
-        kl = torch.exp(logr) - 1 - logr
-    else:
+    """Per-token k1 / k2 / k3 estimate of KL(policy || reference), ``utils.py:42-101``: one elementwise HIP kernel
+    (the arithmetic of the loss kernel's KL term) with its gradient kernel behind autograd.  Computed in fp32 and
+    returned in the inputs' promoted dtype, on the device of ``logprobs``."""
+    if kl_type not in _KL_TYPES:
         raise ValueError(f"Invalid KL type: {kl_type}")
-    if importance_sampling_weights is not None:
-        kl = importance_sampling_weights * kl
-    if output_clamp_value is not None:
-        kl = kl.clamp(min=-output_clamp_value, max=output_clamp_value)
-    return kl
+    tensors = [t for t in (logprobs, logprobs_reference, importance_sampling_weights) if t is not None]
+    out_dtype = tensors[0].dtype
+    for t in tensors[1:]:
+        out_dtype = torch.promote_types(out_dtype, t.dtype)
+    return _CalculateKl.apply(
+        logprobs, logprobs_reference, importance_sampling_weights, _KL_TYPES[kl_type],
+        None if input_clamp_value is None else float(input_clamp_value),
+        None if output_clamp_value is None else float(output_clamp_value), out_dtype, logprobs.device,
+    )
+
+
+class _MaskedMeanRows(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, values2d, mask2d, norm):
+        out, denom = _OPS.masked_mean_rows(values2d, mask2d, norm)
+        ctx.save_for_backward(mask2d, denom)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        mask2d, denom = ctx.saved_tensors
+        return _OPS.masked_mean_rows_bwd(grad.contiguous().float(), mask2d, denom), None, None
 
 
 def masked_mean(
@@ -60,9 +103,34 @@ def masked_mean(
     dim: Optional[int] = None,
     global_normalization_factor: Optional[torch.Tensor | float] = None,
 ):
-    """``sum(values * mask) / (norm + 1e-8)``, ``utils.py:212-224``."""
-    norm = torch.sum(mask, dim=dim) if global_normalization_factor is None else global_normalization_factor
-    return torch.sum(values * mask, dim=dim) / (norm + 1e-8)
+    """``sum(values * mask) / (norm + 1e-8)``, ``utils.py:207-224``, over everything (``dim=None``) or one axis: a
+    row-reduction HIP kernel (sums carried in double) and its gradient kernel for ``values``.  The mask and the
+    normalisation factor are constants of the gradient, as in every use the reference makes of this function."""
+    if dim is not None and not isinstance(dim, int):
+        raise NotImplementedError("masked_mean reduces over everything or over one axis")
+    norm = global_normalization_factor
+    if mask.requires_grad or (isinstance(norm, torch.Tensor) and norm.requires_grad):
+        raise NotImplementedError("masked_mean differentiates with respect to the values only")
+    if isinstance(norm, torch.Tensor) and norm.numel() != 1:
+        raise NotImplementedError("the normalisation factor must be one value")
+    out_dtype = torch.promote_types(values.dtype, mask.dtype)
+    if isinstance(norm, torch.Tensor):
+        out_dtype = torch.promote_types(out_dtype, norm.dtype)
+    if not out_dtype.is_floating_point:
+        out_dtype = torch.float32
+    dev = values.device if values.is_cuda else _gpu_device()
+    v, m = torch.broadcast_tensors(values, mask)
+    if dim is None:
+        v2, m2, out_shape = v.reshape(1, -1), m.reshape(1, -1), ()
+    else:
+        v, m = v.movedim(dim, -1), m.movedim(dim, -1)
+        out_shape = tuple(v.shape[:-1])
+        v2, m2 = v.reshape(-1, v.shape[-1]), m.reshape(-1, m.shape[-1])
+    v2 = v2.to(device=dev, dtype=torch.float32).contiguous()
+    m2 = _staged(m2, dev)
+    norm_t = None if norm is None else torch.as_tensor(norm, dtype=torch.float32).detach().to(dev).reshape(1)
+    out = _MaskedMeanRows.apply(v2, m2, norm_t)
+    return out.reshape(out_shape).to(device=values.device, dtype=out_dtype)
 
 
 def mask_out_neg_inf_logprobs(logprobs: torch.Tensor, mask: torch.Tensor, logprobs_name: str) -> torch.Tensor:

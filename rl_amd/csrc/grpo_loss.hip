@@ -707,6 +707,149 @@ extern "C" int nrl_nll_loss_fwd_bwd(const nrl_grpo_inputs* in, float* loss_out, 
     return check_launch("nll_loss_fwd_bwd");
 }
 
+// ---------------------------------------------------------------------------------------------
+// The two helpers of the loss that the driver also calls on their own (KL in the reward, mean reward):
+// calculate_kl element by element, masked_mean row by row.  [B, S]-sized, latency bound.
+// ---------------------------------------------------------------------------------------------
+struct KlArgs {
+    const float* lp;
+    const float* ref;
+    const float* weight;  // importance sampling weights or NULL
+    int64_t n;
+    int kl_type, has_in, has_out;
+    float in_clamp, out_clamp;
+};
+
+struct KlPoint {
+    float value, d_logr, d_weight;  // clamped value; d value / d (ref - lp); d value / d weight
+};
+
+__device__ __forceinline__ KlPoint kl_point(const KlArgs& a, int64_t i) {
+    float logr = a.ref[i] - a.lp[i];
+    float in_range = 1.f;
+    if (a.has_in) {
+        const float cl = clampf(logr, -a.in_clamp, a.in_clamp);
+        if (!(logr == cl)) in_range = 0.f;  // a clamped token passes no gradient, neither through the KL nor the weight
+        logr = cl;
+    }
+    const float w = a.weight ? a.weight[i] : 1.f;
+    const float k = kl_value(a.kl_type, logr);
+    KlPoint o;
+    o.value = a.weight ? w * k : k;
+    o.d_logr = w * kl_slope(a.kl_type, logr) * in_range;
+    o.d_weight = k * in_range;
+    if (a.has_out) {
+        if (!(o.value >= -a.out_clamp && o.value <= a.out_clamp)) { o.d_logr = 0.f; o.d_weight = 0.f; }
+        o.value = clampf(o.value, -a.out_clamp, a.out_clamp);
+    }
+    return o;
+}
+
+__global__ __launch_bounds__(256) void calculate_kl_kernel(KlArgs a, float* out) {
+    for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < a.n; i += gridDim.x * 256ll) out[i] = kl_point(a, i).value;
+}
+
+__global__ __launch_bounds__(256) void calculate_kl_bwd_kernel(KlArgs a, const float* g, float* d_lp, float* d_ref, float* d_weight) {
+    for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < a.n; i += gridDim.x * 256ll) {
+        const KlPoint p = kl_point(a, i);
+        const float t = g[i] * p.d_logr;
+        if (d_lp) d_lp[i] = -t;
+        if (d_ref) d_ref[i] = t;
+        if (d_weight) d_weight[i] = g[i] * p.d_weight;
+    }
+}
+
+static int kl_args(KlArgs& a, const float* lp, const float* ref, const float* weight, int64_t n, int32_t kl_type,
+                   int32_t has_in, float in_clamp, int32_t has_out, float out_clamp) {
+    if (n < 0 || (n > 0 && (!lp || !ref))) return fail(NRL_E_INVALID, "calculate_kl: null input");
+    if (kl_type < 1 || kl_type > 3) return fail(NRL_E_INVALID, "calculate_kl: kl_type must be 1 (k1), 2 (k2) or 3 (k3)");
+    a = KlArgs{lp, ref, weight, n, kl_type, has_in, has_out, in_clamp, out_clamp};
+    return NRL_OK;
+}
+
+static unsigned small_grid(int64_t n) { return static_cast<unsigned>(n + 255 < 256 * 2048ll ? (n + 255) / 256 : 2048); }
+
+extern "C" int nrl_calculate_kl(const float* logprobs, const float* logprobs_reference, const float* weights, int64_t n,
+                                int32_t kl_type, int32_t has_input_clamp, float input_clamp, int32_t has_output_clamp,
+                                float output_clamp, float* kl_out, void* stream) {
+    KlArgs a;
+    if (int e = kl_args(a, logprobs, logprobs_reference, weights, n, kl_type, has_input_clamp, input_clamp,
+                        has_output_clamp, output_clamp)) return e;
+    if (n == 0) return NRL_OK;
+    if (!kl_out) return fail(NRL_E_INVALID, "calculate_kl: null output");
+    calculate_kl_kernel<<<dim3(small_grid(n)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(a, kl_out);
+    return check_launch("calculate_kl");
+}
+
+extern "C" int nrl_calculate_kl_bwd(const float* grad_kl, const float* logprobs, const float* logprobs_reference,
+                                    const float* weights, int64_t n, int32_t kl_type, int32_t has_input_clamp,
+                                    float input_clamp, int32_t has_output_clamp, float output_clamp, float* dlogprobs_out,
+                                    float* dreference_out, float* dweights_out, void* stream) {
+    KlArgs a;
+    if (int e = kl_args(a, logprobs, logprobs_reference, weights, n, kl_type, has_input_clamp, input_clamp,
+                        has_output_clamp, output_clamp)) return e;
+    if (n == 0) return NRL_OK;
+    if (!grad_kl) return fail(NRL_E_INVALID, "calculate_kl_bwd: null upstream gradient");
+    if (dweights_out && !weights) return fail(NRL_E_INVALID, "calculate_kl_bwd: a weight gradient without weights");
+    calculate_kl_bwd_kernel<<<dim3(small_grid(n)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        a, grad_kl, dlogprobs_out, dreference_out, dweights_out);
+    return check_launch("calculate_kl_bwd");
+}
+
+// one workgroup per row: out[r] = sum_c(values * mask) / (norm + 1e-8), norm = sum_c(mask) unless given
+__global__ __launch_bounds__(kLossBlock) void masked_mean_kernel(const float* values, const float* mask, int64_t n_cols,
+                                                                 const float* norm_dev, float norm_host, int has_norm,
+                                                                 float* out, float* denom_out) {
+    __shared__ double red[kLossBlock / kWave];
+    const int64_t r = blockIdx.x;
+    double sv = 0.0, sm = 0.0;
+    for (int64_t c = threadIdx.x; c < n_cols; c += kLossBlock) {
+        const float m = mask[r * n_cols + c];
+        sv += static_cast<double>(values[r * n_cols + c] * m);
+        sm += static_cast<double>(m);
+    }
+    sv = block_sum<double, kLossBlock / kWave>(sv, red);
+    __syncthreads();
+    sm = block_sum<double, kLossBlock / kWave>(sm, red);
+    if (threadIdx.x == 0) {
+        const float norm = has_norm ? (norm_dev ? norm_dev[0] : norm_host) : static_cast<float>(sm);
+        const float den = norm + 1e-8f;
+        out[r] = static_cast<float>(sv) / den;
+        if (denom_out) denom_out[r] = den;
+    }
+}
+
+__global__ __launch_bounds__(256) void masked_mean_bwd_kernel(const float* g, const float* mask, const float* denom,
+                                                              int64_t n_rows, int64_t n_cols, float* d_values) {
+    const int64_t n = n_rows * n_cols;
+    for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll) {
+        const int64_t r = i / n_cols;
+        d_values[i] = g[r] * mask[i] / denom[r];
+    }
+}
+
+extern "C" int nrl_masked_mean(const float* values, const float* mask, int64_t n_rows, int64_t n_cols,
+                               const float* norm_device, float norm_host, int32_t has_norm, float* out, float* denom_out,
+                               void* stream) {
+    if (n_rows < 0 || n_cols < 0) return fail(NRL_E_INVALID, "masked_mean: negative shape");
+    if (n_rows == 0) return NRL_OK;
+    if (!out || (n_cols > 0 && (!values || !mask))) return fail(NRL_E_INVALID, "masked_mean: null pointer");
+    if (n_rows > 0x7fffffffll) return fail(NRL_E_UNSUPPORTED, "masked_mean: more than 2^31 - 1 rows");
+    masked_mean_kernel<<<dim3((unsigned)n_rows), dim3(kLossBlock), 0, static_cast<hipStream_t>(stream)>>>(
+        values, mask, n_cols, norm_device, norm_host, has_norm, out, denom_out);
+    return check_launch("masked_mean");
+}
+
+extern "C" int nrl_masked_mean_bwd(const float* grad_out, const float* mask, const float* denom, int64_t n_rows,
+                                   int64_t n_cols, float* dvalues_out, void* stream) {
+    if (n_rows < 0 || n_cols < 0) return fail(NRL_E_INVALID, "masked_mean_bwd: negative shape");
+    if (n_rows * n_cols == 0) return NRL_OK;
+    if (!grad_out || !mask || !denom || !dvalues_out) return fail(NRL_E_INVALID, "masked_mean_bwd: null pointer");
+    masked_mean_bwd_kernel<<<dim3(small_grid(n_rows * n_cols)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        grad_out, mask, denom, n_rows, n_cols, dvalues_out);
+    return check_launch("masked_mean_bwd");
+}
+
 static int64_t align8(int64_t v) { return (v + 7) / 8 * 8; }
 
 extern "C" int64_t nrl_fused_workspace_bytes(int64_t batch, int64_t n_inner) {

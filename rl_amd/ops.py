@@ -650,6 +650,88 @@ for _name, _fn in (("grpo_loss", _grpo_loss), ("nll_loss", _nll_loss)):
     _LIB.impl(_name, _fn, "CPU")
 
 
+# the loss helpers that are also called on their own (KL in the reward, mean reward)
+_LIB.define("calculate_kl(Tensor lp, Tensor ref, Tensor? weights, int kl_type, float? input_clamp, float? output_clamp) -> Tensor")
+_LIB.define(
+    "calculate_kl_bwd(Tensor grad, Tensor lp, Tensor ref, Tensor? weights, int kl_type, float? input_clamp, "
+    "float? output_clamp, bool need_lp, bool need_ref, bool need_weights) -> (Tensor, Tensor, Tensor)"
+)
+_LIB.define("masked_mean_rows(Tensor values, Tensor mask, Tensor? norm) -> (Tensor, Tensor)")
+_LIB.define("masked_mean_rows_bwd(Tensor grad, Tensor mask, Tensor denom) -> Tensor")
+
+
+def _flat_f32(*tensors):
+    for t in tensors:
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+            raise ValueError("expected contiguous fp32 tensors")
+    shapes = {tuple(t.shape) for t in tensors if t is not None}
+    if len(shapes) > 1:
+        raise ValueError(f"shapes differ: {sorted(shapes)}")
+
+
+def _clamp_args(value):
+    return (0, 0.0) if value is None else (1, float(value))
+
+
+def _calculate_kl(lp, ref, weights, kl_type, input_clamp, output_clamp):
+    _need_gpu(lp, ref, weights)
+    _flat_f32(lp, ref, weights)
+    out = torch.empty_like(lp)
+    with torch.cuda.device(lp.device):
+        code = _lib.load().nrl_calculate_kl(_ptr(lp), _ptr(ref), _ptr(weights), lp.numel(), int(kl_type),
+                                            *_clamp_args(input_clamp), *_clamp_args(output_clamp), _ptr(out), _stream())
+    _lib.check(code, "nrl_calculate_kl")
+    return out
+
+
+def _calculate_kl_bwd(grad, lp, ref, weights, kl_type, input_clamp, output_clamp, need_lp, need_ref, need_weights):
+    _need_gpu(grad, lp, ref, weights)
+    _flat_f32(grad, lp, ref, weights)
+    empty = lp.new_empty(0)
+    d_lp = torch.empty_like(lp) if need_lp else None
+    d_ref = torch.empty_like(lp) if need_ref else None
+    d_w = torch.empty_like(lp) if need_weights and weights is not None else None
+    with torch.cuda.device(lp.device):
+        code = _lib.load().nrl_calculate_kl_bwd(_ptr(grad), _ptr(lp), _ptr(ref), _ptr(weights), lp.numel(), int(kl_type),
+                                                *_clamp_args(input_clamp), *_clamp_args(output_clamp), _ptr(d_lp),
+                                                _ptr(d_ref), _ptr(d_w), _stream())
+    _lib.check(code, "nrl_calculate_kl_bwd")
+    return tuple(empty if t is None else t for t in (d_lp, d_ref, d_w))
+
+
+def _masked_mean_rows(values, mask, norm):
+    _need_gpu(values, mask, norm)
+    _flat_f32(values, mask)
+    if values.dim() != 2:
+        raise ValueError(f"expected [rows, cols], got {tuple(values.shape)}")
+    if norm is not None and (norm.numel() != 1 or norm.dtype != torch.float32):
+        raise ValueError("the normalisation factor must be one fp32 value")
+    rows, cols = values.shape
+    out = values.new_empty(rows)
+    denom = values.new_empty(rows)
+    with torch.cuda.device(values.device):
+        code = _lib.load().nrl_masked_mean(_ptr(values), _ptr(mask), rows, cols, _ptr(norm), 0.0, int(norm is not None),
+                                           _ptr(out), _ptr(denom), _stream())
+    _lib.check(code, "nrl_masked_mean")
+    return out, denom
+
+
+def _masked_mean_rows_bwd(grad, mask, denom):
+    _need_gpu(grad, mask, denom)
+    rows, cols = mask.shape
+    out = torch.empty_like(mask)
+    with torch.cuda.device(mask.device):
+        code = _lib.load().nrl_masked_mean_bwd(_ptr(grad), _ptr(mask), _ptr(denom), rows, cols, _ptr(out), _stream())
+    _lib.check(code, "nrl_masked_mean_bwd")
+    return out
+
+
+for _name, _fn in (("calculate_kl", _calculate_kl), ("calculate_kl_bwd", _calculate_kl_bwd),
+                   ("masked_mean_rows", _masked_mean_rows), ("masked_mean_rows_bwd", _masked_mean_rows_bwd)):
+    _LIB.impl(_name, _fn, "CUDA")
+    _LIB.impl(_name, _fn, "CPU")
+
+
 _LIB.define("topk_logsoftmax_fwd(Tensor logits, Tensor? indices) -> Tensor")
 _LIB.define("topk_logsoftmax_bwd(Tensor logits, Tensor indices, Tensor logprobs, Tensor grad) -> Tensor")
 _LIB.define(
