@@ -653,22 +653,34 @@ def bench_lmhead(args, torch, w):
         dh, dw = torch.autograd.grad(loss, (hidden, weight))
         del dh, dw
 
-    elapsed, k = timed(torch, ops, args, step)
+    from rl_amd.distributed import model_utils as MU
+
+    # The forward keeps its bf16 logits when they fit ("auto": a quarter of the free memory; 19.9 GB at this shape)
+    # and the backward reads them instead of multiplying a second time.  The reference's way, recomputing, is its
+    # own row below.
     n = b * s
+    kept = MU._keep_lmhead_logits(n, v, dev)
+    elapsed, k = timed(torch, ops, args, step)
     fwd_ms, bwd_ms = k["lmhead_fwd"]["avg_ms"], k["lmhead_bwd"]["avg_ms"]
+    MU.LMHEAD_KEEP_LOGITS = not kept
+    elapsed_other, k_other = timed(torch, ops, args, step)
+    MU.LMHEAD_KEEP_LOGITS = "auto"
     fwd_tf = 2.0 * n * h * v / (fwd_ms * 1e-3) / 1e12
     # the backward products run on the tokens that carry a gradient only (masked prompt tokens and each
     # sequence's last position have a zero row in the logits' gradient)
     live = float(gt.item()) / n
+    products = 2.0 if kept else 3.0                                       # dH, dW (+ the recomputed logits)
     bwd_alg_tf = 4.0 * n * h * v / (bwd_ms * 1e-3) / 1e12                 # dH + dW of every token, the algorithmic count
-    bwd_exec_tf = 6.0 * live * n * h * v / (bwd_ms * 1e-3) / 1e12         # what the matrix cores execute: + recompute, live tokens
-    fills = MEASURED_TRAFFIC.get("c3_fwd") if not args.seqs else None
+    bwd_exec_tf = 2.0 * products * live * n * h * v / (bwd_ms * 1e-3) / 1e12   # what the matrix cores execute, live tokens
+    fills = MEASURED_TRAFFIC.get("c3_fwd") if not args.seqs and not kept else None
     result = {
         "metric": "fused lm_head + GRPO loss fwd/bwd tokens/s; % of bf16 MFMA peak",
         "value": n * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": w["desc"], "tokens": n, "hidden": h, "vocab": v},
+        "config": {"workload": w["desc"], "tokens": n, "hidden": h, "vocab": v,
+                   "logits": ("bf16 logits kept by the forward for the backward (%.1f GB)" % (n * v * 2 / 1e9)) if kept
+                             else "recomputed in the backward"},
         "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel", "achieved": fwd_tf, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": (fills["read"] + fills["write"]) if fills else None,
@@ -677,8 +689,13 @@ def bench_lmhead(args, torch, w):
                          "executed": bwd_exec_tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": bwd_alg_tf / MFMA_BF16_PEAK_TFLOPS, "frac_executed": bwd_exec_tf / MFMA_BF16_PEAK_TFLOPS,
                          "live_token_fraction": live, "avg_launch_ms": bwd_ms,
-                         "note": "achieved counts dH + dW of all tokens (4 N H V); executed counts the three products the matrix "
-                                 "cores run, on the tokens with a non-zero gradient only (6 N_live H V)"},
+                         "note": "achieved counts dH + dW of all tokens (4 N H V); executed counts the products the matrix "
+                                 "cores run (dH, dW and, when the logits are not kept, their recomputation), on the tokens "
+                                 "with a non-zero gradient only"},
+        ("recompute" if kept else "kept_logits"): {
+            "tokens_per_s": n * args.steps / elapsed_other, "ms_per_step": elapsed_other / args.steps * 1e3,
+            "kernel_ms": {kk: round(vv["avg_ms"], 4) for kk, vv in k_other.items()},
+            "note": "the same step with LMHEAD_KEEP_LOGITS = %s" % (not kept)},
         "algorithmic_tflops_end_to_end": 6.0 * n * h * v * args.steps / elapsed / 1e12,
         "kernel_ms": {kk: round(vv["avg_ms"], 4) for kk, vv in k.items()},
     }

@@ -444,8 +444,8 @@ int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* g
                           void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
- * K6  Fused lm_head -> token logprob on the bf16 matrix cores (MFMA), never materialising the
- * [N, V] logits.  Replaces ChunkedDistributedHiddenStatesToLogprobs
+ * K6  Fused lm_head -> token logprob on the bf16 matrix cores (MFMA), without a pass over [N, V]
+ * logits in fp32.  Replaces ChunkedDistributedHiddenStatesToLogprobs
  * (nemo_rl/distributed/model_utils.py:2137-2316) at TP = 1.
  * hidden: bf16 [N, H] rows of stride ldh (token order is the caller's); weight: bf16 [V, H] rows of
  * stride ldw; both 16-byte aligned, H and the strides multiples of 8.  targets: int64 [N], already
@@ -454,19 +454,27 @@ int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* g
  * Backward: grad fp32 [N] -> dhidden_out fp32 [N, H] (row stride ld_dh) and dweight_out bf16 [V, H]
  * (row stride ld_dw), accumulated in fp32 and narrowed once.  Tokens are processed in chunks of 16384:
  * per chunk the gradient of the logits exists as bf16 [chunk, V] (twice, one transposed).
+ * Kept logits (a choice of the caller, who has the memory or not): with logits_out not NULL the forward
+ * also writes the bf16 logits [N, ld_logits] (16-byte aligned, ld_logits a multiple of 8 and >= V; the
+ * columns from V on are unspecified), 2 N ld_logits bytes; handed back as logits_kept the backward reads them
+ * instead of multiplying hidden and weight a second time (the reference always recomputes, :2249-2262, because
+ * its logits are fp32 and its memory a quarter).  Both ways give the same gradients: the kept values are the
+ * rounded logits the recomputation arrives at.
  * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
  * ------------------------------------------------------------------------------------------ */
 int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab);
 int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                            const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                            int64_t vocab_start, int64_t vocab_end, float* logprob_out, float* lse_out,
-                           void* workspace, int64_t workspace_bytes, void* stream);
+                           void* logits_out, int64_t ld_logits, void* workspace, int64_t workspace_bytes,
+                           void* stream);
 int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab);
 int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                            const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                            int64_t vocab_start, int64_t vocab_end, const float* lse, const float* grad,
-                           float* dhidden_out, int64_t ld_dh, void* dweight_out, int64_t ld_dw,
-                           void* workspace, int64_t workspace_bytes, void* stream);
+                           const void* logits_kept, int64_t ld_logits, float* dhidden_out, int64_t ld_dh,
+                           void* dweight_out, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
+                           void* stream);
 
 #ifdef __cplusplus
 }

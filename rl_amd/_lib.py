@@ -113,9 +113,9 @@ SIGNATURES = {
     "nrl_nonzero_indices": (C.c_int, [_P, _I64, _P, _P, _P]),
     "nrl_seq_logprob_error": (C.c_int, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _I64, C.c_int32, C.c_float, _P, _P, _P, _P, _I64, _P]),
     "nrl_lmhead_fwd_workspace_bytes": (_I64, [_I64, _I64]),
-    "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P]),
+    "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _P]),
     "nrl_lmhead_bwd_workspace_bytes": (_I64, [_I64, _I64, _I64]),
-    "nrl_lmhead_logprob_bwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _P, _I64, _P]),
+    "nrl_lmhead_logprob_bwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P]),
     "nrl_group_workspace_bytes": (_I64, [_I64]),
     "nrl_group_baseline_std": (C.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _I32, _I32, _P, _P, _P, _P, _P, _I64, _P]),
 }

@@ -369,9 +369,11 @@ struct LmFwdArgs {
     float* part_m;             // [n_splits, N]
     float* part_s;             // [n_splits, N]
     float* xt;                 // [N] target logit (written by the tile that holds it)
+    uint16_t* logits;          // [N, ldl] bf16 logits kept for the backward, or NULL
+    int64_t ldl;               // multiple of 8, >= V; columns from V on are unspecified
 };
 
-template <class Core>
+template <class Core, bool SAVE>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     constexpr int NI = Core::NI, NJ = Core::NJ, BV = Core::BM, BT = Core::BN;  // vocabulary rows x token columns
     __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
@@ -427,6 +429,18 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
                         const int off = i * 32 + 8 * (e >> 2) + (e & 3);
                         x[e] = (!MASKED || off < limit) ? acc[i][j][e] : -INFINITY;
                         raw = fmaxf(raw, x[e]);
+                    }
+                    if constexpr (SAVE) {
+                        // The lane's 16 values are 4 runs of 4 consecutive vocabulary ids of one token: 8 bytes each,
+                        // next to the 8 bytes of the lane 32 further on; a wave's 4 x 4 blocks fill 256 bytes per token.
+                        if (tok0 + col + j * 32 < a.op.n) {
+                            uint16_t* out = a.logits + (tok0 + col + j * 32) * a.ldl + vb + i * 32;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q)
+                                if (!MASKED || i * 32 + 8 * q < static_cast<int>(a.ldl) - vb)
+                                    *reinterpret_cast<uint2*>(out + 8 * q) =
+                                        uint2{pack_bf16x2(x[4 * q], x[4 * q + 1]), pack_bf16x2(x[4 * q + 2], x[4 * q + 3])};
+                        }
                     }
                     const float mx = fmaxf(run_m[j], round_bf16(raw));
                     const float mx2 = mx * kLog2e;
@@ -685,6 +699,113 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// backward from kept logits: the same G and G^T without the product.  One workgroup turns a tile of 128 tokens x
+// 128 vocabulary ids: a thread reads 16 bytes (8 ids) of 4 consecutive live tokens' rows, writes its part of G
+// straight back (16 bytes of a 256-byte run), and hands the 4 tokens' values of each id to LDS as one 8-byte unit
+// of the transposed tile (unit U of row v at U ^ swizzle(v)), from where G^T leaves in 16-byte pieces after the
+// one-hot term was added to the tokens' target cells.
+// ---------------------------------------------------------------------------------------------
+struct LmGradKeptArgs {
+    const uint16_t* logits;   // [N, ldl] bf16, as the forward left them
+    int64_t ldl;
+    const int32_t* row_map;   // [rows] token (row of logits) of live row r
+    const int32_t* live;      // device count of live tokens
+    int64_t live_from, rows;  // this chunk's live rows are [live_from, live_from + rows) clamped to *live
+    int64_t vocab;
+    const int64_t* targets;   // the live rows' targets, log-sum-exps and upstream gradients
+    int64_t vocab_start;
+    const float* lse;
+    const float* grad;
+    uint16_t* g;              // as in LmGradArgs
+    int64_t ldg;
+    uint16_t* gt;
+    int64_t ldgt;
+};
+
+constexpr int KT = 128;  // tile side of lmhead_grad_kept_kernel
+
+__global__ __launch_bounds__(256) void lmhead_grad_kept_kernel(LmGradKeptArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[KT * KT * 2];
+    __shared__ int tgt_l[KT];
+    __shared__ float lse_l[KT], g_l[KT];
+    __shared__ int64_t row_l[KT];
+    const int tid = threadIdx.x;
+    int64_t m = static_cast<int64_t>(a.live[0]) - a.live_from;
+    m = m < 0 ? 0 : (m > a.rows ? a.rows : m);
+    const int64_t row0 = static_cast<int64_t>(blockIdx.y) * KT, col0 = static_cast<int64_t>(blockIdx.x) * KT;
+    if (row0 >= m) return;
+    const int64_t m_pad = (m + 63) / 64 * 64;
+    if (tid < KT) {
+        const int64_t r = row0 + tid;
+        int64_t t = -1, src = 0;
+        float l = 128.f, g = 0.f;  // rows past the live ones: a finite exponent and a zero gradient
+        if (r < m) { t = a.targets[r] - a.vocab_start; l = a.lse[r]; g = a.grad[r]; src = a.row_map[r]; }
+        tgt_l[tid] = (t >= 0 && t < a.vocab && g != 0.f) ? static_cast<int>(t) : -1;
+        lse_l[tid] = l * kLog2e;
+        g_l[tid] = g;
+        row_l[tid] = src;
+    }
+    __syncthreads();
+    auto swz = [](int v) { return (v ^ (v >> 5)) & 31; };
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int item = pass * 256 + tid, piece = item & 15, t4 = item >> 4;  // 8 ids x 4 tokens
+        const int64_t c = col0 + piece * 8;
+        uint32_t w[4][4];  // [token][pair of ids]
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int t = t4 * 4 + u;
+            float sv[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) sv[k] = 0.f;
+            if (row0 + t < m && c < a.vocab && g_l[t] != 0.f) {
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(a.logits + row_l[t] * a.ldl + c);
+                float x[8];
+                Row<NRL_BF16>::decode(raw, x);
+                const float ng = -g_l[t], ls = lse_l[t];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    sv[k] = c + k < a.vocab ? fast_exp2(__builtin_fmaf(x[k], kLog2e, -ls)) * ng : 0.f;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) w[u][q] = pack_bf16x2(sv[2 * q], sv[2 * q + 1]);
+            if (row0 + t < m_pad && c < a.ldg)
+                *reinterpret_cast<u32x4*>(a.g + (row0 + t) * a.ldg + c) = u32x4{w[u][0], w[u][1], w[u][2], w[u][3]};
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int v = piece * 8 + k, q = k >> 1;
+            uint2 unit;
+            if (k & 1) {
+                unit.x = (w[0][q] >> 16) | (w[1][q] & 0xffff0000u);
+                unit.y = (w[2][q] >> 16) | (w[3][q] & 0xffff0000u);
+            } else {
+                unit.x = (w[0][q] & 0xffffu) | (w[1][q] << 16);
+                unit.y = (w[2][q] & 0xffffu) | (w[3][q] << 16);
+            }
+            *reinterpret_cast<uint2*>(lds + v * (KT * 2) + ((t4 ^ swz(v)) * 8)) = unit;
+        }
+    }
+    __syncthreads();
+    if (tid < KT) {  // the one-hot term of G^T: token `tid` adds its g at its target's row, if that row is in this tile
+        const int v = tgt_l[tid] - static_cast<int>(col0);
+        if (tgt_l[tid] >= 0 && v >= 0 && v < KT) {
+            uint16_t* cell = reinterpret_cast<uint16_t*>(lds + v * (KT * 2) + (((tid >> 2) ^ swz(v)) * 8) + (tid & 3) * 2);
+            *cell = static_cast<uint16_t>(f32_to_bf16_bits(g_l[tid] + bf16_bits_to_f32(*cell)));
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < KT * 16 / 256; ++it) {
+        const int item = it * 256 + tid, v = item >> 4, mq = item & 15;
+        const uint2 lo = *reinterpret_cast<const uint2*>(lds + v * (KT * 2) + (((2 * mq) ^ swz(v)) * 8));
+        const uint2 hi = *reinterpret_cast<const uint2*>(lds + v * (KT * 2) + (((2 * mq + 1) ^ swz(v)) * 8));
+        const int64_t c = col0 + v, r = row0 + 8 * mq;
+        if (c < a.vocab && r < a.ldgt) *reinterpret_cast<u32x4*>(a.gt + c * a.ldgt + r) = u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // plain GEMM with fp32 output: C = A B^T or C += A B^T
 // ---------------------------------------------------------------------------------------------
 template <class Core, bool ACCUM>
@@ -883,7 +1004,9 @@ template <class Core> static void launch_fwd(LmFwdArgs& a, float* ws, hipStream_
     a.n_splits = fwd_splits<Core>(n, a.op.m);
     a.part_m = ws; a.part_s = ws + static_cast<int64_t>(a.n_splits) * n; a.xt = ws + 2 * static_cast<int64_t>(a.n_splits) * n;
     fill_zero_u32<<<dim3(256), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(a.xt), n);
-    lmhead_fwd_kernel<Core><<<dim3((unsigned)patch_grid((n + Core::BN - 1) / Core::BN, a.n_splits)), dim3(GB_THREADS), 0, s>>>(a);
+    const dim3 grid((unsigned)patch_grid((n + Core::BN - 1) / Core::BN, a.n_splits));
+    if (a.logits) lmhead_fwd_kernel<Core, true><<<grid, dim3(GB_THREADS), 0, s>>>(a);
+    else lmhead_fwd_kernel<Core, false><<<grid, dim3(GB_THREADS), 0, s>>>(a);
 }
 
 template <class Core> static void launch_grad(const LmGradArgs& a, hipStream_t s) {
@@ -903,9 +1026,12 @@ template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, 
 extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                                       const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                                       int64_t vocab_start, int64_t vocab_end, float* logprob_out, float* lse_out,
-                                      void* workspace, int64_t workspace_bytes, void* stream) {
+                                      void* logits_out, int64_t ld_logits, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
     if (int e = check_lmhead(hidden, n_tokens, hidden_size, ldh, weight, vocab, ldw, targets)) return e;
     if (vocab_end - vocab_start != vocab) return fail(NRL_E_INVALID, "vocab range does not span the rows of W");
+    if (logits_out && (ld_logits < vocab || ld_logits % 8 || (reinterpret_cast<uintptr_t>(logits_out) & 15)))
+        return fail(NRL_E_INVALID, "kept logits need 16-byte aligned rows: ld_logits a multiple of 8, at least the vocabulary");
     if (n_tokens == 0) return NRL_OK;
     if (!logprob_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
     if (workspace_bytes < nrl_lmhead_fwd_workspace_bytes(n_tokens, vocab)) return fail(NRL_E_WORKSPACE, "workspace too small");
@@ -914,6 +1040,7 @@ extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int6
     a.op.a = static_cast<const uint16_t*>(weight); a.op.b = static_cast<const uint16_t*>(hidden);
     a.op.lda = ldw; a.op.ldb = ldh; a.op.m = vocab; a.op.n = n_tokens; a.op.k = hidden_size;
     a.targets = targets; a.vocab_start = vocab_start;
+    a.logits = static_cast<uint16_t*>(logits_out); a.ldl = ld_logits;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if ((n_tokens + 255) / 256 >= (1ll << 24)) return fail(NRL_E_INVALID, "too many tokens");
     if (hidden_size % CoreB::BK == 0) launch_fwd<CoreB>(a, ws, s);
@@ -945,10 +1072,13 @@ extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidd
 extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                                       const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                                       int64_t vocab_start, int64_t vocab_end, const float* lse, const float* grad,
-                                      float* dhidden_out, int64_t ld_dh, void* dweight_out, int64_t ld_dw, void* workspace,
-                                      int64_t workspace_bytes, void* stream) {
+                                      const void* logits_kept, int64_t ld_logits, float* dhidden_out, int64_t ld_dh,
+                                      void* dweight_out, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
     if (int e = check_lmhead(hidden, n_tokens, hidden_size, ldh, weight, vocab, ldw, targets)) return e;
     if (vocab_end - vocab_start != vocab) return fail(NRL_E_INVALID, "vocab range does not span the rows of W");
+    if (logits_kept && (ld_logits < vocab || ld_logits % 8 || (reinterpret_cast<uintptr_t>(logits_kept) & 15)))
+        return fail(NRL_E_INVALID, "kept logits need 16-byte aligned rows: ld_logits a multiple of 8, at least the vocabulary");
     if (!dweight_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
     if (n_tokens > 0 && (!lse || !grad || !dhidden_out)) return fail(NRL_E_INVALID, "null argument");
     if (n_tokens >= (1ll << 31)) return fail(NRL_E_INVALID, "too many tokens");
@@ -1000,7 +1130,13 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         ga.op.live = count; ga.op.live_from = t0; ga.op.live_dim = 1;
         ga.targets = tgt_c + t0; ga.vocab_start = vocab_start; ga.lse = lse_c + t0; ga.grad = grad_c + t0;
         ga.g = g; ga.ldg = vp; ga.gt = gt; ga.ldgt = chunk;
-        if (h % CoreB::BK == 0) launch_grad<CoreB>(ga, s);
+        if (logits_kept) {
+            LmGradKeptArgs ka;
+            ka.logits = static_cast<const uint16_t*>(logits_kept); ka.ldl = ld_logits; ka.row_map = idx + t0; ka.live = count;
+            ka.live_from = t0; ka.rows = rows; ka.vocab = vocab; ka.targets = ga.targets; ka.vocab_start = vocab_start;
+            ka.lse = ga.lse; ka.grad = ga.grad; ka.g = g; ka.ldg = vp; ka.gt = gt; ka.ldgt = chunk;
+            lmhead_grad_kept_kernel<<<dim3((unsigned)((vp + KT - 1) / KT), (unsigned)((rows + KT - 1) / KT)), dim3(256), 0, s>>>(ka);
+        } else if (h % CoreB::BK == 0) launch_grad<CoreB>(ga, s);
         else launch_grad<CoreA>(ga, s);
         // dH[token of row r] = G [rows, V] * (W^T [H, V])^T, written to the tokens' own rows
         GemmOperands dh;

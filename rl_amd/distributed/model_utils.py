@@ -433,12 +433,30 @@ def from_parallel_logits_to_logprobs_packed_sequences(
 # ------------------------------------------------------------------------------------------------
 # fused lm_head: hidden states -> logprobs
 # ------------------------------------------------------------------------------------------------
+# Whether the forward keeps its bf16 logits [N, V] for the backward, which then reads them instead of multiplying
+# the hidden states and the weights a second time (a quarter of the step's matrix work).  The reference recomputes
+# (``model_utils.py:2249-2262``) because its logits are fp32 and its memory 80 GB; here the logits of 65 536 tokens
+# x 151 936 ids are 20 GB of 288.  True / False force the choice; "auto" keeps them while they take no more than
+# ``LMHEAD_KEEP_FRACTION`` of the memory that is free when the forward runs.  The gradients are the same both ways.
+LMHEAD_KEEP_LOGITS: Any = "auto"
+LMHEAD_KEEP_FRACTION = 0.25
+
+
+def _keep_lmhead_logits(n_tokens: int, vocab: int, device: torch.device) -> bool:
+    if LMHEAD_KEEP_LOGITS != "auto":
+        return bool(LMHEAD_KEEP_LOGITS)
+    need = n_tokens * ((vocab + 7) // 8 * 8) * 2
+    free, _ = torch.cuda.mem_get_info(device)
+    free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)  # the allocator's own free blocks
+    return need <= LMHEAD_KEEP_FRACTION * free
+
+
 class ChunkedDistributedHiddenStatesToLogprobs(torch.autograd.Function):
     """``model_utils.py:2137-2316`` on one rank: ``apply(hidden [S,B,H], target [B,S] (already shifted),
     output_weight [V,H], vocab_start_index, vocab_end_index, chunk_size, tp_group, inference_only)``
     -> fp32 ``[B,S]``.  The product runs on the bf16 matrix cores with the softmax folded into the
     GEMM epilogue; ``chunk_size`` (the reference's sequence chunk) is not needed to bound memory in the
-    forward, and the backward chunks tokens on its own."""
+    forward, and the backward chunks tokens on its own.  See ``LMHEAD_KEEP_LOGITS`` for what the forward saves."""
 
     @staticmethod
     def forward(ctx, tensor_parallel_hidden_states, target, output_weight_layer, vocab_start_index, vocab_end_index,
@@ -451,10 +469,11 @@ class ChunkedDistributedHiddenStatesToLogprobs(torch.autograd.Function):
         hidden2d = hidden.reshape(s * b, h)
         weight = output_weight_layer.detach()
         tgt = _to_device(target, hidden).long().t().contiguous().reshape(-1)  # token order of the hidden rows: (s, b)
-        lp, lse = _OPS.lmhead_logprob_fwd(hidden2d, weight, tgt, vocab_start_index, vocab_end_index)
         ctx.saved = (not inference_only) and (ctx.needs_input_grad[0] or ctx.needs_input_grad[2])
+        keep = ctx.saved and _keep_lmhead_logits(s * b, weight.shape[0], hidden.device)
+        lp, lse, logits = _OPS.lmhead_logprob_fwd(hidden2d, weight, tgt, vocab_start_index, vocab_end_index, keep)
         if ctx.saved:
-            ctx.save_for_backward(hidden2d, weight, tgt, lse)
+            ctx.save_for_backward(hidden2d, weight, tgt, lse, logits)
             ctx.meta = (s, b, h, vocab_start_index, vocab_end_index, tensor_parallel_hidden_states.dtype,
                         output_weight_layer.dtype)
         return lp.view(s, b).t().contiguous()
@@ -463,10 +482,10 @@ class ChunkedDistributedHiddenStatesToLogprobs(torch.autograd.Function):
     def backward(ctx, *grad_outputs):
         if not ctx.saved:
             raise RuntimeError("backward through a logprob computed with inference_only=True")
-        hidden2d, weight, tgt, lse = ctx.saved_tensors
+        hidden2d, weight, tgt, lse, logits = ctx.saved_tensors
         s, b, h, v0, v1, h_dtype, w_dtype = ctx.meta
         grad = grad_outputs[0].float().t().contiguous().reshape(-1)
-        dh, dw = _OPS.lmhead_logprob_bwd(hidden2d, weight, tgt, lse, grad, v0, v1)
+        dh, dw = _OPS.lmhead_logprob_bwd(hidden2d, weight, tgt, lse, grad, v0, v1, logits if logits.numel() else None)
         return dh.view(s, b, h).to(h_dtype), None, dw.to(w_dtype), None, None, None, None, None
 
 

@@ -1179,11 +1179,12 @@ for _name, _fn in (("neg_entropy_fwd", _neg_entropy_fwd), ("neg_entropy_bwd", _n
 # K6: fused lm_head
 # ------------------------------------------------------------------------------------------------
 _LIB.define(
-    "lmhead_logprob_fwd(Tensor hidden, Tensor weight, Tensor targets, int vocab_start, int vocab_end) -> (Tensor, Tensor)"
+    "lmhead_logprob_fwd(Tensor hidden, Tensor weight, Tensor targets, int vocab_start, int vocab_end, bool keep_logits=False) "
+    "-> (Tensor, Tensor, Tensor)"
 )
 _LIB.define(
     "lmhead_logprob_bwd(Tensor hidden, Tensor weight, Tensor targets, Tensor lse, Tensor grad, int vocab_start, "
-    "int vocab_end) -> (Tensor, Tensor)"
+    "int vocab_end, Tensor? logits=None) -> (Tensor, Tensor)"
 )
 
 
@@ -1206,7 +1207,9 @@ def _ws(nbytes, dev):
     return torch.empty(((nbytes + 255) // 256 * 32,), dtype=torch.float64, device=dev)  # 256-byte granules
 
 
-def _lmhead_logprob_fwd(hidden, weight, targets, vocab_start, vocab_end):
+def _lmhead_logprob_fwd(hidden, weight, targets, vocab_start, vocab_end, keep_logits=False):
+    """-> (logprobs [N], log-sum-exps [N], bf16 logits [N, V] kept for the backward or an empty tensor).  The kept
+    logits are a view of rows padded to a multiple of 8 ids."""
     hidden, weight = _check_lmhead(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
@@ -1215,25 +1218,34 @@ def _lmhead_logprob_fwd(hidden, weight, targets, vocab_start, vocab_end):
     with torch.cuda.device(dev):
         lp = torch.empty((n,), dtype=torch.float32, device=dev)
         lse = torch.empty((n,), dtype=torch.float32, device=dev)
+        ldl = (v + 7) // 8 * 8
+        logits = torch.empty((n, ldl), dtype=torch.bfloat16, device=dev)[:, :v] if keep_logits else None
         nbytes = lib.nrl_lmhead_fwd_workspace_bytes(n, v)
         ws = _ws(nbytes, dev)
         with _timed("lmhead_fwd"):
             code = lib.nrl_lmhead_logprob_fwd(
                 _ptr(hidden), n, h, hidden.stride(0), _ptr(weight), v, weight.stride(0), _ptr(targets), vocab_start,
-                vocab_end, _ptr(lp), _ptr(lse), _ptr(ws), ws.numel() * 8, _stream(),
+                vocab_end, _ptr(lp), _ptr(lse), _ptr(logits), ldl, _ptr(ws), ws.numel() * 8, _stream(),
             )
     _lib.check(code, "nrl_lmhead_logprob_fwd")
-    return lp, lse
+    return lp, lse, (logits if keep_logits else lp.new_empty(0, dtype=torch.bfloat16))
 
 
-def _lmhead_logprob_bwd(hidden, weight, targets, lse, grad, vocab_start, vocab_end):
+def _lmhead_logprob_bwd(hidden, weight, targets, lse, grad, vocab_start, vocab_end, logits=None):
     hidden, weight = _check_lmhead(hidden, weight, targets)
-    _need_gpu(lse, grad)
+    _need_gpu(lse, grad, logits)
     n, h = hidden.shape
     v = weight.shape[0]
     for t, name in ((lse, "lse"), (grad, "grad")):
         if t.dtype != torch.float32 or tuple(t.shape) != (n,) or not t.is_contiguous():
             raise ValueError(f"{name} must be a contiguous fp32 [N] tensor")
+    if logits is not None and logits.numel() == 0 and n * v > 0:
+        logits = None
+    if logits is not None:
+        if logits.dtype != torch.bfloat16 or tuple(logits.shape) != (n, v) or (v > 1 and logits.stride(1) != 1):
+            raise ValueError("kept logits must be the bf16 [N, V] tensor the forward returned")
+        if n > 1 and (logits.stride(0) % 8 or logits.stride(0) < v) or logits.data_ptr() % 16:
+            raise ValueError("kept logits need 16-byte aligned rows")
     lib = _lib.load()
     dev = hidden.device
     with torch.cuda.device(dev):
@@ -1241,10 +1253,12 @@ def _lmhead_logprob_bwd(hidden, weight, targets, lse, grad, vocab_start, vocab_e
         dw = torch.empty((v, h), dtype=torch.bfloat16, device=dev)
         nbytes = lib.nrl_lmhead_bwd_workspace_bytes(n, h, v)
         ws = _ws(nbytes, dev)
+        ldl = 0 if logits is None else (logits.stride(0) if n > 1 else (v + 7) // 8 * 8)
         with _timed("lmhead_bwd"):
             code = lib.nrl_lmhead_logprob_bwd(
                 _ptr(hidden), n, h, hidden.stride(0), _ptr(weight), v, weight.stride(0), _ptr(targets), vocab_start,
-                vocab_end, _ptr(lse), _ptr(grad), _ptr(dh), h, _ptr(dw), h, _ptr(ws), ws.numel() * 8, _stream(),
+                vocab_end, _ptr(lse), _ptr(grad), _ptr(logits), ldl, _ptr(dh), h, _ptr(dw), h, _ptr(ws), ws.numel() * 8,
+                _stream(),
             )
     _lib.check(code, "nrl_lmhead_logprob_bwd")
     return dh, dw

@@ -216,13 +216,17 @@ def test_config5_packed_row_full_shape():
     assert (got_lp - want_lp).abs().max().item() <= 2e-3
 
 
-def test_config3_fused_lm_head_full_width_three_chunks():
+@pytest.mark.parametrize("keep_logits", [False, True])
+def test_config3_fused_lm_head_full_width_three_chunks(keep_logits, monkeypatch):
     """Benchmark config 3 at its full width (H = 4096, V = 151936) over 33068 tokens: the backward runs in
     three token chunks, the last one ragged, so dW is accumulated across launches.  Sixteen sampled tokens
     (some in every chunk) are checked against the oracle: their logprobs, their rows of dH, and -- with the
     upstream gradient zero everywhere else -- the whole of dW, which then is exactly what those sixteen
-    contribute.  Every other row of dH must be exactly zero."""
+    contribute.  Every other row of dH must be exactly zero.  Once with the backward recomputing the logits and
+    once with the forward keeping them (10 GB of bf16 here)."""
     from oracle import lmhead as OH
+
+    monkeypatch.setattr(MU, "LMHEAD_KEEP_LOGITS", keep_logits)
 
     n, h, v = 2 * 16384 + 300, 4096, V_QWEN
     g = torch.Generator(device=DEV).manual_seed(3003)

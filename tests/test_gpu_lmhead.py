@@ -90,7 +90,8 @@ def test_lmhead_backward_matches_oracle(s, b, h, v):
     hid2d = hid.reshape(s * b, h)
     tgt = rolled.t().contiguous().reshape(-1)                          # token order of the hidden rows: (s, b)
     up_rows = up.t().contiguous().reshape(-1)
-    _, lse = torch.ops.rl_amd.lmhead_logprob_fwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), 0, v)
+    _, lse, none = torch.ops.rl_amd.lmhead_logprob_fwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), 0, v)
+    assert none.numel() == 0
     dh, dw = torch.ops.rl_amd.lmhead_logprob_bwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), lse, up_rows.to(DEV), 0, v)
     assert dh.dtype == torch.float32
     o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid2d, w, tgt, up_rows)
@@ -118,14 +119,16 @@ def test_lmhead_equals_unfused_path_on_gpu():
     assert err.max().item() <= 1e-2
 
 
-def _bwd_through_the_op(hid2d, w, tgt, up_rows):
+def _bwd_through_the_op(hid2d, w, tgt, up_rows, keep=False):
     v = w.shape[0]
-    _, lse = torch.ops.rl_amd.lmhead_logprob_fwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), 0, v)
-    return torch.ops.rl_amd.lmhead_logprob_bwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), lse, up_rows.to(DEV), 0, v)
+    _, lse, logits = torch.ops.rl_amd.lmhead_logprob_fwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), 0, v, keep)
+    return torch.ops.rl_amd.lmhead_logprob_bwd(hid2d.to(DEV), w.to(DEV), tgt.to(DEV), lse, up_rows.to(DEV), 0, v,
+                                               logits if keep else None)
 
 
+@pytest.mark.parametrize("keep", [False, True])
 @pytest.mark.parametrize("live", ["none", "one", "last_only"])
-def test_lmhead_backward_runs_on_live_tokens_only(live):
+def test_lmhead_backward_runs_on_live_tokens_only(live, keep):
     """The backward products run on the tokens with a non-zero upstream gradient (the others have a zero row in the
     logits' gradient): no such token, a single one, and one at the very end."""
     g = torch.Generator().manual_seed(5)
@@ -138,7 +141,7 @@ def test_lmhead_backward_runs_on_live_tokens_only(live):
         up[137] = 0.5
     elif live == "last_only":
         up[n - 1] = -0.25
-    dh, dw = _bwd_through_the_op(hid, w, tgt, up)
+    dh, dw = _bwd_through_the_op(hid, w, tgt, up, keep)
     o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
     if live == "none":
         assert bool((dh == 0).all()) and bool((dw.float() == 0).all())
@@ -147,7 +150,8 @@ def test_lmhead_backward_runs_on_live_tokens_only(live):
     assert bool(((dh.cpu() - o_dh).abs() <= b_dh).all()) and bool(((dw.float().cpu() - o_dw).abs() <= b_dw).all())
 
 
-def test_lmhead_backward_live_tokens_across_the_chunk_boundary():
+@pytest.mark.parametrize("keep", [False, True])
+def test_lmhead_backward_live_tokens_across_the_chunk_boundary(keep):
     """More live tokens than one backward chunk holds (16384), ending in a partial chunk whose length is not a
     multiple of the 64-wide K slab; masked tokens scattered in between."""
     g = torch.Generator().manual_seed(6)
@@ -158,9 +162,58 @@ def test_lmhead_backward_live_tokens_across_the_chunk_boundary():
     up = torch.randn(n, generator=g) * 1e-3
     up[torch.rand(n, generator=g) < 0.1] = 0.0
     assert 16384 < int((up != 0).sum()) < n and int((up != 0).sum()) % 64 != 0
-    dh, dw = _bwd_through_the_op(hid, w, tgt, up)
+    dh, dw = _bwd_through_the_op(hid, w, tgt, up, keep)
     o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
     assert bool((dh.cpu()[up == 0] == 0).all())
     assert bool(((dh.cpu() - o_dh).abs() <= b_dh).all())
     assert bool(((dw.float().cpu() - o_dw).abs() <= b_dw).all())
     assert ((dh.cpu() - o_dh).norm() / o_dh.norm()).item() <= 1e-4
+
+
+@pytest.mark.parametrize("n,h,v", [(300, 64, 1000), (257, 72, 4099), (515, 128, 777), (64, 256, 32000)])
+def test_lmhead_kept_logits_are_the_rounded_product_and_give_the_same_gradients(n, h, v):
+    """With ``keep_logits`` the forward leaves the bf16 logits and the backward reads them instead of recomputing
+    the product: the kept values are the product rounded to bf16 (to one bf16 step of the fp32 product, the same
+    latitude as the logprobs), logprobs and log-sum-exps do not change, and the gradients equal those of the
+    recomputing backward -- bit for bit, as both take their softmax from the same rounded logits -- and stay within
+    the oracle's narrowing bounds.  Vocabulary sizes that are not a multiple of 8 and token counts that are not a
+    multiple of the 128-wide tile are among the cases."""
+    g = torch.Generator().manual_seed(n + v)
+    hid = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    w = (torch.randn(v, h, generator=g) * 0.05).to(torch.bfloat16)
+    tgt = torch.randint(0, v, (n,), generator=g)
+    up = torch.randn(n, generator=g) * 1e-3
+    up[torch.rand(n, generator=g) < 0.2] = 0.0
+    hd, wd, td, ud = hid.to(DEV), w.to(DEV), tgt.to(DEV), up.to(DEV)
+    lp0, lse0, _ = torch.ops.rl_amd.lmhead_logprob_fwd(hd, wd, td, 0, v)
+    lp1, lse1, logits = torch.ops.rl_amd.lmhead_logprob_fwd(hd, wd, td, 0, v, True)
+    assert logits.shape == (n, v) and logits.dtype == torch.bfloat16
+    assert bool((lp0 == lp1).all()) and bool((lse0 == lse1).all())
+    exact = hid.float() @ w.float().T
+    step = 2.0 ** -8 * exact.abs() + 1e-30
+    assert bool(((logits.float().cpu() - exact).abs() <= step * 1.01 + 1e-6 * exact.abs().max()).all())
+    # the log-sum-exp of the kept logits is the one the forward reported
+    torch.testing.assert_close(torch.logsumexp(logits.float(), -1), lse1, rtol=0, atol=2e-5)
+    dh0, dw0 = torch.ops.rl_amd.lmhead_logprob_bwd(hd, wd, td, lse0, ud, 0, v)
+    dh1, dw1 = torch.ops.rl_amd.lmhead_logprob_bwd(hd, wd, td, lse1, ud, 0, v, logits)
+    o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
+    assert bool(((dh1.cpu() - o_dh).abs() <= b_dh).all()) and bool(((dw1.float().cpu() - o_dw).abs() <= b_dw).all())
+    assert bool((dh0 == dh1).all()) and bool((dw0 == dw1).all())
+
+
+@pytest.mark.parametrize("keep", [True, False, "auto"])
+def test_lmhead_autograd_with_and_without_kept_logits(keep, monkeypatch):
+    s, b, h, v = 130, 2, 128, 2500
+    hid, w, ids, g = _make(s, b, h, v, seed=21)
+    up = torch.randn(b, s - 1, generator=g) * 1e-3
+    monkeypatch.setattr(MU, "LMHEAD_KEEP_LOGITS", False)
+    h0, w0 = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp0 = MU.from_parallel_hidden_states_to_logprobs(h0, w0, False, ids.to(DEV), 0, v, None)
+    (lp0 * up.to(DEV)).sum().backward()
+    monkeypatch.setattr(MU, "LMHEAD_KEEP_LOGITS", keep)
+    h1, w1 = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp1 = MU.from_parallel_hidden_states_to_logprobs(h1, w1, False, ids.to(DEV), 0, v, None)
+    (lp1 * up.to(DEV)).sum().backward()
+    assert bool((lp0 == lp1).all()) and bool((h0.grad == h1.grad).all()) and bool((w0.grad == w1.grad).all())
+    with torch.no_grad():   # nothing is kept when no gradient can be asked for
+        MU.from_parallel_hidden_states_to_logprobs(hid.to(DEV), w.to(DEV), False, ids.to(DEV), 0, v, None, inference_only=True)
