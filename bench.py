@@ -672,7 +672,7 @@ def bench_lmhead(args, torch, w):
     products = 2.0 if kept else 3.0                                       # dH, dW (+ the recomputed logits)
     bwd_alg_tf = 4.0 * n * h * v / (bwd_ms * 1e-3) / 1e12                 # dH + dW of every token, the algorithmic count
     bwd_exec_tf = 2.0 * products * live * n * h * v / (bwd_ms * 1e-3) / 1e12   # what the matrix cores execute, live tokens
-    fills = MEASURED_TRAFFIC.get("c3_fwd") if not args.seqs and not kept else None
+    fills = MEASURED_TRAFFIC.get("c3_fwd_kept" if kept else "c3_fwd") if not args.seqs else None
     result = {
         "metric": "fused lm_head + GRPO loss fwd/bwd tokens/s; % of bf16 MFMA peak",
         "value": n * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
