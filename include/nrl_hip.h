@@ -118,6 +118,16 @@ int nrl_scale_rows(const void* src, void* dst, int32_t dtype, int64_t n_outer, i
                    int64_t src_stride_outer, int64_t src_stride_inner, int64_t dst_stride_outer,
                    int64_t dst_stride_inner, const float* factor, float divisor, void* stream);
 
+/* _pack_input_ids (nemo_rl/algorithms/loss/utils.py:214-261) at CP = 1, on the device and without a host read of
+ * the boundaries: input_ids int64 [batch, width] rows of row_stride -> packed_out int64 [total_out].  Sequence s
+ * fills [cu_seqlens_padded[s], cu_seqlens_padded[s+1]) with its first min(cu_seqlens[s+1] - cu_seqlens[s], width)
+ * ids, rolled by roll_shift inside that span (element j comes from (j - roll_shift) mod span); every other
+ * position, and the positions from cu_seqlens_padded[batch] to total_out, are zero.  Both boundary arrays are
+ * int32 [batch + 1] on the device. */
+int nrl_pack_input_ids(const int64_t* input_ids, int64_t batch, int64_t width, int64_t row_stride,
+                       const int32_t* cu_seqlens, const int32_t* cu_seqlens_padded, int64_t roll_shift,
+                       int64_t* packed_out, int64_t total_out, void* stream);
+
 /* Packed sequences (one [1, T, V] row of logits, sequences delimited by cu_seqlens_padded).
  * Replaces from_parallel_logits_to_logprobs_packed_sequences (model_utils.py:1085-1196) at
  * CP = 1: position p of sequence s (start = cu[s], len = cu[s+1]-cu[s]) uses target

@@ -72,6 +72,7 @@ SIGNATURES = {
     "nrl_logprob_post_fwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P]),
     "nrl_logprob_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _I64, _I64, _P, _I64, _I64, _I64, _P]),
     "nrl_scale_rows": (C.c_int, [_P, _P, _I32, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _F, _P]),
+    "nrl_pack_input_ids": (C.c_int, [_P, _I64, _I64, _I64, _P, _P, _I64, _P, _I64, _P]),
     "nrl_logprob_packed_fwd": (C.c_int, [_P, _I32, _I64, _I64, _I64, _P, _I32, _P, _I64, _I64, _I64, _I64, _F, _I32, _P, _P, _P]),
     "nrl_logprob_packed_bwd": (C.c_int, [_P, _I32, _I64, _I64, _I64, _P, _I32, _P, _I64, _I64, _I64, _I64, _F, _I32, _P, _P, _P, _I64, _P]),
     "nrl_log_softmax_fwd": (C.c_int, [_P, C.c_int32, _I64, _I64, _I64, _P, _I64, _P]),

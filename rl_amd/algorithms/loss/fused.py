@@ -170,7 +170,7 @@ def fused_packed_logits_clipped_pg_loss(logits, data, loss_fn, cu_seqlens_q, cu_
     """``SequencePackingFusionLossWrapper.__call__`` (``loss/wrapper.py:169-228``) in one pass over the packed
     logits: ``prepare_packed_loss_input`` + ``ClippedPGLossFn`` + the backward of the packed logprob op."""
     from ...distributed.model_utils import _checked_cu_seqlens
-    from .utils import _pack_input_ids, _pad_to
+    from .utils import _packed_targets
 
     reason = why_not_fusable_packed(loss_fn, logits, data)
     if reason is not None:
@@ -179,8 +179,7 @@ def fused_packed_logits_clipped_pg_loss(logits, data, loss_fn, cu_seqlens_q, cu_
     dev = logits.device
     input_ids = data["input_ids"]
     x = logits.squeeze(0)
-    targets = _pad_to(_pack_input_ids(input_ids, cu_seqlens_q, cu_seqlens_q_padded, roll_shift=-1), x.shape[0])
-    targets = targets.to(dev).reshape(-1).long().contiguous()
+    targets = _packed_targets(input_ids, cu_seqlens_q, cu_seqlens_q_padded, x.shape[0], dev).reshape(-1)
     cu = _checked_cu_seqlens(cu_seqlens_q_padded, x.shape[0], targets.shape[0], dev)
     beta = loss_fn.reference_policy_kl_penalty
     sample_mask_in = data["sample_mask"]

@@ -109,10 +109,18 @@ def _pack_input_ids(
     return packed.unsqueeze(0)
 
 
-def _pad_to(packed_ids: torch.Tensor, total: int) -> torch.Tensor:
-    """Zero ids for packed positions behind the last sequence (a row padded past ``cu_seqlens_padded[-1]``)."""
-    short = total - packed_ids.shape[1]
-    return torch.nn.functional.pad(packed_ids, (0, short)) if short > 0 else packed_ids
+def _packed_targets(input_ids: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_q_padded: torch.Tensor,
+                    total: int, dev: torch.device) -> torch.Tensor:
+    """``_pack_input_ids(..., roll_shift=-1)`` padded to the ``total`` packed positions, ``[1, total]`` on ``dev``,
+    by one kernel that reads the boundaries where they are: with boundaries that live on the GPU (as the attention
+    kernels need them) the host reads nothing and does not wait for the device."""
+    def on_dev(t):
+        return t.detach().to(device=dev, dtype=torch.int32).contiguous()
+
+    ids = input_ids.to(dev)
+    ids = ids if ids.dtype == torch.int64 else ids.long()
+    ids = ids if ids.dim() != 2 or ids.shape[1] <= 1 or ids.stride(1) == 1 else ids.contiguous()
+    return torch.ops.rl_amd.pack_input_ids(ids, on_dev(cu_seqlens_q), on_dev(cu_seqlens_q_padded), -1, total).unsqueeze(0)
 
 
 def prepare_packed_loss_input(
@@ -137,7 +145,7 @@ def prepare_packed_loss_input(
     input_ids = data["input_ids"]
     rank = vocab_parallel_rank or 0
     vocab = logits.shape[-1]
-    targets = _pad_to(_pack_input_ids(input_ids, cu_seqlens_q, cu_seqlens_q_padded, roll_shift=-1), logits.shape[1])
+    targets = _packed_targets(input_ids, cu_seqlens_q, cu_seqlens_q_padded, logits.shape[1], logits.device)
 
     def logprobs_with(params):
         return from_parallel_logits_to_logprobs_packed_sequences(

@@ -294,7 +294,7 @@ struct FusedArgs {
 struct FusedPos {
     int64_t o, i, tgt;
 };
-__device__ __forceinline__ FusedPos fused_where_packed(const FusedArgs& a, int64_t r) {
+__device__ __forceinline__ FusedPos fused_where_packed(const FusedArgs& a, int64_t r, int64_t total) {
     FusedPos q;
     const int64_t seq = find_seq(a.cu, a.n_seq, r);
     q.o = seq < 0 ? 0 : seq;
@@ -304,6 +304,8 @@ __device__ __forceinline__ FusedPos fused_where_packed(const FusedArgs& a, int64
         const int64_t start = a.cu[seq], len = a.cu[seq + 1] - start, pos = r - start;
         if (pos + 1 < len && pos < a.n_inner) q.i = pos;  // the last position of a sequence predicts nothing
         q.tgt = start + (a.pre_rolled ? pos : (pos + 1 < len ? pos + 1 : 0));
+        // (the targets hold at least `total` entries; boundaries that run past the packed row cannot index beyond them)
+        if (q.tgt >= total) q.tgt = total - 1;
     }
     return q;
 }
@@ -312,7 +314,7 @@ __device__ __forceinline__ FusedPos fused_where_packed(const FusedArgs& a, int64
 __global__ __launch_bounds__(256) void fused_row_pos_kernel(FusedArgs a, int64_t total) {
     const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (r >= total) return;
-    const FusedPos q = fused_where_packed(a, r);
+    const FusedPos q = fused_where_packed(a, r, total);
     a.row_pos[r] = make_int4(static_cast<int>(q.o), static_cast<int>(q.i), static_cast<int>(q.tgt), 0);
 }
 template <bool PACKED>

@@ -246,7 +246,9 @@ __device__ __forceinline__ PackedPos locate(const PackedArgs& a, int64_t p, Pack
 
 __device__ __forceinline__ int64_t packed_target(const PackedArgs& a, const PackedPos& q) {
     const int64_t j = a.pre_rolled ? q.pos : (q.pos + 1 == q.len ? 0 : q.pos + 1);
-    return a.targets[q.start + j];
+    // (the targets hold at least `total` entries; boundaries that run past the packed row cannot index beyond them)
+    const int64_t t = q.start + j;
+    return a.targets[t < a.total ? t : a.total - 1];
 }
 
 template <int DT, int TEMP>
@@ -512,6 +514,26 @@ extern "C" int nrl_logprob_bwd(const nrl_rows* rows, const float* lse, const flo
     return check_launch("logprob_bwd");
 }
 
+// ids [B, S] -> packed ids [total_out]: sequence s fills [cup[s], cup[s+1]) with its first min(cu[s+1] - cu[s], S)
+// ids, rolled by `shift` inside that span (element j comes from (j - shift) mod span), zero elsewhere.
+__global__ __launch_bounds__(256) void pack_ids_kernel(const int64_t* ids, int64_t batch, int64_t width, int64_t ids_stride,
+                                                       const int32_t* cu, const int32_t* cup, int64_t shift, int64_t* out,
+                                                       int64_t total_out) {
+    const int64_t p = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (p >= total_out) return;
+    int64_t v = 0;
+    const int64_t s = find_seq(cup, batch, p);
+    if (s >= 0) {
+        const int64_t start = cup[s], span = cup[s + 1] - start;  // span >= 1: p lies inside it
+        int64_t n_real = static_cast<int64_t>(cu[s + 1]) - cu[s];
+        n_real = n_real < width ? n_real : width;
+        int64_t src = (p - start - shift) % span;
+        if (src < 0) src += span;
+        if (src < n_real) v = ids[s * ids_stride + src];
+    }
+    out[p] = v;
+}
+
 static int check_packed(const void* logits, int32_t dtype, int64_t total, int64_t vocab, const int64_t* targets,
                         const int32_t* cu, int64_t n_seq, int64_t unpacked_seqlen, int64_t vstart, int64_t vend,
                         float temperature, int32_t temp_mode) {
@@ -614,4 +636,16 @@ extern "C" int nrl_scale_rows(const void* src, void* dst, int32_t dtype, int64_t
                                  src, dst, n_inner, vocab, src_stride_outer, src_stride_inner, dst_stride_outer,
                                  dst_stride_inner, factor, divisor));
     return check_launch("scale_rows");
+}
+
+extern "C" int nrl_pack_input_ids(const int64_t* input_ids, int64_t batch, int64_t width, int64_t row_stride,
+                                  const int32_t* cu_seqlens, const int32_t* cu_seqlens_padded, int64_t roll_shift,
+                                  int64_t* packed_out, int64_t total_out, void* stream) {
+    if (batch < 0 || width < 0 || total_out < 0 || row_stride < width) return fail(NRL_E_INVALID, "pack_input_ids: bad shape");
+    if (total_out == 0) return NRL_OK;
+    if (!packed_out || !cu_seqlens || !cu_seqlens_padded || (batch * width > 0 && !input_ids))
+        return fail(NRL_E_INVALID, "pack_input_ids: null pointer");
+    pack_ids_kernel<<<dim3((unsigned)((total_out + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        input_ids, batch, width, row_stride, cu_seqlens, cu_seqlens_padded, roll_shift, packed_out, total_out);
+    return check_launch("pack_input_ids");
 }

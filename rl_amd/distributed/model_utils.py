@@ -372,8 +372,15 @@ class _PackedLogprob(torch.autograd.Function):
 
 
 def _checked_cu_seqlens(cu_seqlens_padded: torch.Tensor, total: int, n_targets: int, device) -> torch.Tensor:
-    """One host read of the sequence boundaries (the reference reads them per sequence): they must be
-    non-decreasing and stay inside the packed buffers, because the kernels index with them."""
+    """The sequence boundaries as int32 on the device.  Boundaries that live on the host are checked there (they
+    should be non-decreasing and stay inside the packed buffers).  Boundaries that live on the GPU are taken as they
+    are, so the host neither reads them nor waits for the device (the reference reads them per sequence): the
+    kernels find a position's sequence by bisection, which ends at a span that contains it whatever the order, and
+    clamp the target index to the packed row, so bad boundaries give wrong numbers but no stray access."""
+    if cu_seqlens_padded.is_cuda:
+        if cu_seqlens_padded.dim() != 1 or cu_seqlens_padded.numel() < 1:
+            raise ValueError("cu_seqlens_padded must be a 1-D tensor with at least one entry")
+        return cu_seqlens_padded.detach().to(device=device, dtype=torch.int32).contiguous()
     host = cu_seqlens_padded.detach().to("cpu", torch.int64)
     if host.dim() != 1 or host.numel() < 1:
         raise ValueError("cu_seqlens_padded must be a 1-D tensor with at least one entry")

@@ -221,6 +221,30 @@ for _name, _fn in (("logprob_fwd", _logprob_fwd), ("logprob_bwd", _logprob_bwd),
 # ------------------------------------------------------------------------------------------------
 # packed sequences
 # ------------------------------------------------------------------------------------------------
+_LIB.define("pack_input_ids(Tensor input_ids, Tensor cu_seqlens, Tensor cu_seqlens_padded, int roll_shift, int total) -> Tensor")
+
+
+def _pack_input_ids(input_ids, cu_seqlens, cu_seqlens_padded, roll_shift, total):
+    """``[B, S]`` int64 ids -> packed ``[total]`` ids; the boundaries are int32 ``[B + 1]`` device tensors that the
+    host never reads."""
+    _need_gpu(input_ids, cu_seqlens, cu_seqlens_padded)
+    if input_ids.dim() != 2 or input_ids.dtype != torch.int64 or (input_ids.shape[1] > 1 and input_ids.stride(1) != 1):
+        raise ValueError("input_ids must be int64 [B, S] with a contiguous last axis")
+    b, s = input_ids.shape
+    for t in (cu_seqlens, cu_seqlens_padded):
+        if t.dtype != torch.int32 or tuple(t.shape) != (b + 1,) or not t.is_contiguous():
+            raise ValueError(f"sequence boundaries must be contiguous int32 [{b + 1}] tensors")
+    with torch.cuda.device(input_ids.device):
+        out = torch.empty((int(total),), dtype=torch.int64, device=input_ids.device)
+        code = _lib.load().nrl_pack_input_ids(_ptr(input_ids), b, s, input_ids.stride(0) if b > 1 else max(s, 1), _ptr(cu_seqlens),
+                                              _ptr(cu_seqlens_padded), int(roll_shift), _ptr(out), int(total), _stream())
+    _lib.check(code, "nrl_pack_input_ids")
+    return out
+
+
+_LIB.impl("pack_input_ids", _pack_input_ids, "CUDA")
+_LIB.impl("pack_input_ids", _pack_input_ids, "CPU")
+
 _LIB.define(
     "logprob_packed_fwd(Tensor logits, Tensor targets, bool pre_rolled, Tensor cu_seqlens, int unpacked_seqlen, "
     "int vocab_start, int vocab_end, float temperature, int temp_mode, bool save_lse) -> (Tensor, Tensor)"

@@ -272,3 +272,34 @@ def test_megatron_loss_post_processor_counteracts_the_schedule_averaging():
         loss.backward()
         assert _close(loss.item(), 3 * want.item(), rel=1e-5)
         assert (x.grad.cpu() - 3 * want_grad).abs().max().item() <= 1e-4 * 3 * want_grad.abs().max().item()
+
+
+@pytest.mark.parametrize("roll", [0, -1, 1, -5])
+@pytest.mark.parametrize("cu_on_gpu", [True, False])
+def test_device_id_packing_matches_the_oracle(roll, cu_on_gpu):
+    """The packing kernel (ids [B, S] -> one packed row, rolled inside every padded span, read from boundaries that
+    stay on the device) against the oracle's loop per sequence: padded spans, an empty sequence, a recorded length
+    beyond the row width, a first boundary above zero and packed rows longer than the last boundary."""
+    from oracle import logprob as OLP
+
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(1, 50, (4, 12), generator=g)
+    cases = [
+        (ids, [0, 5, 17, 17, 26], [0, 8, 24, 24, 36], 36),
+        (ids, [0, 5, 17, 17, 26], [0, 8, 24, 24, 36], 50),
+        (ids[:2], [0, 5, 20], [0, 8, 24], 24),
+        (ids[:3], [3, 9, 9, 21], [4, 12, 12, 24], 31),
+        (ids[:1], [0, 1], [0, 1], 1),
+    ]
+    for rows, cu, cup, total in cases:
+        cu_t, cup_t = torch.tensor(cu), torch.tensor(cup)
+        want = OLP.pack_input_ids(rows, cu_t, cup_t, roll_shift=roll).reshape(-1)
+        want = torch.nn.functional.pad(want, (0, total - want.numel()))
+        where = DEV if cu_on_gpu else "cpu"
+        got = torch.ops.rl_amd.pack_input_ids(rows.to(DEV), cu_t.to(DEV, torch.int32), cup_t.to(DEV, torch.int32), roll, total)
+        assert torch.equal(got.cpu(), want), (cu, cup, total)
+        if roll == -1:
+            from rl_amd.algorithms.loss.utils import _packed_targets
+
+            via = _packed_targets(rows.to(DEV), cu_t.to(where), cup_t.to(where), total, torch.device(DEV))
+            assert via.shape == (1, total) and torch.equal(via.cpu().reshape(-1), want)
