@@ -49,9 +49,10 @@ _PATCHED = {
     "nemo_rl.algorithms.loss.utils": ["prepare_loss_input", "prepare_packed_loss_input"],
     "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn",
                                                "DraftCrossEntropyLossFn"],
-    "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt"],
+    "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt", "calculate_kl", "masked_mean",
+                                 "mask_out_neg_inf_logprobs"],
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling"],
-    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor", "apply_temperature_scaling"],
+    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling"],
     "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking", "dynamic_sampling"],
     "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }
