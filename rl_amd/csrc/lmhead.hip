@@ -333,6 +333,14 @@ template <class Core> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[Cor
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 }
 
+// One accumulator element, moved from its accumulation register when it is used: read this way the epilogue takes
+// the values block by block, where plain uses let the compiler copy all 256 to vector registers first and spill.
+__device__ __forceinline__ float acc_read(float a) {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
 __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
 // Tile coordinates of workgroup w of a 1-D launch over an nbx x nby tile grid.  Workgroups go to the
@@ -395,19 +403,27 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
         tgt_s[tid] = (t >= 0 && t < a.op.m) ? static_cast<int>(t) : -1;
     }
     __syncthreads();
-    const int col = wn * (NJ * 32) + (lane & 31);  // this lane's token column of tile j is col + j * 32
-    float run_m[NJ], run_s[NJ];
+    // Running (max, sum exp) of the lane's NJ token columns.  They live in LDS, not in registers: the K loop of a
+    // tile takes every vector register, and a value that is live across it would be spilled to scratch.  For the
+    // same reason everything derived from the thread index is derived again, from an opaque copy, after the K loop.
+    __shared__ float run_m_s[NJ][GB_THREADS], run_s_s[NJ][GB_THREADS];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) { run_m[j] = -1e30f; run_s[j] = 0.f; }
+    for (int j = 0; j < NJ; ++j) { run_m_s[j][tid] = -1e30f; run_s_s[j][tid] = 0.f; }
 
     for (int64_t tile = split; tile < n_tiles; tile += a.n_splits) {
         const int64_t v0 = tile * BV;
         f32x16 acc[NI][NJ];
         zero_acc<Core>(acc);
         Core::tile(a.op, v0, tok0, acc, lds);
+        int t2 = threadIdx.x;
+        // (the accumulators are read below by instructions the compiler does not look into: the wait a matrix
+        // instruction's result needs before another unit reads it is spelled out)
+        asm volatile("s_nop 15\n s_nop 7" : "+v"(t2));
+        const int lane2 = t2 & 63, wm2 = t2 >> 7, wn2 = (t2 >> 6) & 1;
+        const int col = wn2 * (NJ * 32) + (lane2 & 31);  // this lane's token column of tile j is col + j * 32
         // Accumulator element e of tile i is row `off` = i * 32 + 8 * (e / 4) + e % 4 (a compile-time constant)
         // below this lane's first row vb.  Only the last vocabulary tile needs the rows-past-the-end mask.
-        const int vb = static_cast<int>(v0) + wm * 128 + 4 * (lane >> 5);
+        const int vb = static_cast<int>(v0) + wm2 * 128 + 4 * (lane2 >> 5);
         const int limit = static_cast<int>(a.op.m) - vb;  // rows with off < limit exist
         // One 32 x 32 block (16 accumulator registers) at a time, so that only those 16 values are live next to
         // the accumulators: running maximum and sum are rescaled per block (one extra exponential per 16).
@@ -417,6 +433,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
             for (int j = 0; j < NJ; ++j) {
                 const int tg = tgt_s[col + j * 32];
                 const int toff = tg - vb;  // the target's row as an offset, if it is in this lane at all
+                float run_m = run_m_s[j][t2], run_s = run_s_s[j][t2];
 #pragma unroll
                 for (int i = 0; i < NI; ++i) {
                     __builtin_amdgcn_sched_barrier(0);
@@ -427,7 +444,8 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int off = i * 32 + 8 * (e >> 2) + (e & 3);
-                        x[e] = (!MASKED || off < limit) ? acc[i][j][e] : -INFINITY;
+                        const float r = acc_read(acc[i][j][e]);
+                        x[e] = (!MASKED || off < limit) ? r : -INFINITY;
                         raw = fmaxf(raw, x[e]);
                     }
                     if constexpr (SAVE) {
@@ -442,27 +460,36 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
                                         uint2{pack_bf16x2(x[4 * q], x[4 * q + 1]), pack_bf16x2(x[4 * q + 2], x[4 * q + 3])};
                         }
                     }
-                    const float mx = fmaxf(run_m[j], round_bf16(raw));
+                    const float mx = fmaxf(run_m, round_bf16(raw));
                     const float mx2 = mx * kLog2e;
                     // (the subtraction is exact where an FMA against the rounded mx2 would leave a huge residual
                     // while both maxima are still the -1e30 start value)
-                    float sx = run_s[j] * fast_exp2((run_m[j] - mx) * kLog2e);
+                    float sx = run_s * fast_exp2((run_m - mx) * kLog2e);
 #pragma unroll
                     for (int e = 0; e < 16; ++e) sx += fast_exp2(__builtin_fmaf(round_bf16(x[e]), kLog2e, -mx2));
-                    run_m[j] = mx;
-                    run_s[j] = sx;
+                    run_m = mx;
+                    run_s = sx;
                     if (tg >= 0 && toff >= i * 32 && toff < i * 32 + 32 && (toff & 4) == 0) {  // rare: the target's row is here
+                        // (read again from the accumulators, so that the 16 values above need not stay live for this)
                         float xt = 0.f;
 #pragma unroll
-                        for (int e = 0; e < 16; ++e) xt = toff == i * 32 + 8 * (e >> 2) + (e & 3) ? x[e] : xt;
+                        for (int e = 0; e < 16; ++e) {
+                            const float r = acc_read(acc[i][j][e]);
+                            xt = toff == i * 32 + 8 * (e >> 2) + (e & 3) ? r : xt;
+                        }
                         a.xt[tok0 + col + j * 32] = round_bf16(xt);
                     }
                 }
+                run_m_s[j][t2] = run_m;
+                run_s_s[j][t2] = run_s;
             }
         };
         if (v0 + BV <= a.op.m) fold_tile(std::false_type{});
         else fold_tile(std::true_type{});
     }
+    float run_m[NJ], run_s[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { run_m[j] = run_m_s[j][tid]; run_s[j] = run_s_s[j][tid]; }
     // merge the two half-waves (rows 4 apart), then the two waves that share these token columns
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
