@@ -433,6 +433,15 @@ def bench_topk(args, torch, w):
             del d, loss, loss_input
 
     elapsed, k = timed(torch, ops, args, step)
+    # the same step with the backward streaming the logits again instead of using the forward's record of the kept sets
+    from rl_amd.distributed import sampling_logprob as SL
+
+    record_capacity = SL._record_capacity
+    SL._record_capacity = lambda top_k: 0
+    try:
+        s_elapsed, sk = timed(torch, ops, args, step)
+    finally:
+        SL._record_capacity = record_capacity
     nan = dict(avg_ms=float("nan"))
     fwd, bwd = k.get("topk_topp_fwd", nan), k.get("topk_topp_bwd", nan)
     rows = w["mb_seqs"] * w["seq_len"]
@@ -447,12 +456,21 @@ def bench_topk(args, torch, w):
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
                    "temperature": "divided inside the timed region by the logprob kernels (deferred_temperature), bf16 rounding of a GPU div_"},
-        "algorithmic_bytes_per_token": 3 * row_bytes,
-        "hbm_frac_end_to_end": 3 * row_bytes * tokens * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
-        "roofline": hbm_roofline("topk_topp_stream_kernel (backward)", 2 * row_bytes * rows, bwd["avg_ms"], "c4" if full else None),
+        # the forward reads a row once; the backward writes the gradient row (zeros and the <= 64 kept entries the
+        # forward left on record) without reading the logits again
+        "algorithmic_bytes_per_token": 2 * row_bytes,
+        "hbm_frac_end_to_end": 2 * row_bytes * tokens * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
+        "roofline": hbm_roofline("topk_topp_stream_kernel (backward from the kept-set record: write only)", row_bytes * rows,
+                                 bwd["avg_ms"], "c4" if full else None),
         "roofline_fwd": hbm_roofline("topk_topp_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
                                      "c4_fwd" if full else None),
         "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
+        "streaming_backward": {
+            "value": tokens * args.steps / s_elapsed, "unit": "tokens/s", "ms_per_step": s_elapsed / args.steps * 1e3,
+            "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in sk.items()},
+            "roofline": hbm_roofline("topk_topp_stream_kernel (backward reading the logits)", 2 * row_bytes * rows,
+                                     sk.get("topk_topp_bwd", nan)["avg_ms"], "c4_streaming" if full else None),
+            "note": "without the kept-set record: the backward streams every live row again (3 x V bytes per token)"},
     }
     del mbs
     finish(result, args, torch, w, "topk", cpu_rows=256, gpu_rows=2048)

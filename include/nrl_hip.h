@@ -168,12 +168,20 @@ int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t total_toke
  * ------------------------------------------------------------------------------------------ */
 int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
                               float* thr_out, int32_t* tie_out, float* lse_kept_out,
-                              float* logprob_unfiltered_out, float* lse_full_out, void* stream);
+                              float* logprob_unfiltered_out, float* lse_full_out, int32_t* kept_count_out,
+                              int32_t* kept_index_out, float* kept_value_out, int64_t kept_capacity, void* stream);
 
-/* dlogits_v = keep_v * g * (onehot_v - exp(x_v - lse_kept)); layout arguments as nrl_logprob_bwd. */
+/* dlogits_v = keep_v * g * (onehot_v - exp(x_v - lse_kept)); layout arguments as nrl_logprob_bwd.
+ * The kept-set record (optional, all of it or none; no counterpart in the reference, which keeps the whole filtered
+ * row for autograd): a forward given kept_count_out int32 [rows], kept_index_out int32 [rows, kept_capacity] and
+ * kept_value_out fp32 [rows, kept_capacity] (kept_capacity <= 2048) also writes, for every row whose kept set has
+ * at most kept_capacity elements, their number, their vocabulary indices and their (temperature-scaled) logits,
+ * and -1 as the number for every other row.  A backward given the record back writes the gradient row of a
+ * recorded row as zeros plus those few entries without reading the logits; other rows stream as without it. */
 int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,
                               const float* lse_kept, const float* grad, int64_t grad_stride_outer,
-                              int64_t grad_stride_inner, void* dlogits, int64_t d_n_inner,
+                              int64_t grad_stride_inner, const int32_t* kept_count, const int32_t* kept_index,
+                              const float* kept_value, int64_t kept_capacity, void* dlogits, int64_t d_n_inner,
                               int64_t d_stride_outer, int64_t d_stride_inner, void* stream);
 
 /* Materialises apply_top_k_top_p's outputs from a forward's (thr, tie): filtered logits (-inf outside

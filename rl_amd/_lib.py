@@ -77,8 +77,8 @@ SIGNATURES = {
     "nrl_logprob_packed_bwd": (C.c_int, [_P, _I32, _I64, _I64, _I64, _P, _I32, _P, _I64, _I64, _I64, _I64, _F, _I32, _P, _P, _P, _I64, _P]),
     "nrl_log_softmax_fwd": (C.c_int, [_P, C.c_int32, _I64, _I64, _I64, _P, _I64, _P]),
     "nrl_log_softmax_bwd": (C.c_int, [_P, C.c_int32, _I64, _I64, _I64, _P, _I64, _P, _I64, _P]),
-    "nrl_topk_topp_logprob_fwd": (C.c_int, [C.POINTER(NrlRows), _I64, _F, _P, _P, _P, _P, _P, _P, _P]),
-    "nrl_topk_topp_logprob_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P, _P, _I64, _I64, _P, _I64, _I64, _I64, _P]),
+    "nrl_topk_topp_logprob_fwd": (C.c_int, [C.POINTER(NrlRows), _I64, _F, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
+    "nrl_topk_topp_logprob_bwd": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _P]),
     "nrl_topk_topp_filter": (C.c_int, [C.POINTER(NrlRows), _P, _P, _P, _I64, _I64, _P, _P]),
     "nrl_grpo_loss_workspace_bytes": (_I64, [_I64]),
     "nrl_grpo_loss_fwd_bwd": (C.c_int, [C.POINTER(NrlGrpoCfg), C.POINTER(NrlGrpoInputs), _P, _P, _P, _P, _P, _I64, _P]),

@@ -195,6 +195,11 @@ struct SelArgs {
     float* lse_kept;     // [rows]
     float* logprob_full; // [rows] or NULL: unfiltered logprob of the target
     float* lse_full;     // [rows] or NULL
+    // the kept set itself, for a backward that does not read the row again (all three NULL: not recorded):
+    int32_t* kept_n;     // [rows] number of kept elements, -1 if they do not fit kept_cap (or the row was left to the wide kernel)
+    int32_t* kept_idx;   // [rows, kept_cap] their vocabulary indices, in descending (value, index) order
+    float* kept_x;       // [rows, kept_cap] their (scaled) logits
+    int kept_cap;
 };
 
 // PONLY: top-p without top-k (its own instantiation, so that the mass histogram costs the top-k variants
@@ -492,6 +497,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             if (a.logprob) a.logprob[r] = __builtin_nanf("");
             if (a.lse_full) a.lse_full[r] = lse_full;
             if (a.logprob_full) a.logprob_full[r] = __builtin_nanf("");
+            if (a.kept_n) a.kept_n[r] = -1;
         }
         return;
     }
@@ -555,7 +561,15 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         int tie = 0;
         if (n_keep < n && static_cast<uint32_t>(sh.cand[n_keep] >> 32) == last_key) tie = static_cast<int>(last & 0xffffffffu);
         const float thr = key_value(last_key), lse_kept = m + logf(s);
+        if (a.kept_n && n_keep <= a.kept_cap) {
+            for (int q = tid; q < n_keep; q += kWave) {
+                const unsigned long long c = sh.cand[q];
+                a.kept_idx[r * a.kept_cap + q] = static_cast<int32_t>(c & 0xffffffffu);
+                a.kept_x[r * a.kept_cap + q] = key_value(static_cast<uint32_t>(c >> 32));
+            }
+        }
         if (tid == 0) {
+            if (a.kept_n) a.kept_n[r] = n_keep <= a.kept_cap ? n_keep : -1;
             a.thr[r] = thr;
             a.tie[r] = tie;
             a.lse_kept[r] = lse_kept;
@@ -815,27 +829,57 @@ struct SelBwdArgs {
     void* out;  // dlogits, or filtered logits
     int64_t d_n_inner, ds_outer, ds_inner;
     uint8_t* keep_out;  // [rows, vocab] or NULL (filter mode)
+    const int32_t* kept_n;    // the forward's record of the kept sets (see SelArgs), or NULL
+    const int32_t* kept_idx;
+    const float* kept_x;
+    int kept_cap;
 };
 
 // MODE 0: gradient, MODE 1: filtered logits (-inf outside the kept set) + keep mask
 template <int DT, int TEMP, int MODE>
-__global__ __launch_bounds__(kSelBlock) void topk_topp_stream_kernel(SelBwdArgs a) {
+__device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_t r) {
     constexpr int EPV = Row<DT>::EPV;
     const int tid = threadIdx.x;
-    const int64_t r = blockIdx.x;
     const int64_t o = r / a.d_n_inner, i_in = r - o * a.d_n_inner;
     char* out = static_cast<char*>(a.out) + (o * a.ds_outer + i_in * a.ds_inner) * Row<DT>::BYTES;
     const int64_t vocab = a.vocab;
     float g = 0.f;
     if (MODE == 0 && i_in < a.n_inner) g = a.grad[o * a.gs_outer + i_in * a.gs_inner];
-    if (MODE == 0 && g == 0.f) {  // dropped position or masked token: the gradient row is exactly zero
+    // With the forward's record of the kept set the gradient row is zeros plus the few kept entries, written
+    // without reading the logits again.
+    int n_rec = -1;
+    if (MODE == 0 && g != 0.f && a.kept_n) n_rec = a.kept_n[o * a.n_inner + i_in];
+    if (MODE == 0 && (g == 0.f || n_rec >= 0)) {  // dropped position or masked token: the gradient row is exactly zero
+        __shared__ int32_t rec_idx[kCapSmall];
+        __shared__ float rec_x[kCapSmall];
+        if (n_rec > 0) {  // (uniform over the workgroup)
+            __syncthreads();  // the workgroup's previous row is done with the arrays
+            const int64_t rec = (o * a.n_inner + i_in) * a.kept_cap;
+            for (int q = tid; q < n_rec; q += kSelBlock) { rec_idx[q] = a.kept_idx[rec + q]; rec_x[q] = a.kept_x[rec + q]; }
+            __syncthreads();
+        }
         const int64_t zh = sel_row_head<DT>(out, vocab);
         const int64_t zn = (vocab - zh) / EPV;
+        const int64_t zt = zh + zn * EPV;
         u32x4* zv = reinterpret_cast<u32x4*>(out + zh * Row<DT>::BYTES);
         const u32x4 z = {0u, 0u, 0u, 0u};
         for (int64_t v = tid; v < zn; v += kSelBlock) zv[v] = z;
         if (tid < zh) Row<DT>::store1(out, tid, 0.f);
-        if (zh + zn * EPV + tid < vocab) Row<DT>::store1(out, zh + zn * EPV + tid, 0.f);
+        if (zt + tid < vocab) Row<DT>::store1(out, zt + tid, 0.f);
+        if (n_rec <= 0) return;
+        // Every kept entry is written by the thread that wrote the zeros over it, after them: a thread's own stores
+        // to one address keep their order, so nothing waits for the zeros to land.
+        const float lse_r = a.lse_kept[o * a.n_inner + i_in];
+        const int64_t tg_r = a.targets[o * a.ts_outer + i_in * a.ts_inner];
+        for (int q = 0; q < n_rec; ++q) {
+            const int64_t idx = rec_idx[q];
+            const int64_t owner = idx < zh ? idx : idx >= zt ? idx - zt : ((idx - zh) / EPV) % kSelBlock;
+            if (owner != tid) continue;
+            float d = ((idx == tg_r ? 1.f : 0.f) - fast_exp2((rec_x[q] - lse_r) * kLog2e)) * g;
+            if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
+            if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
+            Row<DT>::store1(out, idx, d);
+        }
         return;
     }
     const int64_t rr = o * a.n_inner + i_in;
@@ -891,6 +935,13 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_stream_kernel(SelBwdArgs 
     }
 }
 
+// One workgroup per row (a fixed set of 512 workgroups walking the rows, which fills memory 10 % faster when it does
+// nothing else, measured no gain here: with few workgroups per compute unit the record staging of a row is exposed).
+template <int DT, int TEMP, int MODE>
+__global__ __launch_bounds__(kSelBlock) void topk_topp_stream_kernel(SelBwdArgs a, int64_t n_rows) {
+    for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) topk_topp_stream_row<DT, TEMP, MODE>(a, r);
+}
+
 static int temp_code3(float temperature, int mode, float* tparam) {
     if (temperature == 1.0f) { *tparam = 1.f; return 0; }
     if (mode == NRL_TEMP_DIV) { *tparam = temperature; return 1; }
@@ -929,7 +980,9 @@ using namespace nrl;
 
 extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
                                          float* thr_out, int32_t* tie_out, float* lse_kept_out,
-                                         float* logprob_unfiltered_out, float* lse_full_out, void* stream) {
+                                         float* logprob_unfiltered_out, float* lse_full_out, int32_t* kept_count_out,
+                                         int32_t* kept_index_out, float* kept_value_out, int64_t kept_capacity,
+                                         void* stream) {
     if (int e = check_sel_rows(rows, logprob_out != nullptr)) return e;
     const bool use_k = top_k > 0, use_p = top_p < 1.0f;
     if (!use_k && !use_p) return fail(NRL_E_INVALID, "neither top-k nor top-p is active");
@@ -937,7 +990,10 @@ extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, fl
     const int64_t n = rows->n_outer * rows->n_inner;
     if (n == 0) return NRL_OK;
     if (!thr_out || !tie_out || !lse_kept_out) return fail(NRL_E_INVALID, "null state output");
+    if (kept_count_out && (!kept_index_out || !kept_value_out || kept_capacity < 1 || kept_capacity > kCapSmall))
+        return fail(NRL_E_INVALID, "kept-set record: index and value outputs and a capacity in [1, %d] are needed", kCapSmall);
     SelArgs a;
+    a.kept_n = kept_count_out; a.kept_idx = kept_index_out; a.kept_x = kept_value_out; a.kept_cap = static_cast<int>(kept_capacity);
     a.logits = rows->logits; a.n_inner = rows->n_inner; a.vocab = rows->vocab;
     a.stride_outer = rows->stride_outer; a.stride_inner = rows->stride_inner;
     a.targets = rows->targets; a.ts_outer = rows->tgt_stride_outer; a.ts_inner = rows->tgt_stride_inner;
@@ -970,7 +1026,8 @@ extern "C" int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, fl
 
 extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,
                                          const float* lse_kept, const float* grad, int64_t grad_stride_outer,
-                                         int64_t grad_stride_inner, void* dlogits, int64_t d_n_inner,
+                                         int64_t grad_stride_inner, const int32_t* kept_count, const int32_t* kept_index,
+                                         const float* kept_value, int64_t kept_capacity, void* dlogits, int64_t d_n_inner,
                                          int64_t d_stride_outer, int64_t d_stride_inner, void* stream) {
     if (int e = check_sel_rows(rows, true)) return e;
     if (d_n_inner < rows->n_inner) return fail(NRL_E_INVALID, "d_n_inner < n_inner");
@@ -986,9 +1043,11 @@ extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr,
     a.gs_outer = grad_stride_outer; a.gs_inner = grad_stride_inner;
     a.out = dlogits; a.d_n_inner = d_n_inner; a.ds_outer = d_stride_outer; a.ds_inner = d_stride_inner;
     a.keep_out = nullptr;
+    if (kept_count && (!kept_index || !kept_value || kept_capacity < 1)) return fail(NRL_E_INVALID, "incomplete kept-set record");
+    a.kept_n = kept_count; a.kept_idx = kept_index; a.kept_x = kept_value; a.kept_cap = static_cast<int>(kept_capacity);
     const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 0><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 0><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a, n));
     return check_launch("topk_topp_logprob_bwd");
 }
 
@@ -1005,8 +1064,9 @@ extern "C" int nrl_topk_topp_filter(const nrl_rows* rows, const float* thr, cons
     a.thr = thr; a.tie = tie; a.lse_kept = thr; a.grad = nullptr; a.gs_outer = 0; a.gs_inner = 0;
     a.out = filtered_out; a.d_n_inner = rows->n_inner; a.ds_outer = f_stride_outer; a.ds_inner = f_stride_inner;
     a.keep_out = keep_out;
+    a.kept_n = nullptr; a.kept_idx = nullptr; a.kept_x = nullptr; a.kept_cap = 0;
     const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 1><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a));
+    NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 1><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a, n));
     return check_launch("topk_topp_filter");
 }

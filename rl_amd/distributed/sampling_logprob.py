@@ -21,6 +21,18 @@ def _norm_p(top_p) -> float:
     return float(top_p) if top_p is not None else 1.0
 
 
+def _record_capacity(top_k: int) -> int:
+    """Entries per row of the kept-set record the forward leaves for the backward (0: none).  Under a top-k the kept
+    set has at most k elements plus ties, a few dozen ids of a 150 000-wide row: with them on record the backward
+    writes a gradient row (zeros and those entries) without reading the logits again.  8 bytes per entry and row;
+    rows whose kept set is larger fall back to the streaming backward one by one."""
+    if 0 < top_k <= 64:
+        return 64
+    if 0 < top_k <= 128:
+        return 128
+    return 128 if top_k <= 0 else 0  # top-p alone: peaked rows keep a small nucleus
+
+
 def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, want_unfiltered=False, temperature=1.0):
     """Shared forward of the filtered-logprob autograd functions: saves the logits (no copy), the targets
     and three numbers per row (threshold, tie index, kept log-sum-exp)."""
@@ -34,12 +46,19 @@ def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, wa
     targets = targets.to(logits.device)
     if targets.dtype != torch.int64:
         targets = targets.long()
-    lp, thr, tie, lse, lpu = _OPS.topk_topp_logprob_fwd(
-        logits, targets, n_inner, _norm_k(top_k), _norm_p(top_p), temperature, NRL_TEMP_RCP, want_unfiltered
-    )
     ctx.saved = (not inference_only) and ctx.needs_input_grad[0]
+    capacity = _record_capacity(_norm_k(top_k)) if ctx.saved else 0
+    if capacity:
+        lp, thr, tie, lse, lpu, *record = _OPS.topk_topp_logprob_fwd_rec(
+            logits, targets, n_inner, _norm_k(top_k), _norm_p(top_p), temperature, NRL_TEMP_RCP, want_unfiltered, capacity
+        )
+    else:
+        record = []
+        lp, thr, tie, lse, lpu = _OPS.topk_topp_logprob_fwd(
+            logits, targets, n_inner, _norm_k(top_k), _norm_p(top_p), temperature, NRL_TEMP_RCP, want_unfiltered
+        )
     if ctx.saved:
-        ctx.save_for_backward(logits, targets, thr, tie, lse)
+        ctx.save_for_backward(logits, targets, thr, tie, lse, *record)
         ctx.n_inner = n_inner
         ctx.temperature = temperature
     return (lp, lpu) if want_unfiltered else lp
@@ -48,9 +67,9 @@ def _sampled_fwd(ctx, logits, targets, n_inner, top_k, top_p, inference_only, wa
 def _sampled_bwd(ctx, grad_lp):
     if not ctx.saved:
         raise RuntimeError("backward through a logprob computed with inference_only=True")
-    logits, targets, thr, tie, lse = ctx.saved_tensors
+    logits, targets, thr, tie, lse, *record = ctx.saved_tensors
     return _OPS.topk_topp_logprob_bwd(
-        logits, targets, thr, tie, lse, grad_lp.float().contiguous(), ctx.n_inner, ctx.temperature, NRL_TEMP_RCP
+        logits, targets, thr, tie, lse, grad_lp.float().contiguous(), ctx.n_inner, ctx.temperature, NRL_TEMP_RCP, *record
     )
 
 

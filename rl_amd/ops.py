@@ -369,16 +369,22 @@ _LIB.define(
     "int temp_mode, bool want_unfiltered) -> (Tensor, Tensor, Tensor, Tensor, Tensor)"
 )
 _LIB.define(
+    "topk_topp_logprob_fwd_rec(Tensor logits, Tensor targets, int n_inner, int top_k, float top_p, float temperature, "
+    "int temp_mode, bool want_unfiltered, int capacity) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)"
+)
+_LIB.define(
     "topk_topp_logprob_bwd(Tensor logits, Tensor targets, Tensor thr, Tensor tie, Tensor lse_kept, Tensor grad, "
-    "int n_inner, float temperature, int temp_mode) -> Tensor"
+    "int n_inner, float temperature, int temp_mode, Tensor? kept_n=None, Tensor? kept_idx=None, Tensor? kept_x=None) -> Tensor"
 )
 _LIB.define(
     "topk_topp_filter(Tensor logits, Tensor thr, Tensor tie, float temperature, int temp_mode) -> (Tensor, Tensor)"
 )
 
 
-def _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, temp_mode, want_unfiltered):
-    """-> (logprob [B,n] (empty without targets), thr, tie, lse_kept, unfiltered logprob (or empty))."""
+def _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, temp_mode, want_unfiltered, capacity=0):
+    """-> (logprob [B,n] (empty without targets), thr, tie, lse_kept, unfiltered logprob (or empty)) and, with a
+    capacity, the record of the kept sets (count [B,n], indices and scaled logits [B,n,capacity]) that lets the
+    backward write a gradient row without reading the logits."""
     _need_gpu(logits, targets)
     b, s, v = logits.shape
     dummy = targets if targets is not None else torch.zeros((b, max(n_inner, 1)), dtype=torch.int64, device=logits.device)
@@ -393,17 +399,32 @@ def _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, 
         tie = torch.empty((b, n_inner), dtype=torch.int32, device=dev)
         lse = torch.empty((b, n_inner), **f32)
         lpu = torch.empty((b, n_inner) if want_unfiltered else (0,), **f32)
+        rec = None
+        if capacity > 0:
+            rec = (torch.empty((b, n_inner), dtype=torch.int32, device=dev),
+                   torch.empty((b, n_inner, capacity), dtype=torch.int32, device=dev),
+                   torch.empty((b, n_inner, capacity), **f32))
         with _timed("topk_topp_fwd"):
             code = _lib.load().nrl_topk_topp_logprob_fwd(
                 C.byref(rows), int(top_k), float(top_p), _ptr(lp if targets is not None else None), _ptr(thr), _ptr(tie),
-                _ptr(lse), _ptr(lpu if want_unfiltered else None), None, _stream(),
+                _ptr(lse), _ptr(lpu if want_unfiltered else None), None, _ptr(rec[0] if rec else None),
+                _ptr(rec[1] if rec else None), _ptr(rec[2] if rec else None), int(capacity), _stream(),
             )
     _lib.check(code, "nrl_topk_topp_logprob_fwd")
+    if capacity > 0:
+        return (lp, thr, tie, lse, lpu) + rec
     return lp, thr, tie, lse, lpu
 
 
-def _topk_topp_logprob_bwd(logits, targets, thr, tie, lse_kept, grad, n_inner, temperature, temp_mode):
-    _need_gpu(logits, targets, thr, tie, lse_kept, grad)
+def _topk_topp_logprob_fwd_rec(logits, targets, n_inner, top_k, top_p, temperature, temp_mode, want_unfiltered, capacity):
+    if capacity < 1:
+        raise ValueError("the kept-set record needs a capacity of at least 1")
+    return _topk_topp_logprob_fwd(logits, targets, n_inner, top_k, top_p, temperature, temp_mode, want_unfiltered, capacity)
+
+
+def _topk_topp_logprob_bwd(logits, targets, thr, tie, lse_kept, grad, n_inner, temperature, temp_mode, kept_n=None,
+                           kept_idx=None, kept_x=None):
+    _need_gpu(logits, targets, thr, tie, lse_kept, grad, kept_n, kept_idx, kept_x)
     b, s, v = logits.shape
     rows = _rows(logits, targets, n_inner, 0, v, temperature, temp_mode)
     for t, name in ((thr, "thr"), (tie, "tie"), (lse_kept, "lse_kept")):
@@ -413,12 +434,23 @@ def _topk_topp_logprob_bwd(logits, targets, thr, tie, lse_kept, grad, n_inner, t
         raise ValueError("thr / lse_kept must be fp32 and tie int32")
     if tuple(grad.shape) != (b, n_inner) or grad.dtype != torch.float32:
         raise ValueError("grad must be fp32 [B, n_inner]")
+    capacity = 0
+    if kept_n is not None:
+        if kept_idx is None or kept_x is None:
+            raise ValueError("the kept-set record is (count, indices, values): all three or none")
+        capacity = kept_idx.shape[-1]
+        ok = (kept_n.dtype == torch.int32 and kept_idx.dtype == torch.int32 and kept_x.dtype == torch.float32
+              and tuple(kept_n.shape) == (b, n_inner) and tuple(kept_idx.shape) == (b, n_inner, capacity)
+              and tuple(kept_x.shape) == (b, n_inner, capacity)
+              and kept_n.is_contiguous() and kept_idx.is_contiguous() and kept_x.is_contiguous() and capacity >= 1)
+        if not ok:
+            raise ValueError("kept-set record: int32 [B, n], int32 [B, n, capacity], fp32 [B, n, capacity], contiguous")
     with torch.cuda.device(logits.device):
         d = _grad_buffer((b, s, v), logits)
         with _timed("topk_topp_bwd"):
             code = _lib.load().nrl_topk_topp_logprob_bwd(
                 C.byref(rows), _ptr(thr), _ptr(tie), _ptr(lse_kept), _ptr(grad), grad.stride(0), grad.stride(1),
-                _ptr(d), s, d.stride(0), d.stride(1), _stream(),
+                _ptr(kept_n), _ptr(kept_idx), _ptr(kept_x), capacity, _ptr(d), s, d.stride(0), d.stride(1), _stream(),
             )
     _lib.check(code, "nrl_topk_topp_logprob_bwd")
     return d
@@ -442,7 +474,8 @@ def _topk_topp_filter(logits, thr, tie, temperature, temp_mode):
     return out, keep
 
 
-for _name, _fn in (("topk_topp_logprob_fwd", _topk_topp_logprob_fwd), ("topk_topp_logprob_bwd", _topk_topp_logprob_bwd),
+for _name, _fn in (("topk_topp_logprob_fwd", _topk_topp_logprob_fwd), ("topk_topp_logprob_fwd_rec", _topk_topp_logprob_fwd_rec),
+                   ("topk_topp_logprob_bwd", _topk_topp_logprob_bwd),
                    ("topk_topp_filter", _topk_topp_filter)):
     _LIB.impl(_name, _fn, "CUDA")
     _LIB.impl(_name, _fn, "CPU")

@@ -336,3 +336,48 @@ def test_sampling_autograd_classes():
     xo = x.clone().requires_grad_(True)
     OL.rows_logprob_sampled(xo, t, 10, 0.9).sum().backward()
     torch.testing.assert_close(ga.cpu(), xo.grad, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 2003), (torch.bfloat16, 4096), (torch.float16, 5001)])
+@pytest.mark.parametrize("k,p,temperature", [(50, 0.95, 0.7), (10, 1.0, 1.0), (None, 0.9, 1.3), (100, 0.99, 1.0)])
+def test_backward_from_the_kept_set_record_equals_the_streaming_backward(dtype, vocab, k, p, temperature):
+    """With the forward's record of the kept sets (count, indices, scaled logits per row) the backward writes a
+    gradient row as zeros plus those entries and never reads the logits; without it, it streams the row.  Both
+    must give the same bits -- also for rows whose kept set exceeds the record's capacity (here: a row of exact ties
+    under top-k, a flat row under top-p), which fall back to streaming inside the same launch, and for rows with a
+    zero upstream gradient."""
+    from rl_amd._lib import NRL_TEMP_DIV, NRL_TEMP_RCP
+
+    g = torch.Generator().manual_seed(vocab + (k or 0))
+    b, s = 3, 9
+    n = s - 1
+    logits = (torch.randn(b, s, vocab, generator=g) * 3.0).to(dtype)
+    logits[1, 2] = 0.5                      # every id tied: the kept set is the whole row (beyond any capacity)
+    logits[2, 4] = (torch.randn(vocab, generator=g) * 0.01).to(dtype)   # flat: thousands of ids under top-p
+    ids = torch.randint(0, vocab, (b, s), generator=g)
+    top = logits.float().argmax(-1)
+    ids[:, 1:] = torch.where(torch.rand(b, n, generator=g) < 0.7, top[:, :-1], ids[:, 1:])
+    up = torch.randn(b, n, generator=g)
+    up[0, 3] = 0.0
+    x, t, u = logits.to(DEV), ids[:, 1:].contiguous().to(DEV), up.to(DEV)
+    kk, pp = (k or 0), (p if p is not None else 1.0)
+    ops = torch.ops.rl_amd
+    for mode in (NRL_TEMP_RCP, NRL_TEMP_DIV):
+        for cap in (8, 64, 128):
+            lp, thr, tie, lse, _ = ops.topk_topp_logprob_fwd(x, t, n, kk, pp, temperature, mode, False)
+            lp2, thr2, tie2, lse2, _, cnt, idx, val = ops.topk_topp_logprob_fwd_rec(x, t, n, kk, pp, temperature, mode, False, cap)
+            assert torch.equal(lp, lp2) and torch.equal(thr, thr2) and torch.equal(tie, tie2) and torch.equal(lse, lse2)
+            assert bool(((cnt >= -1) & (cnt <= cap)).all())
+            if k is not None and cap >= k and dtype == torch.float32:   # (16-bit rows tie at the threshold: more than k kept)
+                assert int(cnt[0, 0]) >= 1                       # an ordinary row is on record
+                assert int(cnt[1, 2]) == -1                      # the all-tied row is not
+            streamed = ops.topk_topp_logprob_bwd(x, t, thr, tie, lse, u, n, temperature, mode)
+            recorded = ops.topk_topp_logprob_bwd(x, t, thr, tie, lse, u, n, temperature, mode, cnt, idx, val)
+            assert torch.equal(streamed.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                               recorded.view(torch.int16 if dtype != torch.float32 else torch.int32))
+            # the record is the kept set: as many entries as the streamed row has kept elements
+            keep_rows = OS.keep_mask_rows((logits.float() / temperature if temperature != 1.0 else logits.float())
+                                          .reshape(-1, vocab), k, p).reshape(b, s, vocab)[:, :-1]
+            on_record = (cnt >= 0).cpu()
+            if temperature == 1.0:
+                assert torch.equal(cnt.cpu()[on_record].long(), keep_rows.sum(-1)[on_record])
