@@ -38,6 +38,8 @@ enum nrl_dtype { NRL_F32 = 0, NRL_BF16 = 1, NRL_F16 = 2 };
  * RCP = round(x * (1/T)) with 1/T rounded to fp32 first, what torch does on the GPU. */
 enum nrl_temp_mode { NRL_TEMP_DIV = 0, NRL_TEMP_RCP = 1 };
 
+/* changes whenever an entry point is added or a signature changes; a binding should refuse a library it was not
+ * written for */
 int nrl_version(void);
 const char* nrl_last_error(void);
 

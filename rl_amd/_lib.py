@@ -124,6 +124,9 @@ SIGNATURES = {
 _lib = None
 
 
+ABI_VERSION = 110  # nrl_version() of the library these signatures describe
+
+
 def load() -> C.CDLL:
     """Load the HIP library (once).  Raises if it has not been built."""
     global _lib
@@ -139,6 +142,11 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
+    built = lib.nrl_version()
+    if built != ABI_VERSION:  # a library of another signature set would be called with the wrong arguments
+        raise RuntimeError(
+            f"{LIB_PATH} has ABI version {built}, these bindings are for {ABI_VERSION}: rebuild it with `python -m rl_amd.build`"
+        )
     _lib = lib
     return lib
 

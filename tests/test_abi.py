@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/nrl_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == declared
-    assert lib.nrl_version() >= 100
+    assert lib.nrl_version() == _lib.ABI_VERSION
 
 
 def test_struct_layouts_match_header_field_order():
