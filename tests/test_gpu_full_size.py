@@ -153,6 +153,14 @@ def test_config4_microbatch_topk_topp_full_vocab():
     (torch.where(wf, want, torch.zeros_like(want)) * upr).sum().backward()
     got_g = torch.stack([gx[bi, si].float().cpu() for bi, si in picks])
     assert _grad_close_bf16(got_g, xo.grad)
+    # autograd took the backward that writes each row from the forward's record of its kept set; the backward that
+    # streams the logits again gives the same tensor bit for bit
+    from rl_amd._lib import NRL_TEMP_RCP
+
+    t = ids[:, 1:].contiguous().to(DEV)
+    _, thr, tie, lse, _ = torch.ops.rl_amd.topk_topp_logprob_fwd(x.detach(), t, s - 1, 50, 0.95, 1.0, NRL_TEMP_RCP, False)
+    streamed = torch.ops.rl_amd.topk_topp_logprob_bwd(x.detach(), t, thr, tie, lse, up.contiguous(), s - 1, 1.0, NRL_TEMP_RCP)
+    assert torch.equal(streamed.view(torch.int16), gx.view(torch.int16))
 
 
 def test_config5_packed_row_full_shape():
