@@ -848,6 +848,9 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
     f32x16 acc[NI][NJ];
     zero_acc<Core>(acc);
     Core::tile(op, row0, col0, acc, lds);
+    // (the write-back reads the accumulators with instructions the compiler does not look into: the wait a matrix
+    // instruction's result needs before another unit reads it is spelled out)
+    asm volatile("s_nop 15\n s_nop 7" ::: "memory");
     if (row_map) {
         // rows of the product are scattered: row r of C goes to row row_map[r] of the output (plain store only)
 #pragma unroll
@@ -869,29 +872,44 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
     const bool interior = row0 + BM <= op.m && col0 + BN <= op.n;
     auto write_back = [&](auto interior_tag) {
         constexpr bool INTERIOR = decltype(interior_tag)::value;
+        // Half of the tile's 16 blocks at a time: with an accumulating epilogue all 128 loads of a half go out before
+        // the first is used, so a tile pays two memory latencies, not one per block.  The accumulators are read one
+        // by one where they are used (plain uses would have the compiler copy them all to vector registers, which
+        // are taken by the loaded values).
+        constexpr int HI = NI / 2 > 0 ? NI / 2 : 1;
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
+        for (int i0 = 0; i0 < NI; i0 += HI) {
+            float prior[HI][NJ][16];
+            if (ACCUM) {
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
-                float* base = c + (row0 + wm * 128 + i * 32) * ldc + col;
-                // all 16 loads of a 32 x 32 block go out before the first is used (one memory latency per
-                // block, not one per element)
-                float prior[16];
-                if (ACCUM) {
+                for (int i = i0; i < i0 + HI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+                        const float* base = c + (row0 + wm * 128 + i * 32) * ldc + col;
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int r = acc_row(e, lane);
+                            prior[i - i0][j][e] =
+                                (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n)) ? base[r * ldc] : 0.f;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int i = i0; i < i0 + HI; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+                    float* base = c + (row0 + wm * 128 + i * 32) * ldc + col;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int r = acc_row(e, lane);
-                        prior[e] = (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n)) ? base[r * ldc] : 0.f;
+                        const float v = acc_read(acc[i][j][e]);
+                        if (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n))
+                            base[r * ldc] = ACCUM ? prior[i - i0][j][e] + v : v;
                     }
                 }
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int r = acc_row(e, lane);
-                    if (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n))
-                        base[r * ldc] = ACCUM ? prior[e] + acc[i][j][e] : acc[i][j][e];
-                }
-            }
+        }
     };
     if (interior) write_back(std::true_type{});
     else write_back(std::false_type{});
