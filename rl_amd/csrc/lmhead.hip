@@ -1099,6 +1099,10 @@ extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int6
 // tokens per backward chunk: long enough that the dW product (K = chunk) amortises its fp32 read-modify-write
 static constexpr int64_t kBwdChunk = 16384;
 static int64_t bwd_chunk(int64_t n) { return n < kBwdChunk ? round_up(n < 1 ? 1 : n, 64) : kBwdChunk; }
+// Row stride (elements) of the two operands of the dW product, whose rows hold a chunk's tokens: one 128-byte line
+// more than the chunk, because rows a power of two apart (16384 tokens = 32 KiB) fall on the same memory channels
+// (measured on the dW product: 1.6 % faster than unpadded; two lines more is 5 % slower, three as good as one).
+static int64_t bwd_ld_t(int64_t chunk) { return chunk + 64; }
 
 extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab) {
     const int64_t n = n_tokens < 1 ? 1 : n_tokens;
@@ -1106,8 +1110,8 @@ extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidd
     int64_t b = 0;
     b += hidden_size * vp * 2;        // W^T
     b += chunk * vp * 2;              // G
-    b += vocab * chunk * 2;           // G^T
-    b += hidden_size * chunk * 2;     // hidden chunk^T
+    b += vocab * bwd_ld_t(chunk) * 2;        // G^T
+    b += hidden_size * bwd_ld_t(chunk) * 2;  // hidden chunk^T
     b += vocab * hidden_size * 4;     // dW accumulator (fp32)
     b += n_pad * hidden_size * 2;     // hidden rows of the tokens that carry a gradient
     b += n_pad * (8 + 4 + 4 + 4);     // their targets, log-sum-exps, gradients and token indices
@@ -1137,8 +1141,9 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
     auto take = [&](int64_t bytes) { char* p = ws; ws += (bytes + 255) / 256 * 256; return p; };
     uint16_t* wt = reinterpret_cast<uint16_t*>(take(h * vp * 2));
     uint16_t* g = reinterpret_cast<uint16_t*>(take(chunk * vp * 2));
-    uint16_t* gt = reinterpret_cast<uint16_t*>(take(vocab * chunk * 2));
-    uint16_t* ht = reinterpret_cast<uint16_t*>(take(h * chunk * 2));
+    const int64_t ld_t = bwd_ld_t(chunk);
+    uint16_t* gt = reinterpret_cast<uint16_t*>(take(vocab * ld_t * 2));
+    uint16_t* ht = reinterpret_cast<uint16_t*>(take(h * ld_t * 2));
     float* dw = reinterpret_cast<float*>(take(vocab * h * 4));
     uint16_t* hid_c = reinterpret_cast<uint16_t*>(take(n_pad * h * 2));
     int64_t* tgt_c = reinterpret_cast<int64_t*>(take(n_pad * 8));
@@ -1174,12 +1179,12 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         ga.op.a = hid_c + t0 * h; ga.op.b = w; ga.op.lda = h; ga.op.ldb = ldw; ga.op.m = rows; ga.op.n = vocab; ga.op.k = h;
         ga.op.live = count; ga.op.live_from = t0; ga.op.live_dim = 1;
         ga.targets = tgt_c + t0; ga.vocab_start = vocab_start; ga.lse = lse_c + t0; ga.grad = grad_c + t0;
-        ga.g = g; ga.ldg = vp; ga.gt = gt; ga.ldgt = chunk;
+        ga.g = g; ga.ldg = vp; ga.gt = gt; ga.ldgt = ld_t;
         if (logits_kept) {
             LmGradKeptArgs ka;
             ka.logits = static_cast<const uint16_t*>(logits_kept); ka.ldl = ld_logits; ka.row_map = idx + t0; ka.live = count;
             ka.live_from = t0; ka.rows = rows; ka.vocab = vocab; ka.targets = ga.targets; ka.vocab_start = vocab_start;
-            ka.lse = ga.lse; ka.grad = ga.grad; ka.g = g; ka.ldg = vp; ka.gt = gt; ka.ldgt = chunk;
+            ka.lse = ga.lse; ka.grad = ga.grad; ka.g = g; ka.ldg = vp; ka.gt = gt; ka.ldgt = ld_t;
             lmhead_grad_kept_kernel<<<dim3((unsigned)((vp + KT - 1) / KT), (unsigned)((rows + KT - 1) / KT)), dim3(256), 0, s>>>(ka);
         } else if (h % CoreB::BK == 0) launch_grad<CoreB>(ga, s);
         else launch_grad<CoreA>(ga, s);
@@ -1190,9 +1195,9 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         launch_gemm<false>(dh, dhidden_out, ld_dh, s, idx + t0);
         // dW += G^T [V, rows] * (hidden^T [H, rows])^T
         transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((rows_pad + 63) / 64)), dim3(256), 0, s>>>(
-            hid_c + t0 * h, rows, h, h, ht, chunk, rows_pad);
+            hid_c + t0 * h, rows, h, h, ht, ld_t, rows_pad);
         GemmOperands dwo;
-        dwo.a = gt; dwo.lda = chunk; dwo.b = ht; dwo.ldb = chunk; dwo.m = vocab; dwo.n = h; dwo.k = rows_pad;
+        dwo.a = gt; dwo.lda = ld_t; dwo.b = ht; dwo.ldb = ld_t; dwo.m = vocab; dwo.n = h; dwo.k = rows_pad;
         dwo.live = count; dwo.live_from = t0; dwo.live_dim = 2;
         launch_gemm<true>(dwo, dw, h, s);
     }
