@@ -384,6 +384,8 @@ struct LmFwdArgs {
 template <class Core, bool SAVE>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     constexpr int NI = Core::NI, NJ = Core::NJ, BV = Core::BM, BT = Core::BN;  // vocabulary rows x token columns
+    // kept logits leave through LDS when a wave's 128 x 128 sub-tile fits its share of the operand buffers
+    constexpr bool STAGE = SAVE && NI == 4 && NJ == 4 && Core::LDS_BYTES >= (GB_THREADS / 64) * 128 * 128 * 2;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
     __shared__ float comb_m[2][BT], comb_s[2][BT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -420,6 +422,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
         // instruction's result needs before another unit reads it is spelled out)
         asm volatile("s_nop 15\n s_nop 7" : "+v"(t2));
         const int lane2 = t2 & 63, wm2 = t2 >> 7, wn2 = (t2 >> 6) & 1;
+        unsigned char* stage = lds + (t2 >> 6) * (128 * 128 * 2);  // STAGE: this wave's quarter of the operand buffers
         const int col = wn2 * (NJ * 32) + (lane2 & 31);  // this lane's token column of tile j is col + j * 32
         // Accumulator element e of tile i is row `off` = i * 32 + 8 * (e / 4) + e % 4 (a compile-time constant)
         // below this lane's first row vb.  Only the last vocabulary tile needs the rows-past-the-end mask.
@@ -448,7 +451,16 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
                         x[e] = (!MASKED || off < limit) ? r : -INFINITY;
                         raw = fmaxf(raw, x[e]);
                     }
-                    if constexpr (SAVE) {
+                    if constexpr (STAGE) {
+                        // The lane's 16 values are 4 runs of 4 consecutive vocabulary ids of one token, 8 bytes each.
+                        // They go to the wave's own quarter of the (now idle) operand buffers, laid out [token][id]:
+                        // 16-byte chunk c of token row t at chunk position c ^ (t & 15).
+                        const int t = j * 32 + (lane2 & 31);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            *reinterpret_cast<uint2*>(stage + t * 256 + (((4 * i + q) ^ (t & 15)) * 16) + (lane2 >> 5) * 8) =
+                                uint2{pack_bf16x2(x[4 * q], x[4 * q + 1]), pack_bf16x2(x[4 * q + 2], x[4 * q + 3])};
+                    } else if constexpr (SAVE) {
                         // The lane's 16 values are 4 runs of 4 consecutive vocabulary ids of one token: 8 bytes each,
                         // next to the 8 bytes of the lane 32 further on; a wave's 4 x 4 blocks fill 256 bytes per token.
                         if (tok0 + col + j * 32 < a.op.n) {
@@ -486,6 +498,31 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
         };
         if (v0 + BV <= a.op.m) fold_tile(std::false_type{});
         else fold_tile(std::true_type{});
+        if constexpr (STAGE) {
+            // The wave's 128 tokens x 128 ids leave as whole 256-byte runs, 16 bytes per lane: a quarter of the
+            // requests the 8-byte pieces of the accumulator layout would make.  All 32 reads go out first (read in
+            // assembly like the fragments: a read the compiler sees would wait for the stores before it).
+            const uint32_t sbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage));
+            const int64_t tokw = tok0 + wn2 * 128, vocw = v0 + wm2 * 128;
+            const int c = lane2 & 15;
+            u32x4 val[32];
+            asm volatile("" ::: "memory");  // the staging writes above are issued before the reads below
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                const int t = 4 * k + (lane2 >> 4);
+                asm volatile("ds_read_b128 %0, %1" : "=v"(val[k]) : "v"(sbase + static_cast<uint32_t>(t * 256 + ((c ^ (t & 15)) * 16))));
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                asm volatile("" : "+v"(val[k]));  // (complete only after the wait above)
+                const int t = 4 * k + (lane2 >> 4);
+                if (tokw + t < a.op.n && vocw + c * 8 < a.ldl)
+                    *reinterpret_cast<u32x4*>(a.logits + (tokw + t) * a.ldl + vocw + c * 8) = val[k];
+            }
+            // every wave is done with its staging area before the next tile's operands land there
+            asm volatile("s_barrier" ::: "memory");
+        }
     }
     float run_m[NJ], run_s[NJ];
 #pragma unroll
