@@ -21,7 +21,11 @@ Pinning status (what fixes each function besides its own text):
                            brute force.  PARITY UNPINNED for which of several
                            exactly tied values at the top-p boundary survives
                            (the reference sorts unstably); this oracle keeps
-                           torch's stable ascending order.
+                           torch's stable ascending order.  Also unpinned: the
+                           one boundary element of a row whose cumulative
+                           probability there lies within fp32 rounding (about
+                           1e-6) of 1 - top_p; softmax and cumsum sum in another
+                           order on every device, the reference's included.
 * ``loss.calculate_kl``    pinned: golden vectors of the reference's unit tests.
 * ``loss.masked_mean``     pinned: closed form.
 * ``loss.clipped_pg_loss`` pinned: closed-form losses of the reference's unit

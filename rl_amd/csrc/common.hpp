@@ -39,7 +39,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     const f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
+// (fp16 only: the values are pinned in fp32 registers first.  Otherwise the compiler folds a preceding multiply into
+// the conversion as v_fma_mix(a, b, +0): one rounding instead of the two of multiply-then-narrow that PyTorch does,
+// and a negative zero product comes out positive.)
 __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    asm volatile("" : "+v"(lo), "+v"(hi));
     const f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
 }
@@ -52,6 +56,7 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t lo16) {
 }
 
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    asm volatile("" : "+v"(f));  // see pack_f16x2
     return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(f)));
 }
 

@@ -868,7 +868,10 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
         if (zt + tid < vocab) Row<DT>::store1(out, zt + tid, 0.f);
         if (n_rec <= 0) return;
         // Every kept entry is written by the thread that wrote the zeros over it, after them: a thread's own stores
-        // to one address keep their order, so nothing waits for the zeros to land.
+        // to one address keep their order, so nothing waits for the zeros to land.  (The compiler is told as much:
+        // the zeros went out as 16-byte vectors, the entries go out as scalars of another type, which it could
+        // otherwise take as never overlapping and reorder.)
+        asm volatile("" ::: "memory");
         const float lse_r = a.lse_kept[o * a.n_inner + i_in];
         const int64_t tg_r = a.targets[o * a.ts_outer + i_in * a.ts_inner];
         for (int q = 0; q < n_rec; ++q) {

@@ -339,11 +339,13 @@ def test_sampling_autograd_classes():
 
 
 @pytest.mark.parametrize("dtype,vocab", [(torch.float32, 2003), (torch.bfloat16, 4096), (torch.float16, 5001)])
-@pytest.mark.parametrize("k,p,temperature", [(50, 0.95, 0.7), (10, 1.0, 1.0), (None, 0.9, 1.3), (100, 0.99, 1.0)])
+@pytest.mark.parametrize("k,p,temperature", [(50, 0.95, 0.7), (10, 1.0, 1.0), (None, 0.9, 1.3), (100, 0.99, 1.0), (1, 1.0, 1.0)])
 def test_backward_from_the_kept_set_record_equals_the_streaming_backward(dtype, vocab, k, p, temperature):
     """With the forward's record of the kept sets (count, indices, scaled logits per row) the backward writes a
     gradient row as zeros plus those entries and never reads the logits; without it, it streams the row.  Both
-    must give the same bits -- also for rows whose kept set exceeds the record's capacity (here: a row of exact ties
+    must give the same bits (with ``top_k = 1`` the one kept entry of a row whose target survived is a zero whose
+    sign is that of ``-g``: the scalar store of the record path and the vector store of the streaming path have to
+    narrow a negative zero alike) -- also for rows whose kept set exceeds the record's capacity (here: a row of exact ties
     under top-k, a flat row under top-p), which fall back to streaming inside the same launch, and for rows with a
     zero upstream gradient."""
     from rl_amd._lib import NRL_TEMP_DIV, NRL_TEMP_RCP
