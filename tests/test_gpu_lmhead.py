@@ -10,7 +10,9 @@ Gradients: the reference forms ``G = g * (onehot - softmax)`` and both backward 
 the hidden states are bf16 already) and narrow ``G`` to bf16 once (round to nearest even, relative error at most
 2^-8 per element) - except the one-hot term of dH, ``g * W[target]``, the one large entry of a row of ``G``,
 which is added in fp32.  The error of an output element is therefore bounded by the narrowing of the terms it
-sums: ``|dH - dH_fp32| <= 2^-8 * (|g * softmax| @ |W|)`` and ``|dW - dW_fp32| <= 2^-8 * (|G|^T @ |hidden|)``
+sums: ``|dH - dH_fp32| <= 2^-8 * (|g * softmax| @ |W|)`` and ``|dW - dW_fp32| <= 2^-8 * ((|g * softmax| + |G|)^T @
+|hidden|)`` (the target's entry of ``G^T`` is ``bf16(g + bf16(-g * softmax))``: both narrowings count, which matters
+for a confident token, where ``|G| = |g| (1 - p)`` is far smaller than the softmax part it is the difference of)
 element by element, to which the checks add as much again for logits that round to the neighbouring bf16 value
 under another accumulation order, 1e-4 of the largest entry for the fp32 accumulation, and for dW its final
 narrowing to bf16.  The fp32 ``dhidden_out`` of the C ABI is what is compared, not its bf16 cast; on the flat
@@ -67,7 +69,7 @@ def narrowing_bounds(hid_rows, w, targets, up_rows):
     eps = 2.0 ** -7                                                   # 2^-8 narrowing of G, as much again for flipped logits
     soft = p * up_rows.abs().unsqueeze(-1)                            # the part of G that dH takes through bf16
     b_h = eps * (soft @ w.float().abs()) + 1e-4 * d_h.abs().max()
-    b_w = eps * (grad.abs().T @ hid_rows.float().abs()) + 1e-4 * d_w.abs().max() + 2.0 ** -8 * d_w.abs()
+    b_w = eps * ((soft + grad.abs()).T @ hid_rows.float().abs()) + 1e-4 * d_w.abs().max() + 2.0 ** -8 * d_w.abs()
     return d_h, d_w, b_h, b_w
 
 
@@ -217,3 +219,27 @@ def test_lmhead_autograd_with_and_without_kept_logits(keep, monkeypatch):
     assert bool((lp0 == lp1).all()) and bool((h0.grad == h1.grad).all()) and bool((w0.grad == w1.grad).all())
     with torch.no_grad():   # nothing is kept when no gradient can be asked for
         MU.from_parallel_hidden_states_to_logprobs(hid.to(DEV), w.to(DEV), False, ids.to(DEV), 0, v, None, inference_only=True)
+
+
+@pytest.mark.parametrize("keep", [False, True])
+def test_lmhead_backward_on_confident_tokens(keep):
+    """Peaked distributions (the target's probability close to 1, as for most tokens of a trained policy): the
+    target's gradient entry ``g (1 - p)`` is the small difference of two large terms, one of which went through bf16;
+    the element-wise bounds hold there too, and a vocabulary of one id (probability exactly 1) gives gradients of
+    rounding size only."""
+    g = torch.Generator().manual_seed(9)
+    n, h, v = 200, 64, 300
+    hid = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    w = (torch.randn(v, h, generator=g) * 0.05).to(torch.bfloat16)
+    tgt = torch.randint(0, v, (n,), generator=g)
+    hid[50:] = (w[tgt[50:]].float() * 150.0).to(torch.bfloat16)     # rows aligned with their target's weights: p -> 1
+    up = torch.randn(n, generator=g) * 1e-2
+    p_t = torch.softmax((hid @ w.T).float(), -1).gather(-1, tgt[:, None])[:, 0]
+    assert float(p_t[50:].median()) > 0.99
+    dh, dw = _bwd_through_the_op(hid, w, tgt, up, keep)
+    o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
+    assert bool(((dh.cpu() - o_dh).abs() <= b_dh).all()) and bool(((dw.float().cpu() - o_dw).abs() <= b_dw).all())
+    one = torch.zeros(n, dtype=torch.long)
+    dh1, dw1 = _bwd_through_the_op(hid, w[:1].contiguous(), one, up, keep)
+    o_dh1, o_dw1, b_dh1, b_dw1 = narrowing_bounds(hid, w[:1], one, up)
+    assert bool(((dh1.cpu() - o_dh1).abs() <= b_dh1).all()) and bool(((dw1.float().cpu() - o_dw1).abs() <= b_dw1).all())
