@@ -66,6 +66,7 @@ __device__ __forceinline__ float key_value(uint32_t k) {
 }
 
 // maximum over the 8 consecutive lanes (aligned to 8) that read one 128-byte line; every lane returns it
+// (written as three hand-placed v_max_f32_dpp the pass has a third fewer vector instructions and takes the same time)
 __device__ __forceinline__ float line_max(float v) {
     int x = __float_as_int(v);
     v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false)));   // quad_perm [1,0,3,2]
@@ -220,6 +221,11 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     const u32x4* xv = reinterpret_cast<const u32x4*>(row + head * Row<DT>::BYTES);
 
     // ---- pass 1: chunk maxima (+ full-row online log-sum-exp) ----
+    // Without the full-row log-sum-exp only maxima leave this pass, and the temperature scaling (a multiplication or
+    // division by a positive number, then rounding to the logits' dtype) is monotone: the maximum of the scaled
+    // values is the scaled maximum, so the raw values are compared and each chunk maximum is scaled once at the end.
+    constexpr bool LATE_SCALE = !FULL_LSE && TEMP != 0;
+    auto scaled = [&](float x) { return LATE_SCALE ? x : scale_logit<DT, TEMP>(x, a.tparam); };
     float mx[kSub];
 #pragma unroll
     for (int u = 0; u < kSub; ++u) mx[u] = -FLT_MAX;
@@ -247,7 +253,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             float vm = -FLT_MAX;
 #pragma unroll
             for (int k = 0; k < EPV; ++k) {
-                t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+                t[k] = scaled(t[k]);
                 v[u * EPV + k] = t[k];
                 vm = fmaxf(vm, t[k]);
             }
@@ -276,7 +282,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                 Row<DT>::decode(xv[vi], t);
 #pragma unroll
                 for (int k = 0; k < EPV; ++k) {
-                    t[k] = scale_logit<DT, TEMP>(t[k], a.tparam);
+                    t[k] = scaled(t[k]);
                     vm = fmaxf(vm, t[k]);
                     if (FULL_LSE) {
                         const float mn = fmaxf(acc.m, t[k]);
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         for (int w = 0; w < 2; ++w) {
             const int64_t e = w == 0 ? e0 : e1;
             if (e < 0) continue;
-            const float x = scale_logit<DT, TEMP>(Row<DT>::load1(row, e), a.tparam);
+            const float x = scaled(Row<DT>::load1(row, e));
             mx[0] = fmaxf(mx[0], x);
             if (FULL_LSE) {
                 const float mn = fmaxf(acc.m, x);
@@ -303,6 +309,10 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                 acc.m = mn;
             }
         }
+    }
+    if (LATE_SCALE) {
+#pragma unroll
+        for (int u = 0; u < kSub; ++u) mx[u] = scale_logit<DT, TEMP>(mx[u], a.tparam);
     }
     uint32_t mx_key[kSub];
 #pragma unroll
