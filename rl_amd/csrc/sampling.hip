@@ -843,6 +843,7 @@ struct SelBwdArgs {
     const int32_t* kept_idx;
     const float* kept_x;
     int kept_cap;
+    int prefilled;  // the whole gradient buffer was zero-filled before this launch: rows on record only add their entries
 };
 
 // MODE 0: gradient, MODE 1: filtered logits (-inf outside the kept set) + keep mask
@@ -859,6 +860,22 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
     // without reading the logits again.
     int n_rec = -1;
     if (MODE == 0 && g != 0.f && a.kept_n) n_rec = a.kept_n[o * a.n_inner + i_in];
+    if (MODE == 0 && a.prefilled && (g == 0.f || n_rec >= 0)) {
+        // the zeros are there already (an earlier launch on the stream): only the kept entries are written
+        const int64_t rec = (o * a.n_inner + i_in) * a.kept_cap;
+        if (n_rec > 0) {
+            const float lse_r = a.lse_kept[o * a.n_inner + i_in];
+            const int64_t tg_r = a.targets[o * a.ts_outer + i_in * a.ts_inner];
+            for (int q = tid; q < n_rec; q += kSelBlock) {
+                const int64_t idx = a.kept_idx[rec + q];
+                float d = ((idx == tg_r ? 1.f : 0.f) - fast_exp2((a.kept_x[rec + q] - lse_r) * kLog2e)) * g;
+                if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
+                if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
+                Row<DT>::store1(out, idx, d);
+            }
+        }
+        return;
+    }
     if (MODE == 0 && (g == 0.f || n_rec >= 0)) {  // dropped position or masked token: the gradient row is exactly zero
         __shared__ int32_t rec_idx[kCapSmall];
         __shared__ float rec_x[kCapSmall];
@@ -945,6 +962,21 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
         bool keep;
         Row<DT>::store1(out, e, elem(Row<DT>::load1(row, e), e, keep));
         if (keep_row) keep_row[e] = keep ? 1 : 0;
+    }
+}
+
+// Zero fill of a contiguous buffer by one workgroup per compute unit in 256 KiB spans: 6.0 TB/s, as a memset, where
+// one workgroup per row reaches 5.5.
+constexpr int kFillGrid = 256;
+constexpr int64_t kFillSpan = 256 * 1024;
+__global__ __launch_bounds__(256) void fill_zero_flat_kernel(char* out, int64_t total_bytes) {
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int64_t s0 = static_cast<int64_t>(blockIdx.x) * kFillSpan; s0 < total_bytes; s0 += static_cast<int64_t>(gridDim.x) * kFillSpan) {
+        u32x4* zv = reinterpret_cast<u32x4*>(out + s0);
+        const int64_t left = total_bytes - s0;
+        const int64_t nv = (left < kFillSpan ? left : kFillSpan) / 16;
+        for (int64_t v = threadIdx.x; v < nv; v += 256) zv[v] = z;
+        if (left < kFillSpan && threadIdx.x < (left & 15)) out[s0 + nv * 16 + threadIdx.x] = 0;
     }
 }
 
@@ -1060,6 +1092,13 @@ extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr,
     a.kept_n = kept_count; a.kept_idx = kept_index; a.kept_x = kept_value; a.kept_cap = static_cast<int>(kept_capacity);
     const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // With the kept sets on record nearly every row is zeros plus a few entries.  A gradient buffer that is one
+    // contiguous block is then zero-filled flat, which writes faster than row by row, and the row launch only adds
+    // the entries (and streams the rows that are not on record).
+    const int64_t elt = rows->dtype == NRL_F32 ? 4 : 2;
+    a.prefilled = kept_count && d_stride_inner == rows->vocab && d_stride_outer == d_n_inner * rows->vocab &&
+                  (reinterpret_cast<uintptr_t>(dlogits) & 15) == 0;
+    if (a.prefilled) fill_zero_flat_kernel<<<dim3(kFillGrid), dim3(256), 0, s>>>(static_cast<char*>(dlogits), n * rows->vocab * elt);
     NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 0><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a, n));
     return check_launch("topk_topp_logprob_bwd");
 }
@@ -1077,7 +1116,7 @@ extern "C" int nrl_topk_topp_filter(const nrl_rows* rows, const float* thr, cons
     a.thr = thr; a.tie = tie; a.lse_kept = thr; a.grad = nullptr; a.gs_outer = 0; a.gs_inner = 0;
     a.out = filtered_out; a.d_n_inner = rows->n_inner; a.ds_outer = f_stride_outer; a.ds_inner = f_stride_inner;
     a.keep_out = keep_out;
-    a.kept_n = nullptr; a.kept_idx = nullptr; a.kept_x = nullptr; a.kept_cap = 0;
+    a.kept_n = nullptr; a.kept_idx = nullptr; a.kept_x = nullptr; a.kept_cap = 0; a.prefilled = 0;
     const int tc = temp_code3(rows->temperature, rows->temp_mode, &a.tparam);
     hipStream_t s = static_cast<hipStream_t>(stream);
     NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 1><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a, n));
