@@ -178,8 +178,10 @@ int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, 
  * row for autograd): a forward given kept_count_out int32 [rows], kept_index_out int32 [rows, kept_capacity] and
  * kept_value_out fp32 [rows, kept_capacity] (kept_capacity <= 2048) also writes, for every row whose kept set has
  * at most kept_capacity elements, their number, their vocabulary indices and their (temperature-scaled) logits,
- * and -1 as the number for every other row.  A backward given the record back writes the gradient row of a
- * recorded row as zeros plus those few entries without reading the logits; other rows stream as without it. */
+ * and -1 as the number for every other row.  A backward given the record back and a dlogits that is one contiguous,
+ * 16-byte aligned block (d_stride_inner == vocab, d_stride_outer == d_n_inner * vocab) zero-fills that block and
+ * writes only those few entries of a recorded row, without reading the logits; other rows stream as without the
+ * record, and so does everything for a strided dlogits. */
 int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,
                               const float* lse_kept, const float* grad, int64_t grad_stride_outer,
                               int64_t grad_stride_inner, const int32_t* kept_count, const int32_t* kept_index,

@@ -843,7 +843,7 @@ struct SelBwdArgs {
     const int32_t* kept_idx;
     const float* kept_x;
     int kept_cap;
-    int prefilled;  // the whole gradient buffer was zero-filled before this launch: rows on record only add their entries
+    int prefilled;  // the record is in use: the whole gradient buffer was zero-filled before this launch, rows on record only add their entries
 };
 
 // MODE 0: gradient, MODE 1: filtered logits (-inf outside the kept set) + keep mask
@@ -859,7 +859,7 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
     // With the forward's record of the kept set the gradient row is zeros plus the few kept entries, written
     // without reading the logits again.
     int n_rec = -1;
-    if (MODE == 0 && g != 0.f && a.kept_n) n_rec = a.kept_n[o * a.n_inner + i_in];
+    if (MODE == 0 && g != 0.f && a.prefilled) n_rec = a.kept_n[o * a.n_inner + i_in];
     if (MODE == 0 && a.prefilled && (g == 0.f || n_rec >= 0)) {
         // the zeros are there already (an earlier launch on the stream): only the kept entries are written
         const int64_t rec = (o * a.n_inner + i_in) * a.kept_cap;
@@ -876,40 +876,14 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
         }
         return;
     }
-    if (MODE == 0 && (g == 0.f || n_rec >= 0)) {  // dropped position or masked token: the gradient row is exactly zero
-        __shared__ int32_t rec_idx[kCapSmall];
-        __shared__ float rec_x[kCapSmall];
-        if (n_rec > 0) {  // (uniform over the workgroup)
-            __syncthreads();  // the workgroup's previous row is done with the arrays
-            const int64_t rec = (o * a.n_inner + i_in) * a.kept_cap;
-            for (int q = tid; q < n_rec; q += kSelBlock) { rec_idx[q] = a.kept_idx[rec + q]; rec_x[q] = a.kept_x[rec + q]; }
-            __syncthreads();
-        }
+    if (MODE == 0 && g == 0.f) {  // dropped position or masked token: the gradient row is exactly zero
         const int64_t zh = sel_row_head<DT>(out, vocab);
         const int64_t zn = (vocab - zh) / EPV;
-        const int64_t zt = zh + zn * EPV;
         u32x4* zv = reinterpret_cast<u32x4*>(out + zh * Row<DT>::BYTES);
         const u32x4 z = {0u, 0u, 0u, 0u};
         for (int64_t v = tid; v < zn; v += kSelBlock) zv[v] = z;
         if (tid < zh) Row<DT>::store1(out, tid, 0.f);
-        if (zt + tid < vocab) Row<DT>::store1(out, zt + tid, 0.f);
-        if (n_rec <= 0) return;
-        // Every kept entry is written by the thread that wrote the zeros over it, after them: a thread's own stores
-        // to one address keep their order, so nothing waits for the zeros to land.  (The compiler is told as much:
-        // the zeros went out as 16-byte vectors, the entries go out as scalars of another type, which it could
-        // otherwise take as never overlapping and reorder.)
-        asm volatile("" ::: "memory");
-        const float lse_r = a.lse_kept[o * a.n_inner + i_in];
-        const int64_t tg_r = a.targets[o * a.ts_outer + i_in * a.ts_inner];
-        for (int q = 0; q < n_rec; ++q) {
-            const int64_t idx = rec_idx[q];
-            const int64_t owner = idx < zh ? idx : idx >= zt ? idx - zt : ((idx - zh) / EPV) % kSelBlock;
-            if (owner != tid) continue;
-            float d = ((idx == tg_r ? 1.f : 0.f) - fast_exp2((rec_x[q] - lse_r) * kLog2e)) * g;
-            if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
-            if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
-            Row<DT>::store1(out, idx, d);
-        }
+        if (zh + zn * EPV + tid < vocab) Row<DT>::store1(out, zh + zn * EPV + tid, 0.f);
         return;
     }
     const int64_t rr = o * a.n_inner + i_in;
@@ -1094,7 +1068,7 @@ extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr,
     hipStream_t s = static_cast<hipStream_t>(stream);
     // With the kept sets on record nearly every row is zeros plus a few entries.  A gradient buffer that is one
     // contiguous block is then zero-filled flat, which writes faster than row by row, and the row launch only adds
-    // the entries (and streams the rows that are not on record).
+    // the entries (and streams the rows that are not on record).  For a strided buffer the record is left unused.
     const int64_t elt = rows->dtype == NRL_F32 ? 4 : 2;
     a.prefilled = kept_count && d_stride_inner == rows->vocab && d_stride_outer == d_n_inner * rows->vocab &&
                   (reinterpret_cast<uintptr_t>(dlogits) & 15) == 0;
