@@ -460,7 +460,7 @@ def bench_topk(args, torch, w):
         # forward left on record) without reading the logits again
         "algorithmic_bytes_per_token": 2 * row_bytes,
         "hbm_frac_end_to_end": 2 * row_bytes * tokens * args.steps / elapsed / 1e9 / HBM_PEAK_GBS,
-        "roofline": hbm_roofline("topk_topp_stream_kernel (backward from the kept-set record: write only)", row_bytes * rows,
+        "roofline": hbm_roofline("fill_zero_flat_kernel + topk_topp_stream_kernel (backward from the kept-set record: write only)", row_bytes * rows,
                                  bwd["avg_ms"], "c4" if full else None),
         "roofline_fwd": hbm_roofline("topk_topp_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
                                      "c4_fwd" if full else None),
