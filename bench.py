@@ -677,7 +677,7 @@ def bench_lmhead(args, torch, w):
     # and the backward reads them instead of multiplying a second time.  The reference's way, recomputing, is its
     # own row below.
     n = b * s
-    kept = MU._keep_lmhead_logits(n, v, dev)
+    kept = MU._keep_lmhead_logits(n, v, dev, h)
     elapsed, k = timed(torch, ops, args, step)
     fwd_ms, bwd_ms = k["lmhead_fwd"]["avg_ms"], k["lmhead_bwd"]["avg_ms"]
     MU.LMHEAD_KEEP_LOGITS = not kept

@@ -444,18 +444,25 @@ def from_parallel_logits_to_logprobs_packed_sequences(
 # the hidden states and the weights a second time (a quarter of the step's matrix work).  The reference recomputes
 # (``model_utils.py:2249-2262``) because its logits are fp32 and its memory 80 GB; here the logits of 65 536 tokens
 # x 151 936 ids are 20 GB of 288.  True / False force the choice; "auto" keeps them while they take no more than
-# ``LMHEAD_KEEP_FRACTION`` of the memory that is free when the forward runs.  The gradients are the same both ways.
+# ``LMHEAD_KEEP_FRACTION`` of the memory that is free when the forward runs and, together with the backward's
+# workspace, no more than half of it.  The gradients are the same both ways.
 LMHEAD_KEEP_LOGITS: Any = "auto"
 LMHEAD_KEEP_FRACTION = 0.25
 
 
-def _keep_lmhead_logits(n_tokens: int, vocab: int, device: torch.device) -> bool:
+def _keep_lmhead_logits(n_tokens: int, vocab: int, device: torch.device, hidden_size: int = 0) -> bool:
     if LMHEAD_KEEP_LOGITS != "auto":
         return bool(LMHEAD_KEEP_LOGITS)
     need = n_tokens * ((vocab + 7) // 8 * 8) * 2
     free, _ = torch.cuda.mem_get_info(device)
     free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)  # the allocator's own free blocks
-    return need <= LMHEAD_KEEP_FRACTION * free
+    # (and the backward's own workspace and outputs must still fit comfortably next to them)
+    later = 0
+    if hidden_size > 0:
+        from .. import _lib
+
+        later = _lib.load().nrl_lmhead_bwd_workspace_bytes(n_tokens, hidden_size, vocab) + n_tokens * hidden_size * 4
+    return need <= LMHEAD_KEEP_FRACTION * free and need + later <= 0.5 * free
 
 
 class ChunkedDistributedHiddenStatesToLogprobs(torch.autograd.Function):
@@ -477,7 +484,7 @@ class ChunkedDistributedHiddenStatesToLogprobs(torch.autograd.Function):
         weight = output_weight_layer.detach()
         tgt = _to_device(target, hidden).long().t().contiguous().reshape(-1)  # token order of the hidden rows: (s, b)
         ctx.saved = (not inference_only) and (ctx.needs_input_grad[0] or ctx.needs_input_grad[2])
-        keep = ctx.saved and _keep_lmhead_logits(s * b, weight.shape[0], hidden.device)
+        keep = ctx.saved and _keep_lmhead_logits(s * b, weight.shape[0], hidden.device, h)
         lp, lse, logits = _OPS.lmhead_logprob_fwd(hidden2d, weight, tgt, vocab_start_index, vocab_end_index, keep)
         if ctx.saved:
             ctx.save_for_backward(hidden2d, weight, tgt, lse, logits)
