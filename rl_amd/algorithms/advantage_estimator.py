@@ -21,7 +21,7 @@ class AdvEstimatorConfig(BaseModel, extra="allow"):
 class GRPOAdvantageEstimator:
     """Leave-one-out (or full) group baseline, optional division by the group std."""
 
-    def __init__(self, estimator_config, loss_config=None):
+    def __init__(self, estimator_config, loss_config):
         self.use_leave_one_out_baseline = estimator_config.use_leave_one_out_baseline
         self.normalize_rewards = estimator_config.normalize_rewards
 

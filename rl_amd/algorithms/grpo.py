@@ -85,7 +85,7 @@ class _NoTimer:
 
 
 def dynamic_sampling(repeated_batch: Any, std: torch.Tensor, baseline: torch.Tensor, dynamic_sampling_num_gen_batches: int,
-                     master_config: Any, timer: Any = None, batch_cache: Any = None):
+                     master_config: Any, timer: Any, batch_cache: Any = None):
     """``grpo.py:1699-1830`` (DAPO dynamic sampling): keep the samples whose prompt group has ``std != 0``,
     collect them in ``batch_cache`` across generation batches until ``num_prompts_per_step *
     num_generations_per_prompt`` are available, then cut to exactly that many.

@@ -91,7 +91,7 @@ def test_dynamic_sampling_keeps_every_group_with_spread():
     batch = _ds_batch(6, [1.0, 0.0, 1.0, 0.5, 0.5, 0.0])
     std = torch.tensor([0.5, 0.5, 0.5, 0.25, 0.25, 0.25])
     baseline = torch.tensor([0.67, 0.67, 0.67, 0.33, 0.33, 0.33])
-    out, complete, cache, metrics = dynamic_sampling(batch, std, baseline, 1, _ds_config(2, 3))
+    out, complete, cache, metrics = dynamic_sampling(batch, std, baseline, 1, _ds_config(2, 3), None)
     assert out.size == 6 and complete is True
     assert torch.allclose(out["std"], std) and torch.allclose(out["baseline"], baseline)
     assert metrics == {"dynamic_sampling_num_discarded_valid_samples": 0}
@@ -103,7 +103,7 @@ def test_dynamic_sampling_drops_groups_without_spread():
     batch = _ds_batch(6, [1.0, 1.0, 1.0, 0.5, 0.5, 0.0])
     std = torch.tensor([0.0, 0.0, 0.0, 0.25, 0.25, 0.25])
     baseline = torch.tensor([1.0, 1.0, 1.0, 0.33, 0.33, 0.33])
-    out, complete, _cache, _ = dynamic_sampling(batch, std, baseline, 1, _ds_config(1, 3))
+    out, complete, _cache, _ = dynamic_sampling(batch, std, baseline, 1, _ds_config(1, 3), None)
     assert out.size == 3 and complete is True
     assert torch.allclose(out["std"], torch.tensor([0.25, 0.25, 0.25]))
     assert torch.allclose(out["baseline"], torch.tensor([0.33, 0.33, 0.33]))
@@ -119,7 +119,7 @@ def test_dynamic_sampling_rows_stay_aligned_through_filter_and_cut():
     std = torch.tensor([0.5, 0.5, 0.5, 0.25, 0.25, 0.25, 0.35, 0.35, 0.35])
     baseline = torch.tensor([0.67, 0.67, 0.67, 0.33, 0.33, 0.33, 0.57, 0.57, 0.57])
     out, complete, _, metrics = dynamic_sampling(batch, std, baseline, dynamic_sampling_num_gen_batches=1,
-                                                 master_config=_ds_config(2, 3))
+                                                 master_config=_ds_config(2, 3), timer=None)
     assert complete is True and out.size == 6
     assert torch.equal(out["mask_sample"], torch.tensor([False, True, False, True, False, True]))
     assert metrics["dynamic_sampling_num_discarded_valid_samples"] == 3
@@ -131,7 +131,7 @@ def test_dynamic_sampling_caches_until_enough_and_gives_up_after_the_limit():
     std = torch.tensor([0.4, 0.4, 0.4])
     baseline = torch.tensor([0.5, 0.5, 0.5])
     cfg = _ds_config(2, 3)
-    out, complete, cache, _ = dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 1, cfg)
+    out, complete, cache, _ = dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 1, cfg, None)
     assert out.size == 3 and complete is False and cache is not None and cache == out
     out, complete, cache, _ = dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 1, cfg, None, cache)
     assert out.size == 6 and complete is True and cache is not None
@@ -139,8 +139,8 @@ def test_dynamic_sampling_caches_until_enough_and_gives_up_after_the_limit():
     out, complete, cache2, _ = dynamic_sampling(_ds_batch(3, [1.0, 1.0, 1.0]), torch.zeros(3), baseline, 2, cfg, None, None)
     assert out.size == 0 and complete is False and cache2 is None
     with pytest.raises(ValueError):
-        dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 6, cfg)
+        dynamic_sampling(_ds_batch(3, [1.0, 0.0, 0.5]), std, baseline, 6, cfg, None)
     # switched off: the batch comes back whole, with baseline and std attached
     batch = _ds_batch(3, [1.0, 1.0, 1.0])
-    out, complete, _, metrics = dynamic_sampling(batch, torch.zeros(3), baseline, 1, _ds_config(2, 3, enabled=False))
+    out, complete, _, metrics = dynamic_sampling(batch, torch.zeros(3), baseline, 1, _ds_config(2, 3, enabled=False), None)
     assert out is batch and complete is True and metrics == {} and torch.equal(out["std"], torch.zeros(3))
