@@ -14,6 +14,7 @@ U[256,1024] masked out; run as microbatches of 16 sequences (19.9 GB of logits e
 from __future__ import annotations
 
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -371,7 +372,7 @@ def finish(result, args, torch, w, kind, cpu_rows, gpu_rows):
                 roof["copy_bandwidth_frac"] = roof["achieved"] / gbs
         result["reference_on_gpu"] = reference_on_gpu(torch, w, kind, gpu_rows)
         result["cpu_baseline"] = cpu_baseline(torch, w, kind, args.cpu_seconds, cpu_rows)
-    print(json.dumps(result))
+    print(json.dumps(result), file=_JSON_OUT, flush=True)
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
@@ -721,7 +722,17 @@ def bench_lmhead(args, torch, w):
     finish(result, args, torch, w, "lmhead", cpu_rows=1024, gpu_rows=1024)
 
 
+# The one JSON line goes to the process's stdout; whatever the measured code prints on the way (the reference's
+# warning about -inf logprobs under top-k / top-p, for one) goes to stderr.
+_JSON_OUT = sys.stdout
+
+
 def main():
+    with contextlib.redirect_stdout(sys.stderr):
+        return _main()
+
+
+def _main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)

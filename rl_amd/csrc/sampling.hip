@@ -859,7 +859,10 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
     // With the forward's record of the kept set the gradient row is zeros plus the few kept entries, written
     // without reading the logits again.
     int n_rec = -1;
-    if (MODE == 0 && g != 0.f && a.prefilled) n_rec = a.kept_n[o * a.n_inner + i_in];
+    if (MODE == 0 && g != 0.f && a.prefilled) {
+        n_rec = a.kept_n[o * a.n_inner + i_in];
+        if (n_rec > a.kept_cap) n_rec = -1;  // not a count the forward writes: stream the row instead
+    }
     if (MODE == 0 && a.prefilled && (g == 0.f || n_rec >= 0)) {
         // the zeros are there already (an earlier launch on the stream): only the kept entries are written
         const int64_t rec = (o * a.n_inner + i_in) * a.kept_cap;
@@ -868,6 +871,7 @@ __device__ __forceinline__ void topk_topp_stream_row(const SelBwdArgs& a, int64_
             const int64_t tg_r = a.targets[o * a.ts_outer + i_in * a.ts_inner];
             for (int q = tid; q < n_rec; q += kSelBlock) {
                 const int64_t idx = a.kept_idx[rec + q];
+                if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(vocab)) continue;
                 float d = ((idx == tg_r ? 1.f : 0.f) - fast_exp2((a.kept_x[rec + q] - lse_r) * kLog2e)) * g;
                 if constexpr (TEMP == 1) d = __fdiv_rn(Row<DT>::round_self(d), a.tparam);
                 if constexpr (TEMP == 2) d = Row<DT>::round_self(d) * a.tparam;
