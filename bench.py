@@ -433,7 +433,17 @@ def bench_topk(args, torch, w):
             (d,) = torch.autograd.grad(loss, leaf)
             del d, loss, loss_input
 
-    elapsed, k = timed(torch, ops, args, step)
+    # the warning about valid tokens whose logprob is -inf is printed when its counts have arrived (opt-in), as the
+    # metric records are; printed at once, as in the reference, it is its own row
+    from rl_amd.algorithms import utils as AU
+
+    AU.DEFER_NEG_INF_WARNING = True
+    try:
+        elapsed, k = timed(torch, ops, args, step)
+    finally:
+        AU.DEFER_NEG_INF_WARNING = False
+        AU.flush_neg_inf_warnings()
+    w_elapsed, wk = timed(torch, ops, args, step)
     # the same step with the backward streaming the logits again instead of using the forward's record of the kept sets
     from rl_amd.distributed import sampling_logprob as SL
 
@@ -456,7 +466,8 @@ def bench_topk(args, torch, w):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
-                   "temperature": "divided inside the timed region by the logprob kernels (deferred_temperature), bf16 rounding of a GPU div_"},
+                   "temperature": "divided inside the timed region by the logprob kernels (deferred_temperature), bf16 rounding of a GPU div_",
+                   "neg_inf_warning": "printed when its counts have arrived (rl_amd.algorithms.utils.DEFER_NEG_INF_WARNING)"},
         # the forward reads a row once; the backward writes the gradient row (zeros and the <= 64 kept entries the
         # forward left on record) without reading the logits again
         "algorithmic_bytes_per_token": 2 * row_bytes,
@@ -466,6 +477,10 @@ def bench_topk(args, torch, w):
         "roofline_fwd": hbm_roofline("topk_topp_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
                                      "c4_fwd" if full else None),
         "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
+        "immediate_warning": {
+            "value": tokens * args.steps / w_elapsed, "unit": "tokens/s", "ms_per_step": w_elapsed / args.steps * 1e3,
+            "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in wk.items()},
+            "note": "mask_out_neg_inf_logprobs waits for its two counts and prints the warning before it returns, once per microbatch"},
         "streaming_backward": {
             "value": tokens * args.steps / s_elapsed, "unit": "tokens/s", "ms_per_step": s_elapsed / args.steps * 1e3,
             "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in sk.items()},

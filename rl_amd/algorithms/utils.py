@@ -7,6 +7,7 @@ kernel instead).  ``mask_out_neg_inf_logprobs`` is [B, S]-sized tensor plumbing 
 
 from __future__ import annotations
 
+import atexit
 from typing import Optional
 
 import torch
@@ -133,17 +134,52 @@ def masked_mean(
     return out.reshape(out_shape).to(device=values.device, dtype=out_dtype)
 
 
-def mask_out_neg_inf_logprobs(logprobs: torch.Tensor, mask: torch.Tensor, logprobs_name: str) -> torch.Tensor:
-    """``utils.py:227-257``: positions that are masked out or infinite become 0 (with the reference's
-    warning when valid tokens are affected)."""
-    is_inf = torch.isinf(logprobs)
-    # both counts in one transfer: the warning is the only reason this function waits for the device at all
-    hit, valid = torch.stack([(is_inf & mask.bool()).sum(), mask.sum().to(torch.int64)]).tolist()
+# Opt-in (not in the reference): with ``DEFER_NEG_INF_WARNING = True`` the two counts behind the warning of
+# ``mask_out_neg_inf_logprobs`` travel to pinned host memory behind the stream and the warning is printed once they
+# have arrived -- at a later call, at ``flush_neg_inf_warnings()`` or when the interpreter exits -- so the caller's
+# thread keeps queueing work (the backward, the next microbatch) instead of waiting for the forward to finish.
+DEFER_NEG_INF_WARNING = False
+_pending_warnings: list = []  # (event, pinned int64[2], name)
+
+
+def _warn_neg_inf(hit: int, valid: int, logprobs_name: str) -> None:
     if hit > 0:
         print(
             f"[WARNING]: {hit}/{valid} valid tokens have -inf in {logprobs_name} "
             "(policy top-k/top-p mismatch). Masking out these positions."
         )
+
+
+def flush_neg_inf_warnings(wait: bool = True) -> None:
+    """Prints the deferred warnings whose counts have arrived, oldest first; with ``wait`` all of them."""
+    while _pending_warnings:
+        event, counts, name = _pending_warnings[0]
+        if not wait and not event.query():
+            return
+        event.synchronize()
+        _pending_warnings.pop(0)
+        _warn_neg_inf(int(counts[0]), int(counts[1]), name)
+
+
+atexit.register(flush_neg_inf_warnings)
+
+
+def mask_out_neg_inf_logprobs(logprobs: torch.Tensor, mask: torch.Tensor, logprobs_name: str) -> torch.Tensor:
+    """``utils.py:227-257``: positions that are masked out or infinite become 0 (with the reference's
+    warning when valid tokens are affected)."""
+    is_inf = torch.isinf(logprobs)
+    # both counts in one transfer: the warning is the only reason this function waits for the device at all
+    counts = torch.stack([(is_inf & mask.bool()).sum(), mask.sum().to(torch.int64)])
+    if DEFER_NEG_INF_WARNING and counts.is_cuda:
+        flush_neg_inf_warnings(wait=False)
+        host = torch.empty(2, dtype=torch.int64, pin_memory=True)
+        host.copy_(counts, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        _pending_warnings.append((event, host, logprobs_name))
+    else:
+        hit, valid = counts.tolist()
+        _warn_neg_inf(hit, valid, logprobs_name)
     keep = mask * (~is_inf).float()
     return torch.where(keep.bool(), logprobs, 0.0)
 
