@@ -1,10 +1,12 @@
 // K6: fused lm_head -> token logprob (hidden @ W^T, never materialising the full logits) and its
 // backward (dH, dW), on the gfx950 matrix cores.
 //
-// Two bf16 MFMA GEMM cores, C[M,N] = A[M,K] * B[N,K]^T with fp32 accumulation (v_mfma_f32_32x32x16_bf16,
-// 4 wave64 in a 2 x 2 grid), serve every product:
-//   * core B, the fast one (K a multiple of 64): 256 x 256 tile, 128 x 128 per wave (256 accumulator
-//     registers, one wave per SIMD), operands double-buffered in LDS by direct global-to-LDS loads;
+// Three bf16 MFMA GEMM cores, C[M,N] = A[M,K] * B[N,K]^T with fp32 accumulation (v_mfma_f32_32x32x16_bf16,
+// 4 wave64, one per SIMD, 256 accumulator registers each), serve every product:
+//   * core B (K a multiple of 64; forward and recomputing gradient): 256 x 256 tile, waves 2 x 2 with 128 x 128
+//     each, both operands double-buffered in LDS by direct global-to-LDS loads;
+//   * core C (K a multiple of 64; the backward's dH and dW products): 256 x 256 tile, waves side by side with
+//     256 x 64 each, operand A through LDS, operand B from a fragment-major copy straight into registers;
 //   * core A, the general one (K a multiple of 8): 256 x 128 tile, operands staged through registers
 //     into one padded LDS buffer.
 // Workgroups are numbered so that the 32 that share an XCD (and its L2) cover a 4 x 8 patch of tiles.
@@ -34,7 +36,7 @@ namespace nrl {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int GB_THREADS = 256;  // 4 wave64 in a 2 x 2 grid, whatever the core
+constexpr int GB_THREADS = 256;  // 4 wave64, whatever the core
 
 struct GemmOperands {
     const uint16_t* a;  // [M, K] row stride lda
@@ -67,7 +69,7 @@ __device__ __forceinline__ int acc_row(int e, int lane) { return 8 * (e >> 2) + 
 // registers while slab k is consumed from one padded LDS buffer (row stride 72 elements).
 // ---------------------------------------------------------------------------------------------
 struct CoreA {
-    static constexpr int BM = 256, BN = 128, NI = 4, NJ = 2, BK = 64, LD = BK + 8;
+    static constexpr int BM = 256, BN = 128, NI = 4, NJ = 2, BK = 64, LD = BK + 8, WAVES_N = 2;
     static constexpr int LDS_BYTES = (BM + BN) * LD * 2;
     static constexpr int A_LOADS = BM * BK / 8 / GB_THREADS, B_LOADS = BN * BK / 8 / GB_THREADS;
     struct Regs {
@@ -162,7 +164,7 @@ struct CoreA {
 // against 12.6 with the key r & 7 and 32 without swizzling.  Per 16-wide k step a wave issues 8 fragment reads for 16 MFMAs.
 // ---------------------------------------------------------------------------------------------
 struct CoreB {
-    static constexpr int BM = 256, BN = 256, NI = 4, NJ = 4, BK = 64;
+    static constexpr int BM = 256, BN = 256, NI = 4, NJ = 4, BK = 64, WAVES_N = 2;
     static constexpr int TILE_BYTES = 256 * BK * 2;  // one operand, one buffer
     static constexpr int LDS_BYTES = 4 * TILE_BYTES;  // A0 A1 B0 B1
     static constexpr int ROUNDS = 256 * BK / 8 / GB_THREADS;  // direct loads per lane, operand and slab: 8
@@ -323,6 +325,194 @@ struct CoreB {
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     }
 };
+
+// ---------------------------------------------------------------------------------------------
+// Core C: 256 x 256 tile, the four waves side by side along N (wave tile 256 x 64: NI = 8, NJ = 2), K a multiple
+// of 64.  Only operand A goes through LDS (four 32 KiB buffers filled by direct global-to-LDS loads, three slabs
+// ahead); each wave reads its own operand-B fragments straight from memory into registers, one slab ahead.  For
+// that B is stored "fragment-major": the 1 KiB that the 64 lanes of a wave feed to one matrix instruction (32 rows
+// x 16 k) is contiguous, lane by lane, and the blocks of a 32-row group follow each other along k -- a wave's load
+// of a fragment is then one fully used 1 KiB burst.  Per 16-wide k step a wave issues 8 LDS fragment reads for 16
+// MFMAs like core B, but the workgroup writes half as much into LDS and no wave reads B from it.
+//   element (n, k) of B sits at ((n / 32 * K16 + k / 16) * 64 + n % 32 + 32 * (k % 16 / 8)) * 8 + k % 8,
+//   K16 = ldb / 16 (ldb: the allocated k extent, a multiple of 64); row groups are allocated up to a multiple of 256 rows.
+// ---------------------------------------------------------------------------------------------
+template <int SPREAD> struct CoreCT {
+    static constexpr int BM = 256, BN = 256, NI = 8, NJ = 2, BK = 64, WAVES_N = 4;
+    static constexpr int KS = BK / 16;
+    static constexpr int NBUF = 4;
+    static constexpr int TILE_BYTES = 256 * BK * 2;
+    static constexpr int LDS_BYTES = NBUF * TILE_BYTES;
+    static constexpr int ROUNDS = 256 * BK / 8 / GB_THREADS;  // 8 direct loads per lane and slab
+
+    struct Ctx {
+        const char* pa;
+        uint32_t voa[ROUNDS];
+        uint32_t aoff[2][KS];   // lane's fragment address for each k step: buffers 0/1 and buffers 2/3 (tile row group 0)
+        uint64_t pb[NJ];        // this wave's two row groups of B at k = 0 (uniform)
+        uint32_t vlane;         // lane * 16
+        int wave;
+    };
+
+    __device__ static __forceinline__ void issue_a(const Ctx& c, unsigned char* lds, int buf, int64_t k0, int j) {
+        unsigned char* dst = lds + buf * TILE_BYTES + (j * GB_THREADS + c.wave * 64) * 16;
+        const char* src = c.pa + k0 * 2 + c.voa[j];
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const __attribute__((address_space(1))) void*>(reinterpret_cast<uintptr_t>(src)),
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+    // fragment (k step ks, row group j) of the slab that starts at k0
+    template <int KSTEP>
+    __device__ static __forceinline__ bf16x8 load_b(const Ctx& c, int64_t k0, int j) {
+        bf16x8 v;
+        const uint64_t base = c.pb[j] + static_cast<uint64_t>(k0) * 64;  // k0 / 16 blocks of 1 KiB
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(v) : "v"(c.vlane), "s"(base), "n"(KSTEP * 1024));
+        return v;
+    }
+    __device__ static __forceinline__ bf16x8 lds_read16(uint32_t addr, int imm) {
+        bf16x8 v;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(imm));
+        return v;
+    }
+    __device__ static __forceinline__ void wait_a(bf16x8 (&a)[NI]) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+    }
+    template <int N> __device__ static __forceinline__ void wait_b(bf16x8 (&b)[KS][NJ]) {
+        asm volatile("s_waitcnt vmcnt(%8)"
+                     : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[2][0]), "+v"(b[2][1]), "+v"(b[3][0]), "+v"(b[3][1])
+                     : "n"(N));
+    }
+
+    static constexpr int LEAD = 2 * KS - 1;  // B fragments are fetched this many k steps ahead
+
+    // fragments of k step `ks` (0 .. 2 KS - 1, counted from the slab that starts at k0) -> the ring of 2 KS register pairs
+    __device__ static __forceinline__ void fetch_b(const Ctx& c, bf16x8 (&bfr)[2][KS][NJ], int set, int ks, int64_t k0, int j) {
+        if (ks == 0) bfr[set][0][j] = load_b<0>(c, k0, j);
+        if (ks == 1) bfr[set][1][j] = load_b<1>(c, k0, j);
+        if (ks == 2) bfr[set][2][j] = load_b<2>(c, k0, j);
+        if (ks == 3) bfr[set][3][j] = load_b<3>(c, k0, j);
+    }
+
+    // One slab out of LDS buffer SLOT; its B fragments are in register set SLOT & 1 of a ring of 2 KS k steps.  On
+    // entry the A fragments of k step 0 are in flight into af[0].  Every k step issues four vector-memory operations,
+    // behind its first MFMAs: the two B fragments of the k step LEAD steps ahead (into the registers that the k
+    // step before this one has just finished with), then two of the eight direct loads of the slab three ahead
+    // (into the buffer that the previous slab's barrier freed).  Memory operations complete in order, so at the
+    // start of a k step "all but the youngest 4 (LEAD - 1) + 2" says that its B fragments are there.  At the start
+    // of the last k step this wave holds every fragment it needs from SLOT; the next slab's direct loads were
+    // issued two slabs ago or, for a tile's second slab, up to 20 operations before this point, hence vmcnt(20),
+    // and the barrier frees SLOT for the slab four ahead.
+    template <int SLOT>
+    __device__ static __forceinline__ void compute(const Ctx& c, unsigned char* lds, f32x16 (&acc)[NI][NJ], bf16x8 (&af)[2][NI],
+                                                   bf16x8 (&bfr)[2][KS][NJ], int64_t k_b1, int64_t k_b2, int64_t k_a) {
+        constexpr int SET = SLOT & 1, NEXT = (SLOT + 1) % NBUF;
+        auto frag_a = [&](int slot, int ks, int set, int f) {
+            af[set][f] = lds_read16(c.aoff[slot >> 1][ks], (slot & 1) * TILE_BYTES + f * 32 * BK * 2);
+        };
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            wait_a(af[ks & 1]);
+            if (ks == KS - 1) {
+                wait_b<20>(bfr[SET]);
+                asm volatile("s_barrier" ::: "memory");
+            } else {
+                wait_b<4 * (LEAD - 1) + 2>(bfr[SET]);
+            }
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int idx = i * NJ + j;
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[SET][ks][j], acc[i][j], 0, 0, 0);
+                    if (idx == 0 || idx == SPREAD) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        // k step ks + LEAD: ks == 0 -> next slab's last k step, otherwise the slab after it
+                        if (ks == 0) fetch_b(c, bfr, SET ^ 1, KS - 1, k_b1, idx / SPREAD);
+                        else fetch_b(c, bfr, SET, ks - 1, k_b2, idx / SPREAD);
+                    }
+                    if (idx == 2 * SPREAD || idx == 3 * SPREAD) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_a(c, lds, (SLOT + 3) % NBUF, k_a, ks * 2 + idx / SPREAD - 2);
+                    }
+                    if (idx < NI) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (ks + 1 < KS) frag_a(SLOT, ks + 1, (ks + 1) & 1, idx);
+                        else frag_a(NEXT, 0, 0, idx);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    __device__ static __forceinline__ void tile(const GemmOperands& op, int64_t row0, int64_t col0, f32x16 (&acc)[NI][NJ],
+                                                unsigned char* lds) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        Ctx c;
+        c.wave = wave;
+        c.vlane = static_cast<uint32_t>(lane * 16);
+        c.pa = reinterpret_cast<const char*>(op.a + row0 * op.lda);
+        const int64_t k16 = op.ldb / 16;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            c.pb[j] = reinterpret_cast<uint64_t>(op.b) + static_cast<uint64_t>(((col0 >> 5) + wave * NJ + j) * k16) * 1024u;
+        const int lr = tid >> 3, cg = (tid & 7) ^ ((lr >> 1) & 7);
+        const int last_a = static_cast<int>(op.m - 1 - row0 < 255 ? op.m - 1 - row0 : 255);
+#pragma unroll
+        for (int j = 0; j < ROUNDS; ++j) {
+            const int r = j * 32 + lr;
+            c.voa[j] = static_cast<uint32_t>((r < last_a ? r : last_a) * op.lda + cg * 8) * 2u;
+        }
+        const int fr = lane & 31, fh = lane >> 5;
+        const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint32_t sw = static_cast<uint32_t>(((ks * 2 + fh) ^ ((fr >> 1) & 7)) * 16);
+            c.aoff[0][ks] = lds_base + static_cast<uint32_t>(fr * BK * 2) + sw;
+            c.aoff[1][ks] = c.aoff[0][ks] + 2 * TILE_BYTES;
+        }
+        const int64_t nk = op.k / BK;
+        const int64_t k_last = (nk - 1) * BK;
+        auto slab_k = [&](int64_t kt) { return kt < nk ? kt * BK : k_last; };
+        bf16x8 af[2][NI], bfr[2][KS][NJ];
+        // order: the B fragments of the first LEAD k steps, then slabs 0, 1, 2 of A (the waits count on it)
+#pragma unroll
+        for (int g = 0; g < LEAD; ++g)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) fetch_b(c, bfr, g / KS, g % KS, g < KS ? 0 : slab_k(1), j);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < ROUNDS; ++j) issue_a(c, lds, 0, 0, j);
+#pragma unroll
+        for (int j = 0; j < ROUNDS; ++j) issue_a(c, lds, 1, slab_k(1), j);
+#pragma unroll
+        for (int j = 0; j < ROUNDS; ++j) issue_a(c, lds, 2, slab_k(2), j);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * ROUNDS) : "memory");  // slab 0 of A has landed everywhere
+#pragma unroll
+        for (int f = 0; f < NI; ++f) af[0][f] = lds_read16(c.aoff[0][0], f * 32 * BK * 2);
+        int64_t kt = 0;
+        for (; kt + 3 < nk; kt += 4) {
+            compute<0>(c, lds, acc, af, bfr, slab_k(kt + 1), slab_k(kt + 2), slab_k(kt + 3));
+            compute<1>(c, lds, acc, af, bfr, slab_k(kt + 2), slab_k(kt + 3), slab_k(kt + 4));
+            compute<2>(c, lds, acc, af, bfr, slab_k(kt + 3), slab_k(kt + 4), slab_k(kt + 5));
+            compute<3>(c, lds, acc, af, bfr, slab_k(kt + 4), slab_k(kt + 5), slab_k(kt + 6));
+        }
+        if (kt < nk) compute<0>(c, lds, acc, af, bfr, slab_k(kt + 1), slab_k(kt + 2), slab_k(kt + 3));
+        if (kt + 1 < nk) compute<1>(c, lds, acc, af, bfr, slab_k(kt + 2), slab_k(kt + 3), slab_k(kt + 4));
+        if (kt + 2 < nk) compute<2>(c, lds, acc, af, bfr, slab_k(kt + 3), slab_k(kt + 4), slab_k(kt + 5));
+        // what the last slabs fetched ahead is never used, but its registers and buffers must stay untouched until it
+        // has arrived
+        wait_a(af[0]);
+        wait_b<0>(bfr[0]);
+        wait_b<0>(bfr[1]);
+        asm volatile("s_barrier" ::: "memory");
+    }
+};
+
+using CoreC = CoreCT<2>;
 
 template <class Core> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[Core::NI][Core::NJ]) {
 #pragma unroll
@@ -877,7 +1067,7 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
     constexpr int NI = Core::NI, NJ = Core::NJ, BM = Core::BM, BN = Core::BN;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / Core::WAVES_N, wn = wave % Core::WAVES_N;
     if (!resolve_live(op)) return;
     int64_t bx, by;
     if (!patch_tile(blockIdx.x, (op.m + BM - 1) / BM, (op.n + BN - 1) / BN, bx, by)) return;
@@ -894,7 +1084,7 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
         for (int i = 0; i < NI; ++i)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int64_t r = row0 + wm * 128 + i * 32 + acc_row(e, lane);
+                const int64_t r = row0 + wm * (NI * 32) + i * 32 + acc_row(e, lane);
                 if (r >= op.m) continue;
                 float* out = c + static_cast<int64_t>(row_map[r]) * ldc;
 #pragma unroll
@@ -923,12 +1113,12 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
 #pragma unroll
                     for (int j = 0; j < NJ; ++j) {
                         const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
-                        const float* base = c + (row0 + wm * 128 + i * 32) * ldc + col;
+                        const float* base = c + (row0 + wm * (NI * 32) + i * 32) * ldc + col;
 #pragma unroll
                         for (int e = 0; e < 16; ++e) {
                             const int r = acc_row(e, lane);
                             prior[i - i0][j][e] =
-                                (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n)) ? base[r * ldc] : 0.f;
+                                (INTERIOR || (row0 + wm * (NI * 32) + i * 32 + r < op.m && col < op.n)) ? base[r * ldc] : 0.f;
                         }
                     }
             }
@@ -937,12 +1127,12 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
                     const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
-                    float* base = c + (row0 + wm * 128 + i * 32) * ldc + col;
+                    float* base = c + (row0 + wm * (NI * 32) + i * 32) * ldc + col;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int r = acc_row(e, lane);
                         const float v = acc_read(acc[i][j][e]);
-                        if (INTERIOR || (row0 + wm * 128 + i * 32 + r < op.m && col < op.n))
+                        if (INTERIOR || (row0 + wm * (NI * 32) + i * 32 + r < op.m && col < op.n))
                             base[r * ldc] = ACCUM ? prior[i - i0][j][e] + v : v;
                     }
                 }
@@ -1012,20 +1202,30 @@ __global__ __launch_bounds__(256) void gather_live_kernel(const uint16_t* hidden
     }
 }
 
-// dst[c, r] = src[r, c] for r < rows, c < cols; dst row stride ldd, columns [rows, pad_cols) zero-filled
-__global__ void transpose_bf16_kernel(const uint16_t* src, int64_t rows, int64_t cols, int64_t lds_, uint16_t* dst,
-                                      int64_t ldd, int64_t pad_cols) {
+// B[n, k] = src[k, n] in core C's fragment-major layout (k extent ldk, a multiple of 64): k < rows and n < cols are
+// copied, everything else up to pad_k and up to the launch's n tiles is zero.  One workgroup per 64 x 64 tile.
+__global__ __launch_bounds__(256) void transpose_to_frag_kernel(const uint16_t* src, int64_t rows, int64_t cols, int64_t lds_,
+                                                                uint16_t* dst, int64_t ldk, int64_t pad_k) {
     __shared__ uint16_t tile[64][66];
-    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 64, c0 = static_cast<int64_t>(blockIdx.x) * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 256 threads: 64 x 4
-    for (int k = ty; k < 64; k += 4) {
-        const int64_t r = r0 + k, c = c0 + tx;
-        tile[k][tx] = (r < rows && c < cols) ? src[r * lds_ + c] : static_cast<uint16_t>(0);
+    const int64_t k0 = static_cast<int64_t>(blockIdx.y) * 64, n0 = static_cast<int64_t>(blockIdx.x) * 64;
+    if (k0 >= pad_k) return;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int kk = ty; kk < 64; kk += 4) {
+        const int64_t r = k0 + kk, c = n0 + tx;
+        tile[kk][tx] = (r < rows && c < cols) ? src[r * lds_ + c] : static_cast<uint16_t>(0);
     }
     __syncthreads();
-    for (int k = ty; k < 64; k += 4) {
-        const int64_t c = c0 + k, r = r0 + tx;
-        if (c < cols && r < pad_cols) dst[c * ldd + r] = tile[tx][k];
+    const int64_t k16 = ldk / 16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int u = h * 256 + threadIdx.x, blk = u >> 6, lane = u & 63;
+        const int ng = blk >> 2, kb = blk & 3;
+        const int nl = ng * 32 + (lane & 31), kl = kb * 16 + (lane >> 5) * 8;
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = static_cast<uint32_t>(tile[kl + 2 * e][nl]) | (static_cast<uint32_t>(tile[kl + 2 * e + 1][nl]) << 16);
+        uint16_t* out = dst + (((n0 / 32 + ng) * k16 + (k0 / 16 + kb)) * 64 + lane) * 8;
+        *reinterpret_cast<u32x4*>(out) = u32x4{w[0], w[1], w[2], w[3]};
     }
 }
 
@@ -1096,13 +1296,10 @@ template <class Core> static void launch_grad(const LmGradArgs& a, hipStream_t s
                                dim3(GB_THREADS), 0, s>>>(a);
 }
 
+// C = or += A B^T with B in core C's fragment-major layout (op.ldb: its k extent); op.k a multiple of 64
 template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, int64_t ldc, hipStream_t s, const int32_t* row_map = nullptr) {
-    if (op.k % CoreB::BK == 0 && op.k > 0)
-        gemm_f32_kernel<CoreB, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreB::BM - 1) / CoreB::BM, (op.n + CoreB::BN - 1) / CoreB::BN)),
-                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
-    else
-        gemm_f32_kernel<CoreA, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreA::BM - 1) / CoreA::BM, (op.n + CoreA::BN - 1) / CoreA::BN)),
-                                        dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
+    gemm_f32_kernel<CoreC, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreC::BM - 1) / CoreC::BM, (op.n + CoreC::BN - 1) / CoreC::BN)),
+                                    dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
 }
 
 extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
@@ -1145,10 +1342,10 @@ extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidd
     const int64_t n = n_tokens < 1 ? 1 : n_tokens;
     const int64_t chunk = bwd_chunk(n_tokens), vp = round_up(vocab, 64), n_pad = round_up(n, chunk);
     int64_t b = 0;
-    b += hidden_size * vp * 2;        // W^T
+    b += round_up(hidden_size, 256) * vp * 2;        // W^T, fragment-major
     b += chunk * vp * 2;              // G
     b += vocab * bwd_ld_t(chunk) * 2;        // G^T
-    b += hidden_size * bwd_ld_t(chunk) * 2;  // hidden chunk^T
+    b += round_up(hidden_size, 256) * bwd_ld_t(chunk) * 2;  // hidden chunk^T, fragment-major
     b += vocab * hidden_size * 4;     // dW accumulator (fp32)
     b += n_pad * hidden_size * 2;     // hidden rows of the tokens that carry a gradient
     b += n_pad * (8 + 4 + 4 + 4);     // their targets, log-sum-exps, gradients and token indices
@@ -1176,11 +1373,12 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
     const int64_t n_pad = round_up(n_tokens < 1 ? 1 : n_tokens, chunk);
     char* ws = static_cast<char*>(workspace);
     auto take = [&](int64_t bytes) { char* p = ws; ws += (bytes + 255) / 256 * 256; return p; };
-    uint16_t* wt = reinterpret_cast<uint16_t*>(take(h * vp * 2));
+    const int64_t h_pad = round_up(h, 256);
+    uint16_t* wt = reinterpret_cast<uint16_t*>(take(h_pad * vp * 2));
     uint16_t* g = reinterpret_cast<uint16_t*>(take(chunk * vp * 2));
     const int64_t ld_t = bwd_ld_t(chunk);
     uint16_t* gt = reinterpret_cast<uint16_t*>(take(vocab * ld_t * 2));
-    uint16_t* ht = reinterpret_cast<uint16_t*>(take(h * ld_t * 2));
+    uint16_t* ht = reinterpret_cast<uint16_t*>(take(h_pad * ld_t * 2));
     float* dw = reinterpret_cast<float*>(take(vocab * h * 4));
     uint16_t* hid_c = reinterpret_cast<uint16_t*>(take(n_pad * h * 2));
     int64_t* tgt_c = reinterpret_cast<int64_t*>(take(n_pad * 8));
@@ -1191,8 +1389,8 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
     const uint16_t* hid = static_cast<const uint16_t*>(hidden);
     const uint16_t* w = static_cast<const uint16_t*>(weight);
 
-    // W^T [H, vp] (zero-padded columns) and a zeroed fp32 dW accumulator
-    transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((vp + 63) / 64)), dim3(256), 0, s>>>(w, vocab, h, ldw, wt, vp, vp);
+    // W^T [H, vp] (zero-padded, fragment-major: operand B of the dH product) and a zeroed fp32 dW accumulator
+    transpose_to_frag_kernel<<<dim3((unsigned)(h_pad / 64), (unsigned)(vp / 64)), dim3(256), 0, s>>>(w, vocab, h, ldw, wt, vp, vp);
     fill_zero_u32<<<dim3(2048), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(dw), vocab * h);
     if (n_tokens == 0) {
         // (nothing to add to dW)
@@ -1231,7 +1429,7 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         dh.live = count; dh.live_from = t0; dh.live_dim = 1;
         launch_gemm<false>(dh, dhidden_out, ld_dh, s, idx + t0);
         // dW += G^T [V, rows] * (hidden^T [H, rows])^T
-        transpose_bf16_kernel<<<dim3((unsigned)((h + 63) / 64), (unsigned)((rows_pad + 63) / 64)), dim3(256), 0, s>>>(
+        transpose_to_frag_kernel<<<dim3((unsigned)(h_pad / 64), (unsigned)(rows_pad / 64)), dim3(256), 0, s>>>(
             hid_c + t0 * h, rows, h, h, ht, ld_t, rows_pad);
         GemmOperands dwo;
         dwo.a = gt; dwo.lda = ld_t; dwo.b = ht; dwo.ldb = ld_t; dwo.m = vocab; dwo.n = h; dwo.k = rows_pad;
