@@ -535,20 +535,23 @@ __device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f
 
 // Tile coordinates of workgroup w of a 1-D launch over an nbx x nby tile grid.  Workgroups go to the
 // 8 XCDs (each with its own L2) round-robin by index, so index w runs on XCD w % 8 as that XCD's
-// (w / 8)-th workgroup; an XCD's 32 compute units hold one 4 x 8 patch of tiles at a time, which share
-// 4 A panels and 8 B panels through that L2.  Patches past the grid yield false.
+// (w / 8)-th workgroup; an XCD's 32 compute units hold one PX x PY patch of tiles at a time (4 x 8 unless said
+// otherwise), which share PX A panels and PY B panels through that L2.  Patches past the grid yield false.
+template <int PX = 4>
 __device__ __forceinline__ bool patch_tile(uint32_t w, int64_t nbx, int64_t nby, int64_t& bx, int64_t& by) {
+    constexpr uint32_t PY = 32 / PX;
+    static_assert(PX * PY == 32, "a patch is what one XCD holds");
     const uint32_t xcd = w & 7, s = w >> 3;
     const uint32_t patch = (s >> 5) * 8 + xcd, t = s & 31;
-    const uint32_t ppy = static_cast<uint32_t>((nby + 7) >> 3);  // patches along y
+    const uint32_t ppy = static_cast<uint32_t>((nby + PY - 1) / PY);  // patches along y
     const uint32_t px = patch / ppy, py = patch - px * ppy;
     // the division runs on the vector unit; hand the (uniform) results back to scalar registers
-    bx = __builtin_amdgcn_readfirstlane(static_cast<int>(px * 4 + (t >> 3)));
-    by = __builtin_amdgcn_readfirstlane(static_cast<int>(py * 8 + (t & 7)));
+    bx = __builtin_amdgcn_readfirstlane(static_cast<int>(px * PX + t / PY));
+    by = __builtin_amdgcn_readfirstlane(static_cast<int>(py * PY + t % PY));
     return bx < nbx && by < nby;
 }
-static int64_t patch_grid(int64_t nbx, int64_t nby) {
-    const int64_t patches = ((nbx + 3) / 4) * ((nby + 7) / 8);
+static int64_t patch_grid(int64_t nbx, int64_t nby, int64_t px = 4) {
+    const int64_t py = 32 / px, patches = ((nbx + px - 1) / px) * ((nby + py - 1) / py);
     return (patches + 7) / 8 * 8 * 32;
 }
 
@@ -571,6 +574,11 @@ struct LmFwdArgs {
     int64_t ldl;               // multiple of 8, >= V; columns from V on are unspecified
 };
 
+// Token tiles per XCD patch of the forward (the other side of the patch counts vocabulary splits).  Without the
+// logits 8 token tiles x 4 splits measured 4 % faster than 4 x 8 (58.9 against 61.3 ms at 65536 tokens, V 151936);
+// with the logits written it measured 1 % slower, and 16 x 2 and 32 x 1 slower either way.
+constexpr int fwd_patch_tokens(bool save) { return save ? 4 : 8; }
+
 template <class Core, bool SAVE>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     constexpr int NI = Core::NI, NJ = Core::NJ, BV = Core::BM, BT = Core::BN;  // vocabulary rows x token columns
@@ -581,7 +589,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     int64_t bx, by;
-    if (!patch_tile(blockIdx.x, (a.op.n + BT - 1) / BT, a.n_splits, bx, by)) return;
+    if (!patch_tile<fwd_patch_tokens(SAVE)>(blockIdx.x, (a.op.n + BT - 1) / BT, a.n_splits, bx, by)) return;
     const int64_t tok0 = bx * BT;
     const int split = static_cast<int>(by);
     const int64_t n_tiles = (a.op.m + BV - 1) / BV;
@@ -1286,7 +1294,7 @@ template <class Core> static void launch_fwd(LmFwdArgs& a, float* ws, hipStream_
     a.n_splits = fwd_splits<Core>(n, a.op.m);
     a.part_m = ws; a.part_s = ws + static_cast<int64_t>(a.n_splits) * n; a.xt = ws + 2 * static_cast<int64_t>(a.n_splits) * n;
     fill_zero_u32<<<dim3(256), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(a.xt), n);
-    const dim3 grid((unsigned)patch_grid((n + Core::BN - 1) / Core::BN, a.n_splits));
+    const dim3 grid((unsigned)patch_grid((n + Core::BN - 1) / Core::BN, a.n_splits, fwd_patch_tokens(a.logits != nullptr)));
     if (a.logits) lmhead_fwd_kernel<Core, true><<<grid, dim3(GB_THREADS), 0, s>>>(a);
     else lmhead_fwd_kernel<Core, false><<<grid, dim3(GB_THREADS), 0, s>>>(a);
 }
