@@ -783,6 +783,9 @@ struct LmGradArgs {
     int64_t ldgt;
 };
 
+// token tiles per XCD patch of the recomputing gradient kernel (x 4 vocabulary tiles): 1.7 % faster than 4 x 8
+constexpr int kGradPatchTokens = 8;
+
 template <class Core>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     constexpr int NI = Core::NI, NJ = Core::NJ, BM = Core::BM, BN = Core::BN;
@@ -793,7 +796,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
     const int wm = wave >> 1, wn = wave & 1;
     if (!resolve_live(a.op)) return;
     int64_t bx, by;
-    if (!patch_tile(blockIdx.x, (a.op.m + BM - 1) / BM, (a.op.n + BN - 1) / BN, bx, by)) return;
+    if (!patch_tile<kGradPatchTokens>(blockIdx.x, (a.op.m + BM - 1) / BM, (a.op.n + BN - 1) / BN, bx, by)) return;
     const int64_t row0 = bx * BM, col0 = by * BN;
     {
         const int64_t grow = row0 + tid;
@@ -1300,7 +1303,7 @@ template <class Core> static void launch_fwd(LmFwdArgs& a, float* ws, hipStream_
 }
 
 template <class Core> static void launch_grad(const LmGradArgs& a, hipStream_t s) {
-    lmhead_grad_kernel<Core><<<dim3((unsigned)patch_grid((a.op.m + Core::BM - 1) / Core::BM, (a.op.n + Core::BN - 1) / Core::BN)),
+    lmhead_grad_kernel<Core><<<dim3((unsigned)patch_grid((a.op.m + Core::BM - 1) / Core::BM, (a.op.n + Core::BN - 1) / Core::BN, kGradPatchTokens)),
                                dim3(GB_THREADS), 0, s>>>(a);
 }
 
