@@ -384,6 +384,7 @@ template <int SPREAD> struct CoreCT {
     }
 
     static constexpr int LEAD = 2 * KS - 1;  // B fragments are fetched this many k steps ahead
+    static_assert(NI == 8 && NJ == 2 && KS == 4 && ROUNDS == 2 * KS, "the waits below list their registers and count the operations of a k step");
 
     // fragments of k step `ks` (0 .. 2 KS - 1, counted from the slab that starts at k0) -> the ring of 2 KS register pairs
     __device__ static __forceinline__ void fetch_b(const Ctx& c, bf16x8 (&bfr)[2][KS][NJ], int set, int ks, int64_t k0, int j) {
