@@ -383,3 +383,31 @@ def test_backward_from_the_kept_set_record_equals_the_streaming_backward(dtype, 
             on_record = (cnt >= 0).cpu()
             if temperature == 1.0:
                 assert torch.equal(cnt.cpu()[on_record].long(), keep_rows.sum(-1)[on_record])
+
+
+def test_record_entries_outside_their_ranges_are_not_followed():
+    """A count above the record's capacity is not a count the forward writes: that row is streamed like a row without
+    a record.  An index outside the vocabulary is skipped.  Neither makes the backward write outside its row."""
+    from rl_amd._lib import NRL_TEMP_RCP
+
+    g = torch.Generator().manual_seed(77)
+    b, s, vocab, cap = 2, 7, 3001, 64
+    n = s - 1
+    x = (torch.randn(b, s, vocab, generator=g) * 3.0).to(torch.bfloat16).to(DEV)
+    t = x.float().argmax(-1)[:, :n].contiguous()
+    u = torch.randn(b, n, generator=g).to(DEV)
+    ops = torch.ops.rl_amd
+    _, thr, tie, lse, _, cnt, idx, val = ops.topk_topp_logprob_fwd_rec(x, t, n, 20, 0.95, 1.0, NRL_TEMP_RCP, False, cap)
+    streamed = ops.topk_topp_logprob_bwd(x, t, thr, tie, lse, u, n, 1.0, NRL_TEMP_RCP)
+    assert int(cnt[0, 1]) > 0 and int(cnt[1, 3]) > 1
+    bad_cnt = cnt.clone()
+    bad_cnt[0, 1] = cap + 5
+    got = ops.topk_topp_logprob_bwd(x, t, thr, tie, lse, u, n, 1.0, NRL_TEMP_RCP, bad_cnt, idx, val)
+    assert torch.equal(got.view(torch.int16), streamed.view(torch.int16))
+    bad_idx = idx.clone()
+    skipped = int(bad_idx[1, 3, 1])
+    bad_idx[1, 3, 1] = vocab + 12345
+    got = ops.topk_topp_logprob_bwd(x, t, thr, tie, lse, u, n, 1.0, NRL_TEMP_RCP, cnt, bad_idx, val)
+    want = streamed.clone()
+    want[1, 3, skipped] = 0.0
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
