@@ -116,6 +116,24 @@ __device__ __forceinline__ void ent_push(Ent& a, float x) {
     a.s += p;
     a.t += p > 0.f ? p * d : 0.f;  // a -inf logit has probability 0 and adds nothing
 }
+// N elements at once: one rescale for the batch's maximum instead of a branch and a rescale per new maximum
+template <int N> __device__ __forceinline__ void ent_push_n(Ent& a, const float (&x)[N]) {
+    float vm = x[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) vm = fmaxf(vm, x[k]);
+    const float mn = fmaxf(a.m, vm);
+    const float d0 = a.m - mn, e = fast_exp2(d0 * kLog2e);
+    float t = e * (a.t + d0 * a.s), s = e * a.s;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        const float d = x[k] - mn, p = fast_exp2(d * kLog2e);
+        s += p;
+        t += p > 0.f ? p * d : 0.f;
+    }
+    a.m = mn;
+    a.s = s;
+    a.t = t;
+}
 __device__ __forceinline__ Ent ent_merge(Ent a, Ent b) {
     const float m = fmaxf(a.m, b.m), da = a.m - m, db = b.m - m;
     const float ea = fast_exp2(da * kLog2e), eb = fast_exp2(db * kLog2e);
@@ -153,7 +171,8 @@ __global__ __launch_bounds__(kDBlock) void neg_entropy_fwd_kernel(RowsView x, fl
     const int64_t r = blockIdx.x;
     const char* row = row_ptr<DT>(x, r);
     Ent acc{-1e30f, 0.f, 0.f};
-    row_for_each<DT>(row, x.vocab, [&](float v) { ent_push(acc, v); });
+    row_for_each_vec<DT>(
+        row, x.vocab, [&](const float(&t)[Row<DT>::EPV]) { ent_push_n<Row<DT>::EPV>(acc, t); }, [&](float v) { ent_push(acc, v); });
     const Ent tot = ent_block(acc, smem);
     if (threadIdx.x == 0) {
         const float log_s = logf(tot.s);
@@ -245,6 +264,25 @@ __device__ __forceinline__ void ce_push(Ce& a, float y, float x) {
     a.s += p;
     a.u += p > 0.f ? p * x : 0.f;
 }
+// N elements at once: one rescale for the batch's maximum instead of a branch and a rescale per new maximum
+template <int N> __device__ __forceinline__ void ce_push_n(Ce& a, const float (&y)[N], const float (&x)[N]) {
+    float vm = y[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) vm = fmaxf(vm, y[k]);
+    const float mn = fmaxf(a.m, vm);
+    const float e = fast_exp2((a.m - mn) * kLog2e);
+    const float mn2 = mn * kLog2e;
+    float s = a.s * e, u = a.u * e;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        const float p = fast_exp2(__builtin_fmaf(y[k], kLog2e, -mn2));
+        s += p;
+        u += p > 0.f ? p * x[k] : 0.f;
+    }
+    a.m = mn;
+    a.s = s;
+    a.u = u;
+}
 __device__ __forceinline__ Ce ce_merge(Ce a, Ce b) {
     const float m = fmaxf(a.m, b.m);
     const float ea = fast_exp2((a.m - m) * kLog2e), eb = fast_exp2((b.m - m) * kLog2e);
@@ -272,8 +310,7 @@ __global__ __launch_bounds__(kDBlock) void soft_ce_fwd_kernel(RowsView x, RowsVi
             Row<DT>::decode(qx, a);
             Row<DT>::decode(qy, b);
             lse_push<EPV>(ax, a);
-#pragma unroll
-            for (int k = 0; k < EPV; ++k) ce_push(ay, b[k], a[k]);
+            ce_push_n<EPV>(ay, b, a);
         };
         int64_t base = 0;
         for (; base + kDUnroll * kDBlock <= nvec; base += kDUnroll * kDBlock) {
