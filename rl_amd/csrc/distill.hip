@@ -106,7 +106,7 @@ struct Ent {
     float m, s, t;
 };
 __device__ __forceinline__ void ent_push(Ent& a, float x) {
-    if (x > a.m) {
+    if (x > a.m) {  // (a batch of 8 with one rescale and no branch measured 4 % slower here, unlike in the soft cross entropy)
         const float d = a.m - x, e = fast_exp2(d * kLog2e);
         a.t = e * (a.t + d * a.s);
         a.s = e * a.s;
@@ -115,24 +115,6 @@ __device__ __forceinline__ void ent_push(Ent& a, float x) {
     const float d = x - a.m, p = fast_exp2(d * kLog2e);
     a.s += p;
     a.t += p > 0.f ? p * d : 0.f;  // a -inf logit has probability 0 and adds nothing
-}
-// N elements at once: one rescale for the batch's maximum instead of a branch and a rescale per new maximum
-template <int N> __device__ __forceinline__ void ent_push_n(Ent& a, const float (&x)[N]) {
-    float vm = x[0];
-#pragma unroll
-    for (int k = 1; k < N; ++k) vm = fmaxf(vm, x[k]);
-    const float mn = fmaxf(a.m, vm);
-    const float d0 = a.m - mn, e = fast_exp2(d0 * kLog2e);
-    float t = e * (a.t + d0 * a.s), s = e * a.s;
-#pragma unroll
-    for (int k = 0; k < N; ++k) {
-        const float d = x[k] - mn, p = fast_exp2(d * kLog2e);
-        s += p;
-        t += p > 0.f ? p * d : 0.f;
-    }
-    a.m = mn;
-    a.s = s;
-    a.t = t;
 }
 __device__ __forceinline__ Ent ent_merge(Ent a, Ent b) {
     const float m = fmaxf(a.m, b.m), da = a.m - m, db = b.m - m;
@@ -171,8 +153,7 @@ __global__ __launch_bounds__(kDBlock) void neg_entropy_fwd_kernel(RowsView x, fl
     const int64_t r = blockIdx.x;
     const char* row = row_ptr<DT>(x, r);
     Ent acc{-1e30f, 0.f, 0.f};
-    row_for_each_vec<DT>(
-        row, x.vocab, [&](const float(&t)[Row<DT>::EPV]) { ent_push_n<Row<DT>::EPV>(acc, t); }, [&](float v) { ent_push(acc, v); });
+    row_for_each<DT>(row, x.vocab, [&](float v) { ent_push(acc, v); });
     const Ent tot = ent_block(acc, smem);
     if (threadIdx.x == 0) {
         const float log_s = logf(tot.s);
