@@ -1,17 +1,33 @@
 """Makes the kernels reachable under NeMo-RL's own dotted paths.
 
-``install()`` either registers ``nemo_rl.distributed.model_utils``, ``nemo_rl.algorithms.loss`` (and
-its sub-modules), ``nemo_rl.algorithms.loss_functions``, ``nemo_rl.algorithms.utils``,
-``nemo_rl.algorithms.logits_sampling_utils``, ``nemo_rl.algorithms.advantage_estimator`` and
-``nemo_rl.models.automodel.train`` / ``nemo_rl.models.megatron.train`` (their post-processors and
-``apply_temperature_scaling``) as
-aliases of the ``rl_amd`` modules (when NeMo-RL is not importable), or replaces the hot-path
-attributes of an existing NeMo-RL install in place.
+``install()`` has two modes.
+
+* NeMo-RL is not importable: the dotted paths ``nemo_rl.distributed.model_utils``,
+  ``nemo_rl.algorithms.loss`` (and its sub-modules), ``nemo_rl.algorithms.loss_functions``,
+  ``nemo_rl.algorithms.utils``, ``nemo_rl.algorithms.logits_sampling_utils``,
+  ``nemo_rl.algorithms.advantage_estimator``, ``nemo_rl.algorithms.grpo`` and
+  ``nemo_rl.models.{automodel,megatron}.train`` are registered as aliases of the ``rl_amd`` modules.
+* NeMo-RL is importable: the hot-path objects of the install are replaced **by identity**.  The
+  reference binds most of them with ``from ... import name`` -- the package ``nemo_rl.algorithms.loss``
+  re-exports its loss classes and input preparation (``algorithms/loss/__init__.py:15-41``), the driver
+  imports ``ClippedPGLossFn`` from that package and ``calculate_baseline_and_std_per_prompt`` by name
+  (``algorithms/grpo.py:32-59``), the workers import the wrappers and ``prepare_loss_input``
+  (``models/automodel/train.py:44-48``, ``models/megatron/train.py:39-50``), the loss module imports
+  ``calculate_kl`` and ``masked_mean`` (``algorithms/loss/loss_functions.py:26``) -- so replacing an
+  attribute of the defining module alone leaves every such copy pointing at the original.  ``install()``
+  therefore records each original object, replaces it in its defining module, and then walks every
+  loaded module and rebinds each global that *is* one of the originals.  In the other direction the
+  ``rl_amd`` classes adopt the install's own ``LossType`` / ``LossInputType`` / ``MetricNormalizer``
+  enums, because the reference's workers compare ``loss_fn.loss_type == LossType.TOKEN_LEVEL``
+  (``models/automodel/data.py:422``) and test ``kind is MetricNormalizer.NONE``
+  (``models/policy/workers/megatron_policy_worker.py:1724``) against their own enum objects.
 """
 
 from __future__ import annotations
 
+import enum
 import importlib
+import importlib.util
 import sys
 import types
 
@@ -31,7 +47,15 @@ _ALIASES = {
     "nemo_rl.algorithms.grpo": "rl_amd.algorithms.grpo",
 }
 
-# attributes replaced on a real NeMo-RL install (module -> names)
+_LOSS_CLASSES = ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn",
+                 "DraftCrossEntropyLossFn"]
+_LOSS_PREPARE = ["prepare_loss_input", "prepare_packed_loss_input"]
+_LOSS_WRAPPERS = ["wrap_loss_fn_with_input_preparation", "SequencePackingLossWrapper",
+                  "SequencePackingFusionLossWrapper"]
+
+# objects replaced on a real NeMo-RL install: defining module -> names.  The package
+# ``nemo_rl.algorithms.loss`` is listed for the case that an install defines a name there directly; its
+# re-exports of the modules below are caught by the identity walk either way.
 _PATCHED = {
     "nemo_rl.distributed.model_utils": [
         "DistributedLogprob", "ChunkedDistributedLogprob", "DistributedLogprobWithSampling",
@@ -44,18 +68,30 @@ _PATCHED = {
         "_compute_distributed_log_softmax", "_compute_distributed_log_softmax_with_grad",
     ],
     "nemo_rl.algorithms.logits_sampling_utils": ["apply_top_k_top_p"],
-    "nemo_rl.algorithms.loss.wrapper": ["wrap_loss_fn_with_input_preparation", "SequencePackingLossWrapper",
-                                        "SequencePackingFusionLossWrapper"],
-    "nemo_rl.algorithms.loss.utils": ["prepare_loss_input", "prepare_packed_loss_input"],
-    "nemo_rl.algorithms.loss.loss_functions": ["ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn",
-                                               "DraftCrossEntropyLossFn"],
     "nemo_rl.algorithms.utils": ["calculate_baseline_and_std_per_prompt", "calculate_kl", "masked_mean",
                                  "mask_out_neg_inf_logprobs"],
+    "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
+    "nemo_rl.algorithms.loss.loss_functions": _LOSS_CLASSES,
+    "nemo_rl.algorithms.loss.utils": _LOSS_PREPARE,
+    "nemo_rl.algorithms.loss.wrapper": _LOSS_WRAPPERS,
+    "nemo_rl.algorithms.loss": _LOSS_CLASSES + _LOSS_PREPARE + _LOSS_WRAPPERS,
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling"],
     "nemo_rl.models.megatron.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling"],
     "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking", "dynamic_sampling"],
-    "nemo_rl.algorithms.advantage_estimator": ["GRPOAdvantageEstimator"],
 }
+
+# modules of an install that need packages a single-GPU DTensor worker may not have (Megatron-Core for the
+# Megatron worker, Ray and the data stack for the driver): skipped when their import fails
+_OPTIONAL = {"nemo_rl.models.megatron.train", "nemo_rl.models.automodel.train", "nemo_rl.algorithms.grpo"}
+
+_ENUMS = ("LossType", "LossInputType", "MetricNormalizer")
+
+_state = {"originals": [], "skipped": [], "replacements": {}}
+
+
+def skipped_modules() -> list[str]:
+    """Modules of the install that the last ``install()`` could not import and therefore left alone."""
+    return list(_state["skipped"])
 
 
 def _real_nemo_rl_present() -> bool:
@@ -68,14 +104,102 @@ def _real_nemo_rl_present() -> bool:
         return False
 
 
-def install(force_alias: bool = False) -> str:
-    """Returns ``"patched"`` or ``"aliased"``."""
-    if _real_nemo_rl_present() and not force_alias:
-        for target, names in _PATCHED.items():
+def _is_ours(name: str) -> bool:
+    return name == "rl_amd" or name.startswith("rl_amd.")
+
+
+def _rebind_by_identity(replacements: dict[int, tuple[object, object]], ours: bool) -> int:
+    """Rebinds, in every loaded module (``rl_amd``'s own when ``ours``, all others otherwise), each global
+    that is one of the recorded objects.  Returns the number of rebindings."""
+    count = 0
+    for name, mod in list(sys.modules.items()):
+        if mod is None or _is_ours(name) != ours:
+            continue
+        namespace = getattr(mod, "__dict__", None)
+        if not isinstance(namespace, dict):
+            continue
+        for attr, value in list(namespace.items()):
+            hit = replacements.get(id(value))
+            if hit is not None and hit[0] is value:
+                try:
+                    setattr(mod, attr, hit[1])
+                except (AttributeError, TypeError):
+                    namespace[attr] = hit[1]
+                count += 1
+    return count
+
+
+def _adopt_reference_enums() -> None:
+    """Makes the ``rl_amd`` modules use the install's ``LossType`` / ``LossInputType`` / ``MetricNormalizer``:
+    module globals are rebound and class attributes that hold a member of one of them are translated by
+    member name (instances read the module globals when they are constructed)."""
+    theirs = importlib.import_module("nemo_rl.algorithms.loss.interfaces")
+    mine = importlib.import_module("rl_amd.algorithms.loss.interfaces")
+    swap: dict[int, tuple[object, object]] = {}
+    for name in _ENUMS:
+        old, new = getattr(mine, name), getattr(theirs, name, None)
+        if new is None or new is old:
+            continue
+        missing = [m.name for m in old if m.name not in new.__members__]
+        if missing:
+            raise RuntimeError(f"nemo_rl.algorithms.loss.interfaces.{name} lacks the members {missing}")
+        swap[id(old)] = (old, new)
+    if not swap:
+        return
+    _state["originals"].extend(old for old, _ in swap.values())
+    _rebind_by_identity(swap, ours=True)
+    for name, mod in list(sys.modules.items()):
+        if mod is None or not _is_ours(name):
+            continue
+        for value in list(vars(mod).values()):
+            if not (isinstance(value, type) and _is_ours(getattr(value, "__module__", ""))):
+                continue
+            for attr, member in list(vars(value).items()):
+                if isinstance(member, enum.Enum) and id(type(member)) in swap:
+                    setattr(value, attr, swap[id(type(member))][1][member.name])
+
+
+def _patch_install() -> None:
+    # kept across calls: a later call also rebinds what a module imported in between may have picked up
+    replacements: dict[int, tuple[object, object]] = _state["replacements"]
+    skipped = []
+    sources = {target: importlib.import_module(_ALIASES[target]) for target in _PATCHED}
+    for target, names in _PATCHED.items():
+        try:
             dst = importlib.import_module(target)
-            src = importlib.import_module(_ALIASES[target])
-            for name in names:
-                setattr(dst, name, getattr(src, name))
+        except ImportError:
+            if target not in _OPTIONAL:
+                raise
+            skipped.append(target)
+            continue
+        for name in names:
+            new = getattr(sources[target], name)
+            old = getattr(dst, name, None)
+            if old is not None and old is not new and not _is_ours(getattr(old, "__module__", "") or ""):
+                replacements[id(old)] = (old, new)
+            setattr(dst, name, new)
+    _state["skipped"] = skipped
+    # (the table references the originals, so their ids cannot be reused while it is in use)
+    _adopt_reference_enums()
+    _rebind_by_identity(replacements, ours=False)
+    short = "nemo_rl.algorithms.loss_functions"  # the short spelling, if the install has no such module
+    if short not in sys.modules and importlib.util.find_spec(short) is None:
+        mod = importlib.import_module(_ALIASES[short])
+        sys.modules[short] = mod
+        setattr(sys.modules["nemo_rl.algorithms"], "loss_functions", mod)
+
+
+def install(force_alias: bool = False) -> str:
+    """Returns ``"patched"`` (a NeMo-RL install was found and its hot-path objects replaced) or
+    ``"aliased"`` (the dotted paths now name the ``rl_amd`` modules).
+
+    On an install, call it in every process that runs a policy worker or the GRPO driver, after the
+    NeMo-RL modules that process uses are imported (what is imported later sees the replaced attributes
+    of the defining modules anyway) and before a loss function, wrapper or post-processor object is
+    constructed: objects built from the original classes stay what they are.  Calling it again is safe
+    and picks up modules that were imported in between."""
+    if _real_nemo_rl_present() and not force_alias:
+        _patch_install()
         return "patched"
     for parent in ("nemo_rl", "nemo_rl.distributed", "nemo_rl.algorithms", "nemo_rl.models", "nemo_rl.models.automodel",
                    "nemo_rl.models.megatron"):

@@ -134,3 +134,115 @@ def packed_grpo_case(lens, pads, width, vocab, dtype, seed, tail=0, empty_mask_r
     gs = sm.sum().float()
     gt = (tm[:, 1:] * sm.unsqueeze(-1)).sum().float()
     return logits, data, cu, cup, gs, gt
+
+
+# A stand-in for a NeMo-RL install: a few lines per module, written for this test, that reproduce how the
+# reference binds its hot-path names -- package re-exports (``algorithms/loss/__init__.py:15-41``), by-name
+# imports in the driver (``algorithms/grpo.py:32-59``), the workers (``models/automodel/train.py:44-48``,
+# ``models/megatron/train.py:39-50``, the latter needing Megatron-Core) and the loss module
+# (``algorithms/loss/loss_functions.py:26``), and an enum comparison outside the replaced code
+# (``models/automodel/data.py:422``).
+_STUB_INSTALL = {
+    "nemo_rl/__init__.py": "",
+    "nemo_rl/distributed/__init__.py": "",
+    "nemo_rl/distributed/model_utils.py": "\n".join(
+        f"def {n}(*a, **k):\n    return 'reference'" for n in (
+            "from_parallel_logits_to_logprobs", "from_parallel_logits_to_logprobs_packed_sequences",
+            "from_parallel_hidden_states_to_logprobs", "get_next_token_logprobs_from_logits",
+            "dtensor_from_parallel_logits_to_logprobs", "get_logprobs_from_vocab_parallel_logits",
+            "get_distillation_topk_logprobs_from_logits", "_compute_distributed_log_softmax",
+            "_compute_distributed_log_softmax_with_grad", "allgather_cp_sharded_tensor")
+    ) + "\n" + "\n".join(
+        f"class {n}:\n    origin = 'reference'" for n in (
+            "DistributedLogprob", "ChunkedDistributedLogprob", "DistributedLogprobWithSampling",
+            "ChunkedDistributedLogprobWithSampling", "ChunkedDistributedHiddenStatesToLogprobs",
+            "ChunkedDistributedEntropy", "ChunkedDistributedGatherLogprob", "DistributedCrossEntropy")
+    ) + "\n",
+    "nemo_rl/algorithms/__init__.py": "",
+    "nemo_rl/algorithms/utils.py": "\n".join(
+        f"def {n}(*a, **k):\n    return 'reference'" for n in (
+            "calculate_kl", "masked_mean", "calculate_baseline_and_std_per_prompt", "mask_out_neg_inf_logprobs",
+            "set_seed")) + "\n",
+    "nemo_rl/algorithms/logits_sampling_utils.py": (
+        "class TrainingSamplingParams:\n    pass\n"
+        "def need_top_k_or_top_p_filtering(p):\n    return False\n"
+        "def apply_top_k_top_p(*a, **k):\n    return 'reference'\n"),
+    "nemo_rl/algorithms/advantage_estimator.py": (
+        "from nemo_rl.algorithms.utils import calculate_baseline_and_std_per_prompt\n"
+        "class GRPOAdvantageEstimator:\n    origin = 'reference'\n"
+        "class ReinforcePlusPlusAdvantageEstimator:\n    origin = 'reference'\n"),
+    "nemo_rl/algorithms/loss/__init__.py": (
+        "from nemo_rl.algorithms.loss.loss_functions import (\n"
+        "    ClippedPGLossConfig, ClippedPGLossFn, DistillationLossFn, DPOLossFn, DraftCrossEntropyLossFn,\n"
+        "    MseValueLossFn, NLLLossFn, PreferenceLossFn)\n"
+        "from nemo_rl.algorithms.loss.utils import prepare_loss_input, prepare_packed_loss_input\n"
+        "from nemo_rl.algorithms.loss.wrapper import (\n"
+        "    SequencePackingFusionLossWrapper, SequencePackingLossWrapper, wrap_loss_fn_with_input_preparation)\n"),
+    "nemo_rl/algorithms/loss/interfaces.py": (
+        "import enum\n"
+        "class LossType(enum.Enum):\n    TOKEN_LEVEL = 'token_level'\n    SEQUENCE_LEVEL = 'sequence_level'\n"
+        "class MetricNormalizer(enum.Enum):\n    TOKENS = 'tokens'\n    SEQUENCES = 'sequences'\n    NONE = 'none'\n"
+        "class LossInputType(enum.Enum):\n    LOGIT = 'logit'\n    LOGPROB = 'logprob'\n"
+        "    DISTILLATION = 'distillation'\n    DISTILLATION_CROSS_TOKENIZER = 'distillation_cross_tokenizer'\n"
+        "    DRAFT = 'draft'\n"
+        "class LossFunction:\n    pass\n"),
+    "nemo_rl/algorithms/loss/loss_functions.py": (
+        "from nemo_rl.algorithms.loss.interfaces import LossFunction, LossInputType, LossType\n"
+        "from nemo_rl.algorithms.utils import calculate_kl, masked_mean\n"
+        "ClippedPGLossConfig = dict\n"
+        + "".join(f"class {n}(LossFunction):\n    origin = 'reference'\n    input_type = LossInputType.LOGPROB\n"
+                  f"    def __init__(self, *a, **k):\n        self.loss_type = LossType.TOKEN_LEVEL\n"
+                  for n in ("ClippedPGLossFn", "NLLLossFn", "PreferenceLossFn", "DPOLossFn", "DistillationLossFn",
+                            "DraftCrossEntropyLossFn"))
+        + "class MseValueLossFn(LossFunction):\n    def __call__(self, *a):\n        return masked_mean(*a)\n"),
+    "nemo_rl/algorithms/loss/utils.py": (
+        "from nemo_rl.distributed.model_utils import (\n"
+        "    from_parallel_logits_to_logprobs_packed_sequences, get_next_token_logprobs_from_logits)\n"
+        "def prepare_loss_input(*a, **k):\n    return 'reference'\n"
+        "def prepare_packed_loss_input(*a, **k):\n    return 'reference'\n"),
+    "nemo_rl/algorithms/loss/wrapper.py": (
+        "def wrap_loss_fn_with_input_preparation(*a, **k):\n    return 'reference'\n"
+        "class SequencePackingLossWrapper:\n    origin = 'reference'\n"
+        "class SequencePackingFusionLossWrapper:\n    origin = 'reference'\n"),
+    "nemo_rl/algorithms/grpo.py": (
+        "from nemo_rl.algorithms.advantage_estimator import GRPOAdvantageEstimator, ReinforcePlusPlusAdvantageEstimator\n"
+        "from nemo_rl.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn\n"
+        "from nemo_rl.algorithms.loss.interfaces import LossFunction\n"
+        "from nemo_rl.algorithms.utils import calculate_baseline_and_std_per_prompt, set_seed\n"
+        "def dynamic_sampling(*a, **k):\n    return 'reference'\n"
+        "def compute_and_apply_seq_logprob_error_masking(*a, **k):\n    return 'reference'\n"
+        "def setup(cfg):\n    return ClippedPGLossFn(cfg)\n"),
+    "nemo_rl/models/__init__.py": "",
+    "nemo_rl/models/automodel/__init__.py": "",
+    "nemo_rl/models/automodel/data.py": (
+        "from nemo_rl.algorithms.loss.interfaces import LossType\n"
+        "def normalises_by_tokens(loss_fn):\n"
+        "    return hasattr(loss_fn, 'loss_type') and loss_fn.loss_type == LossType.TOKEN_LEVEL\n"),
+    "nemo_rl/models/automodel/train.py": (
+        "from nemo_rl.algorithms.logits_sampling_utils import TrainingSamplingParams, apply_top_k_top_p\n"
+        "from nemo_rl.algorithms.loss import SequencePackingLossWrapper, prepare_loss_input\n"
+        "from nemo_rl.algorithms.utils import mask_out_neg_inf_logprobs\n"
+        "from nemo_rl.distributed.model_utils import allgather_cp_sharded_tensor, get_logprobs_from_vocab_parallel_logits\n"
+        "def apply_temperature_scaling(*a, **k):\n    return 'reference'\n"
+        "class LossPostProcessor:\n    origin = 'reference'\n"
+        "class LogprobsPostProcessor:\n    origin = 'reference'\n"
+        "def is_loss_step(fn):\n    return isinstance(fn, LossPostProcessor)\n"),
+    "nemo_rl/models/megatron/__init__.py": "",
+    "nemo_rl/models/megatron/train.py": (
+        "from megatron.core.models.gpt import GPTModel\n"
+        "from nemo_rl.algorithms.loss import wrap_loss_fn_with_input_preparation\n"),
+    "driver_script.py": (
+        "from nemo_rl.algorithms.loss import ClippedPGLossFn\n"
+        "from nemo_rl.algorithms.utils import masked_mean\n"),
+}
+
+
+def write_stub_install(tmp_path) -> str:
+    """Writes the stand-in install under ``tmp_path`` and returns the ``PYTHONPATH`` a child process needs to
+    import it next to this repository."""
+    for rel, text in _STUB_INSTALL.items():
+        path = tmp_path / rel
+        path.parent.mkdir(parents=True, exist_ok=True)
+        path.write_text(text)
+    here = os.path.dirname(os.path.abspath(__file__))
+    return os.pathsep.join([str(tmp_path), os.path.dirname(here), here])

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import rl_amd
-from helpers import load_golden
+from helpers import load_golden, write_stub_install
 from oracle import logprob as OL
 from rl_amd.algorithms.loss import (
     ClippedPGLossConfig,
@@ -145,3 +145,88 @@ def test_lazy_metrics_fetches_once_on_first_use_and_behaves_like_the_dictionary(
         import json
 
         json.dumps(LazyMetrics(build))
+
+
+_STUB_CHECK = r"""
+import json, sys
+import driver_script
+import nemo_rl.algorithms.grpo as grpo
+import nemo_rl.algorithms.loss as pkg
+import nemo_rl.algorithms.loss.loss_functions as lf
+import nemo_rl.algorithms.loss.interfaces as itf
+import nemo_rl.models.automodel.train as train
+import nemo_rl.models.automodel.data as data
+import nemo_rl.algorithms.advantage_estimator as ae
+import rl_amd
+from rl_amd import compat
+
+mode = rl_amd.install()
+again = rl_amd.install()
+import rl_amd.algorithms.loss as mine
+import rl_amd.algorithms.utils as mu
+import rl_amd.algorithms.advantage_estimator as mae
+import rl_amd.models.automodel.train as mtrain
+import nemo_rl.algorithms.loss_functions as short
+
+fn = grpo.setup({"token_level_loss": True})
+seq = pkg.ClippedPGLossFn({"token_level_loss": False})
+out = {
+    "mode": [mode, again],
+    "skipped": compat.skipped_modules(),
+    "pkg.ClippedPGLossFn": pkg.ClippedPGLossFn is mine.ClippedPGLossFn,
+    "lf.ClippedPGLossFn": lf.ClippedPGLossFn is mine.ClippedPGLossFn,
+    "grpo.ClippedPGLossFn": grpo.ClippedPGLossFn is mine.ClippedPGLossFn,
+    "short.ClippedPGLossFn": short.ClippedPGLossFn is mine.ClippedPGLossFn,
+    "script.ClippedPGLossFn": driver_script.ClippedPGLossFn is mine.ClippedPGLossFn,
+    "script.masked_mean": driver_script.masked_mean is mu.masked_mean,
+    "grpo.GRPOAdvantageEstimator": grpo.GRPOAdvantageEstimator is mae.GRPOAdvantageEstimator,
+    "grpo.baseline": grpo.calculate_baseline_and_std_per_prompt is mu.calculate_baseline_and_std_per_prompt,
+    "ae.baseline": ae.calculate_baseline_and_std_per_prompt is mu.calculate_baseline_and_std_per_prompt,
+    "grpo.untouched": grpo.ReinforcePlusPlusAdvantageEstimator.origin == "reference" and grpo.set_seed() == "reference",
+    "grpo.dynamic_sampling": grpo.dynamic_sampling.__module__.startswith("rl_amd."),
+    "pkg.prepare_loss_input": pkg.prepare_loss_input is mine.prepare_loss_input,
+    "pkg.wrap": pkg.wrap_loss_fn_with_input_preparation is mine.wrap_loss_fn_with_input_preparation,
+    "pkg.fusion_wrapper": pkg.SequencePackingFusionLossWrapper is mine.SequencePackingFusionLossWrapper,
+    "train.prepare_loss_input": train.prepare_loss_input is mine.prepare_loss_input,
+    "train.SequencePackingLossWrapper": train.SequencePackingLossWrapper is mine.SequencePackingLossWrapper,
+    "train.apply_top_k_top_p": train.apply_top_k_top_p.__module__.startswith("rl_amd."),
+    "train.mask_out": train.mask_out_neg_inf_logprobs is mu.mask_out_neg_inf_logprobs,
+    "train.LossPostProcessor": train.LossPostProcessor is mtrain.LossPostProcessor,
+    "train.isinstance": train.is_loss_step(object.__new__(mtrain.LossPostProcessor)),
+    "train.get_logprobs": train.get_logprobs_from_vocab_parallel_logits.__module__.startswith("rl_amd."),
+    "train.untouched": train.allgather_cp_sharded_tensor() == "reference",
+    "lf.calculate_kl": lf.calculate_kl is mu.calculate_kl,
+    "lf.masked_mean": lf.masked_mean is mu.masked_mean,
+    "driver builds ours": type(fn) is mine.ClippedPGLossFn,
+    "enum.loss_type": fn.loss_type is itf.LossType.TOKEN_LEVEL and seq.loss_type is itf.LossType.SEQUENCE_LEVEL,
+    "enum.input_type": fn.input_type is itf.LossInputType.LOGPROB
+                       and mine.DistillationLossFn.input_type is itf.LossInputType.DISTILLATION,
+    "enum.normalizer": fn.metric_normalizations["loss"] is itf.MetricNormalizer.TOKENS
+                       and fn.metric_normalizations["num_valid_samples"] is itf.MetricNormalizer.NONE,
+    "enum.compare outside": data.normalises_by_tokens(fn) and not data.normalises_by_tokens(seq),
+    "enum.exports": mine.LossType is itf.LossType and mine.MetricNormalizer is itf.MetricNormalizer,
+    "fusable but for the logits": mine.why_not_fusable(fn, None, {}) == "logits are not a [B, S, V] GPU tensor",
+}
+print("RESULT " + json.dumps(out))
+"""
+
+
+def _run_against_stub_install(tmp_path):
+    import json
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, PYTHONPATH=write_stub_install(tmp_path))
+    done = subprocess.run([sys.executable, "-c", _STUB_CHECK], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-3000:]
+    line = [l for l in done.stdout.splitlines() if l.startswith("RESULT ")][-1]
+    return json.loads(line[len("RESULT "):])
+
+
+def test_install_rebinds_an_existing_install_by_identity(tmp_path):
+    got = _run_against_stub_install(tmp_path)
+    assert got.pop("mode") == ["patched", "patched"]
+    assert got.pop("skipped") == ["nemo_rl.models.megatron.train"]      # Megatron-Core is not installed
+    wrong = [k for k, v in got.items() if v is not True]
+    assert not wrong, wrong
