@@ -181,7 +181,8 @@ int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, 
  * and -1 as the number for every other row.  A backward given the record back and a dlogits that is one contiguous,
  * 16-byte aligned block (d_stride_inner == vocab, d_stride_outer == d_n_inner * vocab) zero-fills that block and
  * writes only those few entries of a recorded row, without reading the logits; other rows stream as without the
- * record, and so does everything for a strided dlogits. */
+ * record, and so does everything for a strided dlogits.  dlogits may alias the logits (in place, same strides);
+ * a dlogits block that overlaps the logits is never cleared first, every row then streams. */
 int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr, const int32_t* tie,
                               const float* lse_kept, const float* grad, int64_t grad_stride_outer,
                               int64_t grad_stride_inner, const int32_t* kept_count, const int32_t* kept_index,

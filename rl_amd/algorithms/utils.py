@@ -17,6 +17,18 @@ from .. import ops as _ops  # noqa: F401
 _OPS = torch.ops.rl_amd
 
 
+def _install_original(name: str):
+    """The function of this name that an existing NeMo-RL install had before ``rl_amd.install()`` replaced it."""
+    from ..compat import original
+
+    return original("nemo_rl.algorithms.utils", name)
+
+
+def _host_only(*tensors) -> bool:
+    """Host tensors in a process that sees no GPU (the GRPO driver of a multi-node run)."""
+    return not torch.cuda.is_available() and all(t is None or not t.is_cuda for t in tensors)
+
+
 def _gpu_device() -> torch.device:
     if not torch.cuda.is_available():
         raise RuntimeError("rl_amd needs an MI355X: no GPU is visible and there is no CPU fallback")
@@ -75,6 +87,12 @@ def calculate_kl(
     if kl_type not in _KL_TYPES:
         raise ValueError(f"Invalid KL type: {kl_type}")
     tensors = [t for t in (logprobs, logprobs_reference, importance_sampling_weights) if t is not None]
+    theirs = _install_original("calculate_kl")
+    if theirs is not None and (_host_only(*tensors) or any(t.dtype == torch.float64 for t in tensors)):
+        # on an install: what the kernels do not cover (a driver process without a GPU, double precision)
+        # stays with the function the install came with
+        return theirs(logprobs, logprobs_reference, kl_type, input_clamp_value, output_clamp_value,
+                      importance_sampling_weights)
     out_dtype = tensors[0].dtype
     for t in tensors[1:]:
         out_dtype = torch.promote_types(out_dtype, t.dtype)
@@ -107,13 +125,21 @@ def masked_mean(
     """``sum(values * mask) / (norm + 1e-8)``, ``utils.py:207-224``, over everything (``dim=None``) or one axis: a
     row-reduction HIP kernel (sums carried in double) and its gradient kernel for ``values``.  The mask and the
     normalisation factor are constants of the gradient, as in every use the reference makes of this function."""
-    if dim is not None and not isinstance(dim, int):
-        raise NotImplementedError("masked_mean reduces over everything or over one axis")
     norm = global_normalization_factor
-    if mask.requires_grad or (isinstance(norm, torch.Tensor) and norm.requires_grad):
-        raise NotImplementedError("masked_mean differentiates with respect to the values only")
-    if isinstance(norm, torch.Tensor) and norm.numel() != 1:
-        raise NotImplementedError("the normalisation factor must be one value")
+    not_covered = None
+    if dim is not None and not isinstance(dim, int):
+        not_covered = "masked_mean reduces over everything or over one axis"
+    elif mask.requires_grad or (isinstance(norm, torch.Tensor) and norm.requires_grad):
+        not_covered = "masked_mean differentiates with respect to the values only"
+    elif isinstance(norm, torch.Tensor) and norm.numel() != 1:
+        not_covered = "the normalisation factor must be one value"
+    theirs = _install_original("masked_mean")
+    if theirs is not None and (not_covered or _host_only(values, mask) or values.dtype == torch.float64):
+        # on an install: argument forms no caller on the hot path uses, a driver process without a GPU and
+        # double precision stay with the function the install came with
+        return theirs(values, mask, dim, global_normalization_factor)
+    if not_covered:
+        raise NotImplementedError(not_covered)
     out_dtype = torch.promote_types(values.dtype, mask.dtype)
     if isinstance(norm, torch.Tensor):
         out_dtype = torch.promote_types(out_dtype, norm.dtype)
@@ -193,6 +219,9 @@ def calculate_baseline_and_std_per_prompt(
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """``utils.py:104-198``: per-prompt (leave-one-out) baseline and std; results come back on the
     device of ``rewards``.  Inputs that live on the host (the driver's default) are staged to the GPU."""
+    theirs = _install_original("calculate_baseline_and_std_per_prompt")
+    if theirs is not None and _host_only(prompts, rewards, valid_mask, std_rewards):
+        return theirs(prompts, rewards, valid_mask, leave_one_out_baseline, std_rewards)  # a driver without a GPU
     baseline, std, _, _ = _group_stats(prompts, rewards, valid_mask, leave_one_out_baseline, std_rewards, False)
     return baseline, std
 

@@ -86,12 +86,19 @@ _OPTIONAL = {"nemo_rl.models.megatron.train", "nemo_rl.models.automodel.train", 
 
 _ENUMS = ("LossType", "LossInputType", "MetricNormalizer")
 
-_state = {"originals": [], "skipped": [], "replacements": {}}
+_state = {"originals": [], "skipped": [], "replacements": {}, "by_name": {}}
 
 
 def skipped_modules() -> list[str]:
     """Modules of the install that the last ``install()`` could not import and therefore left alone."""
     return list(_state["skipped"])
+
+
+def original(module: str, name: str):
+    """What ``module.name`` was on the install before ``install()`` replaced it, or ``None`` (no install, or
+    not replaced).  The driver-side helpers hand the calls they do not cover (host tensors in a process
+    without a GPU, argument forms no caller on the hot path uses) back to it."""
+    return _state["by_name"].get((module, name))
 
 
 def _real_nemo_rl_present() -> bool:
@@ -177,6 +184,7 @@ def _patch_install() -> None:
             old = getattr(dst, name, None)
             if old is not None and old is not new and not _is_ours(getattr(old, "__module__", "") or ""):
                 replacements[id(old)] = (old, new)
+                _state["by_name"].setdefault((target, name), old)
             setattr(dst, name, new)
     _state["skipped"] = skipped
     # (the table references the originals, so their ids cannot be reused while it is in use)

@@ -1086,6 +1086,17 @@ extern "C" int nrl_topk_topp_logprob_bwd(const nrl_rows* rows, const float* thr,
     const int64_t elt = rows->dtype == NRL_F32 ? 4 : 2;
     a.prefilled = kept_count && d_stride_inner == rows->vocab && d_stride_outer == d_n_inner * rows->vocab &&
                   (reinterpret_cast<uintptr_t>(dlogits) & 15) == 0;
+    if (a.prefilled && rows->logits && rows->n_outer * rows->n_inner > 0) {
+        // A gradient written over the logits (allowed, as for nrl_logprob_bwd) must not be cleared first: rows that
+        // are not on record still stream from the logits.  Such a call takes the row-by-row path, which reads a
+        // vector before it overwrites it.
+        const uintptr_t d0 = reinterpret_cast<uintptr_t>(dlogits), d1 = d0 + static_cast<uintptr_t>(n * rows->vocab * elt);
+        const uintptr_t l0 = reinterpret_cast<uintptr_t>(rows->logits);
+        const int64_t so = rows->stride_outer < 0 ? -rows->stride_outer : rows->stride_outer;
+        const int64_t si = rows->stride_inner < 0 ? -rows->stride_inner : rows->stride_inner;
+        const uintptr_t l1 = l0 + static_cast<uintptr_t>(((rows->n_outer - 1) * so + (rows->n_inner - 1) * si + rows->vocab) * elt);
+        if (d0 < l1 && l0 < d1) a.prefilled = 0;
+    }
     if (a.prefilled) fill_zero_flat_kernel<<<dim3(kFillGrid), dim3(256), 0, s>>>(static_cast<char*>(dlogits), n * rows->vocab * elt);
     NRL_SEL_DISPATCH(rows->dtype, tc, topk_topp_stream_kernel<DT, TEMP, 0><<<dim3((unsigned)n), dim3(kSelBlock), 0, s>>>(a, n));
     return check_launch("topk_topp_logprob_bwd");

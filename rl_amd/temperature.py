@@ -10,7 +10,7 @@ That pass costs a full read + write of ``[B, S, V]``.  The logprob kernels can a
 with the same rounding of value and gradient, while they stream the row anyway.  Because nothing in
 the tensor itself can say "not divided yet" without risking a silently unscaled read elsewhere, that is
 an explicit opt-in: inside ``with deferred_temperature():`` ``apply_temperature_scaling`` leaves the
-memory alone and records (storage, T) for the calling thread; the logprob / loss entry points of this
+memory alone and records (storage object, T) for the calling thread, for as long as that storage lives; the logprob / loss entry points of this
 package look the logits they are handed up in that record (views of the recorded tensor share its
 storage) and divide inside their kernels.  Whoever opens the context promises that, until it closes,
 only those entry points read the logits.
@@ -23,7 +23,7 @@ from typing import Any, Optional
 import torch
 
 from . import ops  # noqa: F401  (registers torch.ops.rl_amd)
-from ._deferred import _state, deferred_temperature, pending_temperature  # noqa: F401
+from ._deferred import _state, deferred_temperature, pending_temperature, record_temperature  # noqa: F401
 
 _OPS = torch.ops.rl_amd
 
@@ -61,7 +61,7 @@ def apply_temperature_scaling(logits: torch.Tensor, sampling_params: Optional[An
     if getattr(_state, "depth", 0) > 0:
         if not logits.is_cuda:
             raise RuntimeError("deferred_temperature() needs GPU logits")
-        _state.pending.append((logits.untyped_storage().data_ptr(), t))
+        record_temperature(logits, t)
         return logits
     if not logits.is_cuda:
         raise RuntimeError("rl_amd runs on the GPU only (got CPU logits); there is no CPU fallback")

@@ -411,3 +411,42 @@ def test_record_entries_outside_their_ranges_are_not_followed():
     want = streamed.clone()
     want[1, 3, skipped] = 0.0
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype,vocab", [(torch.bfloat16, 4096), (torch.float32, 2003)])
+def test_record_backward_written_over_the_logits(dtype, vocab):
+    """``dlogits`` may alias the logits, as for ``nrl_logprob_bwd``.  With the kept-set record the out-of-place call
+    clears the gradient block first and only adds the entries; over the logits that would destroy the rows that are
+    not on record (an all-tied row, a flat row) before they are streamed, so such a call must not clear: the in-place
+    result equals the out-of-place one bit for bit."""
+    import ctypes as C
+
+    from rl_amd import _lib
+    from rl_amd._lib import NRL_TEMP_RCP
+    from rl_amd.ops import _ptr, _rows, _stream
+
+    g = torch.Generator().manual_seed(vocab)
+    b, s, cap = 3, 9, 64
+    logits = (torch.randn(b, s, vocab, generator=g) * 3.0).to(dtype)
+    logits[1, 2] = 0.5                      # every id tied: not on record
+    logits[2, 4] = (torch.randn(vocab, generator=g) * 0.01).to(dtype)   # flat under top-p: not on record
+    ids = torch.randint(0, vocab, (b, s), generator=g)
+    ids[:, 1:] = torch.where(torch.rand(b, s - 1, generator=g) < 0.7, logits.float().argmax(-1)[:, :-1], ids[:, 1:])
+    up = torch.randn(b, s - 1, generator=g)
+    up[0, 3] = 0.0
+    n = s - 1
+    x, t, u = logits.to(DEV), ids[:, 1:].contiguous().to(DEV), up.to(DEV)
+    ops = torch.ops.rl_amd
+    _, thr, tie, lse, _, cnt, idx, val = ops.topk_topp_logprob_fwd_rec(x, t, n, 20, 0.95, 1.0, NRL_TEMP_RCP, False, cap)
+    assert int(cnt[1, 2]) == -1 and int(cnt[0, 0]) >= 1
+    want = ops.topk_topp_logprob_bwd(x, t, thr, tie, lse, u, n, 1.0, NRL_TEMP_RCP, cnt, idx, val)
+    over = x.clone()
+    rows = _rows(over, t, n, 0, vocab, 1.0, NRL_TEMP_RCP)
+    with torch.cuda.device(over.device):
+        code = _lib.load().nrl_topk_topp_logprob_bwd(
+            C.byref(rows), _ptr(thr), _ptr(tie), _ptr(lse), _ptr(u), u.stride(0), u.stride(1),
+            _ptr(cnt), _ptr(idx), _ptr(val), cap, _ptr(over), s, over.stride(0), over.stride(1), _stream())
+    _lib.check(code, "nrl_topk_topp_logprob_bwd")
+    torch.cuda.synchronize()
+    bits = torch.int16 if dtype != torch.float32 else torch.int32
+    assert torch.equal(over.view(bits), want.view(bits))

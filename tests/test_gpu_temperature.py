@@ -198,7 +198,8 @@ def test_deferred_temperature_matches_the_eager_divide(dtype):
         out = apply_temperature_scaling(hidden, params)
         assert out is hidden and torch.equal(hidden.detach(), keep)
         assert pending_temperature(hidden) == T and pending_temperature(hidden[:, :-1]) == T
-        assert pending_temperature(leaf_d) == 1.0
+        with pytest.raises(RuntimeError, match="not on record"):   # same width, never went through the function
+            pending_temperature(leaf_d)
         deferred = get_next_token_logprobs_from_logits(ids.to(DEV), out)
         sliced = get_next_token_logprobs_from_logits(ids[:, :5].to(DEV), out[:, :5])
         with pytest.raises(RuntimeError, match="deferred"):
@@ -236,3 +237,28 @@ def test_deferred_temperature_matches_the_eager_divide(dtype):
     l2.backward()
     assert abs(l1.item() - l2.item()) <= 1e-6 * abs(l1.item()) + 1e-7
     _check_twice_rounded(leaf_2.grad, leaf_1.grad.cpu(), dtype)
+
+
+def test_a_recycled_address_is_not_divided():
+    """The record of a deferred divide ends with the storage it was made for: a tensor that the caching
+    allocator places at the address of freed deferred logits has no temperature and its logprobs are those of
+    the undivided values."""
+    from rl_amd.distributed.model_utils import get_next_token_logprobs_from_logits
+
+    vocab = 4096
+    logits, ids, _ = _inputs(torch.bfloat16, vocab, 63, 2, 8)
+    params = TrainingSamplingParams(top_k=None, top_p=1.0, temperature=T)
+    plain = get_next_token_logprobs_from_logits(ids.to(DEV), logits.to(DEV))
+    with deferred_temperature():
+        a = apply_temperature_scaling(logits.to(DEV), params)
+        address = a.data_ptr()
+        assert pending_temperature(a) == T
+        divided = get_next_token_logprobs_from_logits(ids.to(DEV), a)
+        torch.cuda.synchronize()
+        del a
+        b = torch.empty_like(logits, device=DEV)          # same size: the allocator hands the freed block back
+        b.copy_(logits)
+        assert b.data_ptr() == address, "the allocator did not reuse the block; the test needs it to"
+        assert pending_temperature(b) == 1.0
+        again = get_next_token_logprobs_from_logits(ids.to(DEV), b)
+    assert torch.equal(again, plain) and not torch.equal(divided, plain)

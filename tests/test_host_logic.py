@@ -149,6 +149,7 @@ def test_lazy_metrics_fetches_once_on_first_use_and_behaves_like_the_dictionary(
 
 _STUB_CHECK = r"""
 import json, sys
+import torch
 import driver_script
 import nemo_rl.algorithms.grpo as grpo
 import nemo_rl.algorithms.loss as pkg
@@ -205,6 +206,12 @@ out = {
                        and fn.metric_normalizations["num_valid_samples"] is itf.MetricNormalizer.NONE,
     "enum.compare outside": data.normalises_by_tokens(fn) and not data.normalises_by_tokens(seq),
     "enum.exports": mine.LossType is itf.LossType and mine.MetricNormalizer is itf.MetricNormalizer,
+    "uncovered forms go to the install": mu.masked_mean(torch.ones(2, 3), torch.ones(2, 3), (0, 1)) == "reference"
+                                         and mu.masked_mean(torch.ones(3, dtype=torch.float64), torch.ones(3)) == "reference",
+    "driver without a GPU": torch.cuda.is_available() or (
+        mu.masked_mean(torch.ones(3), torch.ones(3)) == "reference"
+        and mu.calculate_kl(torch.zeros(3), torch.zeros(3)) == "reference"
+        and mu.calculate_baseline_and_std_per_prompt(torch.zeros(2, 2, dtype=torch.long), torch.zeros(2), torch.ones(2)) == "reference"),
     "fusable but for the logits": mine.why_not_fusable(fn, None, {}) == "logits are not a [B, S, V] GPU tensor",
 }
 print("RESULT " + json.dumps(out))
@@ -230,3 +237,31 @@ def test_install_rebinds_an_existing_install_by_identity(tmp_path):
     assert got.pop("skipped") == ["nemo_rl.models.megatron.train"]      # Megatron-Core is not installed
     wrong = [k for k, v in got.items() if v is not True]
     assert not wrong, wrong
+
+
+def test_deferred_temperature_record_dies_with_its_storage_and_refuses_copies():
+    import numpy as np
+
+    from rl_amd._deferred import deferred_temperature, pending_temperature, record_temperature
+
+    block = np.zeros(4 * 6 * 32, dtype=np.float32)              # one piece of memory, two storages in turn
+    with deferred_temperature():
+        a = torch.from_numpy(block).view(4, 6, 32)
+        record_temperature(a, 0.7)
+        assert pending_temperature(a) == 0.7 and pending_temperature(a[:, :-1]) == 0.7
+        assert pending_temperature(a.detach().view(24, 32)) == 0.7
+        with pytest.raises(RuntimeError, match="not on record"):
+            pending_temperature(a.clone())                      # a copy carries undivided values
+        assert pending_temperature(a.double()) == 1.0           # another dtype / width is somebody else's tensor
+        assert pending_temperature(torch.zeros(4, 6, 16)) == 1.0
+        view = a[1]
+        del a                                                   # the storage lives on through the view
+        assert pending_temperature(view) == 0.7
+        address = view.untyped_storage().data_ptr()
+        del view                                                # now it is gone, and its record with it
+        b = torch.from_numpy(block).view(4, 6, 32)              # a new storage at the same address
+        assert b.untyped_storage().data_ptr() == address
+        assert pending_temperature(b) == 1.0
+        record_temperature(b, 0.5)
+        assert pending_temperature(b) == 0.5
+    assert pending_temperature(b) == 1.0

@@ -68,10 +68,13 @@ def _run_pair(lib, batch, sm1, seed, token_level, dev):
     ws_bytes = lib.nrl_grpo_loss_workspace_bytes(batch)
     ws = torch.empty(ws_bytes // 8, dtype=torch.float64, device=dev)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # free bytes of the device as the driver reports them: unlike torch's own counters this also sees a hipMalloc
+    # made inside the library (the first call on a device, which resolves the array's address, came before)
+    before = torch.cuda.mem_get_info()[0]
     code = lib.nrl_grpo_loss_fwd_bwd_static(C.byref(cfg), C.byref(inp), _ptr(loss_s), _ptr(dlp_s), None, _ptr(met_s), stream)
     _lib.check(code, "nrl_grpo_loss_fwd_bwd_static")
-    assert torch.cuda.memory_allocated() == before
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == before
     code = lib.nrl_grpo_loss_fwd_bwd(C.byref(cfg), C.byref(inp), _ptr(loss_w), _ptr(dlp_w), None, _ptr(met_w),
                                      _ptr(ws), ws_bytes, stream)
     _lib.check(code, "nrl_grpo_loss_fwd_bwd")
@@ -83,14 +86,56 @@ def _run_pair(lib, batch, sm1, seed, token_level, dev):
     return loss_s.item()
 
 
+def _warm_up(lib, dev):
+    """The first call on a device resolves the address of the library's array (and loads its code object)."""
+    t = _inputs(2, 3, 1, dev)
+    cfg, inp = _structs(t, 2, 3, True)
+    loss, dlp, met = _outputs(2, 3, dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.nrl_grpo_loss_fwd_bwd_static(C.byref(cfg), C.byref(inp), _ptr(loss), _ptr(dlp), None, _ptr(met), stream),
+               "nrl_grpo_loss_fwd_bwd_static")
+    torch.cuda.synchronize()
+
+
 def test_static_scratch_entry_point_matches_the_workspace_one_on_two_calls_in_a_row():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     with torch.cuda.device(dev):
+        _warm_up(lib, dev)
         first = _run_pair(lib, 192, 511, seed=11, token_level=False, dev=dev)
         second = _run_pair(lib, 24, 200, seed=12, token_level=False, dev=dev)   # smaller: stale rows 24..191 stay behind
         third = _run_pair(lib, 7, 33, seed=13, token_level=True, dev=dev)
     assert len({first, second, third}) == 3
+
+
+def test_static_scratch_calls_back_to_back_on_one_stream_without_a_host_wait():
+    """Calls in stream order share the array safely: a large batch immediately followed by a smaller one, no
+    synchronisation in between, each bit-equal to the workspace entry point on the same inputs."""
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    with torch.cuda.device(dev):
+        _warm_up(lib, dev)
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        cases = []
+        for batch, sm1, seed in ((4096, 257, 21), (40, 129, 22), (1, 5, 23)):
+            t = _inputs(batch, sm1, seed, dev)
+            cfg, inp = _structs(t, batch, sm1, False)
+            ws_bytes = lib.nrl_grpo_loss_workspace_bytes(batch)
+            ws = torch.empty(ws_bytes // 8, dtype=torch.float64, device=dev)
+            cases.append((t, cfg, inp, _outputs(batch, sm1, dev), _outputs(batch, sm1, dev), ws, ws_bytes))
+        torch.cuda.synchronize()
+        free = torch.cuda.mem_get_info()[0]
+        for t, cfg, inp, (loss_s, dlp_s, met_s), _, _, _ in cases:          # nothing but launches in between
+            _lib.check(lib.nrl_grpo_loss_fwd_bwd_static(C.byref(cfg), C.byref(inp), _ptr(loss_s), _ptr(dlp_s), None,
+                                                        _ptr(met_s), stream), "nrl_grpo_loss_fwd_bwd_static")
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free
+        for t, cfg, inp, (loss_s, dlp_s, met_s), (loss_w, dlp_w, met_w), ws, ws_bytes in cases:
+            _lib.check(lib.nrl_grpo_loss_fwd_bwd(C.byref(cfg), C.byref(inp), _ptr(loss_w), _ptr(dlp_w), None, _ptr(met_w),
+                                                 _ptr(ws), ws_bytes, stream), "nrl_grpo_loss_fwd_bwd")
+            torch.cuda.synchronize()
+            assert torch.isfinite(loss_s).all()
+            assert torch.equal(loss_s, loss_w) and torch.equal(dlp_s, dlp_w) and torch.equal(met_s, met_w)
 
 
 def test_static_scratch_entry_point_rejects_a_batch_beyond_its_array():
