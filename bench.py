@@ -358,6 +358,57 @@ def copy_bandwidth(torch, dev):
     return 2 * (1 << 32) / (ms * 1e-3) / 1e9
 
 
+def read_write_ceiling(torch, logits, ids, read_bytes, write_bytes):
+    """What this device delivers to the two halves of a gradient kernel taken apart, on the bench's own buffers:
+    a pure read of the logits (the forward logprob kernel, K1) and a pure write of a gradient buffer of the same
+    shape (the backward logprob kernel with every upstream gradient zero: rows are zero-filled, nothing is read).
+    ``mixed_bound_ms`` = the launch's read bytes at the read rate plus its written bytes at the write rate: the time
+    a read + write kernel of that launch would take if the two streams did not disturb each other."""
+    ops = torch.ops.rl_amd
+    b, s, v = logits.shape
+    elt = logits.element_size()
+    n = s - 1
+    targets = ids[:, 1:]
+
+    def ms_of(fn, reps=3):
+        fn()
+        torch.cuda.synchronize()
+        a, z = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        z.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(z) / reps
+
+    with torch.no_grad():
+        lse = torch.zeros((b, n), dtype=torch.float32, device=logits.device)
+        zero = torch.zeros((b, n), dtype=torch.float32, device=logits.device)
+        read_ms = ms_of(lambda: ops.logprob_fwd(logits, targets, n, 0, v, 1.0, 1, False))
+        write_ms = ms_of(lambda: ops.logprob_bwd(logits, targets, lse, zero, n, 0, v, 1.0, 1))
+    read_gbs = b * n * v * elt / (read_ms * 1e-3) / 1e9
+    write_gbs = b * s * v * elt / (write_ms * 1e-3) / 1e9
+    torch.cuda.empty_cache()
+    return {"read_bandwidth_GBps": read_gbs, "write_bandwidth_GBps": write_gbs,
+            "mixed_bound_ms": (read_bytes / read_gbs + write_bytes / write_gbs) / 1e6,
+            "mixed_bound_bytes": {"read": read_bytes, "written": write_bytes}}
+
+
+def worker_scaling(metrics, num_global_batches=1):
+    """What the DTensor worker does with the metrics of a microbatch between the loss call and ``backward()``
+    (``nemo_rl/models/automodel/train.py:525-533``)."""
+    for k in metrics.keys():
+        if "_min" in k or "_max" in k:
+            continue
+        metrics[k] /= num_global_batches
+    return metrics
+
+
+def read_metrics(collected):
+    """The worker's look at the metrics of its microbatches after the step: every value of every record."""
+    return [dict(m.items()) for m in collected]
+
+
 def finish(result, args, torch, w, kind, cpu_rows, gpu_rows):
     """Adds the baseline legs to a workload's record and prints the one JSON line."""
     if not args.no_cpu_baseline:
@@ -380,9 +431,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
 
 def bench_topk(args, torch, w):
     """Config 4: temperature 0.7 + top-k / top-p filtered training logprobs -> DAPO loss -> dlogits (K3 forward +
-    backward).  The temperature divide is inside the timed region, as in the worker
-    (``apply_temperature_scaling`` on the model's output), left to the kernels by ``deferred_temperature()``: no
-    extra pass over the logits."""
+    backward).  The temperature divide is inside the timed region, as in the worker (``apply_temperature_scaling``
+    on the model's output).  Headline: the call sequence with no switch of this package set (an in-place divide pass,
+    the -inf warning printed at once); the opt-in variants (``deferred_temperature()``, ``DEFER_NEG_INF_WARNING``)
+    are rows of their own."""
     from functools import partial
 
     from rl_amd import ops
@@ -399,11 +451,10 @@ def bench_topk(args, torch, w):
     n_mb = (w["seqs"] + w["mb_seqs"] - 1) // w["mb_seqs"]
     mb_bytes = w["mb_seqs"] * w["seq_len"] * w["vocab"] * 2
     free, _ = torch.cuda.mem_get_info()
-    n_buf = max(1, min(n_mb, int((free * 0.9 - mb_bytes * 1.5) // mb_bytes)))
+    n_buf = max(1, min(n_mb, int((free * 0.9 - mb_bytes * 2.6) // mb_bytes)))
     params = TrainingSamplingParams(top_k=w["top_k"], top_p=w["top_p"], temperature=w["temperature"])
     prepare = partial(prepare_loss_input, sampling_params=params)  # as the DTensor worker binds it
     fn = ClippedPGLossFn(ClippedPGLossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0))
-    fn.lazy_metrics = True  # metric records are fetched when read, not once per microbatch
     mbs = []
     for i in range(n_buf):
         m = make_microbatch(torch, dict(w, spike_p=0.0), w["mb_seqs"], 4004 + i, dev)
@@ -422,24 +473,60 @@ def bench_topk(args, torch, w):
     tot_seqs = torch.tensor(float(w["seqs"]), device=dev)
     tot_toks = (sum(m["data"]["token_mask"][:, 1:].sum() for m in mbs) * (n_mb / n_buf)).float()
 
-    def step():
+    class _ModelOutput(torch.autograd.Function):
+        """Hands the resident logits buffer out as a non-leaf tensor, as a model's forward would: the worker's
+        in-place ``logits.div_(T)`` is only legal on such a tensor.  No copy; the gradient stops here."""
+
+        @staticmethod
+        def forward(ctx, buffer, anchor):
+            return buffer.detach()
+
+        @staticmethod
+        def backward(ctx, grad):
+            return None, grad.new_zeros(())
+
+    anchor = torch.zeros((), device=dev, requires_grad=True)
+    one = torch.ones((), device=dev)
+    restore_events = []
+
+    def step(defer=True):
+        collected = []
         for i in range(n_mb):
             m = mbs[i % n_buf]
-            leaf = m["logits"].requires_grad_(True)
-            with deferred_temperature():
-                logits = apply_temperature_scaling(leaf, params)
+            with (deferred_temperature() if defer else contextlib.nullcontext()):
+                out = _ModelOutput.apply(m["logits"], anchor)
+                logits = apply_temperature_scaling(out, params)     # eager: one in-place pass over [B, S, V]
                 loss_input, data = prepare(logits=logits, data=m["data"], loss_fn=fn)
-                loss, _ = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
-            (d,) = torch.autograd.grad(loss, leaf)
-            del d, loss, loss_input
+                loss, metrics = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+            collected.append(worker_scaling(metrics))
+            torch.autograd.grad(loss, anchor)
+            del loss, loss_input, logits, out
+            if not defer:
+                # Not part of the step: the bench keeps its logits resident, so after an in-place divide it multiplies
+                # them back (a worker gets fresh logits from its model).  Timed with events and taken off the clock.
+                a, z = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                torch.ops.rl_amd.scale_rows_(m["logits"], one, 1.0 / w["temperature"])
+                z.record()
+                restore_events.append((a, z))
+        read_metrics(collected)
 
-    # the warning about valid tokens whose logprob is -inf is printed when its counts have arrived (opt-in), as the
-    # metric records are; printed at once, as in the reference, it is its own row
+    def timed_eager():
+        """-> (seconds without the restoring passes, kernel summary)."""
+        restore_events.clear()
+        total, k = timed(torch, ops, args, lambda: step(defer=False))
+        restore_ms = sum(a.elapsed_time(z) for a, z in restore_events[-args.steps * n_mb:])
+        k.get("scale_rows", {}).pop("total_ms", None)
+        return total - restore_ms * 1e-3, k, restore_ms / (args.steps * n_mb)
+
+    # Opt-ins of this package, each its own row: the divide left to the kernels (deferred_temperature), and on top of
+    # that the warning about valid tokens whose logprob is -inf printed when its counts have arrived instead of
+    # before mask_out_neg_inf_logprobs returns.  The row without any of them is the headline.
     from rl_amd.algorithms import utils as AU
 
     AU.DEFER_NEG_INF_WARNING = True
     try:
-        elapsed, k = timed(torch, ops, args, step)
+        o_elapsed, ok_ = timed(torch, ops, args, step)
     finally:
         AU.DEFER_NEG_INF_WARNING = False
         AU.flush_neg_inf_warnings()
@@ -453,12 +540,20 @@ def bench_topk(args, torch, w):
         s_elapsed, sk = timed(torch, ops, args, step)
     finally:
         SL._record_capacity = record_capacity
+    # last, because the in-place divides and their restoring passes leave the logits a few roundings off
+    elapsed, k, restore_avg_ms = timed_eager()
     nan = dict(avg_ms=float("nan"))
     fwd, bwd = k.get("topk_topp_fwd", nan), k.get("topk_topp_bwd", nan)
     rows = w["mb_seqs"] * w["seq_len"]
     row_bytes = w["vocab"] * 2
     tokens = w["seqs"] * w["seq_len"]
     full = not args.seqs
+
+    def row(seconds, kernels, note):
+        return {"value": tokens * args.steps / seconds, "unit": "tokens/s", "ms_per_step": seconds / args.steps * 1e3,
+                "hbm_frac_end_to_end": 2 * row_bytes * tokens * args.steps / seconds / 1e9 / HBM_PEAK_GBS,
+                "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in kernels.items()}, "note": note}
+
     result = {
         "metric": "top-k/top-p filtered logprob + DAPO loss fwd/bwd tokens/s at V=151936; % of HBM peak",
         "value": tokens * args.steps / elapsed, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -466,8 +561,13 @@ def bench_topk(args, torch, w):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
-                   "temperature": "divided inside the timed region by the logprob kernels (deferred_temperature), bf16 rounding of a GPU div_",
-                   "neg_inf_warning": "printed when its counts have arrived (rl_amd.algorithms.utils.DEFER_NEG_INF_WARNING)"},
+                   "temperature": "apply_temperature_scaling as the worker calls it: one in-place pass over the logits "
+                                  "(bf16 rounding of a GPU div_) before the loss, one pass over the gradient in the backward",
+                   "neg_inf_warning": "printed before mask_out_neg_inf_logprobs returns (one wait per microbatch)",
+                   "metrics": "worker loop: metrics[k] /= num_global_batches after every loss call, every record read after "
+                              "the last microbatch; no rl_amd-specific switch is set",
+                   "clock": "wall clock of the steps minus the event-timed passes that multiply the resident logits back "
+                            "after each in-place divide (%.3f ms each; a worker's logits come fresh from its model)" % restore_avg_ms},
         # the forward reads a row once; the backward writes the gradient row (zeros and the <= 64 kept entries the
         # forward left on record) without reading the logits again
         "algorithmic_bytes_per_token": 2 * row_bytes,
@@ -476,17 +576,20 @@ def bench_topk(args, torch, w):
                                  bwd["avg_ms"], "c4" if full else None),
         "roofline_fwd": hbm_roofline("topk_topp_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
                                      "c4_fwd" if full else None),
+        "roofline_temperature": hbm_roofline("scale_rows_kernel (the eager divide and its backward; also the restoring pass)",
+                                             2 * row_bytes * rows, k.get("scale_rows", nan)["avg_ms"]),
         "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
-        "immediate_warning": {
-            "value": tokens * args.steps / w_elapsed, "unit": "tokens/s", "ms_per_step": w_elapsed / args.steps * 1e3,
-            "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in wk.items()},
-            "note": "mask_out_neg_inf_logprobs waits for its two counts and prints the warning before it returns, once per microbatch"},
+        "deferred_temperature": row(w_elapsed, wk, "with deferred_temperature(): the divide is applied by the kernels that read "
+                                                    "the logits, no pass of its own; warning printed at once"),
+        "deferred_temperature_and_warning": row(o_elapsed, ok_, "deferred_temperature() and DEFER_NEG_INF_WARNING: no pass for the "
+                                                                "divide, no wait for the warning's counts"),
         "streaming_backward": {
             "value": tokens * args.steps / s_elapsed, "unit": "tokens/s", "ms_per_step": s_elapsed / args.steps * 1e3,
             "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in sk.items()},
             "roofline": hbm_roofline("topk_topp_stream_kernel (backward reading the logits)", 2 * row_bytes * rows,
                                      sk.get("topk_topp_bwd", nan)["avg_ms"], "c4_streaming" if full else None),
-            "note": "without the kept-set record: the backward streams every live row again (3 x V bytes per token)"},
+            "note": "deferred_temperature(), without the kept-set record: the backward streams every live row again "
+                    "(3 x V bytes per token)"},
     }
     del mbs
     finish(result, args, torch, w, "topk", cpu_rows=256, gpu_rows=2048)
@@ -597,7 +700,6 @@ def bench_packed(args, torch, w):
     prefix = torch.randint(256, 1025, (nseq, 1), generator=g, device=dev)
     token_mask = ((torch.arange(smax, device=dev).unsqueeze(0) >= prefix) & in_seq).to(torch.int64)
     fn = ClippedPGLossFn(ClippedPGLossConfig(token_level_loss=False, reference_policy_kl_penalty=0.001))
-    fn.lazy_metrics = True  # metric records are fetched when read, not once per microbatch
     with torch.no_grad():
         targets = torch.cat([ids[i, : lens[i]].roll(-1) for i in range(nseq)]).unsqueeze(0)
         cur = from_parallel_logits_to_logprobs_packed_sequences(logits, targets, cu, smax, 0, v, None,
@@ -617,16 +719,20 @@ def bench_packed(args, torch, w):
 
     def step():
         x = logits.requires_grad_(True)
-        loss, _m = wrapped(x, data, gs, gt)
+        loss, metrics = wrapped(x, data, gs, gt)
+        worker_scaling(metrics)
         (d,) = torch.autograd.grad(loss, x)
         del d, loss
+        read_metrics([metrics])
 
     def three_pass_step():
         x = logits.requires_grad_(True)
         loss_input, prepared = prepare_packed_loss_input(x, data, fn, cu, cu)
-        loss, _m = fn(data=prepared, global_valid_seqs=gs, global_valid_toks=gt, **loss_input)
+        loss, metrics = fn(data=prepared, global_valid_seqs=gs, global_valid_toks=gt, **loss_input)
+        worker_scaling(metrics)
         (d,) = torch.autograd.grad(loss, x)
         del d, loss, loss_input
+        read_metrics([metrics])
 
     elapsed, km = timed(torch, ops, args, step)
     row_bytes = v * 2
@@ -678,14 +784,15 @@ def bench_lmhead(args, torch, w):
             "prev_logprobs": prev, "generation_logprobs": prev,
             "reference_policy_logprobs": cur + 0.05 * torch.randn((b, s), generator=g, device=dev)}
     fn = ClippedPGLossFn(ClippedPGLossConfig(), use_fused_linear_logprobs=True)
-    fn.lazy_metrics = True  # metric records are fetched when read, not once per microbatch
     gs, gt = torch.tensor(float(b), device=dev), tm[:, 1:].sum().float()
 
     def step():
         lp = from_parallel_hidden_states_to_logprobs(hidden, weight, False, ids, 0, v, None)
-        loss, _ = fn(next_token_logprobs=lp, data=data, global_valid_seqs=gs, global_valid_toks=gt)
+        loss, metrics = fn(next_token_logprobs=lp, data=data, global_valid_seqs=gs, global_valid_toks=gt)
+        worker_scaling(metrics)
         dh, dw = torch.autograd.grad(loss, (hidden, weight))
         del dh, dw
+        read_metrics([metrics])
 
     from rl_amd.distributed import model_utils as MU
 
@@ -785,9 +892,8 @@ def _main():
     torch.cuda.synchronize()
 
     fn = ClippedPGLossFn(ClippedPGLossConfig())  # eps 0.2/0.2, k3 KL beta 0.01, token-level mean
-    # the metrics record of every microbatch is fetched when it is read (here: never inside the step), the way a
-    # worker collects per-microbatch metrics and looks at them after the step; the eager default is its own row
-    fn.lazy_metrics = True
+    # No switch of this package is set: the step is the worker's loop -- loss, the per-metric division by the number
+    # of global batches, backward, per microbatch -- followed by one read of every microbatch's metrics.
     tot_seqs = torch.tensor(float(w["seqs"]), device=dev)
     tot_toks = sum((m["data"]["token_mask"][:, 1:].sum() for m in mbs)) * (n_mb / n_buf)
     tot_toks = tot_toks.float()
@@ -811,35 +917,44 @@ def _main():
     def step():
         # the drop-in call: logits + batch -> loss; dispatches to the single-pass kernel when the loss
         # configuration allows it (this one does), and autograd hands back d loss / d logits
+        collected = []
         for i in range(n_mb):
             m = mbs[i % n_buf]
             if grouped is not None:
                 m["data"]["advantages"] = grouped["estimator"].compute_advantage(grouped["prompts"], grouped["rewards"],
                                                                                  m["data"]["token_mask"])
             logits = m["logits"].requires_grad_(True)
-            loss, _metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare, 0, None, None)
+            loss, metrics = wrap_loss_fn_with_input_preparation(logits, m["data"], tot_seqs, tot_toks, fn, prepare, 0, None, None)
+            collected.append(worker_scaling(metrics))
             (dlogits,) = torch.autograd.grad(loss, logits)
             del dlogits, loss
+        read_metrics(collected)
 
     def three_pass_step():
         # the reference's call structure spelled out: logprobs (pass 1), loss on logprobs, backward (passes 2+3)
+        collected = []
         for i in range(n_mb):
             m = mbs[i % n_buf]
             logits = m["logits"].requires_grad_(True)
             loss_input, data = prepare_loss_input(logits, m["data"], fn)
-            loss, _metrics = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+            loss, metrics = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+            collected.append(worker_scaling(metrics))
             (dlogits,) = torch.autograd.grad(loss, logits)
             del dlogits, loss, loss_input
+        read_metrics(collected)
 
     def in_place_step():
         # the gradient written over the logits (the logits are dead after the loss in a training step): no second
         # [B, S, V] buffer, and the read and the write of a row hit the same DRAM pages
+        collected = []
         for i in range(n_mb):
             m = mbs[i % n_buf]
             logits = m["logits"].requires_grad_(True)
-            loss, _metrics = fused_logits_clipped_pg_loss(logits, m["data"], fn, tot_seqs, tot_toks, in_place=True)
+            loss, metrics = fused_logits_clipped_pg_loss(logits, m["data"], fn, tot_seqs, tot_toks, in_place=True)
+            collected.append(worker_scaling(metrics))
             (dlogits,) = torch.autograd.grad(loss, logits)
             del dlogits, loss
+        read_metrics(collected)
 
     elapsed, kernels = timed(torch, ops, args, step)
     tokens_per_step = w["seqs"] * w["seq_len"]
@@ -865,7 +980,9 @@ def _main():
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
                    "loss": "ClippedPGLoss eps=0.2/0.2, k3 KL beta=0.01, token-level",
-                   "metrics": "all diagnostics computed per microbatch; records fetched lazily (loss_fn.lazy_metrics = True)",
+                   "metrics": "all diagnostics computed per microbatch; after every loss call the worker's metrics[k] /= "
+                              "num_global_batches, after the last microbatch every value of every record is read (inside the "
+                              "timed step); no rl_amd-specific switch is set",
                    "api": "wrap_loss_fn_with_input_preparation(logits, batch, ..., prepare_fn=partial(prepare_loss_input, "
                           "sampling_params=, d2t=, chunk_size=)) + autograd.grad -> nrl_fused_logits_grpo_loss (seq stats + single "
                           "pass + term reduce + finish)"},
@@ -874,15 +991,15 @@ def _main():
         "roofline": hbm_roofline("fused_logits_loss_kernel", alg_launch, fk["avg_ms"], args.workload if full else None),
         "kernel_ms": {k: round(v["avg_ms"], 4) for k, v in kernels.items()},
     }
-    # ---- the same call with the default eager metrics: the host waits for every microbatch's record ----
+    # ---- the same step with a plain dictionary filled before every loss call returns ----
     fn.lazy_metrics = False
     e_elapsed, e_kernels = timed(torch, ops, args, step)
     fn.lazy_metrics = True
     result["eager_metrics"] = {
         "value": tokens_per_step * args.steps / e_elapsed, "unit": "tokens/s", "ms_per_step": e_elapsed / args.steps * 1e3,
         "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / e_elapsed / 1e9 / HBM_PEAK_GBS,
-        "note": "ClippedPGLossFn.lazy_metrics = False: the metrics dictionary is filled before the call returns (one device -> "
-                "host wait per microbatch, the reference's behaviour)",
+        "note": "ClippedPGLossFn.lazy_metrics = False: a plain dict filled before the call returns (one device -> host wait "
+                "per microbatch)",
     }
     # ---- the three-pass path (its own row: 3 * V * sizeof per token) ----
     t_elapsed, t_kernels = timed(torch, ops, args, three_pass_step)
@@ -908,6 +1025,10 @@ def _main():
         "hbm_frac_end_to_end": 2 * row_bytes * tokens_per_step * args.steps / i_elapsed / 1e9 / HBM_PEAK_GBS,
         "roofline": hbm_roofline("fused_logits_loss_kernel (dlogits over logits)", alg_launch, ik["avg_ms"]),
     }
+    if not args.no_cpu_baseline:
+        live = float(mbs[0]["data"]["token_mask"][:, 1:].sum().item())
+        result.update(read_write_ceiling(torch, mbs[0]["logits"].detach(), mbs[0]["data"]["input_ids"],
+                                         read_bytes=live * row_bytes, write_bytes=rows_per_launch * row_bytes))
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)  # 4 GiB
         dst = torch.empty_like(src)

@@ -9,7 +9,6 @@ dozen element-wise kernels and a synchronisation per metric.
 
 from __future__ import annotations
 
-from collections.abc import MutableMapping
 from typing import Any, Optional
 
 import torch
@@ -69,92 +68,172 @@ def _global_valid(seqs, toks, dev) -> torch.Tensor:
     return torch.stack(parts)
 
 
-class LazyMetrics(MutableMapping):
-    """The metrics of a loss call, fetched from the device on first use (opt-in: ``loss_fn.lazy_metrics = True``).
+class PendingMetric:
+    """One value of a ``StepMetrics`` mapping whose record has not been read yet.
+
+    It stands for ``record[key]`` times the factors it has been multiplied or divided by since: ``value / n`` and
+    ``value * n`` with a plain number give another ``PendingMetric`` and touch nothing (that is what the DTensor
+    worker does to every metric right after the loss call, ``models/automodel/train.py:525-533``); every other use
+    -- ``float()``, comparison, addition, formatting, pickling -- waits for the record and continues with the
+    ``float``."""
+
+    __slots__ = ("_owner", "_key", "_steps")
+
+    def __init__(self, owner, key, steps=()):
+        self._owner, self._key, self._steps = owner, key, steps
+
+    def _value(self):
+        v = self._owner._resolve()[self._key]
+        for divide, n in self._steps:
+            v = v / n if divide else v * n
+        return v
+
+    def _scaled(self, divide, n):
+        if type(n) in (int, float):
+            return PendingMetric(self._owner, self._key, self._steps + ((divide, n),))
+        return self._value() / n if divide else self._value() * n
+
+    def __truediv__(self, n): return self._scaled(True, n)
+    def __mul__(self, n): return self._scaled(False, n)
+    __rmul__ = __mul__
+    def __rtruediv__(self, n): return n / self._value()
+    def __add__(self, o): return self._value() + o
+    def __radd__(self, o): return o + self._value()
+    def __sub__(self, o): return self._value() - o
+    def __rsub__(self, o): return o - self._value()
+    def __neg__(self): return -self._value()
+    def __pos__(self): return self._value()
+    def __abs__(self): return abs(self._value())
+    def __pow__(self, o): return self._value() ** o
+    def __float__(self): return float(self._value())
+    def __int__(self): return int(self._value())
+    def __bool__(self): return bool(self._value())
+    def __round__(self, n=None): return round(self._value(), n)
+    def __eq__(self, o): return self._value() == o
+    def __ne__(self, o): return self._value() != o
+    def __lt__(self, o): return self._value() < o
+    def __le__(self, o): return self._value() <= o
+    def __gt__(self, o): return self._value() > o
+    def __ge__(self, o): return self._value() >= o
+    def __hash__(self): return hash(self._value())
+    def __repr__(self): return repr(self._value())
+    def __str__(self): return str(self._value())
+    def __format__(self, spec): return format(self._value(), spec)
+    def __reduce__(self):
+        v = self._value()
+        return (type(v), (v,))
+
+
+class StepMetrics(dict):
+    """The metrics of a loss call: a ``dict`` whose values arrive from the device behind the stream.
 
     The reference ends every loss call with about fifteen ``.item()`` calls, each of which stalls the host until
-    the device has caught up; by default this package returns the same plain ``{name: float}`` dictionary after
-    ONE such wait.  With ``lazy_metrics`` set the wait moves to the first time anything reads, writes or iterates
-    the mapping: a worker that collects the metrics of its microbatches and looks at them after the step (as the
-    Megatron schedule does) then launches the backward pass and the next microbatch without idling the device in
-    between.  Deliberately not a ``dict`` subclass: C-level consumers (``json.dumps``) read a dict subclass's
-    storage directly and would see it empty; ``dict(metrics)`` gives the plain dictionary."""
+    the device has caught up.  Here the 24-float record of a call travels to pinned host memory behind the kernels
+    and the host does not wait for it: until it is there, ``metrics[key]`` hands out a ``PendingMetric`` and
+    ``metrics[key] = ...`` stores whatever it is given, so the DTensor worker's ``metrics[k] /= num_global_batches``
+    between the loss call and ``backward()`` (``models/automodel/train.py:525-547``) records the division instead of
+    stalling, and the backward pass and the next microbatch are queued while the device is still busy.  Everything
+    that hands out the values wholesale or shows them -- ``items()``, ``values()``, ``get()``, ``pop()``, ``copy()``,
+    ``repr()``, comparison, ``json.dumps``, pickling -- waits for the record first and from then on the mapping holds
+    plain numbers, as it does from the start when the record has already arrived by the time it is first touched
+    (a Megatron worker reads its metrics after ``forward_backward_func`` has returned).  Copies that read the
+    storage directly (``dict(metrics)``, ``{**metrics}``) before that hold ``PendingMetric`` values, each of which
+    still resolves by itself.
+    ``loss_fn.lazy_metrics = False`` gives a plain ``dict`` filled before the call returns instead."""
 
-    __slots__ = ("_pending", "_data")
+    def __init__(self, keys, fetch):
+        super().__init__()
+        self._fetch = fetch
+        self._record = None
+        for key in keys:
+            dict.__setitem__(self, key, PendingMetric(self, key))
 
-    def __init__(self, build):
-        self._pending = build
-        self._data = None
+    def _resolve(self) -> dict:
+        if self._record is None:
+            self._record = self._fetch()
+            self._fetch = None
+            for key, value in list(dict.items(self)):
+                if isinstance(value, PendingMetric):
+                    dict.__setitem__(self, key, value._value())
+        return self._record
 
-    def _fill(self) -> dict:
-        if self._data is None:
-            self._data = self._pending()
-            self._pending = None
-        return self._data
+    def _settle(self, wait: bool):
+        if self._record is None and (wait or self._fetch.ready()):
+            self._resolve()
 
-    def __getitem__(self, key): return self._fill()[key]
-    def __setitem__(self, key, value): self._fill()[key] = value
-    def __delitem__(self, key): del self._fill()[key]
-    def __iter__(self): return iter(self._fill())
-    def __len__(self): return len(self._fill())
-    def __repr__(self): return repr(self._fill())
-    def __reduce_ex__(self, protocol): return (dict, (dict(self._fill()),))
-    def copy(self): return dict(self._fill())
+    def __getitem__(self, key):
+        self._settle(False)
+        return dict.__getitem__(self, key)
+
+    def __setitem__(self, key, value):
+        if isinstance(value, PendingMetric) and self._record is not None:
+            value = value._value()
+        dict.__setitem__(self, key, value)
+
+    def items(self): self._settle(True); return dict.items(self)
+    def values(self): self._settle(True); return dict.values(self)
+    def get(self, key, default=None): self._settle(True); return dict.get(self, key, default)
+    def pop(self, *args): self._settle(True); return dict.pop(self, *args)
+    def popitem(self): self._settle(True); return dict.popitem(self)
+    def setdefault(self, key, default=None): self._settle(True); return dict.setdefault(self, key, default)
+    def copy(self): self._settle(True); return dict(dict.items(self))
+    def __eq__(self, other): self._settle(True); return dict.__eq__(self, other)
+    def __ne__(self, other): self._settle(True); return dict.__ne__(self, other)
+    def __or__(self, other): self._settle(True); return dict.__or__(dict(dict.items(self)), other)
+    def __repr__(self): self._settle(True); return dict.__repr__(self)
+    def __reduce_ex__(self, protocol): self._settle(True); return (dict, (dict(dict.items(self)),))
+    __hash__ = None
 
 
 def fetch_later(record: torch.Tensor):
     """Starts the copy of a small device record to pinned host memory on the current stream and returns a function
-    that waits for that copy alone (not for work enqueued afterwards) and yields the values as a list."""
+    that waits for that copy alone (not for work enqueued afterwards) and yields the values as a list; its
+    ``ready()`` says without waiting whether the copy has arrived."""
     if not record.is_cuda:
-        return record.tolist
+        values = record.tolist
+        fetch = lambda: values()  # noqa: E731
+        fetch.ready = lambda: True
+        return fetch
     host = torch.empty(record.shape, dtype=record.dtype, pin_memory=True)
     host.copy_(record, non_blocking=True)
     done = torch.cuda.Event()
     done.record()
 
-    def values():
-        done.synchronize()
+    def fetch():
+        if not done.query():
+            done.synchronize()
         return host.tolist()
 
-    return values
+    fetch.ready = done.query
+    return fetch
 
 
 def metrics_record_to_dict(metrics: torch.Tensor, loss_fn, sample_mask_in: torch.Tensor) -> dict:
     """The kernels' metrics record -> the dictionary ``ClippedPGLossFn`` returns (``loss_functions.py:767-788``).
-    Fetching the record is the one device -> host wait of a loss call; with ``loss_fn.lazy_metrics`` it is put off
-    until the metrics are first used (``LazyMetrics``)."""
+    Fetching the record is the one device -> host wait of a loss call; it is put off until the values are needed
+    (``StepMetrics``) unless ``loss_fn.lazy_metrics`` is switched off."""
     beta = loss_fn.reference_policy_kl_penalty
     with_oob = loss_fn.truncated_importance_sampling_ratio is not None
     as_float = sample_mask_in.is_floating_point()
     values = fetch_later(metrics)
+    keys = ["loss", "probs_ratio", "probs_ratio_clamped", "probs_ratio_min", "probs_ratio_max", "probs_ratio_clamped_min",
+            "probs_ratio_clamped_max", "kl_penalty", "token_mult_prob_error", "gen_kl_error", "policy_kl_error",
+            "js_divergence_error", "sampling_importance_ratio", "num_valid_samples", "approx_entropy"]
+    if with_oob:
+        keys.append("is_oob_ratio")
+    keys.append("positive_nll_loss")
 
     def build():
         m = values()
         get = lambda name: m[METRIC_SLOTS[name]]  # noqa: E731
+        out = {key: get(key) for key in keys if key not in ("kl_penalty", "num_valid_samples")}
+        out["kl_penalty"] = get("kl") / beta if (beta != 0 and get("kl") != 0) else 0
         n_valid = get("num_valid_samples")
-        out = {
-            "loss": get("loss"),
-            "probs_ratio": get("probs_ratio"),
-            "probs_ratio_clamped": get("probs_ratio_clamped"),
-            "probs_ratio_min": get("probs_ratio_min"),
-            "probs_ratio_max": get("probs_ratio_max"),
-            "probs_ratio_clamped_min": get("probs_ratio_clamped_min"),
-            "probs_ratio_clamped_max": get("probs_ratio_clamped_max"),
-            "kl_penalty": get("kl") / beta if (beta != 0 and get("kl") != 0) else 0,
-            "token_mult_prob_error": get("token_mult_prob_error"),
-            "gen_kl_error": get("gen_kl_error"),
-            "policy_kl_error": get("policy_kl_error"),
-            "js_divergence_error": get("js_divergence_error"),
-            "sampling_importance_ratio": get("sampling_importance_ratio"),
-            "num_valid_samples": n_valid if as_float else int(n_valid),
-            "approx_entropy": get("approx_entropy"),
-        }
-        if with_oob:
-            out["is_oob_ratio"] = get("is_oob_ratio")
-        out["positive_nll_loss"] = get("positive_nll_loss")
-        return out
+        out["num_valid_samples"] = n_valid if as_float else int(n_valid)
+        return {key: out[key] for key in keys}
 
-    return LazyMetrics(build) if getattr(loss_fn, "lazy_metrics", False) else build()
+    build.ready = values.ready
+    return StepMetrics(keys, build) if getattr(loss_fn, "lazy_metrics", True) else build()
 
 
 class _FusedLoss(torch.autograd.Function):
@@ -186,10 +265,11 @@ class ClippedPGLossFn(LossFunction):
     ``L = E_t[max(-A r, -A clip(r, 1-eps_lo, 1+eps_hi))] + beta * KL(pi || pi_ref)`` with the variants
     selected by the configuration flags (see ``ClippedPGLossConfig``).
 
-    ``lazy_metrics`` (not in the reference; set it on the instance): return the metrics as a ``LazyMetrics``
-    mapping that waits for the device only when first read, instead of a plain dictionary."""
+    The metrics come back as a ``StepMetrics`` dictionary, which waits for the device when its values are first
+    needed rather than before the call returns; ``lazy_metrics = False`` (not in the reference; set it on the
+    instance) gives a plain dictionary filled at once."""
 
-    lazy_metrics = False
+    lazy_metrics = True
 
     input_type = LossInputType.LOGPROB
 

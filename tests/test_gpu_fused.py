@@ -355,22 +355,71 @@ def test_fused_packed_rejects_what_it_cannot_take():
                                             torch.tensor([0, 5, 40], dtype=torch.int32), gs, gt)
 
 
-def test_lazy_metrics_hold_the_same_values_as_the_eager_dictionary():
-    from rl_amd.algorithms.loss.loss_functions import LazyMetrics
+def test_step_metrics_hold_the_same_values_as_the_eager_dictionary():
+    from rl_amd.algorithms.loss.loss_functions import PendingMetric, StepMetrics
 
     logits, data, gs, gt = _batch(3, 20, 4096, torch.bfloat16, seed=77)
     ddev = {k: v.to(DEV) for k, v in data.items()}
     fn = ClippedPGLossFn(ClippedPGLossConfig())
+    fn.lazy_metrics = False
     eager_loss, eager = fused_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, fn, gs.to(DEV), gt.to(DEV))
     assert type(eager) is dict
-    fn.lazy_metrics = True
+    fn.lazy_metrics = True                   # the default
     x = logits.to(DEV).requires_grad_(True)
     lazy_loss, lazy = fused_logits_clipped_pg_loss(x, ddev, fn, gs.to(DEV), gt.to(DEV))
-    assert isinstance(lazy, LazyMetrics)
+    assert isinstance(lazy, StepMetrics) and isinstance(lazy, dict)
     lazy_loss.backward()                     # more work goes onto the stream before the record is looked at
     torch.ops.rl_amd.logprob_fwd(logits.to(DEV), ddev["input_ids"], 20, 0, 4096, 1.0, 1, False)
-    assert dict(lazy) == eager and lazy_loss.item() == eager_loss.item()
-    # the three-pass loss honours the switch as well
+    assert lazy == eager and dict(lazy.items()) == eager and lazy_loss.item() == eager_loss.item()
+    assert list(lazy) == list(eager) and all(type(v) in (float, int) for v in lazy.values())
+    # the three-pass loss returns the same kind of mapping
     loss_input, d2 = prepare_loss_input(logits.to(DEV), dict(ddev), fn)
     _, m3 = fn(data=d2, global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV), **loss_input)
-    assert isinstance(m3, LazyMetrics) and set(m3) == set(eager)
+    assert isinstance(m3, StepMetrics) and set(m3) == set(eager)
+
+
+def test_the_worker_loop_does_not_wait_for_the_device_between_loss_and_backward(monkeypatch):
+    """The DTensor worker divides every metric but the extrema by the number of global batches right after the loss
+    call and only then calls ``backward`` (``models/automodel/train.py:525-547``).  With the metrics of a call still on
+    their way that loop must not wait for the device: no event or stream synchronisation happens before ``backward``
+    is queued, and what is read afterwards is the eager value divided by the same number."""
+    from rl_amd.algorithms.loss.loss_functions import PendingMetric
+
+    logits, data, gs, gt = _batch(4, 64, 32768, torch.bfloat16, seed=78)
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    gsd, gtd = gs.to(DEV), gt.to(DEV)
+    fn = ClippedPGLossFn(ClippedPGLossConfig())
+    fn.lazy_metrics = False
+    _, eager = fused_logits_clipped_pg_loss(logits.to(DEV).requires_grad_(True), ddev, fn, gsd, gtd)
+    fn.lazy_metrics = True
+    xs = [logits.to(DEV).requires_grad_(True) for _ in range(3)]
+    torch.cuda.synchronize()
+
+    waits = []
+    real_event_sync, real_sync = torch.cuda.Event.synchronize, torch.cuda.synchronize
+    monkeypatch.setattr(torch.cuda.Event, "synchronize", lambda self: (waits.append("event"), real_event_sync(self))[1])
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda *a, **k: (waits.append("device"), real_sync(*a, **k))[1])
+    monkeypatch.setattr(torch.Tensor, "item", lambda self: (waits.append("item"), self.tolist())[1])
+    num_global_batches = 4
+    collected = []
+    torch.cuda._sleep(400_000_000)                     # keeps the device busy (about 0.2 s) while the host runs the loop
+    for x in xs:                                       # three microbatches queued back to back
+        loss, metrics = fused_logits_clipped_pg_loss(x, ddev, fn, gsd, gtd)
+        for k in metrics.keys():
+            if "_min" in k or "_max" in k:
+                continue
+            metrics[k] /= num_global_batches
+        (loss * 2).backward()
+        collected.append(metrics)
+    assert waits == [], waits                          # nothing waited while the device was still working
+    pending = sum(isinstance(v, PendingMetric) for v in dict.values(collected[-1]))
+    monkeypatch.undo()
+    assert pending > 0                                 # (the last call's record had indeed not arrived)
+    for metrics in collected:
+        metrics["lr"] = 1e-5
+        assert metrics["num_valid_samples"] > 0
+        for k, v in metrics.items():
+            if k == "lr":
+                continue
+            want = eager[k] if ("_min" in k or "_max" in k) else eager[k] / num_global_batches
+            assert type(v) in (float, int) and v == want, (k, v, want)

@@ -115,36 +115,65 @@ def test_multi_rank_groups_are_rejected(monkeypatch):
         mu.from_parallel_logits_to_logprobs(torch.zeros(1, 2, 4), torch.zeros(1, 2, dtype=torch.long), 0, 4, "tp2")
 
 
-def test_lazy_metrics_fetches_once_on_first_use_and_behaves_like_the_dictionary():
-    import pickle
-
-    from rl_amd.algorithms.loss.loss_functions import LazyMetrics
+def _step_metrics(record, arrived):
+    from rl_amd.algorithms.loss.loss_functions import StepMetrics
 
     calls = []
 
-    def build():
+    def fetch():
         calls.append(1)
-        return {"loss": 0.5, "num_valid_samples": 4}
+        return dict(record)
 
-    m = LazyMetrics(build)
-    assert calls == []                       # nothing fetched by construction
-    assert m["loss"] == 0.5 and calls == [1]
-    assert list(m) == ["loss", "num_valid_samples"] and len(m) == 2 and "loss" in m and calls == [1]
+    fetch.ready = lambda: arrived[0]
+    return StepMetrics(list(record), fetch), calls
+
+
+def test_step_metrics_wait_only_when_values_are_needed():
+    import json
+    import pickle
+
+    from rl_amd.algorithms.loss.loss_functions import PendingMetric
+
+    record = {"loss": 0.5, "probs_ratio_max": 3.0, "num_valid_samples": 4}
+    arrived = [False]
+    m, calls = _step_metrics(record, arrived)
+    assert isinstance(m, dict) and calls == []
+    # what the DTensor worker does between the loss call and backward(): nothing is fetched
+    for k in m.keys():
+        if "_min" in k or "_max" in k:
+            continue
+        m[k] /= 4
     m["lr"] = 1e-5
-    m["loss"] /= 2
-    assert dict(m) == {"loss": 0.25, "num_valid_samples": 4, "lr": 1e-5}
-    for use in (lambda x: list(x.items()), lambda x: x.get("loss"), lambda x: repr(x), lambda x: x == {"loss": 0.5, "num_valid_samples": 4},
-                lambda x: {**x}, lambda x: x.copy(), lambda x: x.update(a=1), lambda x: x.setdefault("b", 2)):
-        calls.clear()
-        fresh = LazyMetrics(build)
-        use(fresh)
-        assert calls == [1]
-    restored = pickle.loads(pickle.dumps(LazyMetrics(build)))
-    assert type(restored) is dict and restored == {"loss": 0.5, "num_valid_samples": 4}
-    with pytest.raises(TypeError):           # not a dict subclass on purpose: C-level consumers must not see it empty
-        import json
+    assert calls == [] and len(m) == 4 and "loss" in m and list(m.keys())[:3] == list(record)
+    assert isinstance(m["loss"], PendingMetric) and calls == []
+    # the first real use fetches once; afterwards the mapping holds plain numbers
+    assert m["num_valid_samples"] > 0 and calls == [1]
+    assert dict.__getitem__(m, "loss") == 0.125 and type(dict.__getitem__(m, "loss")) is float
+    assert m == {"loss": 0.125, "probs_ratio_max": 3.0, "num_valid_samples": 1.0, "lr": 1e-5} and calls == [1]
+    assert json.loads(json.dumps(m))["loss"] == 0.125
 
-        json.dumps(LazyMetrics(build))
+    # a record that has arrived by the first touch (the Megatron worker reads after the schedule returned)
+    arrived = [True]
+    m, calls = _step_metrics(record, arrived)
+    assert type(m["loss"]) is float and calls == [1]
+
+    # every way of handing the values out wholesale waits, once
+    for use in (lambda x: list(x.items()), lambda x: list(x.values()), lambda x: x.get("loss"), lambda x: repr(x),
+                lambda x: x == record, lambda x: x.copy(), lambda x: x.pop("loss"), lambda x: x.setdefault("b", 2),
+                lambda x: json.dumps(x), lambda x: pickle.dumps(x), lambda x: x | {"a": 1},
+                lambda x: float(x["loss"]), lambda x: x["loss"] + 1, lambda x: f"{x['loss']:.3f}", lambda x: x["loss"] < 1):
+        m, calls = _step_metrics(record, [False])
+        use(m)
+        assert calls == [1], use
+    m, calls = _step_metrics(record, [False])
+    restored = pickle.loads(pickle.dumps(m))
+    assert type(restored) is dict and restored == record
+    # values that escaped before the record arrived still resolve by themselves, scaled as recorded
+    m, calls = _step_metrics(record, [False])
+    early = {k: v for k, v in zip(m.keys(), dict.values(m))}
+    scaled = early["loss"] / 2 * 3
+    assert calls == [] and scaled == 0.75 and calls == [1] and pickle.loads(pickle.dumps(early["loss"])) == 0.5
+    assert early["num_valid_samples"] / torch.tensor(2.0) == torch.tensor(2.0)   # a non-number operand resolves at once
 
 
 _STUB_CHECK = r"""
