@@ -21,7 +21,8 @@ from functools import partial
 import torch
 
 import nemo_rl.algorithms.grpo as grpo                    # binds the originals by name, as the driver does
-from nemo_rl.algorithms.loss import prepare_loss_input as before
+import nemo_rl.algorithms.loss as _pkg_before
+before = [_pkg_before.prepare_loss_input]               # in a list: install() rebinds module globals, this script's too
 import nemo_rl.models.automodel.train as train
 import rl_amd
 
@@ -58,7 +59,7 @@ got, metrics = pkg.wrap_loss_fn_with_input_preparation(
 got.backward()
 print("RESULT " + json.dumps({
     "mode": mode,
-    "rebinding": before is not pkg.prepare_loss_input and train.prepare_loss_input is pkg.prepare_loss_input,
+    "rebinding": before[0] is not pkg.prepare_loss_input and train.prepare_loss_input is pkg.prepare_loss_input,
     "fusable": why_not_fusable(fn, xg, ddev),
     "single_pass_calls": len(calls),
     "loss": [got.item(), want.item()],
