@@ -23,7 +23,8 @@
 //
 // Rows whose candidate list would exceed the LDS capacity (very flat distributions under top-p
 // alone, thousands of exact ties, or a top_k in the thousands) are marked and finished by
-// topk_topp_wide_kernel, which finds the same predicate by bitwise threshold search over the row.
+// topk_topp_wide_kernel, which finds the same predicate by a radix descent over the row's order keys
+// (a histogram pass per key digit: two to three passes for 16-bit logits).
 
 #include <float.h>
 #include <math.h>
@@ -39,7 +40,7 @@ constexpr int kSelWaves = kSelBlock / kWave;
 constexpr int kMassBins = 64;
 constexpr int kLooseHits = 768;  // top-p alone: more hit chunks than this under the chunk maxima's bound -> bound from the row
 constexpr int kMassCopies = 8;  // copies of the histogram, by lane: most elements fall into the few lowest bins
-constexpr int kWideGrid = 2048;  // workgroups of the threshold-search kernel (more in flight measured faster than fewer)
+constexpr int kWideGrid = 2048;  // workgroups of the kernel that finishes the marked rows
 constexpr int32_t kTieUnresolved = -1;  // tie[] marker: the row's kept set did not fit the candidate list
 constexpr int kSub = 8;                      // chunk maxima per thread
 constexpr int kChunks = kSelBlock * kSub;    // 2048
@@ -501,9 +502,19 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     bound_key = bound_from_row();
     }
     if (n > CAP || n == 0) {
-        // the kept set does not fit the candidate list (or the row holds no finite value)
+        // the kept set does not fit the candidate list (or the row holds no finite value); the kernel that finishes
+        // such a row finds its largest (scaled) logit in thr
+        float row_max = mx[0];
+#pragma unroll
+        for (int u = 1; u < kSub; ++u) row_max = fmaxf(row_max, mx[u]);
+        row_max = wave_max(row_max);
+        __syncthreads();
+        if ((tid & (kWave - 1)) == 0) sh.lse_w[tid / kWave].m = row_max;
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kSelWaves; ++q) row_max = fmaxf(row_max, sh.lse_w[q].m);
         if (tid == 0) {
-            a.thr[r] = __builtin_nanf("");
+            a.thr[r] = n > CAP ? row_max : __builtin_nanf("");
             a.tie[r] = n > CAP ? kTieUnresolved : 0;  // unresolved rows are finished by topk_topp_wide_kernel
             a.lse_kept[r] = __builtin_nanf("");
             if (a.logprob) a.logprob[r] = __builtin_nanf("");
@@ -603,30 +614,87 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// rows whose kept set does not fit the on-chip candidate list (top-p alone over a flat distribution, or a
-// very large top_k): the same keep predicate found without a sort, by searching the threshold key bit by
-// bit with one streaming pass over the row per two bits.  The row (at most a few hundred KB) stays in L2
-// between passes.  Sums are carried in double, so the cumulative mass at the boundary differs from the
-// sorted fp32 running sum of the fast path only in which of two nearly equal neighbours falls first.
+// rows whose kept set does not fit the on-chip candidate list (top-p alone over a flat distribution, thousands
+// of exact ties, or a very large top_k): the same keep predicate found without a sort, by a radix descent over
+// the order keys.  A pass streams the row once and fills a histogram over one digit of the keys that share the
+// digits chosen so far: the number of elements per bin, which is what top-k descends by (the largest key with at
+// least top_k keys at or above it), and their probability mass per bin, which is what top-p descends by (the
+// smallest key whose cumulative mass from below exceeds (1 - p) Z).  A 16-bit logit has 16 significant key bits:
+// two digits, so top-k and top-p together take three passes (the first histogram serves both), top-p alone two;
+// fp16 adds a three-bit digit, fp32 has four digits.  One more pass over the row and a look at one block of it
+// find the first survivor among the elements that tie with the top-p threshold.  The row (at most a few hundred
+// KB) comes from cache after the first pass.
+//
+// Masses are summed as 64-bit fixed-point integers (exp(x - max) * 2^S with S chosen from the row length so that a
+// whole row cannot overflow): integer addition is associative, so the LDS atomics that fill the histogram give
+// the same sums whatever order they arrive in, and the row's result does not depend on scheduling.  The fixed
+// point resolves 2^-45 of the largest element's mass at V = 151936; what it drops is below the rounding of the
+// reference's fp32 sums by orders of magnitude, and which of two nearly equal neighbours at the top-p boundary
+// falls first may differ from a sorted fp32 running sum, as it may between any two summation orders.
 // ---------------------------------------------------------------------------------------------
-template <typename T> __device__ __forceinline__ void block_sum3(T (&v)[3], T* shm) {
+constexpr int kRadixBins = 256;
+constexpr int kRadixCopies = 8;   // histogram copies by lane: logits of one magnitude share their leading digit
+constexpr int kTieBlocks = kRadixBins * kRadixCopies;  // index blocks of the tie search (they reuse the count bins)
+
+// digits of an order key from the top, by element type: 16-bit types leave the low key bits constant for a given sign
+template <int DT> struct KeyDigits;
+template <> struct KeyDigits<NRL_F32> {
+    static constexpr int N = 4, LOW = 0;
+    __device__ static constexpr int shift(int l) { return 24 - 8 * l; }
+    __device__ static constexpr int bits(int) { return 8; }
+};
+template <> struct KeyDigits<NRL_BF16> {
+    static constexpr int N = 2, LOW = 16;
+    __device__ static constexpr int shift(int l) { return 24 - 8 * l; }
+    __device__ static constexpr int bits(int) { return 8; }
+};
+template <> struct KeyDigits<NRL_F16> {
+    static constexpr int N = 3, LOW = 13;
+    __device__ static constexpr int shift(int l) { return l == 2 ? 13 : 24 - 8 * l; }
+    __device__ static constexpr int bits(int l) { return l == 2 ? 3 : 8; }
+};
+
+struct WideShared {
+    unsigned long long mass[kRadixBins * kRadixCopies];
+    unsigned int cnt[kRadixBins * kRadixCopies];
+    unsigned long long scan64[kSelWaves];
+    unsigned int scan32[kSelWaves];
+    // what the thread that owns the chosen bin tells the others
+    unsigned int pick_bin, pick_cnt;
+    unsigned long long pick_a, pick_b;
+};
+
+template <typename T> __device__ __forceinline__ T wide_scan_excl(T v, T* shm, T& total) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    T inc = v;
 #pragma unroll
-    for (int c = 0; c < 3; ++c)
-#pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) v[c] += __shfl_down(v[c], off, kWave);
-    __syncthreads();  // the previous round's readers are done with shm
-    if (lane == 0)
-#pragma unroll
-        for (int c = 0; c < 3; ++c) shm[wave * 3 + c] = v[c];
-    __syncthreads();
-#pragma unroll
-    for (int c = 0; c < 3; ++c) {
-        T t = shm[c];
-#pragma unroll
-        for (int w = 1; w < kSelWaves; ++w) t += shm[w * 3 + c];
-        v[c] = t;
+    for (int off = 1; off < kWave; off <<= 1) {
+        const T t = __shfl_up(inc, off, kWave);
+        if (lane >= off) inc += t;
     }
+    __syncthreads();  // the previous scan's readers are done with shm
+    if (lane == kWave - 1) shm[wave] = inc;
+    __syncthreads();
+    T base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kSelWaves; ++w) {
+        const T part = shm[w];
+        if (w < wave) base += part;
+        tot += part;
+    }
+    total = tot;
+    return base + inc - v;
+}
+
+// exp(x - m) as a fixed-point integer with fx_shift fraction bits (x <= m); zero below its resolution
+__device__ __forceinline__ unsigned long long wide_mass(float x, float m, int fx_shift) {
+    const uint32_t b = __float_as_uint(fast_exp2((x - m) * kLog2e));
+    int ex = static_cast<int>((b >> 23) & 0xffu);
+    if (ex == 0 || ex == 255 || (b >> 31)) return 0ull;  // zero / subnormal; never infinite or NaN for finite x <= m
+    if (ex > 127) ex = 127;
+    const unsigned long long mant = (b & 0x7fffffu) | 0x800000u;
+    const int sh = ex + fx_shift - 150;
+    return sh >= 0 ? mant << sh : (sh > -24 ? mant >> (-sh) : 0ull);
 }
 
 template <int DT, int TEMP> struct WideRow {
@@ -649,13 +717,51 @@ template <int DT, int TEMP> struct WideRow {
     }
 };
 
+// One histogram pass: bin = digit `level` of the keys whose higher digits equal `prefix` (every key at level 0).
+// Thread b returns the number of such elements in bin b and their mass.
+template <int DT, int TEMP>
+__device__ __forceinline__ void wide_hist_pass(const WideRow<DT, TEMP>& w, WideShared& sh, float m, int fx_shift, int level,
+                                               uint32_t prefix, unsigned int& my_cnt, unsigned long long& my_mass) {
+    const int tid = threadIdx.x;
+    const int shift = KeyDigits<DT>::shift(level), bits = KeyDigits<DT>::bits(level);
+    const uint32_t mask = (1u << bits) - 1u;
+    __syncthreads();  // whoever still reads the bins of the pass before
+    for (int i = tid; i < kRadixBins * kRadixCopies; i += kSelBlock) { sh.mass[i] = 0ull; sh.cnt[i] = 0u; }
+    __syncthreads();
+    const int copy = tid & (kRadixCopies - 1);
+    if (level == 0) {
+        w.for_each([&](float x, int64_t) {
+            const int slot = static_cast<int>((order_key(x) >> shift) & mask) * kRadixCopies + copy;
+            atomicAdd(&sh.cnt[slot], 1u);
+            atomicAdd(&sh.mass[slot], wide_mass(x, m, fx_shift));
+        });
+    } else {
+        w.for_each([&](float x, int64_t) {
+            const uint32_t key = order_key(x);
+            if ((key >> (shift + bits)) == prefix) {
+                const int slot = static_cast<int>((key >> shift) & mask) * kRadixCopies + copy;
+                atomicAdd(&sh.cnt[slot], 1u);
+                atomicAdd(&sh.mass[slot], wide_mass(x, m, fx_shift));
+            }
+        });
+    }
+    __syncthreads();
+    my_cnt = 0u;
+    my_mass = 0ull;
+#pragma unroll
+    for (int q = 0; q < kRadixCopies; ++q) {
+        my_cnt += sh.cnt[tid * kRadixCopies + q];
+        my_mass += sh.mass[tid * kRadixCopies + q];
+    }
+}
+
 template <int DT, int TEMP>
 __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, int64_t n_rows) {
-    __shared__ double shm_d[kSelWaves * 3];
-    __shared__ long long shm_i[kSelWaves * 3];
-    __shared__ float shm_m[kSelWaves];
+    static_assert(kRadixBins == kSelBlock, "one histogram bin per thread");
+    __shared__ WideShared sh;
+    using KD = KeyDigits<DT>;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const bool use_k = a.top_k > 0, use_p = a.top_p < 1.0f;
+    const bool use_p = a.top_p < 1.0f;
     {
         // the usual case is that no row of this workgroup is marked: look at all of them at once and leave
         bool mine = false;
@@ -663,6 +769,9 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
             mine |= a.tie[r] == kTieUnresolved;
         if (!__syncthreads_or(mine)) return;
     }
+    int clog2 = 0;
+    while ((int64_t{1} << clog2) < a.vocab) ++clog2;
+    const int fx_shift = 63 - clog2 < 46 ? 63 - clog2 : 46;  // a row of `vocab` largest elements still fits 63 bits
     for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
         if (a.tie[r] != kTieUnresolved) continue;  // the same word for every thread of the workgroup
         const int64_t o = r / a.n_inner, i_in = r - o * a.n_inner;
@@ -674,134 +783,168 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
         w.tail0 = w.head + w.nvec * Row<DT>::EPV;
         w.xv = reinterpret_cast<const u32x4*>(w.row + w.head * Row<DT>::BYTES);
         w.tparam = a.tparam;
+        const float m = a.thr[r];  // the row's largest (scaled) logit, left here by the kernel that marked the row
+        const bool use_k = a.top_k > 0 && a.top_k < w.vocab;
 
-        // row maximum
-        float m = -FLT_MAX;
-        w.for_each([&](float x, int64_t) { m = fmaxf(m, x); });
-#pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) m = fmaxf(m, __shfl_down(m, off, kWave));
-        __syncthreads();
-        if (lane == 0) shm_m[wave] = m;
-        __syncthreads();
-        m = shm_m[0];
-#pragma unroll
-        for (int q = 1; q < kSelWaves; ++q) m = fmaxf(m, shm_m[q]);
-        const uint32_t max_key = order_key(m);
+        // ---- first digit, every element: serves the top-k and the top-p descent alike ----
+        unsigned int hc[KD::N];         // this thread's bin along the top-k descent (or just level 0), per level
+        unsigned long long hm[KD::N];
+        uint32_t hprefix[KD::N];
+        int h_levels = 1;
+        hprefix[0] = 0u;
+        wide_hist_pass<DT, TEMP>(w, sh, m, fx_shift, 0, 0u, hc[0], hm[0]);
+        unsigned long long total_mass = 0ull;
+        wide_scan_excl(hm[0], sh.scan64, total_mass);
 
-        // top-k: the largest key with at least top_k keys at or above it (ties at that key are all kept)
+        // ---- top-k: the largest key with at least top_k keys at or above it (ties at that key are all kept) ----
         uint32_t k_key = 0u;
-        if (use_k && a.top_k < w.vocab) {
-            for (int bit = 30; bit >= 0; bit -= 2) {
-                long long cnt[3] = {0, 0, 0};
-                const uint32_t c1 = k_key | (1u << bit), c2 = k_key | (2u << bit), c3 = k_key | (3u << bit);
-                w.for_each([&](float x, int64_t) {
-                    const uint32_t key = order_key(x);
-                    cnt[0] += key >= c1;
-                    cnt[1] += key >= c2;
-                    cnt[2] += key >= c3;
-                });
-                block_sum3(cnt, shm_i);
-                const uint32_t step = cnt[2] >= a.top_k ? 3u : cnt[1] >= a.top_k ? 2u : cnt[0] >= a.top_k ? 1u : 0u;
-                k_key |= step << bit;
+        unsigned long long mass_below_k = 0ull;
+        unsigned int cnt_at_k = 0u;
+        if (use_k) {
+            unsigned int need = static_cast<unsigned int>(a.top_k);
+            uint32_t prefix = 0u;
+#pragma unroll
+            for (int l = 0; l < KD::N; ++l) {
+                if (l > 0) {
+                    hprefix[l] = prefix;
+                    wide_hist_pass<DT, TEMP>(w, sh, m, fx_shift, l, prefix, hc[l], hm[l]);
+                    h_levels = l + 1;
+                }
+                unsigned int tot_c = 0u;
+                unsigned long long tot_m = 0ull;
+                const unsigned int excl_c = wide_scan_excl(hc[l], sh.scan32, tot_c);
+                const unsigned long long excl_m = wide_scan_excl(hm[l], sh.scan64, tot_m);
+                const unsigned int at_or_above = tot_c - excl_c, above = at_or_above - hc[l];
+                if (at_or_above >= need && above < need) {
+                    sh.pick_bin = static_cast<unsigned int>(tid);
+                    sh.pick_cnt = hc[l];
+                    sh.pick_a = need - above;
+                    sh.pick_b = excl_m;
+                }
+                __syncthreads();
+                prefix = (prefix << KD::bits(l)) | sh.pick_bin;
+                need = static_cast<unsigned int>(sh.pick_a);
+                mass_below_k += sh.pick_b;
+                cnt_at_k = sh.pick_cnt;
+                __syncthreads();  // everyone has read the pick
             }
+            k_key = prefix << KD::LOW;
+            if (KD::LOW > 0 && !(k_key >> 31)) k_key |= (1u << KD::LOW) - 1u;  // a negative value's low key bits are ones
         }
-
-        // mass of the top-k survivors (Z) and of the whole row
-        auto wexp = [&](float x) { return static_cast<double>(fast_exp2((x - m) * kLog2e)); };
-        double mass[3] = {0.0, 0.0, 0.0};
-        w.for_each([&](float x, int64_t) {
-            const double e = wexp(x);
-            mass[0] += order_key(x) >= k_key ? e : 0.0;
-            mass[1] += e;
-        });
-        block_sum3(mass, shm_d);
-        const double z = mass[0];
-        const float lse_full = m + logf(static_cast<float>(mass[1]));
+        const unsigned long long z = total_mass - mass_below_k;  // mass of the top-k survivors
 
         uint32_t thr_key = k_key;
         int32_t tie = 0;
-        double kept_mass = z;
+        unsigned long long kept_mass = z;
         if (use_p) {
-            // ascending cumulative probability; elements fall while it stays <= 1 - p.  The threshold is
-            // the largest key c whose strictly-lower survivors together weigh <= (1 - p) Z.  `base` carries
-            // the mass of the survivors below c from round to round, so a round only looks at the keys in
-            // the still undecided range [c, c + 3 * 2^bit): after the first few rounds nearly every element
-            // is skipped before its exponential.
-            const double target = static_cast<double>(1.0f - a.top_p) * z;
-            uint32_t c = 0u;
-            double base = 0.0;
-            for (int bit = 30; bit >= 0; bit -= 2) {
-                const uint32_t c1 = c | (1u << bit), c2 = c | (2u << bit), c3 = c | (3u << bit);
-                const uint32_t lo = c > k_key ? c : k_key;
-                double seg[3] = {0.0, 0.0, 0.0};  // survivors in [c, c1), [c1, c2), [c2, c3)
-                w.for_each([&](float x, int64_t) {
-                    const uint32_t key = order_key(x);
-                    if (key >= lo && key < c3) {
-                        const double e = wexp(x);
-                        seg[0] += key < c1 ? e : 0.0;
-                        seg[1] += (key >= c1 && key < c2) ? e : 0.0;
-                        seg[2] += key >= c2 ? e : 0.0;
-                    }
-                });
-                block_sum3(seg, shm_d);
-                const double l1 = base + seg[0], l2 = l1 + seg[1], l3 = l2 + seg[2];
-                if (l3 <= target) { c = c3; base = l3; }
-                else if (l2 <= target) { c = c2; base = l2; }
-                else if (l1 <= target) { c = c1; base = l1; }
+            // ascending cumulative probability over the survivors; elements fall while it stays <= (1 - p) Z.  Counted
+            // over the whole row that is: mass below the key <= (1 - p) Z + mass below the top-k threshold.
+            const double target_d = static_cast<double>(1.0f - a.top_p) * static_cast<double>(z);
+            const unsigned long long target = target_d <= 0.0 ? 0ull : static_cast<unsigned long long>(target_d);
+            unsigned long long room = target + mass_below_k;  // what may still lie below the digit being chosen
+            unsigned long long below_all = 0ull;
+            unsigned int n_eq = 0u;
+            uint32_t prefix = 0u;
+#pragma unroll
+            for (int l = 0; l < KD::N; ++l) {
+                unsigned int bc = hc[l];
+                unsigned long long bm = hm[l];
+                if (l >= h_levels || hprefix[l] != prefix) wide_hist_pass<DT, TEMP>(w, sh, m, fx_shift, l, prefix, bc, bm);
+                unsigned int tot_c = 0u;
+                unsigned long long tot_m = 0ull;
+                const unsigned int excl_c = wide_scan_excl(bc, sh.scan32, tot_c);
+                const unsigned long long excl_m = wide_scan_excl(bm, sh.scan64, tot_m);
+                // the bin in which the cumulative mass first exceeds the room; if it never does (top_p -> 0), the
+                // highest bin that holds anything: the largest element always survives
+                const bool crossing = tot_m > room ? (excl_m + bm > room && excl_m <= room)
+                                                   : (bc > 0u && tot_c - excl_c - bc == 0u);
+                if (crossing) {
+                    sh.pick_bin = static_cast<unsigned int>(tid);
+                    sh.pick_cnt = bc;
+                    sh.pick_a = room - excl_m;
+                    sh.pick_b = excl_m;
+                }
+                __syncthreads();
+                prefix = (prefix << KD::bits(l)) | sh.pick_bin;
+                room = sh.pick_a;
+                below_all += sh.pick_b;
+                n_eq = sh.pick_cnt;
+                __syncthreads();
             }
-            bool clamped = false;
-            if (c > max_key) { c = max_key; clamped = true; }  // the largest element always survives
-            if (c < k_key) { c = k_key; clamped = true; }
+            uint32_t c = prefix << KD::LOW;
+            if (KD::LOW > 0 && !(c >> 31)) c |= (1u << KD::LOW) - 1u;
+            unsigned long long below = 0ull;  // mass of the survivors strictly below the threshold
+            if (c <= k_key) { c = k_key; if (use_k) n_eq = cnt_at_k; }
+            else below = below_all - mass_below_k;
             thr_key = c;
             // how many of the elements equal to the threshold fall too (the ones with the smallest indices)
-            double below[3] = {clamped ? 0.0 : base, 0.0, 0.0};
-            long long n_eq[3] = {0, 0, 0};
-            if (clamped) {
-                w.for_each([&](float x, int64_t) {
-                    const uint32_t key = order_key(x);
-                    below[0] += (key >= k_key && key < c) ? wexp(x) : 0.0;
-                    n_eq[0] += key == c;
+            const unsigned long long e_thr = wide_mass(key_value(c), m, fx_shift);
+            unsigned long long drop = 0ull;
+            if (e_thr > 0ull && n_eq > 1u && target >= below) {
+                drop = (target - below) / e_thr;
+                if (drop > n_eq - 1u) drop = n_eq - 1u;
+            }
+            if (drop > 0ull) {
+                // index of the first survivor among the equal elements, the one with `drop` equal elements before it:
+                // equal elements counted per block of indices, then one look at the block that holds it
+                int ishift = clog2 - 11;
+                if (ishift < 0) ishift = 0;
+                __syncthreads();
+                for (int i = tid; i < kTieBlocks; i += kSelBlock) sh.cnt[i] = 0u;
+                __syncthreads();
+                w.for_each([&](float x, int64_t j) {
+                    if (order_key(x) == c) atomicAdd(&sh.cnt[j >> ishift], 1u);
                 });
-                block_sum3(below, shm_d);
-            } else {
-                w.for_each([&](float x, int64_t) { n_eq[0] += order_key(x) == c; });
-            }
-            block_sum3(n_eq, shm_i);
-            const double e_thr = wexp(key_value(c));
-            long long drop = 0;
-            if (e_thr > 0.0 && n_eq[0] > 1) {
-                const double room = (target - below[0]) / e_thr;
-                drop = room <= 0.0 ? 0 : room >= static_cast<double>(n_eq[0] - 1) ? n_eq[0] - 1 : static_cast<long long>(room);
-                while (drop + 1 <= n_eq[0] - 1 && below[0] + static_cast<double>(drop + 1) * e_thr <= target) ++drop;
-                while (drop > 0 && below[0] + static_cast<double>(drop) * e_thr > target) --drop;
-            }
-            if (drop > 0) {
-                // index of the first survivor among the equal elements: the largest index with at most
-                // `drop` equal elements before it
-                int64_t idx = 0;
-                int top_bit = 0;
-                while ((int64_t{1} << (top_bit + 1)) < w.vocab) ++top_bit;
-                top_bit |= 1;  // pairs of bits, so start from an odd position
-                for (int bit = top_bit - 1; bit >= 0; bit -= 2) {
-                    long long before[3] = {0, 0, 0};
-                    const int64_t i1 = idx | (int64_t{1} << bit), i2 = idx | (int64_t{2} << bit), i3 = idx | (int64_t{3} << bit);
-                    w.for_each([&](float x, int64_t j) {
-                        const bool eq = order_key(x) == c;
-                        before[0] += eq && j < i1;
-                        before[1] += eq && j < i2;
-                        before[2] += eq && j < i3;
-                    });
-                    block_sum3(before, shm_i);
-                    const int64_t step = before[2] <= drop ? 3 : before[1] <= drop ? 2 : before[0] <= drop ? 1 : 0;
-                    idx |= step << bit;
+                __syncthreads();
+                unsigned int mine8[kRadixCopies], sum8 = 0u;
+#pragma unroll
+                for (int q = 0; q < kRadixCopies; ++q) { mine8[q] = sh.cnt[tid * kRadixCopies + q]; sum8 += mine8[q]; }
+                unsigned int tot_eq = 0u;
+                unsigned int before = wide_scan_excl(sum8, sh.scan32, tot_eq);
+                if (before <= drop && drop < before + sum8) {
+#pragma unroll
+                    for (int q = 0; q < kRadixCopies; ++q) {
+                        if (before <= drop && drop < before + mine8[q]) {
+                            sh.pick_bin = static_cast<unsigned int>(tid * kRadixCopies + q);
+                            sh.pick_cnt = static_cast<unsigned int>(drop) - before;
+                        }
+                        before += mine8[q];
+                    }
                 }
-                tie = static_cast<int32_t>(idx);
+                __syncthreads();
+                const int64_t first = static_cast<int64_t>(sh.pick_bin) << ishift;
+                int64_t stop = first + (int64_t{1} << ishift);
+                if (stop > w.vocab) stop = w.vocab;
+                unsigned int seen = 0u;
+                const unsigned int want = sh.pick_cnt;
+                for (int64_t j0 = first; j0 < stop; j0 += kSelBlock) {
+                    const int64_t j = j0 + tid;
+                    const bool eq = j < stop && order_key(scale_logit<DT, TEMP>(Row<DT>::load1(w.row, j), a.tparam)) == c;
+                    const unsigned long long bal = __ballot(eq);
+                    const unsigned int in_wave = static_cast<unsigned int>(__popcll(bal & ((1ull << lane) - 1ull)));
+                    __syncthreads();
+                    if (lane == 0) sh.scan32[wave] = static_cast<unsigned int>(__popcll(bal));
+                    __syncthreads();
+                    unsigned int ahead = seen, chunk = 0u;
+#pragma unroll
+                    for (int q = 0; q < kSelWaves; ++q) {
+                        if (q < wave) ahead += sh.scan32[q];
+                        chunk += sh.scan32[q];
+                    }
+                    if (eq && ahead + in_wave == want) sh.pick_a = static_cast<unsigned long long>(j);
+                    seen += chunk;
+                }
+                __syncthreads();
+                tie = static_cast<int32_t>(sh.pick_a);
             }
-            kept_mass = z - below[0] - static_cast<double>(drop) * e_thr;
-            if (!(kept_mass > 0.0)) kept_mass = e_thr;
+            kept_mass = z - below - drop * e_thr;
+            if (kept_mass == 0ull || kept_mass > z) kept_mass = e_thr;
         }
         const float thr = key_value(thr_key);
-        const float lse_kept = m + logf(static_cast<float>(kept_mass));
+        const float unit = __uint_as_float(static_cast<uint32_t>(127 - fx_shift) << 23);  // 2^-fx_shift
+        const float lse_kept = m + logf(static_cast<float>(static_cast<double>(kept_mass) * static_cast<double>(unit)));
+        const float lse_full = m + logf(static_cast<float>(static_cast<double>(total_mass) * static_cast<double>(unit)));
+        __syncthreads();      // every thread has read thr[r] (the row maximum) and tie[r] == unresolved before they are replaced
         if (tid == 0) {
             a.thr[r] = thr;
             a.lse_kept[r] = lse_kept;
@@ -818,9 +961,8 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
                 a.logprob[r] = lp;
                 if (a.logprob_full) a.logprob_full[r] = lpf;
             }
+            a.tie[r] = tie;
         }
-        __syncthreads();      // every thread has read tie[r] == unresolved before it is replaced
-        if (tid == 0) a.tie[r] = tie;
     }
 }
 
