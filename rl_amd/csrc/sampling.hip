@@ -482,6 +482,9 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
     };
     constexpr int kBatch = 4;
     for (int i0 = tid; i0 < n_items; i0 += kBatch * kSelBlock) {
+        // a list that has overflowed is not used (the bound is raised, or the row goes to the wide kernel): stop feeding
+        // it -- on a flat row every element would otherwise queue up on the one counter
+        if (*reinterpret_cast<volatile int*>(&sh.count) > CAP) break;
         int64_t vi[kBatch];
         u32x4 q[kBatch];
 #pragma unroll
@@ -686,15 +689,16 @@ template <typename T> __device__ __forceinline__ T wide_scan_excl(T v, T* shm, T
     return base + inc - v;
 }
 
-// exp(x - m) as a fixed-point integer with fx_shift fraction bits (x <= m); zero below its resolution
+// exp(x - m) as a fixed-point integer with fx_shift fraction bits (x <= m, 23 <= fx_shift <= 46); zero below its
+// resolution.  Without branches: the 24-bit significand is placed where the value 1.0 belongs and moved down by
+// the exponent's distance from 1.0's.
 __device__ __forceinline__ unsigned long long wide_mass(float x, float m, int fx_shift) {
-    const uint32_t b = __float_as_uint(fast_exp2((x - m) * kLog2e));
-    int ex = static_cast<int>((b >> 23) & 0xffu);
-    if (ex == 0 || ex == 255 || (b >> 31)) return 0ull;  // zero / subnormal; never infinite or NaN for finite x <= m
-    if (ex > 127) ex = 127;
-    const unsigned long long mant = (b & 0x7fffffu) | 0x800000u;
-    const int sh = ex + fx_shift - 150;
-    return sh >= 0 ? mant << sh : (sh > -24 ? mant >> (-sh) : 0ull);
+    const uint32_t b = __float_as_uint(fast_exp2((x - m) * kLog2e)) & 0x7fffffffu;
+    const int ex = static_cast<int>(b >> 23);
+    const unsigned long long top = static_cast<unsigned long long>((b & 0x7fffffu) | 0x800000u) << (fx_shift - 23);
+    int down = 127 - ex;              // 0 for 1.0; 127 for zero and subnormals (flushed); negative never for x <= m
+    down = down < 0 ? 0 : down > 63 ? 63 : down;
+    return ex == 255 ? 0ull : top >> down;   // (a NaN logit weighs nothing)
 }
 
 template <int DT, int TEMP> struct WideRow {
@@ -705,8 +709,22 @@ template <int DT, int TEMP> struct WideRow {
     // f(scaled logit, vocabulary index) for every element of the row, each exactly once
     template <typename F> __device__ __forceinline__ void for_each(F f) const {
         constexpr int EPV = Row<DT>::EPV;
+        constexpr int kLoads = 8;  // vector loads in flight per thread: a pass is bound by their latency otherwise
         const int tid = threadIdx.x;
-        for (int64_t vi = tid; vi < nvec; vi += kSelBlock) {
+        int64_t vi = tid;
+        for (; vi + (kLoads - 1) * kSelBlock < nvec; vi += kLoads * kSelBlock) {
+            u32x4 q[kLoads];
+#pragma unroll
+            for (int u = 0; u < kLoads; ++u) q[u] = xv[vi + u * kSelBlock];
+#pragma unroll
+            for (int u = 0; u < kLoads; ++u) {
+                float t[EPV];
+                Row<DT>::decode(q[u], t);
+#pragma unroll
+                for (int k = 0; k < EPV; ++k) f(scale_logit<DT, TEMP>(t[k], tparam), head + (vi + u * kSelBlock) * EPV + k);
+            }
+        }
+        for (; vi < nvec; vi += kSelBlock) {
             float t[EPV];
             Row<DT>::decode(xv[vi], t);
 #pragma unroll
@@ -718,8 +736,9 @@ template <int DT, int TEMP> struct WideRow {
 };
 
 // One histogram pass: bin = digit `level` of the keys whose higher digits equal `prefix` (every key at level 0).
-// Thread b returns the number of such elements in bin b and their mass.
-template <int DT, int TEMP>
+// Thread b returns the mass of such elements in bin b and, with CNT, their number (0 otherwise: the top-p descent
+// needs counts at its last digit only, and every atomic less shortens the pass).
+template <int DT, int TEMP, bool CNT>
 __device__ __forceinline__ void wide_hist_pass(const WideRow<DT, TEMP>& w, WideShared& sh, float m, int fx_shift, int level,
                                                uint32_t prefix, unsigned int& my_cnt, unsigned long long& my_mass) {
     const int tid = threadIdx.x;
@@ -732,7 +751,7 @@ __device__ __forceinline__ void wide_hist_pass(const WideRow<DT, TEMP>& w, WideS
     if (level == 0) {
         w.for_each([&](float x, int64_t) {
             const int slot = static_cast<int>((order_key(x) >> shift) & mask) * kRadixCopies + copy;
-            atomicAdd(&sh.cnt[slot], 1u);
+            if (CNT) atomicAdd(&sh.cnt[slot], 1u);
             atomicAdd(&sh.mass[slot], wide_mass(x, m, fx_shift));
         });
     } else {
@@ -740,7 +759,7 @@ __device__ __forceinline__ void wide_hist_pass(const WideRow<DT, TEMP>& w, WideS
             const uint32_t key = order_key(x);
             if ((key >> (shift + bits)) == prefix) {
                 const int slot = static_cast<int>((key >> shift) & mask) * kRadixCopies + copy;
-                atomicAdd(&sh.cnt[slot], 1u);
+                if (CNT) atomicAdd(&sh.cnt[slot], 1u);
                 atomicAdd(&sh.mass[slot], wide_mass(x, m, fx_shift));
             }
         });
@@ -792,7 +811,8 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
         uint32_t hprefix[KD::N];
         int h_levels = 1;
         hprefix[0] = 0u;
-        wide_hist_pass<DT, TEMP>(w, sh, m, fx_shift, 0, 0u, hc[0], hm[0]);
+        if (use_k) wide_hist_pass<DT, TEMP, true>(w, sh, m, fx_shift, 0, 0u, hc[0], hm[0]);
+        else wide_hist_pass<DT, TEMP, KD::N == 1>(w, sh, m, fx_shift, 0, 0u, hc[0], hm[0]);
         unsigned long long total_mass = 0ull;
         wide_scan_excl(hm[0], sh.scan64, total_mass);
 
@@ -807,7 +827,7 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
             for (int l = 0; l < KD::N; ++l) {
                 if (l > 0) {
                     hprefix[l] = prefix;
-                    wide_hist_pass<DT, TEMP>(w, sh, m, fx_shift, l, prefix, hc[l], hm[l]);
+                    wide_hist_pass<DT, TEMP, true>(w, sh, m, fx_shift, l, prefix, hc[l], hm[l]);
                     h_levels = l + 1;
                 }
                 unsigned int tot_c = 0u;
@@ -849,15 +869,16 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_wide_kernel(SelArgs a, in
             for (int l = 0; l < KD::N; ++l) {
                 unsigned int bc = hc[l];
                 unsigned long long bm = hm[l];
-                if (l >= h_levels || hprefix[l] != prefix) wide_hist_pass<DT, TEMP>(w, sh, m, fx_shift, l, prefix, bc, bm);
-                unsigned int tot_c = 0u;
+                if (l >= h_levels || hprefix[l] != prefix) {
+                    if (l == KD::N - 1) wide_hist_pass<DT, TEMP, true>(w, sh, m, fx_shift, l, prefix, bc, bm);
+                    else wide_hist_pass<DT, TEMP, false>(w, sh, m, fx_shift, l, prefix, bc, bm);
+                }
                 unsigned long long tot_m = 0ull;
-                const unsigned int excl_c = wide_scan_excl(bc, sh.scan32, tot_c);
                 const unsigned long long excl_m = wide_scan_excl(bm, sh.scan64, tot_m);
                 // the bin in which the cumulative mass first exceeds the room; if it never does (top_p -> 0), the
-                // highest bin that holds anything: the largest element always survives
+                // highest bin with any mass, which holds the largest element: that one always survives
                 const bool crossing = tot_m > room ? (excl_m + bm > room && excl_m <= room)
-                                                   : (bc > 0u && tot_c - excl_c - bc == 0u);
+                                                   : (bm > 0ull && tot_m - excl_m - bm == 0ull);
                 if (crossing) {
                     sh.pick_bin = static_cast<unsigned int>(tid);
                     sh.pick_cnt = bc;
