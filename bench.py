@@ -592,6 +592,30 @@ def bench_topk(args, torch, w):
                     "(3 x V bytes per token)"},
     }
     del mbs
+    torch.cuda.empty_cache()
+    # ---- flat rows: top-p alone over N(0, 1) logits (an early-training policy) -- every row's nucleus is far wider
+    # than the on-chip candidate list, so every row is finished by the radix descent of topk_topp_wide_kernel ----
+    flat_rows = w["mb_seqs"] * w["seq_len"] if full else min(4096, w["mb_seqs"] * w["seq_len"])
+    gen = torch.Generator(device=dev).manual_seed(4044)
+    flat = torch.empty((1, flat_rows + 1, w["vocab"]), dtype=torch.bfloat16, device=dev).normal_(0.0, 1.0, generator=gen)
+    flat_ids = torch.randint(0, w["vocab"], (1, flat_rows + 1), generator=gen, device=dev)
+    flat_params = TrainingSamplingParams(top_k=None, top_p=w["top_p"], temperature=1.0)
+
+    def flat_step():
+        with torch.no_grad():
+            get_next_token_logprobs_from_logits(flat_ids, flat, sampling_params=flat_params)
+
+    f_elapsed, fk = timed(torch, ops, args, flat_step)
+    f_ms = fk.get("topk_topp_fwd", nan)["avg_ms"]
+    result["c4_flat"] = {
+        "value": flat_rows * args.steps / f_elapsed, "unit": "tokens/s", "ms_per_step": f_elapsed / args.steps * 1e3,
+        "rows": flat_rows, "us_per_row": f_ms * 1e3 / flat_rows,
+        "roofline": hbm_roofline("topk_topp_fwd_kernel + topk_topp_wide_kernel (every row wide)", row_bytes * flat_rows, f_ms),
+        "note": "forward only: top_p=%.2f alone on bf16 N(0,1) logits; the kept set of every row (~10^5 ids) exceeds the "
+                "4096-entry candidate list, so the forward marks the row and the wide kernel finds threshold, tie index and "
+                "kept log-sum-exp in three more passes over the row (two key digits + the tie search); algorithmic bytes = "
+                "one read of the row" % w["top_p"]}
+    del flat
     finish(result, args, torch, w, "topk", cpu_rows=256, gpu_rows=2048)
 
 

@@ -144,6 +144,11 @@ WIDE = [
     (3000, 1.0, 20000, 2.5, torch.float32),      # top_k beyond the candidate list's reach
     (3000, 0.8, 20000, 1.0, torch.float32),
     (5000, 0.9, 8199, 1.0, torch.bfloat16),      # bf16: many exact ties at both boundaries
+    (None, 0.95, 40000, 1.0, torch.float16),     # fp16 keys: two 8-bit digits and one of three bits
+    (6000, 0.9, 151936, 1.0, torch.float16),
+    (8000, 0.7, 151936, 3.0, torch.bfloat16),    # the top-k and the top-p threshold lie in different leading digits
+    (None, 0.999, 151936, 1.0, torch.float32),   # four digits, the threshold among the negative logits
+    (20000, 0.6, 50257, 1.5, torch.float32),
 ]
 
 
@@ -450,3 +455,22 @@ def test_record_backward_written_over_the_logits(dtype, vocab):
     torch.cuda.synchronize()
     bits = torch.int16 if dtype != torch.float32 else torch.int32
     assert torch.equal(over.view(bits), want.view(bits))
+
+
+def test_wide_rows_come_out_the_same_every_time():
+    """The histograms of the wide-row kernel are filled with LDS atomics in whatever order the waves arrive; its
+    masses are integers, so the sums, and with them threshold, tie index and log-sum-exp, do not depend on that
+    order: repeated calls agree bit for bit."""
+    from rl_amd._lib import NRL_TEMP_RCP
+
+    g = torch.Generator().manual_seed(5)
+    vocab, n = 151936, 24
+    x = torch.randn(1, n + 1, vocab, generator=g).to(torch.bfloat16).to(DEV)
+    t = torch.randint(0, vocab, (1, n), generator=g).to(DEV)
+    ops = torch.ops.rl_amd
+    first = ops.topk_topp_logprob_fwd(x, t, n, 0, 0.95, 0.7, NRL_TEMP_RCP, True)
+    assert bool((first[2] >= 0).all())                       # every row resolved
+    for _ in range(4):
+        again = ops.topk_topp_logprob_fwd(x, t, n, 0, 0.95, 0.7, NRL_TEMP_RCP, True)
+        for a, b in zip(first, again):
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32))
