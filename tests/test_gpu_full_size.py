@@ -163,6 +163,84 @@ def test_config4_microbatch_topk_topp_full_vocab():
     assert torch.equal(streamed.view(torch.int16), gx.view(torch.int16))
 
 
+def test_config4_as_benchmarked_deferred_temperature_full_vocab():
+    """Config 4 the way ``bench.py --workload c4`` runs it with the divide left to the kernels: ``apply_temperature_scaling``
+    inside ``deferred_temperature()`` (the logits stay undivided in memory), ``prepare_loss_input`` with top-k 50 /
+    top-p 0.95 -> DAPO clip-higher loss -> backward from the forward's kept-set record, at V = 151936 bf16.  Against the
+    oracle on sampled rows: the divide as a GPU ``div_`` rounds it (``x * fp32(1/T)`` narrowed to bf16), the filtered
+    log-softmax, and autograd through both, i.e. the gradient rounded to bf16 twice."""
+    from functools import partial
+
+    from rl_amd.algorithms.loss import prepare_loss_input
+    from rl_amd.temperature import apply_temperature_scaling, deferred_temperature
+
+    b, s, v, temp = 2, 8192, V_QWEN, 0.7
+    g = torch.Generator().manual_seed(4104)
+    logits = _randn_bf16((b, s, v), 3.0, 4104)
+    rcp = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(temp, dtype=torch.float32)
+    ids = torch.randint(0, v, (b, s), generator=g)
+    top = torch.stack([logits[bi].float().argmax(-1) for bi in range(b)]).cpu()
+    ids[:, 1:] = torch.where(torch.rand(b, s - 1, generator=g) < 0.8, top[:, :-1], ids[:, 1:])
+    params = TrainingSamplingParams(top_k=50, top_p=0.95, temperature=temp)
+    tm = torch.ones(b, s, dtype=torch.int64)
+    tm[:, :300] = 0
+    gen = torch.Generator().manual_seed(7)
+    keep_bits = logits.clone()
+    leaf = logits.requires_grad_(True)
+    fn = ClippedPGLossFn(ClippedPGLossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0))
+    with torch.no_grad(), deferred_temperature():
+        cur = MU.get_next_token_logprobs_from_logits(ids.to(DEV), apply_temperature_scaling(leaf.detach(), params), sampling_params=params)
+    cur0 = torch.nan_to_num(cur, neginf=0.0).cpu()
+    prev = torch.cat([torch.zeros(b, 1), cur0 + 0.05 * torch.randn(b, s - 1, generator=gen)], 1)
+    data = {"input_ids": ids, "token_mask": tm, "sample_mask": torch.ones(b), "advantages": torch.randn(b, 1, generator=gen).expand(b, s).contiguous(),
+            "prev_logprobs": prev, "generation_logprobs": prev}
+    ddev = {k: t.to(DEV) for k, t in data.items()}
+    gs = torch.tensor(float(b), device=DEV)
+    gt = tm[:, 1:].sum().float().to(DEV)
+    prepare = partial(prepare_loss_input, sampling_params=params)
+    with deferred_temperature():
+        x = apply_temperature_scaling(leaf, params)     # deferred: the tensor is not touched, so a leaf may go in
+        assert x is leaf
+        loss_input, prepared = prepare(logits=x, data=ddev, loss_fn=fn)
+        loss, metrics = fn(data=prepared, global_valid_seqs=gs, global_valid_toks=gt, **loss_input)
+    loss.backward()
+    assert torch.equal(leaf.detach().view(torch.int16), keep_bits.view(torch.int16))      # never divided in memory
+    lp = loss_input["next_token_logprobs"].detach()
+    assert bool(torch.isfinite(lp).all())                     # -inf targets were masked to 0 by prepare_loss_input
+    gx = leaf.grad
+    assert bool((gx[:, :299] == 0).all()) and bool((gx[:, -1] == 0).all())
+    # the whole step on the CPU for a few sequences' worth of sampled rows
+    picks = [(0, 299), (0, 300), (0, 4095), (1, 1017), (1, 8190), (1, 5000), (0, 7777)]
+    rows = torch.stack([keep_bits[bi, si].cpu() for bi, si in picks])                     # bf16, undivided
+    tgt = torch.stack([ids[bi, si + 1] for bi, si in picks])
+    xo = rows.clone().requires_grad_(True)
+    scaled = (xo.float() * rcp).to(torch.bfloat16)                                          # logits.div_(T) as the GPU rounds it
+    want_lp = OL.rows_logprob_sampled(scaled.float(), tgt, 50, 0.95)
+    finite = torch.isfinite(want_lp.detach())
+    got_lp = torch.stack([lp[bi, si] for bi, si in picks]).cpu()
+    live = torch.tensor([float(tm[bi, si + 1]) for bi, si in picks]) > 0
+    ok = finite & live
+    assert ok.any() and (got_lp[ok] - want_lp.detach()[ok]).abs().max().item() <= 2e-3
+    assert bool((got_lp[~ok] == 0).all())
+    # d loss / d logprob of those tokens comes from the loss kernel (pinned elsewhere): take it from autograd of the
+    # oracle loss on the GPU logprobs, then push it through the oracle's logprob backward
+    lpo = lp.cpu().clone().requires_grad_(True)
+    want_loss, _ = O.clipped_pg_loss(O.LossConfig(ratio_clip_min=0.2, ratio_clip_max=0.28, reference_policy_kl_penalty=0.0), lpo,
+                                     {k: t for k, t in data.items()}, gs.cpu(), gt.cpu())
+    want_loss.backward()
+    assert abs(loss.item() - want_loss.item()) <= 1e-4 * abs(want_loss.item()) + 1e-7
+    assert abs(float(metrics["loss"]) - want_loss.item()) <= 1e-4 * abs(want_loss.item()) + 1e-7
+    up = torch.stack([lpo.grad[bi, si] for bi, si in picks])
+    up = torch.where(ok, up, torch.zeros_like(up))
+    (torch.where(ok, want_lp, torch.zeros_like(want_lp)) * up).sum().backward()
+    got_g = torch.stack([gx[bi, si].float().cpu() for bi, si in picks])
+    want_g = xo.grad.float()
+    scale = want_g.abs().max().item()
+    assert scale > 0
+    assert (got_g == want_g).float().mean().item() > 0.999       # rows of zeros with a few dozen entries
+    assert bool(((got_g - want_g).abs() <= want_g.abs() * 2 * 2.0 ** -8 + 1e-6 * scale).all())
+
+
 def test_config5_packed_row_full_shape():
     """benchmark config 5: one packed row of 131072 tokens (lengths U[2048, 32768]), V = 131072 bf16."""
     v, total = 131072, 131072
