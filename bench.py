@@ -26,20 +26,36 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+def source_fingerprint(name):
+    """First 12 hex digits of the SHA-256 of ``rl_amd/csrc/<name>``: what a row of the traffic table is tied to."""
+    import hashlib
+
+    try:
+        with open(os.path.join(ROOT, "rl_amd", "csrc", name), "rb") as fh:
+            return hashlib.sha256(fh.read()).hexdigest()[:12]
+    except OSError:
+        return None
+
+
 def load_measured_traffic():
     """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, from the committed table
-    ``profiles/measured_traffic.md`` (key -> dict(kernel, read, write, profile)); each row names the profile
-    summary it was taken from, so a figure that no longer matches its kernel can be traced and re-measured."""
+    ``profiles/measured_traffic.md`` (key -> dict(kernel, read, write, profile)).  Each row names the profile summary
+    it was taken from and the kernel's source file with that file's fingerprint at the time of the measurement; a
+    row whose source has changed since is dropped here, so the JSON line says ``traffic: null`` instead of quoting
+    bytes that belong to another version of the kernel."""
     table = {}
     path = os.path.join(ROOT, "profiles", "measured_traffic.md")
     try:
         with open(path) as fh:
             for line in fh:
                 cells = [c.strip() for c in line.strip().strip("|").split("|")]
-                if len(cells) == 6 and cells[0] not in ("key", "---") and not set(cells[0]) <= set("-"):
+                if len(cells) == 7 and cells[0] not in ("key", "---") and not set(cells[0]) <= set("-"):
                     try:
+                        name, _, stamp = cells[5].partition("@")
+                        if source_fingerprint(name.strip()) != stamp.strip():
+                            continue
                         table[cells[0]] = dict(kernel=cells[1], shape=cells[2], read=float(cells[3]), write=float(cells[4]),
-                                               profile=cells[5])
+                                               profile=cells[6])
                     except ValueError:
                         pass
     except OSError:
@@ -102,6 +118,8 @@ def parse_args():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 4 GiB device-to-device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--source-fingerprints", action="store_true",
+                    help="print the fingerprints of the kernel sources (for the rows of profiles/measured_traffic.md) and exit")
     return ap.parse_args()
 
 
@@ -880,6 +898,12 @@ def main():
 
 def _main():
     args = parse_args()
+    if args.source_fingerprints:
+        import glob
+
+        for path in sorted(glob.glob(os.path.join(ROOT, "rl_amd", "csrc", "*.hip"))):
+            print("%s@%s" % (os.path.basename(path), source_fingerprint(os.path.basename(path))), file=_JSON_OUT)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
