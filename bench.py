@@ -609,6 +609,9 @@ def bench_topk(args, torch, w):
             "note": "deferred_temperature(), without the kept-set record: the backward streams every live row again "
                     "(3 x V bytes per token)"},
     }
+    if not args.no_cpu_baseline:
+        result.update(read_write_ceiling(torch, mbs[0]["logits"].detach(), mbs[0]["data"]["input_ids"],
+                                         read_bytes=rows * row_bytes, write_bytes=rows * row_bytes))
     del mbs
     torch.cuda.empty_cache()
     # ---- flat rows: top-p alone over N(0, 1) logits (an early-training policy) -- every row's nucleus is far wider
@@ -678,6 +681,10 @@ def bench_distill(args, torch, w):
         "roofline": hbm_roofline(worst, passes[worst] * tensor_bytes, km[worst]["avg_ms"]),
         "kernels": kernels,
     }
+    if not args.no_cpu_baseline:
+        ids0 = torch.zeros(student.shape[:2], dtype=torch.int64, device=student.device)
+        nbytes = student.numel() * student.element_size()
+        result.update(read_write_ceiling(torch, student.detach(), ids0, read_bytes=nbytes, write_bytes=nbytes))
     del student, teacher
     finish(result, args, torch, w, "distill", cpu_rows=512, gpu_rows=2048)
 
@@ -713,6 +720,9 @@ def bench_post(args, torch, w):
         "roofline": hbm_roofline("logprob_post_fwd_kernel", live_rows * v * 2, km["logprob_post_fwd"]["avg_ms"]),
         "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in km.items()},
     }
+    if not args.no_cpu_baseline:
+        result.update(read_write_ceiling(torch, logits, ids, read_bytes=result["roofline"]["algorithmic_bytes_per_launch"],
+                                         write_bytes=0))
     del logits
     finish(result, args, torch, w, "post", cpu_rows=4096, gpu_rows=4096)
 
@@ -799,6 +809,9 @@ def bench_packed(args, torch, w):
                "backward -> nrl_logprob_packed_bwd",
         "kernel_ms": {k: round(x["avg_ms"], 4) for k, x in tk.items()},
     }
+    if not args.no_cpu_baseline:
+        out.update(read_write_ceiling(torch, logits.detach(), torch.zeros((1, total), dtype=torch.int64, device=dev),
+                                      read_bytes=live_rows * row_bytes, write_bytes=total * row_bytes))
     del logits
     finish(out, args, torch, w, "packed", cpu_rows=2048, gpu_rows=4096)
 
