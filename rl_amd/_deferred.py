@@ -66,6 +66,14 @@ def pending_temperature(logits: Any) -> float:
     return 1.0
 
 
+def drop_record(logits: torch.Tensor) -> None:
+    """Forgets what is on record for the storage of ``logits`` (its divide has been applied)."""
+    if getattr(_state, "depth", 0) == 0:
+        return
+    storage = logits.untyped_storage()
+    _state.pending = [e for e in _state.pending if e[0]() is not None and e[0]() is not storage]
+
+
 def refuse_pending(logits: Any, what: str) -> None:
     """For entry points that read logits but have no fused temperature: fail instead of reading unscaled values."""
     t = pending_temperature(logits)

@@ -33,6 +33,12 @@ def prepare_loss_input(
 ) -> tuple[dict[str, Any], Any]:
     """``loss/utils.py:37-120``.  Returns ``({"next_token_logprobs": [B, S-1]}, data)``; with top-k /
     top-p active ``data`` gains ``curr_logprobs_unfiltered`` when the loss has a KL penalty."""
+    if loss_fn.input_type != LossInputType.LOGPROB or getattr(loss_fn, "use_fused_linear_logprobs", False):
+        # these readers have no fused temperature (the loss takes the logits as they are, or reduces them with
+        # kernels that do not scale): a divide left to the kernels by deferred_temperature() is applied here
+        from ...temperature import materialise_pending
+
+        logits = materialise_pending(logits)
     if loss_fn.input_type == LossInputType.LOGIT:
         return {"logits": logits}, data
     if loss_fn.input_type == LossInputType.DISTILLATION:  # ``loss/utils.py:122-141``

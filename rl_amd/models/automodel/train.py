@@ -1,4 +1,5 @@
-"""``LogprobsPostProcessor`` (``nemo_rl/models/automodel/train.py:655-864``) on the HIP kernels.
+"""The DTensor worker's post-processors (``nemo_rl/models/automodel/train.py:540-864``) on the HIP kernels and the
+function that feeds them, ``forward_with_post_processing_fn`` (``:308-441``).
 
 The policy worker runs this forward-only pass twice per step (``prev_logprobs`` and
 ``reference_policy_logprobs``) on the same logits shapes as training.  Here one launch emits the
@@ -22,6 +23,100 @@ from ...algorithms.logits_sampling_utils import TrainingSamplingParams, need_top
 from ...algorithms.loss.utils import mask_out_neg_inf_logprobs
 from ...distributed import model_utils as MU
 from ...temperature import apply_temperature_scaling, deferred_temperature  # noqa: F401
+
+
+# The model-side helpers of ``forward_with_post_processing_fn`` (``model_forward``, ``extract_logits``,
+# ``_needs_kv_cache_for_shared_layers``) and the post-processors this package does not replace
+# (``TopkLogitsPostProcessor``, ``FullLogitsPostProcessor``, ``ScorePostProcessor``) are the install's own: they are
+# looked up in the globals of the function this one replaces.  A caller without an install may provide them here.
+MODEL_HELPERS: Optional[dict] = None
+
+
+def _helpers() -> dict:
+    if MODEL_HELPERS is not None:
+        return MODEL_HELPERS
+    from ...compat import original
+
+    theirs = original("nemo_rl.models.automodel.train", "forward_with_post_processing_fn")
+    if theirs is None:
+        raise NotImplementedError("forward_with_post_processing_fn runs the model with the helpers of a NeMo-RL install "
+                                  "(model_forward, extract_logits); none is installed and MODEL_HELPERS is not set")
+    return theirs.__globals__
+
+
+def forward_with_post_processing_fn(
+    model: Any,
+    post_processing_fn: Any,
+    processed_mb: Any,
+    is_reward_model: bool = False,
+    allow_flash_attn_args: bool = True,
+    global_valid_seqs: Optional[torch.Tensor] = None,
+    global_valid_toks: Optional[torch.Tensor] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+    sequence_dim: int = 1,
+):
+    """``models/automodel/train.py:308-441``: model forward, temperature, post-processing; same arguments, same
+    ``(result, metrics, processed_mb)``.
+
+    The one difference is where the temperature divide happens.  The reference divides the logits tensor in place
+    and hands it to the post-processor, and autograd later sends the gradient back through that divide: two read +
+    write passes over ``[B, S, V]``.  When the post-processor is this package's ``LossPostProcessor`` or
+    ``LogprobsPostProcessor`` nothing else reads the tensor in between (it is deleted on return), so the divide is
+    left to the kernel that reads the logits next (``deferred_temperature``), with the same roundings of value and
+    gradient; a loss that takes the raw logits gets them divided after all (``materialise_pending``).  Every other
+    post-processor sees the in-place divide."""
+    h = _helpers()
+    data_dict = processed_mb.data_dict
+    processed_inputs = processed_mb.processed_inputs
+    kv_cache = h.get("_needs_kv_cache_for_shared_layers")
+    outputs = h["model_forward"](model, processed_inputs, is_reward_model=is_reward_model,
+                                 allow_flash_attn_args=allow_flash_attn_args,
+                                 use_cache=kv_cache(model) if kv_cache is not None else False)
+    logits = h["extract_logits"](model, outputs)
+    del outputs
+
+    def is_a(name):
+        cls = h.get(name)
+        return cls is not None and isinstance(post_processing_fn, cls)
+
+    ours = isinstance(post_processing_fn, (LossPostProcessor, LogprobsPostProcessor))
+    defer = ours and type(logits) is torch.Tensor and logits.is_cuda
+    with (deferred_temperature() if defer else _nothing()):
+        if ours or is_a("TopkLogitsPostProcessor") or is_a("FullLogitsPostProcessor"):
+            logits = apply_temperature_scaling(logits, sampling_params)
+        if isinstance(post_processing_fn, LossPostProcessor):
+            result, metrics = post_processing_fn(
+                logits=logits, data_dict=data_dict, processed_inputs=processed_inputs, global_valid_seqs=global_valid_seqs,
+                global_valid_toks=global_valid_toks, sequence_dim=sequence_dim)
+        elif isinstance(post_processing_fn, LogprobsPostProcessor) or is_a("TopkLogitsPostProcessor"):
+            result = post_processing_fn(
+                logits=logits, data_dict=data_dict, processed_inputs=processed_inputs,
+                original_batch_size=processed_mb.original_batch_size, original_seq_len=processed_mb.original_seq_len,
+                sequence_dim=sequence_dim)
+            if isinstance(post_processing_fn, LogprobsPostProcessor):
+                metrics = {"logprobs": result}
+            else:
+                vals, idx = result
+                metrics = {"topk_logits": vals, "topk_indices": idx}
+        elif is_a("FullLogitsPostProcessor"):
+            result = post_processing_fn(
+                logits=logits, data_dict=data_dict, processed_inputs=processed_inputs,
+                original_batch_size=processed_mb.original_batch_size, original_seq_len=processed_mb.original_seq_len,
+                sequence_dim=sequence_dim)
+            metrics = {"full_logits": result}
+        elif is_a("ScorePostProcessor"):
+            result = post_processing_fn(logits=logits)
+            metrics = {"scores": result}
+        else:
+            raise TypeError(f"Unknown post-processing function type: {type(post_processing_fn)}")
+    del logits
+    return result, metrics, processed_mb
+
+
+def _nothing():
+    import contextlib
+
+    return contextlib.nullcontext()
 
 
 class LossPostProcessor:

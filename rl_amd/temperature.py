@@ -23,7 +23,7 @@ from typing import Any, Optional
 import torch
 
 from . import ops  # noqa: F401  (registers torch.ops.rl_amd)
-from ._deferred import _state, deferred_temperature, pending_temperature, record_temperature  # noqa: F401
+from ._deferred import _state, deferred_temperature, drop_record, pending_temperature, record_temperature  # noqa: F401
 
 _OPS = torch.ops.rl_amd
 
@@ -51,6 +51,18 @@ class _DivideInPlace(torch.autograd.Function):
         return _OPS.scale_rows(g3, _one(grad.device), ctx.temperature).view(grad.shape), None
 
 
+def _divide_now(logits: torch.Tensor, t: float) -> torch.Tensor:
+    if not logits.is_cuda:
+        raise RuntimeError("rl_amd runs on the GPU only (got CPU logits); there is no CPU fallback")
+    if logits.dim() < 1 or logits.stride(-1) != 1 or not logits.is_contiguous():
+        raise ValueError("apply_temperature_scaling expects a contiguous logits tensor")
+    if torch.is_grad_enabled() and logits.requires_grad:
+        return _DivideInPlace.apply(logits, t)
+    view = logits if logits.dim() == 3 else logits.view(-1, 1, logits.shape[-1])
+    _OPS.scale_rows_(view, _one(logits.device), t)
+    return logits
+
+
 def apply_temperature_scaling(logits: torch.Tensor, sampling_params: Optional[Any]) -> torch.Tensor:
     """Same contract as the reference function: returns ``logits``, divided in place by the temperature
     when there is one and it is not 1.  Inside ``deferred_temperature()`` the divide is left to the
@@ -63,12 +75,21 @@ def apply_temperature_scaling(logits: torch.Tensor, sampling_params: Optional[An
             raise RuntimeError("deferred_temperature() needs GPU logits")
         record_temperature(logits, t)
         return logits
-    if not logits.is_cuda:
-        raise RuntimeError("rl_amd runs on the GPU only (got CPU logits); there is no CPU fallback")
-    if logits.dim() < 1 or logits.stride(-1) != 1 or not logits.is_contiguous():
-        raise ValueError("apply_temperature_scaling expects a contiguous logits tensor")
-    if torch.is_grad_enabled() and logits.requires_grad:
-        return _DivideInPlace.apply(logits, t)
-    view = logits if logits.dim() == 3 else logits.view(-1, 1, logits.shape[-1])
-    _OPS.scale_rows_(view, _one(logits.device), t)
-    return logits
+    return _divide_now(logits, t)
+
+
+def materialise_pending(logits: Any) -> Any:
+    """For a reader without a fused temperature (a loss that takes raw logits, the distillation reductions): a
+    divide that ``apply_temperature_scaling`` left to the kernels is applied now, in place and through autograd
+    exactly as the eager call would have, and taken off the record.  The tensor must be the whole of the recorded
+    storage: dividing a slice would leave the rest of it undivided with nothing on record."""
+    if not isinstance(logits, torch.Tensor):
+        return logits
+    t = pending_temperature(logits)
+    if t == 1.0:
+        return logits
+    if logits.storage_offset() != 0 or logits.numel() * logits.element_size() != logits.untyped_storage().nbytes():
+        raise RuntimeError("a view of logits whose temperature divide is still deferred reached a reader that cannot apply "
+                           "it; hand over the whole tensor, or divide eagerly outside deferred_temperature()")
+    drop_record(logits)
+    return _divide_now(logits, t)

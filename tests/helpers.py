@@ -226,6 +226,15 @@ _STUB_INSTALL = {
         "def apply_temperature_scaling(*a, **k):\n    return 'reference'\n"
         "class LossPostProcessor:\n    origin = 'reference'\n"
         "class LogprobsPostProcessor:\n    origin = 'reference'\n"
+        "class TopkLogitsPostProcessor:\n    def __call__(self, logits, **k):\n        return logits.topk(2).values, logits.topk(2).indices\n"
+        "class FullLogitsPostProcessor:\n    def __call__(self, logits, **k):\n        return logits\n"
+        "class ScorePostProcessor:\n    def __call__(self, logits):\n        return logits.sum(-1)\n"
+        "def _needs_kv_cache_for_shared_layers(model):\n    return False\n"
+        "def model_forward(model, processed_inputs, is_reward_model=False, allow_flash_attn_args=True, use_cache=False):\n"
+        "    return model(processed_inputs)\n"
+        "def extract_logits(model, outputs):\n    return outputs['logits']\n"
+        "def forward_with_post_processing_fn(*a, **k):\n    return 'reference'\n"
+        "def automodel_forward_backward(model, mb, fn, **k):\n    return forward_with_post_processing_fn(model, fn, mb, **k)\n"
         "def is_loss_step(fn):\n    return isinstance(fn, LossPostProcessor)\n"),
     "nemo_rl/models/megatron/__init__.py": "",
     "nemo_rl/models/megatron/train.py": (

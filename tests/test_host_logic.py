@@ -192,6 +192,27 @@ from rl_amd import compat
 
 mode = rl_amd.install()
 again = rl_amd.install()
+
+
+def _forward_dispatch(train):
+    # post-processors this package leaves alone keep working through the replaced forward function (no temperature
+    # here: the in-place divide needs a GPU)
+    import types
+
+    mb = types.SimpleNamespace(data_dict={}, processed_inputs="inputs", original_batch_size=1, original_seq_len=3)
+    x = torch.arange(12.0).view(1, 3, 4)
+    model = lambda inputs: {"logits": x}
+    score, m1, back = train.automodel_forward_backward(model, mb, train.ScorePostProcessor())
+    (vals, idx), m2, _ = train.forward_with_post_processing_fn(model, train.TopkLogitsPostProcessor(), mb, sampling_params=None)
+    full, m3, _ = train.forward_with_post_processing_fn(model, train.FullLogitsPostProcessor(), mb)
+    try:
+        train.forward_with_post_processing_fn(model, object(), mb)
+        unknown = False
+    except TypeError:
+        unknown = True
+    return (back is mb and torch.equal(score, x.sum(-1)) and torch.equal(m1["scores"], score) and torch.equal(vals, x.topk(2).values)
+            and set(m2) == {"topk_logits", "topk_indices"} and full is x and m3["full_logits"] is x and unknown)
+
 import rl_amd.algorithms.loss as mine
 import rl_amd.algorithms.utils as mu
 import rl_amd.algorithms.advantage_estimator as mae
@@ -225,6 +246,8 @@ out = {
     "train.isinstance": train.is_loss_step(object.__new__(mtrain.LossPostProcessor)),
     "train.get_logprobs": train.get_logprobs_from_vocab_parallel_logits.__module__.startswith("rl_amd."),
     "train.untouched": train.allgather_cp_sharded_tensor() == "reference",
+    "train.forward": train.forward_with_post_processing_fn is mtrain.forward_with_post_processing_fn,
+    "train.forward dispatches": _forward_dispatch(train),
     "lf.calculate_kl": lf.calculate_kl is mu.calculate_kl,
     "lf.masked_mean": lf.masked_mean is mu.masked_mean,
     "driver builds ours": type(fn) is mine.ClippedPGLossFn,
