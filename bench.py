@@ -449,10 +449,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
 
 def bench_topk(args, torch, w):
     """Config 4: temperature 0.7 + top-k / top-p filtered training logprobs -> DAPO loss -> dlogits (K3 forward +
-    backward).  The temperature divide is inside the timed region, as in the worker (``apply_temperature_scaling``
-    on the model's output).  Headline: the call sequence with no switch of this package set (an in-place divide pass,
-    the -inf warning printed at once); the opt-in variants (``deferred_temperature()``, ``DEFER_NEG_INF_WARNING``)
-    are rows of their own."""
+    backward).  Headline: the DTensor worker's sequence, ``forward_with_post_processing_fn`` with a ``LossPostProcessor``
+    (model output -> ``apply_temperature_scaling`` -> ``prepare_loss_input`` -> loss), with no switch of this package
+    set; the function leaves the temperature divide to the kernels because this package's post-processor reads the
+    logits next.  Rows of their own: the -inf warning printed at once, the divide as an in-place pass of its own (the Megatron
+    worker's step), the backward without the kept-set record, and a forward over flat rows."""
     from functools import partial
 
     from rl_amd import ops
@@ -507,18 +508,36 @@ def bench_topk(args, torch, w):
     one = torch.ones((), device=dev)
     restore_events = []
 
+    # The DTensor worker's own sequence: forward_with_post_processing_fn(model, LossPostProcessor, microbatch, ...)
+    # (models/automodel/train.py:308-441, 593-653), here with the resident logits standing for the model's output.
+    import types
+
+    from rl_amd.models.automodel import train as AT
+
+    AT.MODEL_HELPERS = {"model_forward": lambda model, inputs, **kw: model(inputs), "extract_logits": lambda model, out: out}
+    post = AT.LossPostProcessor(fn, {}, None, None, None, 1, 1, False, params)
+
     def step(defer=True):
         collected = []
         for i in range(n_mb):
             m = mbs[i % n_buf]
-            with (deferred_temperature() if defer else contextlib.nullcontext()):
+            if defer:
+                # (the function leaves the divide to the kernels by itself: this package's post-processor comes next)
+                mb = types.SimpleNamespace(data_dict=m["data"], processed_inputs=None, original_batch_size=w["mb_seqs"],
+                                           original_seq_len=w["seq_len"])
+                loss, metrics, _ = AT.forward_with_post_processing_fn(
+                    lambda inputs: _ModelOutput.apply(m["logits"], anchor), post, mb, global_valid_seqs=tot_seqs,
+                    global_valid_toks=tot_toks, sampling_params=params)
+            else:
+                # the Megatron worker's sequence (models/megatron/train.py:329-336): the divide on its own, in place
                 out = _ModelOutput.apply(m["logits"], anchor)
-                logits = apply_temperature_scaling(out, params)     # eager: one in-place pass over [B, S, V]
+                logits = apply_temperature_scaling(out, params)
                 loss_input, data = prepare(logits=logits, data=m["data"], loss_fn=fn)
                 loss, metrics = fn(data=data, global_valid_seqs=tot_seqs, global_valid_toks=tot_toks, **loss_input)
+                del loss_input, logits, out
             collected.append(worker_scaling(metrics))
             torch.autograd.grad(loss, anchor)
-            del loss, loss_input, logits, out
+            del loss
             if not defer:
                 # Not part of the step: the bench keeps its logits resident, so after an in-place divide it multiplies
                 # them back (a worker gets fresh logits from its model).  Timed with events and taken off the clock.
@@ -537,18 +556,18 @@ def bench_topk(args, torch, w):
         k.get("scale_rows", {}).pop("total_ms", None)
         return total - restore_ms * 1e-3, k, restore_ms / (args.steps * n_mb)
 
-    # Opt-ins of this package, each its own row: the divide left to the kernels (deferred_temperature), and on top of
-    # that the warning about valid tokens whose logprob is -inf printed when its counts have arrived instead of
-    # before mask_out_neg_inf_logprobs returns.  The row without any of them is the headline.
+    # The headline is the DTensor worker's sequence with no switch of this package set.  Rows of their own: the same
+    # with the warning about valid tokens whose logprob is -inf printed before mask_out_neg_inf_logprobs returns, as the
+    # reference prints it (one wait per microbatch), and the divide as a pass of its own.
     from rl_amd.algorithms import utils as AU
 
-    AU.DEFER_NEG_INF_WARNING = True
+    elapsed, k = timed(torch, ops, args, step)
+    AU.flush_neg_inf_warnings()
+    AU.DEFER_NEG_INF_WARNING = False
     try:
         o_elapsed, ok_ = timed(torch, ops, args, step)
     finally:
-        AU.DEFER_NEG_INF_WARNING = False
-        AU.flush_neg_inf_warnings()
-    w_elapsed, wk = timed(torch, ops, args, step)
+        AU.DEFER_NEG_INF_WARNING = True
     # the same step with the backward streaming the logits again instead of using the forward's record of the kept sets
     from rl_amd.distributed import sampling_logprob as SL
 
@@ -559,7 +578,7 @@ def bench_topk(args, torch, w):
     finally:
         SL._record_capacity = record_capacity
     # last, because the in-place divides and their restoring passes leave the logits a few roundings off
-    elapsed, k, restore_avg_ms = timed_eager()
+    e_elapsed, ek, restore_avg_ms = timed_eager()
     nan = dict(avg_ms=float("nan"))
     fwd, bwd = k.get("topk_topp_fwd", nan), k.get("topk_topp_bwd", nan)
     rows = w["mb_seqs"] * w["seq_len"]
@@ -579,13 +598,13 @@ def bench_topk(args, torch, w):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "sequences": w["seqs"], "seq_len": w["seq_len"], "vocab": w["vocab"],
                    "microbatches": n_mb, "resident_logit_buffers": n_buf,
-                   "temperature": "apply_temperature_scaling as the worker calls it: one in-place pass over the logits "
-                                  "(bf16 rounding of a GPU div_) before the loss, one pass over the gradient in the backward",
-                   "neg_inf_warning": "printed before mask_out_neg_inf_logprobs returns (one wait per microbatch)",
-                   "metrics": "worker loop: metrics[k] /= num_global_batches after every loss call, every record read after "
-                              "the last microbatch; no rl_amd-specific switch is set",
-                   "clock": "wall clock of the steps minus the event-timed passes that multiply the resident logits back "
-                            "after each in-place divide (%.3f ms each; a worker's logits come fresh from its model)" % restore_avg_ms},
+                   "api": "forward_with_post_processing_fn(model, LossPostProcessor(ClippedPGLossFn, sampling_params), microbatch, "
+                          "..., sampling_params) of the DTensor worker, then metrics[k] /= num_global_batches and backward, per "
+                          "microbatch; every metrics record read after the last one; no rl_amd-specific switch is set",
+                   "temperature": "apply_temperature_scaling inside that function; because this package's post-processor reads "
+                                  "the logits next, the divide is applied by the kernels (bf16 rounding of a GPU div_, value and "
+                                  "gradient) instead of a pass over the logits",
+                   "neg_inf_warning": "printed when its two counts have arrived from the device (the package's default)"},
         # the forward reads a row once; the backward writes the gradient row (zeros and the <= 64 kept entries the
         # forward left on record) without reading the logits again
         "algorithmic_bytes_per_token": 2 * row_bytes,
@@ -594,20 +613,22 @@ def bench_topk(args, torch, w):
                                  bwd["avg_ms"], "c4" if full else None),
         "roofline_fwd": hbm_roofline("topk_topp_fwd_kernel", row_bytes * w["mb_seqs"] * (w["seq_len"] - 1), fwd["avg_ms"],
                                      "c4_fwd" if full else None),
-        "roofline_temperature": hbm_roofline("scale_rows_kernel (the eager divide and its backward; also the restoring pass)",
-                                             2 * row_bytes * rows, k.get("scale_rows", nan)["avg_ms"]),
         "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in k.items()},
-        "deferred_temperature": row(w_elapsed, wk, "with deferred_temperature(): the divide is applied by the kernels that read "
-                                                    "the logits, no pass of its own; warning printed at once"),
-        "deferred_temperature_and_warning": row(o_elapsed, ok_, "deferred_temperature() and DEFER_NEG_INF_WARNING: no pass for the "
-                                                                "divide, no wait for the warning's counts"),
+        "immediate_warning": row(o_elapsed, ok_, "DEFER_NEG_INF_WARNING = False: mask_out_neg_inf_logprobs waits for its two counts and "
+                                                 "prints the warning before it returns, once per microbatch"),
+        "in_place_divide": dict(
+            row(e_elapsed, ek, "the divide as the Megatron worker's step makes it: apply_temperature_scaling on its own, one "
+                               "in-place pass over the logits, and a second pass when autograd sends the gradient back through it"),
+            roofline=hbm_roofline("scale_rows_kernel (the eager divide and its backward; also the restoring pass)",
+                                  2 * row_bytes * rows, ek.get("scale_rows", nan)["avg_ms"]),
+            clock="wall clock of the steps minus the event-timed passes that multiply the resident logits back after each "
+                  "in-place divide (%.3f ms each; a worker's logits come fresh from its model)" % restore_avg_ms),
         "streaming_backward": {
             "value": tokens * args.steps / s_elapsed, "unit": "tokens/s", "ms_per_step": s_elapsed / args.steps * 1e3,
             "kernel_ms": {n: round(v["avg_ms"], 4) for n, v in sk.items()},
             "roofline": hbm_roofline("topk_topp_stream_kernel (backward reading the logits)", 2 * row_bytes * rows,
                                      sk.get("topk_topp_bwd", nan)["avg_ms"], "c4_streaming" if full else None),
-            "note": "deferred_temperature(), without the kept-set record: the backward streams every live row again "
-                    "(3 x V bytes per token)"},
+            "note": "without the kept-set record: the backward streams every live row again (3 x V bytes per token)"},
     }
     if not args.no_cpu_baseline:
         result.update(read_write_ceiling(torch, mbs[0]["logits"].detach(), mbs[0]["data"]["input_ids"],
@@ -906,7 +927,13 @@ _JSON_OUT = sys.stdout
 
 def main():
     with contextlib.redirect_stdout(sys.stderr):
-        return _main()
+        try:
+            return _main()
+        finally:
+            # warnings whose counts were still on their way are printed here, not after the JSON line at exit
+            utils = sys.modules.get("rl_amd.algorithms.utils")
+            if utils is not None:
+                utils.flush_neg_inf_warnings()
 
 
 def _main():

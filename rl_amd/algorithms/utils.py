@@ -160,11 +160,12 @@ def masked_mean(
     return out.reshape(out_shape).to(device=values.device, dtype=out_dtype)
 
 
-# Opt-in (not in the reference): with ``DEFER_NEG_INF_WARNING = True`` the two counts behind the warning of
-# ``mask_out_neg_inf_logprobs`` travel to pinned host memory behind the stream and the warning is printed once they
-# have arrived -- at a later call, at ``flush_neg_inf_warnings()`` or when the interpreter exits -- so the caller's
-# thread keeps queueing work (the backward, the next microbatch) instead of waiting for the forward to finish.
-DEFER_NEG_INF_WARNING = False
+# The warning of ``mask_out_neg_inf_logprobs`` needs two counts from the device.  The reference fetches them and
+# prints before it returns, which stalls the caller's thread until the forward pass has finished, once per
+# microbatch.  Here the counts travel to pinned host memory behind the stream and the same line is printed once they
+# have arrived -- at a later call, at ``flush_neg_inf_warnings()`` or when the interpreter exits -- so the caller keeps
+# queueing work (the backward, the next microbatch).  ``DEFER_NEG_INF_WARNING = False`` prints before returning.
+DEFER_NEG_INF_WARNING = True
 _pending_warnings: list = []  # (event, pinned int64[2], name)
 
 

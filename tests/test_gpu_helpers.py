@@ -125,24 +125,27 @@ def test_masked_mean_closed_forms_and_mask_broadcast():
 
 def test_neg_inf_warning_immediate_and_deferred(capsys):
     """``utils.py:227-257``: masked-out and infinite positions become 0 and the warning counts the valid tokens that
-    were infinite.  With the opt-in switch the same warning is printed once its counts have arrived."""
+    were infinite.  By default the warning is printed once its counts have arrived from the device; with the switch
+    off, before the function returns, as in the reference."""
     from oracle import logprob as OL
 
     lp = torch.tensor([[-1.0, float("-inf"), -2.0, float("-inf")], [-0.5, -0.25, float("-inf"), -3.0]], device=DEV)
     mask = torch.tensor([[1.0, 1.0, 0.0, 0.0], [1.0, 1.0, 1.0, 0.0]], device=DEV)
     want = OL.mask_out_neg_inf_logprobs(lp.cpu(), mask.cpu())
+    assert U.DEFER_NEG_INF_WARNING is True
+    U.flush_neg_inf_warnings()
     capsys.readouterr()
-    got = U.mask_out_neg_inf_logprobs(lp, mask, "curr_logprobs")
-    assert torch.equal(got.cpu(), want)
-    assert "2/5 valid tokens have -inf in curr_logprobs" in capsys.readouterr().out
-    U.DEFER_NEG_INF_WARNING = True
+    U.DEFER_NEG_INF_WARNING = False
     try:
-        got = U.mask_out_neg_inf_logprobs(lp, mask, "prev_logprobs")
-        quiet = U.mask_out_neg_inf_logprobs(lp[:, :1], mask[:, :1], "prev_logprobs")  # nothing infinite: no warning
-        assert torch.equal(got.cpu(), want) and torch.equal(quiet, lp[:, :1])
+        got = U.mask_out_neg_inf_logprobs(lp, mask, "curr_logprobs")
+        assert torch.equal(got.cpu(), want)
+        assert "2/5 valid tokens have -inf in curr_logprobs" in capsys.readouterr().out
     finally:
-        U.DEFER_NEG_INF_WARNING = False
-        U.flush_neg_inf_warnings()
+        U.DEFER_NEG_INF_WARNING = True
+    got = U.mask_out_neg_inf_logprobs(lp, mask, "prev_logprobs")
+    quiet = U.mask_out_neg_inf_logprobs(lp[:, :1], mask[:, :1], "prev_logprobs")  # nothing infinite: no warning
+    assert torch.equal(got.cpu(), want) and torch.equal(quiet, lp[:, :1])
+    U.flush_neg_inf_warnings()
     out = capsys.readouterr().out
     assert out.count("[WARNING]") == 1 and "2/5 valid tokens have -inf in prev_logprobs" in out
     U.flush_neg_inf_warnings()  # nothing left
