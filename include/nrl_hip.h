@@ -165,8 +165,10 @@ int nrl_logprob_packed_bwd(const void* logits, int32_t dtype, int64_t total_toke
  * was filtered out.  logprob_unfiltered_out / lse_full_out (may be NULL): the same row's unfiltered
  * logprob (what the KL penalty needs, loss/utils.py:104-118) from the same pass.
  * Rows whose kept set exceeds the on-chip candidate list (4096 entries: a flat distribution under
- * top-p alone, many exact ties, a top_k in the thousands) take a second, slower kernel in the same
- * call that searches the threshold instead of sorting; there is no limit on top_k or on the kept set.
+ * top-p alone, many exact ties, a top_k in the thousands) take a second kernel in the same call that
+ * finds the threshold by a radix descent over the logits' order keys instead of sorting (two to four
+ * more passes over the row; its sums are integers, so results do not depend on scheduling); there is
+ * no limit on top_k or on the kept set.
  * ------------------------------------------------------------------------------------------ */
 int nrl_topk_topp_logprob_fwd(const nrl_rows* rows, int64_t top_k, float top_p, float* logprob_out,
                               float* thr_out, int32_t* tie_out, float* lse_kept_out,

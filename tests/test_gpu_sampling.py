@@ -154,7 +154,7 @@ WIDE = [
 
 @pytest.mark.parametrize("k,p,vocab,sigma,dtype", WIDE)
 def test_kept_sets_beyond_the_candidate_list(k, p, vocab, sigma, dtype):
-    """Rows whose kept set exceeds the 4096-entry on-chip list take the threshold-search kernel.  Same
+    """Rows whose kept set exceeds the 4096-entry on-chip list take the wide-row kernel (a radix descent over the order keys).  Same
     oracle; the top-p boundary may move by a few near-equal elements (see _boundary_only), which moves
     the kept mass by parts in 1e5, hence the 1e-4 bound on the logprobs."""
     g = torch.Generator().manual_seed(vocab + (k or 7))
@@ -227,7 +227,7 @@ def test_top_p_cut_at_multiples_of_the_wave_width():
 
 def test_wide_rows_with_masked_vocabulary_entries():
     """-inf logits (a masked part of the vocabulary) carry no mass and are never kept, also on the
-    threshold-search path; a top_k that reaches into them keeps only finite entries plus nothing else."""
+    wide-row path; a top_k that reaches into them keeps only finite entries plus nothing else."""
     g = torch.Generator().manual_seed(77)
     vocab = 30011
     x = torch.randn(1, 3, vocab, generator=g) * 0.5
