@@ -8,12 +8,15 @@ tensor (how a GPU ``div_`` by a scalar rounds), differentiable like ``div_``.
 
 That pass costs a full read + write of ``[B, S, V]``.  The logprob kernels can apply the same divide,
 with the same rounding of value and gradient, while they stream the row anyway.  Because nothing in
-the tensor itself can say "not divided yet" without risking a silently unscaled read elsewhere, that is
-an explicit opt-in: inside ``with deferred_temperature():`` ``apply_temperature_scaling`` leaves the
-memory alone and records (storage object, T) for the calling thread, for as long as that storage lives; the logprob / loss entry points of this
+the tensor itself can say "not divided yet" without risking a silently unscaled read elsewhere, a bare
+call never does that: only inside ``with deferred_temperature():`` does ``apply_temperature_scaling`` leave the
+memory alone and record (storage object, T) for the calling thread, for as long as that storage lives; the logprob / loss entry points of this
 package look the logits they are handed up in that record (views of the recorded tensor share its
 storage) and divide inside their kernels.  Whoever opens the context promises that, until it closes,
-only those entry points read the logits.
+only those entry points read the logits -- as ``forward_with_post_processing_fn`` of the DTensor worker's mirror
+does, which knows that a post-processor of this package comes next.  Readers of this package that have no fused
+temperature either refuse such logits or, where they sit on a worker's path (``prepare_loss_input`` for a loss that
+takes raw logits), apply the divide after all (``materialise_pending``).
 """
 
 from __future__ import annotations
