@@ -129,24 +129,31 @@ class StepMetrics(dict):
 
     The reference ends every loss call with about fifteen ``.item()`` calls, each of which stalls the host until
     the device has caught up.  Here the 24-float record of a call travels to pinned host memory behind the kernels
-    and the host does not wait for it: until it is there, ``metrics[key]`` hands out a ``PendingMetric`` and
-    ``metrics[key] = ...`` stores whatever it is given, so the DTensor worker's ``metrics[k] /= num_global_batches``
-    between the loss call and ``backward()`` (``models/automodel/train.py:525-547``) records the division instead of
-    stalling, and the backward pass and the next microbatch are queued while the device is still busy.  Everything
-    that hands out the values wholesale or shows them -- ``items()``, ``values()``, ``get()``, ``pop()``, ``copy()``,
-    ``repr()``, comparison, ``json.dumps``, pickling -- waits for the record first and from then on the mapping holds
-    plain numbers, as it does from the start when the record has already arrived by the time it is first touched
-    (a Megatron worker reads its metrics after ``forward_backward_func`` has returned).  Copies that read the
-    storage directly (``dict(metrics)``, ``{**metrics}``) before that hold ``PendingMetric`` values, each of which
-    still resolves by itself.
+    and the host waits for it only when a value is first needed: ``metrics[key]``, ``items()``, ``values()``,
+    ``get()``, ``pop()``, ``copy()``, ``repr()``, comparison, ``json.dumps`` and pickling all wait once, and from then
+    on the mapping holds plain numbers.  A Megatron worker reads its metrics after ``forward_backward_func`` has
+    returned, by when the records have long arrived, so it never waits.
+
+    The DTensor worker does touch them earlier: ``metrics[k] /= num_global_batches`` between the loss call and
+    ``backward()`` (``models/automodel/train.py:525-547``).  For that caller, which the ``LossPostProcessor`` of that
+    worker's mirror announces with ``defer_scaling()``, ``metrics[key]`` hands out a ``PendingMetric`` while the record
+    is still on its way and ``metrics[key] = ...`` stores whatever it is given, so the division is recorded instead of
+    waited for and the backward pass and the next microbatch are queued while the device is still busy.  Without
+    that announcement every value that leaves the mapping is a plain number, whatever the timing.
     ``loss_fn.lazy_metrics = False`` gives a plain ``dict`` filled before the call returns instead."""
 
     def __init__(self, keys, fetch):
         super().__init__()
         self._fetch = fetch
         self._record = None
+        self._pending_ok = False
         for key in keys:
             dict.__setitem__(self, key, PendingMetric(self, key))
+
+    def defer_scaling(self):
+        """From now on ``metrics[key]`` may hand out a ``PendingMetric`` (see the class text).  Returns ``self``."""
+        self._pending_ok = True
+        return self
 
     def _resolve(self) -> dict:
         if self._record is None:
@@ -162,7 +169,7 @@ class StepMetrics(dict):
             self._resolve()
 
     def __getitem__(self, key):
-        self._settle(False)
+        self._settle(not self._pending_ok)
         return dict.__getitem__(self, key)
 
     def __setitem__(self, key, value):
@@ -177,6 +184,7 @@ class StepMetrics(dict):
     def popitem(self): self._settle(True); return dict.popitem(self)
     def setdefault(self, key, default=None): self._settle(True); return dict.setdefault(self, key, default)
     def copy(self): self._settle(True); return dict(dict.items(self))
+    def __iter__(self): self._settle(not self._pending_ok); return dict.__iter__(self)   # (dict(metrics) comes this way)
     def __eq__(self, other): self._settle(True); return dict.__eq__(self, other)
     def __ne__(self, other): self._settle(True); return dict.__ne__(self, other)
     def __or__(self, other): self._settle(True); return dict.__or__(dict(dict.items(self)), other)

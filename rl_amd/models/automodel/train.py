@@ -160,8 +160,13 @@ class LossPostProcessor:
             wrapped = SequencePackingLossWrapper(loss_fn=self.loss_fn, prepare_fn=prepare, cu_seqlens_q=cu,
                                                  cu_seqlens_q_padded=cu)
             return wrapped(logits, data_dict, global_valid_seqs, global_valid_toks)
-        return wrap_loss_fn_with_input_preparation(logits, data_dict, global_valid_seqs, global_valid_toks, self.loss_fn,
-                                                   prepare)
+        loss, metrics = wrap_loss_fn_with_input_preparation(logits, data_dict, global_valid_seqs, global_valid_toks,
+                                                            self.loss_fn, prepare)
+        if hasattr(metrics, "defer_scaling"):
+            # this worker's loop divides every metric by the number of global batches before it calls backward()
+            # (``train.py:525-547``): let the mapping record that instead of waiting for the device
+            metrics.defer_scaling()
+        return loss, metrics
 
 
 class LogprobsPostProcessor:

@@ -403,8 +403,11 @@ def test_the_worker_loop_does_not_wait_for_the_device_between_loss_and_backward(
     num_global_batches = 4
     collected = []
     torch.cuda._sleep(400_000_000)                     # keeps the device busy (about 0.2 s) while the host runs the loop
+    from rl_amd.models.automodel.train import LossPostProcessor
+
+    post = LossPostProcessor(fn, {}, None, None, None, 1, 1)   # the DTensor worker's post-processor announces the scaling
     for x in xs:                                       # three microbatches queued back to back
-        loss, metrics = fused_logits_clipped_pg_loss(x, ddev, fn, gsd, gtd)
+        loss, metrics = post(logits=x, data_dict=ddev, processed_inputs=None, global_valid_seqs=gsd, global_valid_toks=gtd)
         for k in metrics.keys():
             if "_min" in k or "_max" in k:
                 continue

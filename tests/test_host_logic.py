@@ -135,42 +135,57 @@ def test_step_metrics_wait_only_when_values_are_needed():
     from rl_amd.algorithms.loss.loss_functions import PendingMetric
 
     record = {"loss": 0.5, "probs_ratio_max": 3.0, "num_valid_samples": 4}
+    # as returned by the loss: nothing is fetched until a value is needed, and every value that leaves is a number
+    m, calls = _step_metrics(record, [False])
+    assert isinstance(m, dict) and calls == [] and len(m) == 3 and "loss" in m and list(m.keys()) == list(record)
+    m["lr"] = 1e-5
+    assert calls == []
+    assert type(m["loss"]) is float and calls == [1]
+    m, calls = _step_metrics(record, [False])
+    assert dict(m) == record and all(type(v) in (float, int) for v in dict(m).values()) and calls == [1]
+    m, calls = _step_metrics(record, [False])
+    assert {**m} == record and calls == [1]
+
+    # announced by the DTensor worker's post-processor: what that worker does between the loss call and backward()
+    # fetches nothing
     arrived = [False]
     m, calls = _step_metrics(record, arrived)
-    assert isinstance(m, dict) and calls == []
-    # what the DTensor worker does between the loss call and backward(): nothing is fetched
+    assert m.defer_scaling() is m
     for k in m.keys():
         if "_min" in k or "_max" in k:
             continue
         m[k] /= 4
     m["lr"] = 1e-5
-    assert calls == [] and len(m) == 4 and "loss" in m and list(m.keys())[:3] == list(record)
+    assert calls == [] and len(m) == 4
     assert isinstance(m["loss"], PendingMetric) and calls == []
     # the first real use fetches once; afterwards the mapping holds plain numbers
     assert m["num_valid_samples"] > 0 and calls == [1]
     assert dict.__getitem__(m, "loss") == 0.125 and type(dict.__getitem__(m, "loss")) is float
     assert m == {"loss": 0.125, "probs_ratio_max": 3.0, "num_valid_samples": 1.0, "lr": 1e-5} and calls == [1]
     assert json.loads(json.dumps(m))["loss"] == 0.125
-
-    # a record that has arrived by the first touch (the Megatron worker reads after the schedule returned)
-    arrived = [True]
-    m, calls = _step_metrics(record, arrived)
+    # ... and a record that has arrived by the first touch gives numbers at once
+    m, calls = _step_metrics(record, [True])
+    m.defer_scaling()
     assert type(m["loss"]) is float and calls == [1]
 
-    # every way of handing the values out wholesale waits, once
-    for use in (lambda x: list(x.items()), lambda x: list(x.values()), lambda x: x.get("loss"), lambda x: repr(x),
-                lambda x: x == record, lambda x: x.copy(), lambda x: x.pop("loss"), lambda x: x.setdefault("b", 2),
-                lambda x: json.dumps(x), lambda x: pickle.dumps(x), lambda x: x | {"a": 1},
-                lambda x: float(x["loss"]), lambda x: x["loss"] + 1, lambda x: f"{x['loss']:.3f}", lambda x: x["loss"] < 1):
-        m, calls = _step_metrics(record, [False])
-        use(m)
-        assert calls == [1], use
+    # every way of handing the values out wholesale waits, once, announced or not
+    for announce in (False, True):
+        for use in (lambda x: list(x.items()), lambda x: list(x.values()), lambda x: x.get("loss"), lambda x: repr(x),
+                    lambda x: x == record, lambda x: x.copy(), lambda x: x.pop("loss"), lambda x: x.setdefault("b", 2),
+                    lambda x: json.dumps(x), lambda x: pickle.dumps(x), lambda x: x | {"a": 1},
+                    lambda x: float(x["loss"]), lambda x: x["loss"] + 1, lambda x: f"{x['loss']:.3f}", lambda x: x["loss"] < 1):
+            m, calls = _step_metrics(record, [False])
+            if announce:
+                m.defer_scaling()
+            use(m)
+            assert calls == [1], use
     m, calls = _step_metrics(record, [False])
     restored = pickle.loads(pickle.dumps(m))
     assert type(restored) is dict and restored == record
     # values that escaped before the record arrived still resolve by themselves, scaled as recorded
     m, calls = _step_metrics(record, [False])
-    early = {k: v for k, v in zip(m.keys(), dict.values(m))}
+    m.defer_scaling()
+    early = {k: m[k] for k in m.keys()}
     scaled = early["loss"] / 2 * 3
     assert calls == [] and scaled == 0.75 and calls == [1] and pickle.loads(pickle.dumps(early["loss"])) == 0.5
     assert early["num_valid_samples"] / torch.tensor(2.0) == torch.tensor(2.0)   # a non-number operand resolves at once
