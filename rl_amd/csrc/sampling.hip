@@ -411,26 +411,74 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         return bound_from_bins();
     };
     bool whole_row = true;  // top-p alone: the bound already rests on the whole row
+    bool force_wide = false;  // top-p alone: the chunk maxima show that the kept set cannot fit the candidate list
     if (use_k) {
         if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, mx_key, a.top_k);
     } else {
         clear_bins();
+        // (how many elements the chunks hold whose maxima fall into each bin is counted too, in integers: see below)
+        int* max_cnt = reinterpret_cast<int*>(sh.cand);  // the candidate list is not in use yet
+        if (tid <= kMassBins) max_cnt[tid] = 0;
         __syncthreads();
+        {
+            // this lane's chunks are the lines of the iterations i = lane8, lane8 + 8, ... <= n_full (the ragged last
+            // iteration counted whole); chunk 0 also took one element of the unaligned head and of the tail
+            const int n_full_iter = static_cast<int>(nvec / (kSub * kSelBlock));
+            const int lines = n_full_iter >= lane8 ? (n_full_iter - lane8) / 8 + 1 : 0;
 #pragma unroll
-        for (int u = 0; u < kSub; ++u) bin(mx[u]);
+            for (int u = 0; u < kSub; ++u) {
+                bin(mx[u]);
+                const int elems = lines * 8 * EPV + (u == 0 ? 2 : 0);
+                int j = kMassBins;  // maxima under the first bin's lower edge
+                if (mx[u] > hb) {
+                    j = static_cast<int>((mx[u] - hb) * to_bin);
+                    j = j < kMassBins - 1 ? j : kMassBins - 1;
+                }
+                atomicAdd(&max_cnt[j], elems);
+            }
+        }
         __syncthreads();
         bound_key = bound_from_bins();
         whole_row = bound_key == order_key(b0) + 1u;  // the maxima alone prove nothing: go to the row at once
         if (whole_row) {
-            __syncthreads();  // every wave is done with the bins
-            bound_key = bound_from_row();
+            // A row whose kept set cannot fit the candidate list is not worth the two passes that would find that
+            // out.  No element outweighs the maximum of its chunk, so the CAP heaviest elements of the row weigh at
+            // most what all elements of the chunks with the heaviest maxima would, taken chunk by chunk until CAP
+            // elements are reached, each at its chunk's maximum; if even that stays under top_p, more than CAP
+            // elements are kept and the row goes to the wide kernel now.  The maxima are taken at the upper edge of
+            // their bin and the elements counted in integers, so the decision does not depend on the order in which
+            // atomics arrived (both paths find the same kept set up to near-equal elements at the boundary, but a row
+            // should take the same path every time).
+            static_assert(kMassBins == kWave, "one bin per lane");
+            const int lane_b = tid & (kWave - 1);
+            int c_above = max_cnt[lane_b];   // becomes: elements of the chunks whose maxima lie in bins >= lane_b
+            // their weight, each at the bin's upper edge (the last bin: at probability 1)
+            const float edge = lane_b == kMassBins - 1 ? 0.f : fminf(hb + static_cast<float>(lane_b + 1) / to_bin - lse_full, 0.f);
+            float w_above = static_cast<float>(c_above) * expf(edge);
+#pragma unroll
+            for (int off = 1; off < kWave; off <<= 1) {
+                const int cu = __shfl_down(c_above, off, kWave);
+                const float wu = __shfl_down(w_above, off, kWave);
+                if (lane_b + off < kWave) { c_above += cu; w_above += wu; }
+            }
+            const unsigned long long enough = __ballot(c_above >= CAP);
+            const int jstar = enough ? 63 - __builtin_clzll(enough) : 0;
+            const float w_star = __shfl(w_above, jstar, kWave);
+            const int c_star = __shfl(c_above, jstar, kWave);
+            // chunks whose maxima were not binned lie under hb
+            const float heaviest = w_star + static_cast<float>(c_star < CAP ? CAP - c_star : 0) * expf(hb - lse_full);
+            force_wide = heaviest < 0.98f * a.top_p;
+            if (!force_wide) {
+                __syncthreads();  // every wave is done with the bins
+                bound_key = bound_from_row();
+            }
         }
     }
 
     // ---- pass 2: collect candidates (top-p alone: once more with the bound from the whole row if the list
     // did not hold what the chunk maxima's bound lets through) ----
-    int n = 0;
-    for (;;) {
+    int n = force_wide ? CAP + 1 : 0;
+    for (; !force_wide;) {
     // Only the chunks whose maximum reaches the bound can hold candidates (with top-k that is about k of the
     // 2048 chunks, a few percent of the row).
     auto push = [&](uint32_t key, int64_t index) {
