@@ -416,9 +416,11 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
         if (a.top_k <= kChunks) bound_key = select_kth_largest(sh, mx_key, a.top_k);
     } else {
         clear_bins();
-        // (how many elements the chunks hold whose maxima fall into each bin is counted too, in integers: see below)
+        // (how many elements the chunks hold whose maxima fall into each bin, and what they would weigh if each
+        // weighed as much as its chunk's maximum, is summed too, in integers: see below)
         int* max_cnt = reinterpret_cast<int*>(sh.cand);  // the candidate list is not in use yet
-        if (tid <= kMassBins) max_cnt[tid] = 0;
+        unsigned long long* max_w = sh.cand + kMassBins;  // 32.32 fixed point
+        if (tid <= kMassBins) { max_cnt[tid] = 0; max_w[tid] = 0ull; }
         __syncthreads();
         {
             // this lane's chunks are the lines of the iterations i = lane8, lane8 + 8, ... <= n_full (the ragged last
@@ -435,6 +437,8 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
                     j = j < kMassBins - 1 ? j : kMassBins - 1;
                 }
                 atomicAdd(&max_cnt[j], elems);
+                const float w = expf(fminf(mx[u] - lse_full, 0.f)) * 4294967296.0f;  // NaN (no finite row sum) -> 0
+                atomicAdd(&max_w[j], static_cast<unsigned long long>(w) * static_cast<unsigned long long>(elems));
             }
         }
         __syncthreads();
@@ -445,28 +449,35 @@ __global__ __launch_bounds__(kSelBlock) void topk_topp_fwd_kernel(SelArgs a) {
             // out.  No element outweighs the maximum of its chunk, so the CAP heaviest elements of the row weigh at
             // most what all elements of the chunks with the heaviest maxima would, taken chunk by chunk until CAP
             // elements are reached, each at its chunk's maximum; if even that stays under top_p, more than CAP
-            // elements are kept and the row goes to the wide kernel now.  The maxima are taken at the upper edge of
-            // their bin and the elements counted in integers, so the decision does not depend on the order in which
-            // atomics arrived (both paths find the same kept set up to near-equal elements at the boundary, but a row
-            // should take the same path every time).
+            // elements are kept and the row goes to the wide kernel now.  Counts and weights are summed as integers,
+            // so the decision does not depend on the order in which atomics arrived (both paths find the same kept
+            // set up to near-equal elements at the boundary, but a row should take the same path every time).
             static_assert(kMassBins == kWave, "one bin per lane");
             const int lane_b = tid & (kWave - 1);
             int c_above = max_cnt[lane_b];   // becomes: elements of the chunks whose maxima lie in bins >= lane_b
-            // their weight, each at the bin's upper edge (the last bin: at probability 1)
-            const float edge = lane_b == kMassBins - 1 ? 0.f : fminf(hb + static_cast<float>(lane_b + 1) / to_bin - lse_full, 0.f);
-            float w_above = static_cast<float>(c_above) * expf(edge);
+            unsigned long long w_above = max_w[lane_b];  // their weight, each element at its chunk's maximum
 #pragma unroll
             for (int off = 1; off < kWave; off <<= 1) {
                 const int cu = __shfl_down(c_above, off, kWave);
-                const float wu = __shfl_down(w_above, off, kWave);
+                const unsigned long long wu = __shfl_down(w_above, off, kWave);
                 if (lane_b + off < kWave) { c_above += cu; w_above += wu; }
             }
             const unsigned long long enough = __ballot(c_above >= CAP);
             const int jstar = enough ? 63 - __builtin_clzll(enough) : 0;
-            const float w_star = __shfl(w_above, jstar, kWave);
+            const float w_star = static_cast<float>(__shfl(w_above, jstar, kWave)) * (1.0f / 4294967296.0f);
             const int c_star = __shfl(c_above, jstar, kWave);
             // chunks whose maxima were not binned lie under hb
-            const float heaviest = w_star + static_cast<float>(c_star < CAP ? CAP - c_star : 0) * expf(hb - lse_full);
+            float heaviest = w_star + static_cast<float>(c_star < CAP ? CAP - c_star : 0) * expf(hb - lse_full);
+            if (enough) {
+                // of bin jstar only as many elements as the list still has room for, each at the bin's upper edge
+                const int up = jstar + 1 < kWave ? jstar + 1 : jstar;
+                const unsigned long long w_up = __shfl(w_above, up, kWave);
+                const int c_up = __shfl(c_above, up, kWave);
+                const float w_next = jstar + 1 < kWave ? static_cast<float>(w_up) * (1.0f / 4294967296.0f) : 0.f;
+                const int c_next = jstar + 1 < kWave ? c_up : 0;
+                const float edge = jstar == kMassBins - 1 ? 0.f : fminf(hb + static_cast<float>(jstar + 1) / to_bin - lse_full, 0.f);
+                heaviest = fminf(heaviest, w_next + static_cast<float>(CAP - c_next) * expf(edge));
+            }
             force_wide = heaviest < 0.98f * a.top_p;
             if (!force_wide) {
                 __syncthreads();  // every wave is done with the bins
