@@ -486,6 +486,9 @@ int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* g
  * its logits are fp32 and its memory a quarter).  Both ways give the same gradients: the kept values are the
  * rounded logits the recomputation arrives at.
  * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
+ * Environment: NRL_LMHEAD_ALIGN (read once per process) -- the forward's workgroups that share an L2 wait for
+ * each other before their first tile (unset), before every N-th tile (N > 0), or never (0); the results are
+ * the same either way.
  * ------------------------------------------------------------------------------------------ */
 int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab);
 int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
