@@ -480,27 +480,31 @@ int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* g
  * (row stride ld_dw), accumulated in fp32 and narrowed once.  Tokens are processed in chunks of 16384:
  * per chunk the gradient of the logits exists as bf16 [chunk, V] (twice, one transposed).
  * Kept logits (a choice of the caller, who has the memory or not): with logits_out not NULL the forward
- * also writes the bf16 logits [N, ld_logits] (16-byte aligned, ld_logits a multiple of 8 and >= V; the
- * columns from V on are unspecified), 2 N ld_logits bytes; handed back as logits_kept the backward reads them
- * instead of multiplying hidden and weight a second time (the reference always recomputes, :2249-2262, because
- * its logits are fp32 and its memory a quarter).  Both ways give the same gradients: the kept values are the
- * rounded logits the recomputation arrives at.
+ * also writes the bf16 logits into that buffer (16-byte aligned, nrl_lmhead_kept_logits_bytes(N, V) bytes:
+ * 2 bytes per token and id, both rounded up to multiples of 32); handed back as logits_kept the backward reads
+ * them instead of multiplying hidden and weight a second time (the reference always recomputes, :2249-2262,
+ * because its logits are fp32 and its memory a quarter).  Both ways give the same gradients: the kept values are
+ * the rounded logits the recomputation arrives at.  The buffer is for the backward only; its layout is the one
+ * the matrix instructions leave in registers: blocks of 32 ids x 32 tokens, 2 KiB each, ceil(V / 32) blocks per
+ * token block; inside a block [half p = 0, 1][lane = 32 h + token % 32][8 values], the 8 values being the ids
+ * 16 p + 8 q + 4 h + e of the block (q = 0, 1; e = 0..3).  Ids and tokens past the end hold unspecified values.
  * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
  * Environment: NRL_LMHEAD_ALIGN (read once per process) -- the forward's workgroups that share an L2 wait for
  * each other before their first tile (unset), before every N-th tile (N > 0), or never (0); the results are
  * the same either way.
  * ------------------------------------------------------------------------------------------ */
 int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab);
+int64_t nrl_lmhead_kept_logits_bytes(int64_t n_tokens, int64_t vocab);
 int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                            const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                            int64_t vocab_start, int64_t vocab_end, float* logprob_out, float* lse_out,
-                           void* logits_out, int64_t ld_logits, void* workspace, int64_t workspace_bytes,
+                           void* logits_out, int64_t logits_bytes, void* workspace, int64_t workspace_bytes,
                            void* stream);
 int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab);
 int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                            const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                            int64_t vocab_start, int64_t vocab_end, const float* lse, const float* grad,
-                           const void* logits_kept, int64_t ld_logits, float* dhidden_out, int64_t ld_dh,
+                           const void* logits_kept, int64_t logits_bytes, float* dhidden_out, int64_t ld_dh,
                            void* dweight_out, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
                            void* stream);
 

@@ -114,6 +114,7 @@ SIGNATURES = {
     "nrl_nonzero_indices": (C.c_int, [_P, _I64, _P, _P, _P]),
     "nrl_seq_logprob_error": (C.c_int, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _I64, C.c_int32, C.c_float, _P, _P, _P, _P, _I64, _P]),
     "nrl_lmhead_fwd_workspace_bytes": (_I64, [_I64, _I64]),
+    "nrl_lmhead_kept_logits_bytes": (_I64, [_I64, _I64]),
     "nrl_lmhead_logprob_fwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _P]),
     "nrl_lmhead_bwd_workspace_bytes": (_I64, [_I64, _I64, _I64]),
     "nrl_lmhead_logprob_bwd": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P]),
@@ -124,7 +125,7 @@ SIGNATURES = {
 _lib = None
 
 
-ABI_VERSION = 110  # nrl_version() of the library these signatures describe
+ABI_VERSION = 111  # nrl_version() of the library these signatures describe
 
 
 def load() -> C.CDLL:

@@ -27,6 +27,6 @@ int check_launch(const char* what) {
 
 }  // namespace nrl
 
-extern "C" int nrl_version(void) { return 110; }
+extern "C" int nrl_version(void) { return 111; }
 
 extern "C" const char* nrl_last_error(void) { return nrl::error_slot(); }

@@ -564,6 +564,19 @@ static int64_t patch_grid(int64_t nbx, int64_t nby, int64_t px = 4) {
 // and 16 rows, so with the vocabulary along the rows the whole log-sum-exp reduction of a tile stays
 // inside the lane (NJ token columns per lane, 2 registers of running state each) and no cross-lane
 // traffic happens until the very end.
+// Kept logits are stored as the forward's accumulators hold them, block by block: a block is 32 vocabulary ids x 32
+// tokens, 2 KiB, laid out [half p][lane][8 bf16] with lane = 32 h + token % 32, and the lane's 8 values of half p are
+// the ids 16 p + 8 q + 4 h + e of the block (q = 0, 1; e = 0..3), in that order.  Blocks follow each other along the
+// vocabulary (ceil(V / 32) of them), then along the tokens (ceil(N / 32)).  The forward writes a block with two
+// 1 KiB stores per wave and no shuffle; the backward reads 16 bytes per token and half and regroups in registers.
+// Ids past V and tokens past N of the last blocks hold unspecified values.
+__host__ __device__ __forceinline__ int64_t kept_block(int64_t token_block, int64_t vocab_block, int64_t n_vb) {
+    return (token_block * n_vb + vocab_block) * 2048;
+}
+static int64_t kept_logits_bytes(int64_t n_tokens, int64_t vocab) {
+    return kept_block((n_tokens + 31) / 32, 0, (vocab + 31) / 32);
+}
+
 struct LmFwdArgs {
     GemmOperands op;           // a = W [V,H] (m = V), b = hidden [N,H] (n = N)
     const int64_t* targets;    // [N]
@@ -572,8 +585,8 @@ struct LmFwdArgs {
     float* part_m;             // [n_splits, N]
     float* part_s;             // [n_splits, N]
     float* xt;                 // [N] target logit (written by the tile that holds it)
-    uint16_t* logits;          // [N, ldl] bf16 logits kept for the backward, or NULL
-    int64_t ldl;               // multiple of 8, >= V; columns from V on are unspecified
+    unsigned char* logits;     // bf16 logits kept for the backward in the block layout (kept_block), or NULL
+    int64_t n_vb;              // its vocabulary blocks per token block: ceil(V / 32)
     unsigned int* arrive;      // one zeroed counter per XCD patch of workgroups, or NULL: see patch_cross
     unsigned align_every;      // the patch re-aligns before every align_every-th tile
 };
@@ -610,8 +623,6 @@ constexpr int fwd_patch_tokens(bool save) { return save ? 4 : 8; }
 template <class Core, bool SAVE>
 __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     constexpr int NI = Core::NI, NJ = Core::NJ, BV = Core::BM, BT = Core::BN;  // vocabulary rows x token columns
-    // kept logits leave through LDS when a wave's 128 x 128 sub-tile fits its share of the operand buffers
-    constexpr bool STAGE = SAVE && NI == 4 && NJ == 4 && Core::LDS_BYTES >= (GB_THREADS / 64) * 128 * 128 * 2;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
     __shared__ float comb_m[2][BT], comb_s[2][BT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -665,7 +676,6 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
         // instruction's result needs before another unit reads it is spelled out)
         asm volatile("s_nop 15\n s_nop 7" : "+v"(t2));
         const int lane2 = t2 & 63, wm2 = t2 >> 7, wn2 = (t2 >> 6) & 1;
-        unsigned char* stage = lds + (t2 >> 6) * (128 * 128 * 2);  // STAGE: this wave's quarter of the operand buffers
         const int col = wn2 * (NJ * 32) + (lane2 & 31);  // this lane's token column of tile j is col + j * 32
         // Accumulator element e of tile i is row `off` = i * 32 + 8 * (e / 4) + e % 4 (a compile-time constant)
         // below this lane's first row vb.  Only the last vocabulary tile needs the rows-past-the-end mask.
@@ -694,25 +704,18 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
                         x[e] = (!MASKED || off < limit) ? r : -INFINITY;
                         raw = fmaxf(raw, x[e]);
                     }
-                    if constexpr (STAGE) {
-                        // The lane's 16 values are 4 runs of 4 consecutive vocabulary ids of one token, 8 bytes each.
-                        // They go to the wave's own quarter of the (now idle) operand buffers, laid out [token][id]:
-                        // 16-byte chunk c of token row t at chunk position c ^ (t & 15).
-                        const int t = j * 32 + (lane2 & 31);
+                    if constexpr (SAVE) {
+                        // The block leaves as it lies in the accumulators (kept_block): the lane's 16 values are two
+                        // 16-byte pieces, and the wave's 64 pieces of one half are 1 KiB contiguous, so each of the
+                        // two stores is one full burst, straight from the registers.
+                        const int64_t tb = (tok0 + wn2 * (NJ * 32) + j * 32) >> 5, vblk = (v0 + wm2 * (NI * 32) + i * 32) >> 5;
+                        if (tb * 32 < a.op.n && vblk < a.n_vb) {
+                            unsigned char* out = a.logits + kept_block(tb, vblk, a.n_vb) + lane2 * 16;
 #pragma unroll
-                        for (int q = 0; q < 4; ++q)
-                            *reinterpret_cast<uint2*>(stage + t * 256 + (((4 * i + q) ^ (t & 15)) * 16) + (lane2 >> 5) * 8) =
-                                uint2{pack_bf16x2(x[4 * q], x[4 * q + 1]), pack_bf16x2(x[4 * q + 2], x[4 * q + 3])};
-                    } else if constexpr (SAVE) {
-                        // The lane's 16 values are 4 runs of 4 consecutive vocabulary ids of one token: 8 bytes each,
-                        // next to the 8 bytes of the lane 32 further on; a wave's 4 x 4 blocks fill 256 bytes per token.
-                        if (tok0 + col + j * 32 < a.op.n) {
-                            uint16_t* out = a.logits + (tok0 + col + j * 32) * a.ldl + vb + i * 32;
-#pragma unroll
-                            for (int q = 0; q < 4; ++q)
-                                if (!MASKED || i * 32 + 8 * q < static_cast<int>(a.ldl) - vb)
-                                    *reinterpret_cast<uint2*>(out + 8 * q) =
-                                        uint2{pack_bf16x2(x[4 * q], x[4 * q + 1]), pack_bf16x2(x[4 * q + 2], x[4 * q + 3])};
+                            for (int p = 0; p < 2; ++p)
+                                *reinterpret_cast<u32x4*>(out + p * 1024) =
+                                    u32x4{pack_bf16x2(x[8 * p], x[8 * p + 1]), pack_bf16x2(x[8 * p + 2], x[8 * p + 3]),
+                                          pack_bf16x2(x[8 * p + 4], x[8 * p + 5]), pack_bf16x2(x[8 * p + 6], x[8 * p + 7])};
                         }
                     }
                     const float mx = fmaxf(run_m, round_bf16(raw));
@@ -741,31 +744,6 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
         };
         if (v0 + BV <= a.op.m) fold_tile(std::false_type{});
         else fold_tile(std::true_type{});
-        if constexpr (STAGE) {
-            // The wave's 128 tokens x 128 ids leave as whole 256-byte runs, 16 bytes per lane: a quarter of the
-            // requests the 8-byte pieces of the accumulator layout would make.  All 32 reads go out first (read in
-            // assembly like the fragments: a read the compiler sees would wait for the stores before it).
-            const uint32_t sbase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(stage));
-            const int64_t tokw = tok0 + wn2 * 128, vocw = v0 + wm2 * 128;
-            const int c = lane2 & 15;
-            u32x4 val[32];
-            asm volatile("" ::: "memory");  // the staging writes above are issued before the reads below
-#pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                const int t = 4 * k + (lane2 >> 4);
-                asm volatile("ds_read_b128 %0, %1" : "=v"(val[k]) : "v"(sbase + static_cast<uint32_t>(t * 256 + ((c ^ (t & 15)) * 16))));
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                asm volatile("" : "+v"(val[k]));  // (complete only after the wait above)
-                const int t = 4 * k + (lane2 >> 4);
-                if (tokw + t < a.op.n && vocw + c * 8 < a.ldl)
-                    *reinterpret_cast<u32x4*>(a.logits + (tokw + t) * a.ldl + vocw + c * 8) = val[k];
-            }
-            // every wave is done with its staging area before the next tile's operands land there
-            asm volatile("s_barrier" ::: "memory");
-        }
     }
     float run_m[NJ], run_s[NJ];
 #pragma unroll
@@ -1010,14 +988,16 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_grad_kernel(LmGradArgs a) {
 
 // ---------------------------------------------------------------------------------------------
 // backward from kept logits: the same G and G^T without the product.  One workgroup turns a tile of 128 tokens x
-// 128 vocabulary ids: a thread reads 16 bytes (8 ids) of 4 consecutive live tokens' rows, writes its part of G
+// 128 vocabulary ids: a thread reads 16 bytes of 4 consecutive live tokens (two runs of 4 ids, 8 ids apart: what a
+// lane of the forward held; the neighbouring thread holds the runs in between, and the two swap a run each so that
+// both end up with 8 consecutive ids), writes its part of G
 // straight back (16 bytes of a 256-byte run), and hands the 4 tokens' values of each id to LDS as one 8-byte unit
 // of the transposed tile (unit U of row v at U ^ swizzle(v)), from where G^T leaves in 16-byte pieces after the
 // one-hot term was added to the tokens' target cells.
 // ---------------------------------------------------------------------------------------------
 struct LmGradKeptArgs {
-    const uint16_t* logits;   // [N, ldl] bf16, as the forward left them
-    int64_t ldl;
+    const unsigned char* logits;  // bf16 logits as the forward left them (kept_block)
+    int64_t n_vb;
     const int32_t* row_map;   // [rows] token (row of logits) of live row r
     const int32_t* live;      // device count of live tokens
     int64_t live_from, rows;  // this chunk's live rows are [live_from, live_from + rows) clamped to *live
@@ -1068,8 +1048,26 @@ __global__ __launch_bounds__(256) void lmhead_grad_kept_kernel(LmGradKeptArgs a)
             float sv[8];
 #pragma unroll
             for (int k = 0; k < 8; ++k) sv[k] = 0.f;
-            if (row0 + t < m && c < a.vocab && g_l[t] != 0.f) {
-                const u32x4 raw = *reinterpret_cast<const u32x4*>(a.logits + row_l[t] * a.ldl + c);
+            // (the swap below runs in every lane: whether a token is live is the same for both partners, whether the
+            // ids exist is not)
+            u32x4 raw = u32x4{0u, 0u, 0u, 0u};
+            const bool live = row0 + t < m && g_l[t] != 0.f;
+            if (live && (c & ~15) < a.vocab) {
+                // piece = 4 * (block of the tile) + 2 * (half p) + h
+                const int64_t src = row_l[t];
+                raw = *reinterpret_cast<const u32x4*>(a.logits + kept_block(src >> 5, (col0 >> 5) + (piece >> 2), a.n_vb) +
+                                                     ((piece >> 1) & 1) * 1024 + ((piece & 1) * 32 + (src & 31)) * 16);
+            }
+            {
+                // this lane (h) holds the ids 16 p + 4 h + {0..3} and + 8 + {0..3}; the lane with the other h sits next
+                // to it.  h = 0 keeps its first run and takes the partner's first run, h = 1 takes the partner's
+                // second run and keeps its own second: 8 consecutive ids, the ids c .. c + 7 of the tile.
+                const bool hi = piece & 1;
+                const uint32_t give0 = hi ? raw.x : raw.z, give1 = hi ? raw.y : raw.w;
+                const uint32_t got0 = __shfl_xor(give0, 1, kWave), got1 = __shfl_xor(give1, 1, kWave);
+                raw = hi ? u32x4{got0, got1, raw.z, raw.w} : u32x4{raw.x, raw.y, got0, got1};
+            }
+            if (live && c < a.vocab) {
                 float x[8];
                 Row<NRL_BF16>::decode(raw, x);
                 const float ng = -g_l[t], ls = lse_l[t];
@@ -1390,15 +1388,19 @@ template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, 
                                     dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
 }
 
+extern "C" int64_t nrl_lmhead_kept_logits_bytes(int64_t n_tokens, int64_t vocab) {
+    return n_tokens < 0 || vocab < 0 ? 0 : kept_logits_bytes(n_tokens, vocab);
+}
+
 extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                                       const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                                       int64_t vocab_start, int64_t vocab_end, float* logprob_out, float* lse_out,
-                                      void* logits_out, int64_t ld_logits, void* workspace, int64_t workspace_bytes,
+                                      void* logits_out, int64_t logits_bytes, void* workspace, int64_t workspace_bytes,
                                       void* stream) {
     if (int e = check_lmhead(hidden, n_tokens, hidden_size, ldh, weight, vocab, ldw, targets)) return e;
     if (vocab_end - vocab_start != vocab) return fail(NRL_E_INVALID, "vocab range does not span the rows of W");
-    if (logits_out && (ld_logits < vocab || ld_logits % 8 || (reinterpret_cast<uintptr_t>(logits_out) & 15)))
-        return fail(NRL_E_INVALID, "kept logits need 16-byte aligned rows: ld_logits a multiple of 8, at least the vocabulary");
+    if (logits_out && (logits_bytes < kept_logits_bytes(n_tokens, vocab) || (reinterpret_cast<uintptr_t>(logits_out) & 15)))
+        return fail(NRL_E_INVALID, "kept logits need a 16-byte aligned buffer of nrl_lmhead_kept_logits_bytes() bytes");
     if (n_tokens == 0) return NRL_OK;
     if (!logprob_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
     if (workspace_bytes < nrl_lmhead_fwd_workspace_bytes(n_tokens, vocab)) return fail(NRL_E_WORKSPACE, "workspace too small");
@@ -1407,7 +1409,7 @@ extern "C" int nrl_lmhead_logprob_fwd(const void* hidden, int64_t n_tokens, int6
     a.op.a = static_cast<const uint16_t*>(weight); a.op.b = static_cast<const uint16_t*>(hidden);
     a.op.lda = ldw; a.op.ldb = ldh; a.op.m = vocab; a.op.n = n_tokens; a.op.k = hidden_size;
     a.targets = targets; a.vocab_start = vocab_start;
-    a.logits = static_cast<uint16_t*>(logits_out); a.ldl = ld_logits;
+    a.logits = static_cast<unsigned char*>(logits_out); a.n_vb = (vocab + 31) / 32;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if ((n_tokens + 255) / 256 >= (1ll << 24)) return fail(NRL_E_INVALID, "too many tokens");
     if (hidden_size % CoreB::BK == 0) launch_fwd<CoreB>(a, ws, s);
@@ -1443,13 +1445,13 @@ extern "C" int64_t nrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidd
 extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int64_t hidden_size, int64_t ldh,
                                       const void* weight, int64_t vocab, int64_t ldw, const int64_t* targets,
                                       int64_t vocab_start, int64_t vocab_end, const float* lse, const float* grad,
-                                      const void* logits_kept, int64_t ld_logits, float* dhidden_out, int64_t ld_dh,
+                                      const void* logits_kept, int64_t logits_bytes, float* dhidden_out, int64_t ld_dh,
                                       void* dweight_out, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
                                       void* stream) {
     if (int e = check_lmhead(hidden, n_tokens, hidden_size, ldh, weight, vocab, ldw, targets)) return e;
     if (vocab_end - vocab_start != vocab) return fail(NRL_E_INVALID, "vocab range does not span the rows of W");
-    if (logits_kept && (ld_logits < vocab || ld_logits % 8 || (reinterpret_cast<uintptr_t>(logits_kept) & 15)))
-        return fail(NRL_E_INVALID, "kept logits need 16-byte aligned rows: ld_logits a multiple of 8, at least the vocabulary");
+    if (logits_kept && (logits_bytes < kept_logits_bytes(n_tokens, vocab) || (reinterpret_cast<uintptr_t>(logits_kept) & 15)))
+        return fail(NRL_E_INVALID, "kept logits need a 16-byte aligned buffer of nrl_lmhead_kept_logits_bytes() bytes");
     if (!dweight_out || !workspace) return fail(NRL_E_INVALID, "null output or workspace");
     if (n_tokens > 0 && (!lse || !grad || !dhidden_out)) return fail(NRL_E_INVALID, "null argument");
     if (n_tokens >= (1ll << 31)) return fail(NRL_E_INVALID, "too many tokens");
@@ -1505,7 +1507,7 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         ga.g = g; ga.ldg = vp; ga.gt = gt; ga.ldgt = ld_t;
         if (logits_kept) {
             LmGradKeptArgs ka;
-            ka.logits = static_cast<const uint16_t*>(logits_kept); ka.ldl = ld_logits; ka.row_map = idx + t0; ka.live = count;
+            ka.logits = static_cast<const unsigned char*>(logits_kept); ka.n_vb = (vocab + 31) / 32; ka.row_map = idx + t0; ka.live = count;
             ka.live_from = t0; ka.rows = rows; ka.vocab = vocab; ka.targets = ga.targets; ka.vocab_start = vocab_start;
             ka.lse = ga.lse; ka.grad = ga.grad; ka.g = g; ka.ldg = vp; ka.gt = gt; ka.ldgt = ld_t;
             lmhead_grad_kept_kernel<<<dim3((unsigned)((vp + KT - 1) / KT), (unsigned)((rows + KT - 1) / KT)), dim3(256), 0, s>>>(ka);

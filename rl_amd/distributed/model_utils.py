@@ -453,7 +453,7 @@ LMHEAD_KEEP_FRACTION = 0.25
 def _keep_lmhead_logits(n_tokens: int, vocab: int, device: torch.device, hidden_size: int = 0) -> bool:
     if LMHEAD_KEEP_LOGITS != "auto":
         return bool(LMHEAD_KEEP_LOGITS)
-    need = n_tokens * ((vocab + 7) // 8 * 8) * 2
+    need = ((n_tokens + 31) // 32 * 32) * ((vocab + 31) // 32 * 32) * 2
     free, _ = torch.cuda.mem_get_info(device)
     free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)  # the allocator's own free blocks
     # (and the backward's own workspace and outputs must still fit comfortably next to them)

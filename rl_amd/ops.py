@@ -1265,8 +1265,9 @@ def _ws(nbytes, dev):
 
 
 def _lmhead_logprob_fwd(hidden, weight, targets, vocab_start, vocab_end, keep_logits=False):
-    """-> (logprobs [N], log-sum-exps [N], bf16 logits [N, V] kept for the backward or an empty tensor).  The kept
-    logits are a view of rows padded to a multiple of 8 ids."""
+    """-> (logprobs [N], log-sum-exps [N], the bf16 logits kept for the backward or an empty tensor).  The kept
+    logits are a flat buffer in the layout the kernels exchange (``lmhead_unpack_kept_logits`` turns it into
+    ``[N, V]``)."""
     hidden, weight = _check_lmhead(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
@@ -1275,14 +1276,14 @@ def _lmhead_logprob_fwd(hidden, weight, targets, vocab_start, vocab_end, keep_lo
     with torch.cuda.device(dev):
         lp = torch.empty((n,), dtype=torch.float32, device=dev)
         lse = torch.empty((n,), dtype=torch.float32, device=dev)
-        ldl = (v + 7) // 8 * 8
-        logits = torch.empty((n, ldl), dtype=torch.bfloat16, device=dev)[:, :v] if keep_logits else None
+        logits = torch.empty((lib.nrl_lmhead_kept_logits_bytes(n, v) // 2,), dtype=torch.bfloat16, device=dev) if keep_logits else None
         nbytes = lib.nrl_lmhead_fwd_workspace_bytes(n, v)
         ws = _ws(nbytes, dev)
         with _timed("lmhead_fwd"):
             code = lib.nrl_lmhead_logprob_fwd(
                 _ptr(hidden), n, h, hidden.stride(0), _ptr(weight), v, weight.stride(0), _ptr(targets), vocab_start,
-                vocab_end, _ptr(lp), _ptr(lse), _ptr(logits), ldl, _ptr(ws), ws.numel() * 8, _stream(),
+                vocab_end, _ptr(lp), _ptr(lse), _ptr(logits), 0 if logits is None else logits.numel() * 2, _ptr(ws),
+                ws.numel() * 8, _stream(),
             )
     _lib.check(code, "nrl_lmhead_logprob_fwd")
     return lp, lse, (logits if keep_logits else lp.new_empty(0, dtype=torch.bfloat16))
@@ -1298,27 +1299,35 @@ def _lmhead_logprob_bwd(hidden, weight, targets, lse, grad, vocab_start, vocab_e
             raise ValueError(f"{name} must be a contiguous fp32 [N] tensor")
     if logits is not None and logits.numel() == 0 and n * v > 0:
         logits = None
-    if logits is not None:
-        if logits.dtype != torch.bfloat16 or tuple(logits.shape) != (n, v) or (v > 1 and logits.stride(1) != 1):
-            raise ValueError("kept logits must be the bf16 [N, V] tensor the forward returned")
-        if n > 1 and (logits.stride(0) % 8 or logits.stride(0) < v) or logits.data_ptr() % 16:
-            raise ValueError("kept logits need 16-byte aligned rows")
     lib = _lib.load()
+    if logits is not None:
+        if (logits.dtype != torch.bfloat16 or logits.dim() != 1 or not logits.is_contiguous() or logits.data_ptr() % 16
+                or logits.numel() * 2 != lib.nrl_lmhead_kept_logits_bytes(n, v)):
+            raise ValueError("kept logits must be the bf16 buffer the forward returned for these shapes")
     dev = hidden.device
     with torch.cuda.device(dev):
         dh = torch.empty((n, h), dtype=torch.float32, device=dev)
         dw = torch.empty((v, h), dtype=torch.bfloat16, device=dev)
         nbytes = lib.nrl_lmhead_bwd_workspace_bytes(n, h, v)
         ws = _ws(nbytes, dev)
-        ldl = 0 if logits is None else (logits.stride(0) if n > 1 else (v + 7) // 8 * 8)
         with _timed("lmhead_bwd"):
             code = lib.nrl_lmhead_logprob_bwd(
                 _ptr(hidden), n, h, hidden.stride(0), _ptr(weight), v, weight.stride(0), _ptr(targets), vocab_start,
-                vocab_end, _ptr(lse), _ptr(grad), _ptr(logits), ldl, _ptr(dh), h, _ptr(dw), h, _ptr(ws), ws.numel() * 8,
-                _stream(),
+                vocab_end, _ptr(lse), _ptr(grad), _ptr(logits), 0 if logits is None else logits.numel() * 2, _ptr(dh), h,
+                _ptr(dw), h, _ptr(ws), ws.numel() * 8, _stream(),
             )
     _lib.check(code, "nrl_lmhead_logprob_bwd")
     return dh, dw
+
+
+def lmhead_unpack_kept_logits(kept: torch.Tensor, n_tokens: int, vocab: int) -> torch.Tensor:
+    """The kept logits of ``lmhead_logprob_fwd`` as a bf16 ``[N, V]`` tensor (a copy, for inspection: the backward
+    reads the buffer as it is).  The buffer holds blocks of 32 ids x 32 tokens, ``ceil(V / 32)`` per token block; a
+    block is ``[p][h][token % 32][q][e]`` with id ``16 p + 8 q + 4 h + e``."""
+    n_tb, n_vb = (n_tokens + 31) // 32, (vocab + 31) // 32
+    blocks = kept.view(n_tb, n_vb, 2, 2, 32, 2, 4)  # tb, vb, p, h, token, q, e
+    rows = blocks.permute(0, 4, 1, 2, 5, 3, 6).reshape(n_tb * 32, n_vb * 32)  # (tb, token) x (vb, p, q, h, e)
+    return rows[:n_tokens, :vocab].contiguous()
 
 
 for _name, _fn in (("lmhead_logprob_fwd", _lmhead_logprob_fwd), ("lmhead_logprob_bwd", _lmhead_logprob_bwd)):

@@ -23,6 +23,7 @@ import torch
 
 from oracle import lmhead as OH
 from oracle import logprob as OL
+from rl_amd import ops
 from rl_amd.distributed import model_utils as MU
 
 pytestmark = pytest.mark.gpu
@@ -188,7 +189,8 @@ def test_lmhead_kept_logits_are_the_rounded_product_and_give_the_same_gradients(
     up[torch.rand(n, generator=g) < 0.2] = 0.0
     hd, wd, td, ud = hid.to(DEV), w.to(DEV), tgt.to(DEV), up.to(DEV)
     lp0, lse0, _ = torch.ops.rl_amd.lmhead_logprob_fwd(hd, wd, td, 0, v)
-    lp1, lse1, logits = torch.ops.rl_amd.lmhead_logprob_fwd(hd, wd, td, 0, v, True)
+    lp1, lse1, kept = torch.ops.rl_amd.lmhead_logprob_fwd(hd, wd, td, 0, v, True)
+    logits = ops.lmhead_unpack_kept_logits(kept, n, v)
     assert logits.shape == (n, v) and logits.dtype == torch.bfloat16
     assert bool((lp0 == lp1).all()) and bool((lse0 == lse1).all())
     exact = hid.float() @ w.float().T
@@ -197,7 +199,7 @@ def test_lmhead_kept_logits_are_the_rounded_product_and_give_the_same_gradients(
     # the log-sum-exp of the kept logits is the one the forward reported
     torch.testing.assert_close(torch.logsumexp(logits.float(), -1), lse1, rtol=0, atol=2e-5)
     dh0, dw0 = torch.ops.rl_amd.lmhead_logprob_bwd(hd, wd, td, lse0, ud, 0, v)
-    dh1, dw1 = torch.ops.rl_amd.lmhead_logprob_bwd(hd, wd, td, lse1, ud, 0, v, logits)
+    dh1, dw1 = torch.ops.rl_amd.lmhead_logprob_bwd(hd, wd, td, lse1, ud, 0, v, kept)
     o_dh, o_dw, b_dh, b_dw = narrowing_bounds(hid, w, tgt, up)
     assert bool(((dh1.cpu() - o_dh).abs() <= b_dh).all()) and bool(((dw1.float().cpu() - o_dw).abs() <= b_dw).all())
     assert bool((dh0 == dh1).all()) and bool((dw0 == dw1).all())
