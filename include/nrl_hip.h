@@ -489,9 +489,10 @@ int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* g
  * token block; inside a block [half p = 0, 1][lane = 32 h + token % 32][8 values], the 8 values being the ids
  * 16 p + 8 q + 4 h + e of the block (q = 0, 1; e = 0..3).  Ids and tokens past the end hold unspecified values.
  * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
- * Environment: NRL_LMHEAD_ALIGN (read once per process) -- the forward's workgroups that share an L2 wait for
- * each other before their first tile (unset), before every N-th tile (N > 0), or never (0); the results are
- * the same either way.
+ * Environment (read once per process): NRL_LMHEAD_ALIGN -- the forward's workgroups that share an L2 wait for
+ * each other before their first tile (unset), before every N-th tile (N > 0), or never (0);
+ * NRL_LMHEAD_ALIGN_SPINS -- polls after which a workgroup stops waiting (default 4096; the wait is always
+ * bounded).  The results are the same whatever they say.
  * ------------------------------------------------------------------------------------------ */
 int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab);
 int64_t nrl_lmhead_kept_logits_bytes(int64_t n_tokens, int64_t vocab);

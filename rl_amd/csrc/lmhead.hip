@@ -589,6 +589,7 @@ struct LmFwdArgs {
     int64_t n_vb;              // its vocabulary blocks per token block: ceil(V / 32)
     unsigned int* arrive;      // one zeroed counter per XCD patch of workgroups, or NULL: see patch_cross
     unsigned align_every;      // the patch re-aligns before every align_every-th tile
+    unsigned align_spins;      // polls after which a workgroup stops waiting for its patch
 };
 
 // The 32 workgroups of an XCD patch share their operand panels through that XCD's L2 only while they read the same
@@ -600,12 +601,12 @@ struct LmFwdArgs {
 // patch walks on unaligned, which costs bandwidth, not correctness.
 constexpr unsigned kAlignSpins = 4096;
 constexpr unsigned kAlignOpen = 1u << 24;  // added by a workgroup that gives up: every later target is below it
-__device__ __forceinline__ void patch_cross(unsigned int* ctr, unsigned target) {
+__device__ __forceinline__ void patch_cross(unsigned int* ctr, unsigned target, unsigned max_spins) {
     if (threadIdx.x == 0) {
         __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         unsigned spins = 0;
         while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-            if (++spins > kAlignSpins) {
+            if (++spins > max_spins) {
                 __hip_atomic_fetch_add(ctr, kAlignOpen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 break;
             }
@@ -665,7 +666,7 @@ __global__ __launch_bounds__(GB_THREADS) void lmhead_fwd_kernel(LmFwdArgs a) {
     for (int64_t tile = split; tile < n_tiles; tile += a.n_splits) {
         const int64_t v0 = tile * BV;
         if (arrive && epoch < common) {
-            if (epoch % a.align_every == 0) patch_cross(arrive, members * (epoch / a.align_every + 1));
+            if (epoch % a.align_every == 0) patch_cross(arrive, members * (epoch / a.align_every + 1), a.align_spins);
             ++epoch;
         }
         f32x16 acc[NI][NJ];
@@ -1356,6 +1357,16 @@ static unsigned fwd_align_every() {
     }();
     return n;
 }
+// polls before a workgroup walks on alone: kAlignSpins unless NRL_LMHEAD_ALIGN_SPINS says otherwise (0: at once; how
+// the give-up path is tested)
+static unsigned fwd_align_spins() {
+    static const unsigned n = [] {
+        const char* v = getenv("NRL_LMHEAD_ALIGN_SPINS");
+        const long k = v ? atol(v) : -1;
+        return k < 0 ? kAlignSpins : static_cast<unsigned>(k > (1 << 20) ? (1 << 20) : k);
+    }();
+    return n;
+}
 static bool fwd_align_enabled() {
     static const bool on = [] {
         const char* v = getenv("NRL_LMHEAD_ALIGN");
@@ -1372,6 +1383,7 @@ template <class Core> static void launch_fwd(LmFwdArgs& a, float* ws, hipStream_
     // xt and, right behind it, the patches' arrival counters are cleared together
     a.arrive = fwd_align_enabled() ? reinterpret_cast<unsigned int*>(a.xt + n) : nullptr;
     a.align_every = fwd_align_every();
+    a.align_spins = fwd_align_spins();
     fill_zero_u32<<<dim3(256), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(a.xt), n + (a.arrive ? grid.x / 32 : 0));
     if (a.logits) lmhead_fwd_kernel<Core, true><<<grid, dim3(GB_THREADS), 0, s>>>(a);
     else lmhead_fwd_kernel<Core, false><<<grid, dim3(GB_THREADS), 0, s>>>(a);

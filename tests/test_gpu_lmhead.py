@@ -245,3 +245,60 @@ def test_lmhead_backward_on_confident_tokens(keep):
     dh1, dw1 = _bwd_through_the_op(hid, w[:1].contiguous(), one, up, keep)
     o_dh1, o_dw1, b_dh1, b_dw1 = narrowing_bounds(hid, w[:1], one, up)
     assert bool(((dh1.cpu() - o_dh1).abs() <= b_dh1).all()) and bool(((dw1.float().cpu() - o_dw1).abs() <= b_dw1).all())
+
+
+_ALIGN_SCRIPT = r"""
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+from rl_amd import ops
+g = torch.Generator().manual_seed(5)
+n, h, v = 2600, 128, 9000      # 11 token tiles x several vocabulary splits: whole and partial XCD patches
+hid = torch.randn(n, h, generator=g).to(torch.bfloat16).cuda()
+w = (torch.randn(v, h, generator=g) * 0.05).to(torch.bfloat16).cuda()
+tgt = torch.randint(0, v, (n,), generator=g).cuda()
+out = []
+for keep in (False, True):
+    lp, lse, kept = torch.ops.rl_amd.lmhead_logprob_fwd(hid, w, tgt, 0, v, keep)
+    if keep:
+        kept = ops.lmhead_unpack_kept_logits(kept, n, v)   # (the buffer's padding is not written)
+    out += [lp.cpu(), lse.cpu(), kept.cpu()]
+torch.save(out, sys.argv[2])
+"""
+
+
+def _forward_in_child(tmp_dir, name, extra_env):
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = tmp_dir / "fwd.py"
+    script.write_text(_ALIGN_SCRIPT)
+    child_env = {k: v for k, v in os.environ.items() if not k.startswith("NRL_LMHEAD_ALIGN")}
+    child_env.update(extra_env)
+    out = tmp_dir / f"{name}.pt"
+    done = subprocess.run([sys.executable, str(script), root, str(out)], env=child_env, capture_output=True, text=True,
+                          timeout=240)
+    assert done.returncode == 0, done.stderr[-2000:]
+    return torch.load(out, weights_only=True)
+
+
+@pytest.fixture(scope="module")
+def default_forward(tmp_path_factory):
+    return _forward_in_child(tmp_path_factory.mktemp("lmhead_align"), "default", {})
+
+
+@pytest.mark.parametrize("env", [{"NRL_LMHEAD_ALIGN": "0"}, {"NRL_LMHEAD_ALIGN": "1"}, {"NRL_LMHEAD_ALIGN": "3"},
+                                 {"NRL_LMHEAD_ALIGN_SPINS": "0"}, {"NRL_LMHEAD_ALIGN": "2", "NRL_LMHEAD_ALIGN_SPINS": "1"}])
+def test_lmhead_forward_is_the_same_however_its_workgroups_wait_for_each_other(env, default_forward, tmp_path):
+    """The forward's workgroups that share an L2 wait for each other before their first tile (the default), before every
+    N-th tile, or never (``NRL_LMHEAD_ALIGN``); a workgroup that is not joined within ``NRL_LMHEAD_ALIGN_SPINS`` polls
+    walks on alone (0: every workgroup gives up at once).  None of this touches the arithmetic: logprobs, log-sum-exps
+    and kept logits are bit-identical.  The settings are read once per process, hence the child processes."""
+    variant = _forward_in_child(tmp_path, "variant", env)
+    assert len(variant) == len(default_forward) == 6
+    for a, b in zip(default_forward, variant):
+        assert a.shape == b.shape
+        if a.dtype == torch.bfloat16:
+            a, b = a.view(torch.int16), b.view(torch.int16)
+        assert bool((a == b).all())
