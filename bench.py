@@ -557,7 +557,7 @@ def bench_topk(args, torch, w):
                     lambda inputs: _ModelOutput.apply(m["logits"], anchor), post, mb, global_valid_seqs=tot_seqs,
                     global_valid_toks=tot_toks, sampling_params=params)
             else:
-                # the Megatron worker's sequence (models/megatron/train.py:329-336): the divide on its own, in place
+                # apply_temperature_scaling called on its own, outside the workers' forward functions: in place
                 out = _ModelOutput.apply(m["logits"], anchor)
                 logits = apply_temperature_scaling(out, params)
                 loss_input, data = prepare(logits=logits, data=m["data"], loss_fn=fn)
@@ -648,7 +648,7 @@ def bench_topk(args, torch, w):
         "immediate_warning": row(o_elapsed, ok_, "DEFER_NEG_INF_WARNING = False: mask_out_neg_inf_logprobs waits for its two counts and "
                                                  "prints the warning before it returns, once per microbatch"),
         "in_place_divide": dict(
-            row(e_elapsed, ek, "the divide as the Megatron worker's step makes it: apply_temperature_scaling on its own, one "
+            row(e_elapsed, ek, "apply_temperature_scaling called on its own (outside the workers' forward functions): one "
                                "in-place pass over the logits, and a second pass when autograd sends the gradient back through it"),
             roofline=hbm_roofline("scale_rows_kernel (the eager divide and its backward; also the restoring pass)",
                                   2 * row_bytes * rows, ek.get("scale_rows", nan)["avg_ms"]),

@@ -77,7 +77,8 @@ _PATCHED = {
     "nemo_rl.algorithms.loss": _LOSS_CLASSES + _LOSS_PREPARE + _LOSS_WRAPPERS,
     "nemo_rl.models.automodel.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling",
                                        "forward_with_post_processing_fn"],
-    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling"],
+    "nemo_rl.models.megatron.train": ["LogprobsPostProcessor", "LossPostProcessor", "apply_temperature_scaling",
+                                      "forward_with_post_processing_fn"],
     "nemo_rl.algorithms.grpo": ["compute_and_apply_seq_logprob_error_masking", "dynamic_sampling"],
 }
 

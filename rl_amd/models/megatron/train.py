@@ -1,8 +1,8 @@
-"""``LogprobsPostProcessor`` of the Megatron worker (``nemo_rl/models/megatron/train.py:599-684``) on the
-HIP kernels.
+"""The Megatron worker's post-processors (``nemo_rl/models/megatron/train.py:442-684``) on the HIP kernels, and
+its forward step with the temperature divide left to those kernels (``:220-362``).
 
-The reference class returns a function that the Megatron forward step applies to the model's output
-tensor; that function yields ``(dummy_loss, {"logprobs": [B, S]})``.  Here the plain path is one
+The reference classes return a function that the Megatron forward step applies to the model's output
+tensor.  ``LogprobsPostProcessor``'s yields ``(dummy_loss, {"logprobs": [B, S]})``: here the plain path is one
 forward-only launch that writes the ``[B, S]`` result with its zero column directly, the packed path
 is the packed logprob kernel, and top-k / top-p go through the sampling kernels.  One GPU: the
 tensor- and context-parallel groups of the reference are of size one, so the vocabulary range is
@@ -16,7 +16,7 @@ from typing import Any, Callable, Dict, Optional, Tuple
 import torch
 
 from ... import ops  # noqa: F401  (registers torch.ops.rl_amd)
-from ..._deferred import pending_temperature
+from ..._deferred import drop_record, pending_temperature, record_temperature
 from ..._lib import NRL_TEMP_RCP
 from ...algorithms.logits_sampling_utils import TrainingSamplingParams, need_top_k_or_top_p_filtering
 from ...algorithms.loss.utils import mask_out_neg_inf_logprobs
@@ -144,3 +144,69 @@ class LogprobsPostProcessor:
             return torch.tensor(0.0, device=token_logprobs.device), {"logprobs": token_logprobs}
 
         return processor_fn_inner
+
+
+def _forward_deferring_temperature(post_processing_fn: Any, sampling_params: Any, use_fused_linear_logprobs: bool,
+                                   call: Callable[[], Any]) -> Any:
+    """Runs the install's forward step (``call``) so that its ``apply_temperature_scaling`` -- this package's, through
+    the module global -- records the temperature instead of dividing, and hands the record on to the function the
+    step returns, which Megatron-Core's schedule applies to the output tensor next
+    (``megatron/core/pipeline_parallel/schedules.py``: ``output_tensor, loss_func = forward_step_func(...)`` and then
+    ``loss_func(output_tensor)``).  Only when what follows is a post-processor of this package and the output is
+    logits: with ``use_fused_linear_logprobs`` the model returns logprobs, which the reference divides all the same."""
+    ours = isinstance(post_processing_fn, (LossPostProcessor, LogprobsPostProcessor))
+    if (not ours or sampling_params is None or sampling_params.temperature == 1.0 or use_fused_linear_logprobs):
+        return call()
+    with deferred_temperature():
+        output_tensor, wrapped = call()
+        temperature = 1.0
+        if type(output_tensor) is torch.Tensor and output_tensor.is_cuda:
+            temperature = pending_temperature(output_tensor)
+            drop_record(output_tensor)
+    if temperature == 1.0:  # nothing was put off (the install's step did not scale this output)
+        return output_tensor, wrapped
+
+    def with_the_divide_pending(output: torch.Tensor, *args: Any, **kwargs: Any) -> Any:
+        # Whatever the schedule hands over is the step's output or a copy of it: undivided values either way.
+        with deferred_temperature():
+            record_temperature(output, temperature)
+            return wrapped(output, *args, **kwargs)
+
+    return output_tensor, with_the_divide_pending
+
+
+def forward_with_post_processing_fn(
+    data_iterator: Any,
+    model: Any,
+    post_processing_fn: Any,
+    defer_fp32_logits: Optional[bool] = False,
+    global_valid_seqs: Optional[torch.Tensor] = None,
+    global_valid_toks: Optional[torch.Tensor] = None,
+    sampling_params: Optional[TrainingSamplingParams] = None,
+    straggler_timer: Any = None,
+    draft_model: Any = None,
+    enable_hidden_capture: Optional[bool] = False,
+    use_fused_linear_logprobs: bool = False,
+    use_router_replay: bool = False,
+    router_replay_train: bool = False,
+) -> Tuple[torch.Tensor, Callable]:
+    """``nemo_rl/models/megatron/train.py:220-362`` on a NeMo-RL install: the install's own function does the work
+    (the Megatron-Core model forward, router replay, hidden-state capture); this one only decides where the
+    temperature divide happens.  The reference scales the output in place (``:336``) and autograd later sends the
+    gradient back through that divide, two read + write passes over ``[B, S, V]`` per microbatch; here, when a
+    ``LossPostProcessor`` or ``LogprobsPostProcessor`` of this package consumes the output, the kernels that read
+    the logits anyway apply the divide, with the same rounding of value and gradient.  The output tensor then keeps
+    its undivided values."""
+    from ...compat import original
+
+    theirs = original("nemo_rl.models.megatron.train", "forward_with_post_processing_fn")
+    if theirs is None:
+        raise RuntimeError("forward_with_post_processing_fn of the Megatron worker wraps the function of a NeMo-RL install "
+                           "(it needs Megatron-Core's model forward); rl_amd.install() found none to wrap")
+    return _forward_deferring_temperature(
+        post_processing_fn, sampling_params, use_fused_linear_logprobs,
+        lambda: theirs(data_iterator, model, post_processing_fn, defer_fp32_logits=defer_fp32_logits,
+                       global_valid_seqs=global_valid_seqs, global_valid_toks=global_valid_toks,
+                       sampling_params=sampling_params, straggler_timer=straggler_timer, draft_model=draft_model,
+                       enable_hidden_capture=enable_hidden_capture, use_fused_linear_logprobs=use_fused_linear_logprobs,
+                       use_router_replay=use_router_replay, router_replay_train=router_replay_train))

@@ -239,17 +239,39 @@ _STUB_INSTALL = {
     "nemo_rl/models/megatron/__init__.py": "",
     "nemo_rl/models/megatron/train.py": (
         "from megatron.core.models.gpt import GPTModel\n"
-        "from nemo_rl.algorithms.loss import wrap_loss_fn_with_input_preparation\n"),
+        "from nemo_rl.algorithms.loss import wrap_loss_fn_with_input_preparation\n"
+        "def apply_temperature_scaling(*a, **k):\n    return 'reference'\n"
+        "class LossPostProcessor:\n    origin = 'reference'\n"
+        "class LogprobsPostProcessor:\n    origin = 'reference'\n"
+        "class TopkLogitsPostProcessor:\n    def __call__(self, data_dict):\n        return lambda output: ('topk', output)\n"
+        "def forward_with_post_processing_fn(data_iterator, model, post_processing_fn, sampling_params=None, **k):\n"
+        "    mb = next(data_iterator)\n"
+        "    output = model(mb)\n"
+        "    apply_temperature_scaling(output, sampling_params)\n"
+        "    return output, post_processing_fn(data_dict=mb)\n"
+        "def megatron_forward_backward(model, data_iterator, fn, **k):\n"
+        "    return forward_with_post_processing_fn(data_iterator, model, fn, **k)\n"),
     "driver_script.py": (
         "from nemo_rl.algorithms.loss import ClippedPGLossFn\n"
         "from nemo_rl.algorithms.utils import masked_mean\n"),
 }
 
 
-def write_stub_install(tmp_path) -> str:
+# a stand-in for Megatron-Core, just enough for the stand-in Megatron worker module to import
+_STUB_MEGATRON = {
+    "megatron/__init__.py": "",
+    "megatron/core/__init__.py": "",
+    "megatron/core/models/__init__.py": "",
+    "megatron/core/models/gpt.py": "class GPTModel:\n    pass\n",
+}
+
+
+def write_stub_install(tmp_path, with_megatron: bool = False) -> str:
     """Writes the stand-in install under ``tmp_path`` and returns the ``PYTHONPATH`` a child process needs to
-    import it next to this repository."""
-    for rel, text in _STUB_INSTALL.items():
+    import it next to this repository.  ``with_megatron`` adds a stand-in ``megatron.core``, so that the Megatron
+    worker module of the stand-in imports."""
+    files = dict(_STUB_INSTALL, **(_STUB_MEGATRON if with_megatron else {}))
+    for rel, text in files.items():
         path = tmp_path / rel
         path.parent.mkdir(parents=True, exist_ok=True)
         path.write_text(text)

@@ -262,3 +262,82 @@ def test_a_recycled_address_is_not_divided():
         assert pending_temperature(b) == 1.0
         again = get_next_token_logprobs_from_logits(ids.to(DEV), b)
     assert torch.equal(again, plain) and not torch.equal(divided, plain)
+
+
+@pytest.mark.parametrize("what", ["loss", "logprobs", "fused_linear", "foreign"])
+def test_megatron_forward_step_leaves_the_divide_to_the_kernels(what):
+    """The Megatron worker's forward step scales the model output in place and drops the return value
+    (``nemo_rl/models/megatron/train.py:336``); Megatron-Core's schedule then applies the function the step returned
+    to that output.  Wrapped by this package, the step of an install (a stand-in here: model call, the scaling, the
+    dispatch on the post-processor's type) records the temperature instead, the output keeps its undivided values and
+    the returned function divides inside the kernels: same loss, metrics and logprobs as after the in-place divide,
+    the gradient equal up to its two roundings.  With ``use_fused_linear_logprobs`` (the output holds logprobs, which
+    the reference divides all the same) and for a post-processor that is not this package's the step runs as it is."""
+    from rl_amd.algorithms.loss import ClippedPGLossConfig, ClippedPGLossFn
+    from rl_amd.models.megatron import train as MT
+
+    dtype, vocab, b, s = torch.bfloat16, 4096, 2, 8
+    logits, ids, _ = _inputs(dtype, vocab, 71, b, s)
+    params = TrainingSamplingParams(top_k=None, top_p=1.0, temperature=T)
+    g = torch.Generator().manual_seed(72)
+    base_lp = torch.log_softmax((logits.float() * (1 / T)), -1)[:, :-1].gather(-1, ids[:, 1:, None])[..., 0]
+    data, gs, gt = _loss_data(b, s, base_lp, g)
+    data["input_ids"] = ids
+    ddev = {k: v.to(DEV) for k, v in data.items()}
+    cfg = {"sequence_packing": {"enabled": False}}
+
+    class Foreign:  # stands for the install's TopkLogitsPostProcessor: reads the scaled tensor itself
+        def __call__(self, data_dict, **kwargs):
+            return lambda output: (output.float().sum(), {})
+
+    def post_processor():
+        if what == "loss":
+            return MT.LossPostProcessor(ClippedPGLossFn(ClippedPGLossConfig()), cfg, sampling_params=params)
+        if what == "foreign":
+            return Foreign()
+        return MT.LogprobsPostProcessor(cfg, sampling_params=params, use_fused_linear_logprobs=what == "fused_linear")
+
+    def install_step(data_iterator, model, post_processing_fn, sampling_params=None, global_valid_seqs=None,
+                     global_valid_toks=None, **unused):
+        mb = next(data_iterator)
+        output = model(mb)
+        MT.apply_temperature_scaling(output, sampling_params)  # in place, return value dropped
+        if isinstance(post_processing_fn, MT.LossPostProcessor):
+            return output, post_processing_fn(data_dict=mb, packed_seq_params=None, global_valid_seqs=global_valid_seqs,
+                                              global_valid_toks=global_valid_toks)
+        if isinstance(post_processing_fn, MT.LogprobsPostProcessor):
+            return output, post_processing_fn(data_dict=mb, input_ids=mb["input_ids"], cu_seqlens_padded=None)
+        return output, post_processing_fn(data_dict=mb)
+
+    def run(deferring):
+        leaf = logits.to(DEV).requires_grad_(what == "loss")
+        post = post_processor()
+        step = lambda: install_step(iter([dict(ddev)]), lambda mb: leaf * 1, post, sampling_params=params,  # noqa: E731
+                                    global_valid_seqs=gs.to(DEV), global_valid_toks=gt.to(DEV))
+        if deferring:
+            output, fn = MT._forward_deferring_temperature(post, params, what == "fused_linear", step)
+        else:
+            output, fn = step()
+        raw = output.detach().clone()
+        first, second = fn(output)
+        if what == "loss":
+            first.backward()
+        return raw, first, second, leaf.grad
+
+    raw_e, first_e, second_e, grad_e = run(False)
+    raw_d, first_d, second_d, grad_d = run(True)
+    assert not torch.equal(raw_e, logits.to(DEV))            # the reference's way: the output holds divided values
+    if what in ("loss", "logprobs"):
+        assert torch.equal(raw_d, logits.to(DEV))            # the output kept its undivided values
+    else:
+        assert torch.equal(raw_d, raw_e)                     # nothing was put off
+    if what == "loss":
+        assert abs(first_e.item() - first_d.item()) <= 1e-6 * abs(first_e.item()) + 1e-7
+        for k in second_e:
+            a, c = float(second_e[k]), float(second_d[k])
+            assert abs(a - c) <= 1e-5 * abs(a) + 1e-7, k
+        _check_twice_rounded(grad_d, grad_e.cpu(), dtype)
+    elif what == "foreign":
+        assert torch.equal(first_e, first_d)
+    else:
+        assert torch.equal(second_e["logprobs"], second_d["logprobs"])

@@ -306,6 +306,53 @@ def test_install_rebinds_an_existing_install_by_identity(tmp_path):
     assert not wrong, wrong
 
 
+_STUB_MEGATRON_CHECK = r"""
+import json
+import torch
+import nemo_rl.models.megatron.train as mtrain
+import rl_amd
+from rl_amd import compat
+import rl_amd.models.megatron.train as mine
+
+before = [mtrain.forward_with_post_processing_fn]
+mode = rl_amd.install()
+# a post-processor this package does not replace: the install's own step runs, its scaling included (a GPU is not
+# needed for that: the stand-in's apply_temperature_scaling was replaced, and this package's returns CPU logits
+# untouched only when there is no temperature)
+x = torch.arange(6.0).view(1, 2, 3)
+output, fn = mtrain.megatron_forward_backward(lambda mb: x, iter([{"k": 1}]), mtrain.TopkLogitsPostProcessor(), sampling_params=None)
+out = {
+    "mode": mode,
+    "skipped": compat.skipped_modules(),
+    "forward replaced": mtrain.forward_with_post_processing_fn is mine.forward_with_post_processing_fn,
+    "original kept": compat.original("nemo_rl.models.megatron.train", "forward_with_post_processing_fn") is before[0],
+    "LossPostProcessor": mtrain.LossPostProcessor is mine.LossPostProcessor,
+    "LogprobsPostProcessor": mtrain.LogprobsPostProcessor is mine.LogprobsPostProcessor,
+    "apply_temperature_scaling": mtrain.apply_temperature_scaling is mine.apply_temperature_scaling,
+    "passes through": output is x and fn(output) == ("topk", x),
+}
+print("RESULT " + json.dumps(out))
+"""
+
+
+def test_install_wraps_the_megatron_forward_step(tmp_path):
+    """With Megatron-Core importable the Megatron worker module of an install is patched too: its forward step is
+    wrapped (the original stays reachable for the wrapper), its post-processors and ``apply_temperature_scaling`` are
+    replaced, and a post-processor that stays the install's own runs through the wrapper unchanged."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, PYTHONPATH=write_stub_install(tmp_path, with_megatron=True))
+    done = subprocess.run([sys.executable, "-c", _STUB_MEGATRON_CHECK], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-3000:]
+    got = json.loads([l for l in done.stdout.splitlines() if l.startswith("RESULT ")][-1][len("RESULT "):])
+    assert got.pop("mode") == "patched" and got.pop("skipped") == []
+    wrong = [k for k, v in got.items() if v is not True]
+    assert not wrong, wrong
+
+
 def test_deferred_temperature_record_dies_with_its_storage_and_refuses_copies():
     import numpy as np
 
