@@ -683,7 +683,8 @@ def bench_topk(args, torch, w):
     result["c4_flat"] = {
         "value": flat_rows * args.steps / f_elapsed, "unit": "tokens/s", "ms_per_step": f_elapsed / args.steps * 1e3,
         "rows": flat_rows, "us_per_row": f_ms * 1e3 / flat_rows,
-        "roofline": hbm_roofline("topk_topp_fwd_kernel + topk_topp_wide_kernel (every row wide)", row_bytes * flat_rows, f_ms),
+        "roofline": hbm_roofline("topk_topp_fwd_kernel + topk_topp_wide_kernel (every row wide)", row_bytes * flat_rows, f_ms,
+                                 "c4_flat" if flat_rows == 65536 and w["vocab"] == 151936 else None),
         "note": "forward only: top_p=%.2f alone on bf16 N(0,1) logits; the kept set of every row (~10^5 ids) exceeds the "
                 "4096-entry candidate list, so the forward marks the row and the wide kernel finds threshold, tie index and "
                 "kept log-sum-exp in three more passes over the row (two key digits + the tie search); algorithmic bytes = "
