@@ -430,16 +430,19 @@ __global__ __launch_bounds__(kBlock) void log_softmax_bwd_kernel(const void* __r
 // rows' dtype.  The factor lives on the device so that the host never waits for it; when dst is src and the
 // quotient is exactly 1 every workgroup leaves after reading it and no row is touched.
 template <int DT>
-__global__ __launch_bounds__(kBlock) void scale_rows_kernel(const void* src, void* dst, int64_t n_inner, int64_t vocab,
+__global__ __launch_bounds__(kBlock) void scale_rows_kernel(const void* src, void* dst, int64_t n_rows, int64_t n_inner, int64_t vocab,
                                                             int64_t src_outer, int64_t src_inner, int64_t dst_outer,
                                                             int64_t dst_inner, const float* __restrict__ factor, float divisor) {
     const float f = factor[0] / divisor;
     if (f == 1.f && src == dst) return;
-    const int64_t r = blockIdx.x;
-    const int64_t o = r / n_inner, i = r - o * n_inner;
-    const char* in = static_cast<const char*>(src) + (o * src_outer + i * src_inner) * Row<DT>::BYTES;
-    char* out = static_cast<char*>(dst) + (o * dst_outer + i * dst_inner) * Row<DT>::BYTES;
-    row_apply<DT, false>(in, nullptr, out, vocab, [&](float x, float) { return x * f; });
+    // (a bounded grid walking the rows: the launch that finds nothing to do costs a few microseconds, not one
+    // workgroup per row)
+    for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
+        const int64_t o = r / n_inner, i = r - o * n_inner;
+        const char* in = static_cast<const char*>(src) + (o * src_outer + i * src_inner) * Row<DT>::BYTES;
+        char* out = static_cast<char*>(dst) + (o * dst_outer + i * dst_inner) * Row<DT>::BYTES;
+        row_apply<DT, false>(in, nullptr, out, vocab, [&](float x, float) { return x * f; });
+    }
 }
 
 #define NRL_DISPATCH(DT_, TC_, ...)                                                         \
@@ -632,8 +635,9 @@ extern "C" int nrl_scale_rows(const void* src, void* dst, int32_t dtype, int64_t
     if (!src || !dst || !factor) return fail(NRL_E_INVALID, "null src, dst or factor");
     if (n >= (1ll << 31)) return fail(NRL_E_INVALID, "more than 2^31 rows in one launch");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    NRL_DISPATCH(dtype, 0, (void)TEMP; scale_rows_kernel<DT><<<dim3((unsigned)n), dim3(kBlock), 0, s>>>(
-                                 src, dst, n_inner, vocab, src_stride_outer, src_stride_inner, dst_stride_outer,
+    constexpr int64_t kScaleGrid = 4096;  // 16 workgroups per compute unit; each walks its share of the rows
+    NRL_DISPATCH(dtype, 0, (void)TEMP; scale_rows_kernel<DT><<<dim3((unsigned)(n < kScaleGrid ? n : kScaleGrid)), dim3(kBlock), 0, s>>>(
+                                 src, dst, n, n_inner, vocab, src_stride_outer, src_stride_inner, dst_stride_outer,
                                  dst_stride_inner, factor, divisor));
     return check_launch("scale_rows");
 }
