@@ -557,22 +557,42 @@ __global__ __launch_bounds__(kFusedBlock) void fused_logits_loss_kernel(FusedArg
     }
 }
 
-// one workgroup per sequence: token term records -> the sequence's row of partials
+// one workgroup per sequence: token term records -> the sequence's row of partials.  Thread t sums the records of
+// tokens t, t + 256, ... in that order (the assignment of the three-pass kernel, so both give the same sums); a
+// record is read as ten 8-byte pairs, four records in flight per thread (eight measured slower).
 __global__ __launch_bounds__(kLossBlock) void grpo_terms_reduce_kernel(FusedArgs a) {
     __shared__ double sm_d[kLossWaves];
     __shared__ float sm_f[kLossWaves];
+    static_assert(T_COUNT % 2 == 0, "records are read as 8-byte pairs");
+    constexpr int kPairs = T_COUNT / 2, kAhead = 4;
     const int64_t b = blockIdx.x, n = a.n_inner;
     double acc[P_R_MIN];
 #pragma unroll
     for (int k = 0; k < P_R_MIN; ++k) acc[k] = 0;
     float r_min = INFINITY, r_max = -INFINITY, rc_min = INFINITY, rc_max = -INFINITY;
-    for (int64_t t = threadIdx.x; t < n; t += kLossBlock) {
-        const float* rec = a.terms + (b * n + t) * T_COUNT;
+    for (int64_t t0 = threadIdx.x; t0 < n; t0 += kAhead * kLossBlock) {
+        float2 v[kAhead][kPairs];
 #pragma unroll
-        for (int k = 0; k < P_SAMPLE_MASK; ++k) acc[k] += rec[k];
-        if (rec[T_SELECTED] != 0.f) {
-            r_min = fminf(r_min, rec[T_RATIO]); r_max = fmaxf(r_max, rec[T_RATIO]);
-            rc_min = fminf(rc_min, rec[T_RATIO_CL]); rc_max = fmaxf(rc_max, rec[T_RATIO_CL]);
+        for (int u = 0; u < kAhead; ++u) {
+            const int64_t t = t0 + u * kLossBlock;
+            if (t < n) {
+                const float2* rec = reinterpret_cast<const float2*>(a.terms + (b * n + t) * T_COUNT);  // 8-byte aligned: T_COUNT is even
+#pragma unroll
+                for (int k = 0; k < kPairs; ++k) v[u][k] = rec[k];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            if (t0 + u * kLossBlock >= n) break;
+            float rec[T_COUNT];
+#pragma unroll
+            for (int k = 0; k < kPairs; ++k) { rec[2 * k] = v[u][k].x; rec[2 * k + 1] = v[u][k].y; }
+#pragma unroll
+            for (int k = 0; k < P_SAMPLE_MASK; ++k) acc[k] += rec[k];
+            if (rec[T_SELECTED] != 0.f) {
+                r_min = fminf(r_min, rec[T_RATIO]); r_max = fmaxf(r_max, rec[T_RATIO]);
+                rc_min = fminf(rc_min, rec[T_RATIO_CL]); rc_max = fmaxf(rc_max, rec[T_RATIO_CL]);
+            }
         }
     }
     SeqStats st;
