@@ -491,7 +491,7 @@ int nrl_seq_logprob_error(const float* prev, int64_t prev_stride, const float* g
  * Workspaces: nrl_lmhead_*_workspace_bytes(), 256-byte aligned.
  * Environment (read once per process): NRL_LMHEAD_ALIGN -- the forward's workgroups that share an L2 wait for
  * each other before their first tile (unset), before every N-th tile (N > 0), or never (0);
- * NRL_LMHEAD_ALIGN_SPINS -- polls after which a workgroup stops waiting (default 4096; the wait is always
+ * NRL_LMHEAD_ALIGN_SPINS -- polls after which a workgroup stops waiting (default 512; the wait is always
  * bounded).  The results are the same whatever they say.
  * ------------------------------------------------------------------------------------------ */
 int64_t nrl_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t vocab);

@@ -599,7 +599,9 @@ struct LmFwdArgs {
 // bounded: a workgroup that has not seen the others after
 // kAlignSpins polls (they may not all be resident, e.g. next to another kernel) opens the counter for good, and the
 // patch walks on unaligned, which costs bandwidth, not correctness.
-constexpr unsigned kAlignSpins = 4096;
+// (512 polls, well under a millisecond, align as well as 4096 did -- 58.7 M KiB of fills against 58.6 M; 64 do not:
+// 64.5 M -- and bound what a patch can lose when its workgroups cannot all be resident)
+constexpr unsigned kAlignSpins = 512;
 constexpr unsigned kAlignOpen = 1u << 24;  // added by a workgroup that gives up: every later target is below it
 __device__ __forceinline__ void patch_cross(unsigned int* ctr, unsigned target, unsigned max_spins) {
     if (threadIdx.x == 0) {
