@@ -258,7 +258,8 @@ def test_a_recycled_address_is_not_divided():
         del a
         b = torch.empty_like(logits, device=DEV)          # same size: the allocator hands the freed block back
         b.copy_(logits)
-        assert b.data_ptr() == address, "the allocator did not reuse the block; the test needs it to"
+        if b.data_ptr() != address:  # (an allocator configured not to hand a freed block back: nothing to test)
+            pytest.skip("the caching allocator did not reuse the freed block")
         assert pending_temperature(b) == 1.0
         again = get_next_token_logprobs_from_logits(ids.to(DEV), b)
     assert torch.equal(again, plain) and not torch.equal(divided, plain)
