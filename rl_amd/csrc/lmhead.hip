@@ -1117,21 +1117,33 @@ __global__ __launch_bounds__(256) void lmhead_grad_kept_kernel(LmGradKeptArgs a)
 }
 
 // ---------------------------------------------------------------------------------------------
-// plain GEMM with fp32 output: C = A B^T or C += A B^T
+// plain GEMM with fp32 accumulation: C = A B^T or C += A B^T.  MODE bit 0 (ACCUM): the product is added to what c
+// holds; bit 1 (NARROW): the result goes to cb, bf16 with c's row stride, instead of to c.  The two are not
+// combined: with the prior values in flight next to the narrowing stores the compiler spills accumulators inside the
+// K loop.  A product whose k extent turns out empty on the device still delivers zeros without ACCUM; with ACCUM there
+// is nothing to do.
 // ---------------------------------------------------------------------------------------------
-template <class Core, bool ACCUM>
-__global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, float* c, int64_t ldc, const int32_t* row_map) {
+constexpr int GEMM_ACCUM = 1, GEMM_NARROW = 2;
+template <class Core, int MODE>
+__global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, float* c, int64_t ldc, const int32_t* row_map,
+                                                              uint16_t* cb) {
+    constexpr bool ACCUM = (MODE & GEMM_ACCUM) != 0, NARROW = (MODE & GEMM_NARROW) != 0;
+    static_assert(!(ACCUM && NARROW), "accumulate in fp32, narrow in a pass of its own");
     constexpr int NI = Core::NI, NJ = Core::NJ, BM = Core::BM, BN = Core::BN;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[Core::LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / Core::WAVES_N, wn = wave % Core::WAVES_N;
-    if (!resolve_live(op)) return;
+    const bool runs = resolve_live(op);
+    if (!runs) {
+        // only an empty k extent leaves anything to write, and only where the output is not simply kept as it is
+        if (op.m <= 0 || op.n <= 0 || row_map || ACCUM) return;
+    }
     int64_t bx, by;
     if (!patch_tile(blockIdx.x, (op.m + BM - 1) / BM, (op.n + BN - 1) / BN, bx, by)) return;
     const int64_t row0 = bx * BM, col0 = by * BN;
     f32x16 acc[NI][NJ];
     zero_acc<Core>(acc);
-    Core::tile(op, row0, col0, acc, lds);
+    if (runs) Core::tile(op, row0, col0, acc, lds);
     // (the write-back reads the accumulators with instructions the compiler does not look into: the wait a matrix
     // instruction's result needs before another unit reads it is spelled out)
     asm volatile("s_nop 15\n s_nop 7" ::: "memory");
@@ -1184,13 +1196,17 @@ __global__ __launch_bounds__(GB_THREADS) void gemm_f32_kernel(GemmOperands op, f
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
                     const int64_t col = col0 + wn * (NJ * 32) + j * 32 + (lane & 31);
+                    // (cb has c's row stride: one set of offsets serves the prior values and the narrowed result)
                     float* base = c + (row0 + wm * (NI * 32) + i * 32) * ldc + col;
+                    uint16_t* base_b = cb + (row0 + wm * (NI * 32) + i * 32) * ldc + col;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int r = acc_row(e, lane);
                         const float v = acc_read(acc[i][j][e]);
-                        if (INTERIOR || (row0 + wm * (NI * 32) + i * 32 + r < op.m && col < op.n))
-                            base[r * ldc] = ACCUM ? prior[i - i0][j][e] + v : v;
+                        if (INTERIOR || (row0 + wm * (NI * 32) + i * 32 + r < op.m && col < op.n)) {
+                            if (NARROW) base_b[r * ldc] = static_cast<uint16_t>(f32_to_bf16_bits(ACCUM ? prior[i - i0][j][e] + v : v));
+                            else base[r * ldc] = ACCUM ? prior[i - i0][j][e] + v : v;
+                        }
                     }
                 }
         }
@@ -1397,9 +1413,10 @@ template <class Core> static void launch_grad(const LmGradArgs& a, hipStream_t s
 }
 
 // C = or += A B^T with B in core C's fragment-major layout (op.ldb: its k extent); op.k a multiple of 64
-template <bool ACCUM> static void launch_gemm(const GemmOperands& op, float* c, int64_t ldc, hipStream_t s, const int32_t* row_map = nullptr) {
-    gemm_f32_kernel<CoreC, ACCUM><<<dim3((unsigned)patch_grid((op.m + CoreC::BM - 1) / CoreC::BM, (op.n + CoreC::BN - 1) / CoreC::BN)),
-                                    dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map);
+template <int MODE> static void launch_gemm(const GemmOperands& op, float* c, int64_t ldc, hipStream_t s, const int32_t* row_map = nullptr,
+                                            uint16_t* cb = nullptr) {
+    gemm_f32_kernel<CoreC, MODE><<<dim3((unsigned)patch_grid((op.m + CoreC::BM - 1) / CoreC::BM, (op.n + CoreC::BN - 1) / CoreC::BN)),
+                                   dim3(GB_THREADS), 0, s>>>(op, c, ldc, row_map, cb);
 }
 
 extern "C" int64_t nrl_lmhead_kept_logits_bytes(int64_t n_tokens, int64_t vocab) {
@@ -1493,11 +1510,13 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
     const uint16_t* hid = static_cast<const uint16_t*>(hidden);
     const uint16_t* w = static_cast<const uint16_t*>(weight);
 
-    // W^T [H, vp] (zero-padded, fragment-major: operand B of the dH product) and a zeroed fp32 dW accumulator
+    // W^T [H, vp] (zero-padded, fragment-major: operand B of the dH product)
     transpose_to_frag_kernel<<<dim3((unsigned)(h_pad / 64), (unsigned)(vp / 64)), dim3(256), 0, s>>>(w, vocab, h, ldw, wt, vp, vp);
-    fill_zero_u32<<<dim3(2048), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(dw), vocab * h);
     if (n_tokens == 0) {
-        // (nothing to add to dW)
+        // no token: dW is zero (rows of h bf16 = h / 2 words, row stride ld_dw / 2 words: both are multiples of 8)
+        for (int64_t r = 0; r < vocab; r += 65535)
+            fill_zero_rows_kernel<<<dim3((unsigned)(vocab - r < 65535 ? vocab - r : 65535)), dim3(256), 0, s>>>(
+                reinterpret_cast<float*>(static_cast<uint16_t*>(dweight_out) + r * ld_dw), ld_dw / 2, h / 2);
     } else {
         // Tokens with a zero upstream gradient (prompt tokens, masked samples, each sequence's dropped last position)
         // have a zero row in G: the three products run on the other tokens only.  How many those are stays on the
@@ -1510,6 +1529,10 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
                 dhidden_out + r * ld_dh, ld_dh, h);
     }
 
+    // dW is summed over the chunks in an fp32 buffer and narrowed once at the end.  The first chunk's product starts
+    // the buffer (no zero fill, no read; zeros if the chunk turns out to hold no live token); when there is only one
+    // chunk its product is written as bf16 straight to the output.
+    const bool single = n_tokens <= chunk && ld_dw == h;
     for (int64_t t0 = 0; t0 < n_tokens; t0 += chunk) {
         const int64_t rows = n_tokens - t0 < chunk ? n_tokens - t0 : chunk;   // upper bound: the live rows of this chunk
         const int64_t rows_pad = round_up(rows, 64);
@@ -1531,21 +1554,19 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
         GemmOperands dh;
         dh.a = g; dh.lda = vp; dh.b = wt; dh.ldb = vp; dh.m = rows; dh.n = h; dh.k = vp;
         dh.live = count; dh.live_from = t0; dh.live_dim = 1;
-        launch_gemm<false>(dh, dhidden_out, ld_dh, s, idx + t0);
+        launch_gemm<0>(dh, dhidden_out, ld_dh, s, idx + t0);
         // dW += G^T [V, rows] * (hidden^T [H, rows])^T
         transpose_to_frag_kernel<<<dim3((unsigned)(h_pad / 64), (unsigned)(rows_pad / 64)), dim3(256), 0, s>>>(
             hid_c + t0 * h, rows, h, h, ht, ld_t, rows_pad);
         GemmOperands dwo;
         dwo.a = gt; dwo.lda = ld_t; dwo.b = ht; dwo.ldb = ld_t; dwo.m = vocab; dwo.n = h; dwo.k = rows_pad;
         dwo.live = count; dwo.live_from = t0; dwo.live_dim = 2;
-        launch_gemm<true>(dwo, dw, h, s);
+        // (the narrowing epilogue writes with the accumulator's row stride)
+        if (single) launch_gemm<GEMM_NARROW>(dwo, dw, h, s, nullptr, static_cast<uint16_t*>(dweight_out));
+        else if (t0 == 0) launch_gemm<0>(dwo, dw, h, s);
+        else launch_gemm<GEMM_ACCUM>(dwo, dw, h, s);
     }
-    if (n_tokens > 0)  // the one-hot term of dH in fp32, on the tokens' own rows
-        for (int64_t r = 0; r < n_tokens; r += 65535)
-            lmhead_onehot_dh_kernel<<<dim3((unsigned)(n_tokens - r < 65535 ? n_tokens - r : 65535)), dim3(256), 0, s>>>(
-                dhidden_out + r * ld_dh, ld_dh, grad + r, targets + r, vocab_start, vocab, w, ldw, h);
-    // narrow dW once
-    {
+    if (n_tokens > 0 && !single) {
         uint16_t* out = static_cast<uint16_t*>(dweight_out);
         if (ld_dw == h) {
             f32_to_bf16_kernel<<<dim3(2048), dim3(256), 0, s>>>(dw, out, vocab * h);
@@ -1553,5 +1574,9 @@ extern "C" int nrl_lmhead_logprob_bwd(const void* hidden, int64_t n_tokens, int6
             for (int64_t r = 0; r < vocab; ++r) f32_to_bf16_kernel<<<dim3(4), dim3(256), 0, s>>>(dw + r * h, out + r * ld_dw, h);
         }
     }
+    if (n_tokens > 0)  // the one-hot term of dH in fp32, on the tokens' own rows
+        for (int64_t r = 0; r < n_tokens; r += 65535)
+            lmhead_onehot_dh_kernel<<<dim3((unsigned)(n_tokens - r < 65535 ? n_tokens - r : 65535)), dim3(256), 0, s>>>(
+                dhidden_out + r * ld_dh, ld_dh, grad + r, targets + r, vocab_start, vocab, w, ldw, h);
     return check_launch("lmhead_logprob_bwd");
 }
